@@ -1,0 +1,100 @@
+/* C ABI of the MI355X tree-mask attention / Gated DeltaNet library (libspinf_tree.so).
+ *
+ * Plain pointers and sizes only; every function returns SPINF_OK (0) or a negative SPINF_E_* code and never throws.
+ * spinf_last_error() returns a thread-local message for the last failing call.  Device pointers are HIP device
+ * pointers of the current device; `stream` is a hipStream_t passed as void* (NULL = the default stream).  All
+ * launches are asynchronous on that stream.
+ *
+ * Each entry point names the reference interface (file:line under the reference tree) that it stands in for.
+ */
+#ifndef SPINF_TREE_H
+#define SPINF_TREE_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SPINF_OK 0
+#define SPINF_E_ARG (-1)      /* bad argument (null pointer, unsupported shape, misaligned stride) */
+#define SPINF_E_HIP (-2)      /* a HIP runtime call failed */
+#define SPINF_E_NOMEM (-3)    /* host allocation failed */
+
+#define SPINF_QTILE 128       /* query tokens per tile (the reference's BLOCK, spinf_serve/packer.py:22) */
+#define SPINF_KTILE 64        /* key tokens per tile entry */
+#define SPINF_SUB 32          /* rows / keys of one sub-tile bit */
+
+const char* spinf_last_error(void);
+int spinf_version(void);
+
+/* ------------------------------------------------------------------------------------------------ tile plan
+ * Replaces block_tables() (spinf_serve/packer.py:426-491) and the BlockMask built from it
+ * (spinf_serve/scorer.py:207-238): the stream metadata is compiled into, per 128-token query tile, the ascending list
+ * of 64-key tiles it may see.  No dense mask and no nb x nb table is built.  Host only, deterministic, thread-safe.
+ *
+ *   art, end, pos   [n] int32 host arrays: job slot (-1 pad), exclusive subtree end, depth on the path
+ *   window          sliding window of the layer (pos[q] - pos[k] < window); <= 0 for the global layers
+ *
+ * Entry e of query tile t (qt_ptr[t] <= e < qt_ptr[t+1]) names key tile kv_idx[e]; kv_bits[e] bit (2*w + s) says that
+ * rows 32w..32w+31 of the query tile see at least one key of keys 32s..32s+31 of the key tile, bit 8 + (2*w + s) that
+ * some pair of that 32 x 32 block is masked (the kernel then evaluates spinf_serve/scorer.py:173-177 per element).
+ * order[] lists the query tiles job by job, heaviest first inside a job (a launch order, it does not change results).
+ */
+typedef struct spinf_tileplan spinf_tileplan;
+
+int spinf_tileplan_build(const int32_t* art, const int32_t* end, const int32_t* pos, int64_t n, int32_t window,
+                         spinf_tileplan** out);
+/* counts[0] query tiles, [1] entries, [2] active 32x32 blocks, [3] masked 32x32 blocks, [4] n */
+int spinf_tileplan_counts(const spinf_tileplan* plan, int64_t counts[5]);
+/* qt_ptr [n_qtiles+1], kv_idx [entries], kv_bits [entries], order [n_qtiles]: caller-allocated host arrays */
+int spinf_tileplan_export(const spinf_tileplan* plan, int32_t* qt_ptr, int32_t* kv_idx, uint32_t* kv_bits, int32_t* order);
+void spinf_tileplan_free(spinf_tileplan* plan);
+
+/* ------------------------------------------------------------------------------------------------ attention
+ * Replaces the compiled flex_attention call of tree_flex_forward (spinf_serve/models/gemma4.py:107-118) and of
+ * tree_attention (spinf_serve/models/qwen35/qwen.py:614,620): out = softmax(scale * Q K^T under the tree mask) V with
+ * GQA (query head h reads key/value head h / (hq / hkv)).  bf16 in, fp32 softmax and accumulation, bf16 out.
+ *
+ *   q [n, hq, d], k / v [n, hkv, d], out [n, hq, d]: bf16 device tensors, d contiguous; *_tok / *_head are the token
+ *   and head strides in elements (multiples of 8).  d is 64, 128 or 256.
+ *   art, end, pos, qt_ptr, kv_idx, kv_bits, order: device copies of the metadata and of the exported plan
+ *   window: the window the plan was built with (<= 0 global)
+ */
+typedef struct spinf_attn_args {
+    const void* q; const void* k; const void* v; void* out;
+    int64_t q_tok, q_head, k_tok, k_head, v_tok, v_head, o_tok, o_head;
+    int64_t n; int32_t hq, hkv, d; float scale; int32_t window;
+    const int32_t* art; const int32_t* end; const int32_t* pos;
+    const int32_t* qt_ptr; const int32_t* kv_idx; const uint32_t* kv_bits; const int32_t* order;
+    int64_t n_qtiles;
+    int32_t variant;   /* 0 = default kernel choice; other values select a tuning variant (same results) */
+} spinf_attn_args;
+
+int spinf_tree_attn_fwd(const spinf_attn_args* args, void* stream);
+
+/* ------------------------------------------------------------------------------------------------ Gated DeltaNet
+ * Replaces gdn.recurrent / gdn.chunked (spinf_serve/models/qwen35/gdn.py:197-235 and :109-133): the gated delta rule
+ * over a set of segments; segment s covers call rows cu[s] .. cu[s+1]-1, call row r is stream row idx[r] (idx NULL:
+ * row r itself); it starts from h0[h0_idx[s]] (h0 or h0_idx NULL, or index < 0: zero state) and, where ht_idx[s] >= 0,
+ * leaves its final state in ht[ht_idx[s]].  States are fp32 [*, hv, dk, dv].
+ *
+ *   q, k [rows, h, dk] (l2-normalised), v, o [rows, hv, dv] bf16; g [rows, hv] fp32 log decay; beta [rows, hv] bf16;
+ *   strides in elements (q and k share q_tok, g and beta share g_tok; heads are dense inside a row); dk = dv = 128.
+ *   cu, idx, h0_idx, ht_idx: int64 device arrays.  mode 0 = token by token, 1 = chunk-64 WY form.
+ */
+typedef struct spinf_gdn_args {
+    const void* q; const void* k; const void* v; const float* g; const void* beta; void* o;
+    int64_t q_tok, v_tok, g_tok, o_tok;
+    int32_t h, hv, dk, dv; float scale;
+    const int64_t* cu; const int64_t* idx; int64_t n_seg; int64_t max_len;
+    const float* h0; const int64_t* h0_idx; float* ht; const int64_t* ht_idx;
+    int32_t mode;
+} spinf_gdn_args;
+
+int spinf_gdn_fwd(const spinf_gdn_args* args, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

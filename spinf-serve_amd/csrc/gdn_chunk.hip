@@ -1,0 +1,438 @@
+// Gated DeltaNet, chunk-64 WY form, one fused kernel: stands in for gdn.chunked (spinf_serve/models/qwen35/gdn.py:109-133),
+// i.e. for fla's cumsum -> intra-chunk WY solve -> state recurrence (gdn.py:21-106) -> output pipeline, without writing
+// the per-chunk state snapshots or the w / u / v_new intermediates to memory.
+//
+// One workgroup (4 waves) owns one (segment, value head) and walks its 64-token chunks in order.  The state S [K=128, V=128]
+// lives in fp32 MFMA accumulators (wave w owns key rows 32w..32w+31) and is mirrored once per chunk as bf16 S^T in LDS,
+// where it serves as an MFMA operand.  Per chunk, with G = cumsum(g), D_ij = exp(G_i - G_j):
+//     A   = -strict_tril(beta_i (K K^T)_ij D_ij)         T = (I - A)^-1        (fp32, blocked forward substitution)
+//     U   = T diag(beta) V          W = T diag(beta e^G) K                     (bf16 MFMA, fp32 accumulate)
+//     V'  = U - W S                 O = s e^{G_i} (Q S)_i + tril(s (Q K^T) D) V'
+//     S  <- e^{G_L} S + (K e^{G_L - G})^T V'
+// Every product is computed in the orientation whose result has the token index on the lanes, so results go to LDS or to
+// memory as 8-byte row-major vectors; operands whose contraction index is their row index are read with
+// ds_read_b64_tr_b16.
+#include <hip/hip_runtime.h>
+
+#include "spinf_tree.h"
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(8))) short s16x8;
+
+struct GdnParams {
+    const __bf16* q; const __bf16* k; const __bf16* v; const float* g; const __bf16* beta; __bf16* o;
+    long q_tok, v_tok, g_tok, o_tok;
+    int h, hv, dk, dv; float scale;
+    const long* cu; const long* idx; long n_seg;
+    const float* h0; const long* h0_idx; float* ht; const long* ht_idx;
+};
+
+namespace {
+
+constexpr int C = 64;          // chunk
+constexpr int KD = 128;        // key head dim
+constexpr int VD = 128;        // value head dim
+constexpr int LD = 136;        // row stride (elements) of the [*, 128] bf16 tiles: 272 B, b128 row reads hit 16 distinct bank groups
+constexpr int LT = 72;         // row stride of the [64, 64] bf16 tiles
+constexpr int LA = 68;         // row stride (floats) of the fp32 [64, 64] matrix
+
+// LDS map (bytes)
+constexpr int OFF_K = 0;                         // K   [64][LD] bf16
+constexpr int OFF_Q = OFF_K + C * LD * 2;        // Q   [64][LD]
+constexpr int OFF_V = OFF_Q + C * LD * 2;        // V, later V' [64][LD]
+constexpr int OFF_A = OFF_V + C * LD * 2;        // A / T fp32 [64][LA]; later V' e^{G_L - G} bf16 [64][LD] (same size)
+constexpr int OFF_TU = OFF_A + C * LD * 2;       // T diag(beta)            bf16 [64][LT]
+constexpr int OFF_TW = OFF_TU + C * LT * 2;      // -T diag(beta e^G)       bf16 [64][LT]
+constexpr int OFF_P = OFF_TW + C * LT * 2;       // tril(s Q K^T D)         bf16 [64][LT]
+constexpr int OFF_W = OFF_P + C * LT * 2;        // -W  [64][LD] bf16
+constexpr int OFF_ST = OFF_W + C * LD * 2;       // S^T [128][LD] bf16
+constexpr int OFF_G = OFF_ST + VD * LD * 2;      // G [64] fp32, beta [64] fp32, idx rows [64] int64
+constexpr int OFF_X = OFF_G + 64 * 4 * 2 + 64 * 8;   // scratch fp32 [32][36] for the block merges
+constexpr int LDS_BYTES = OFF_X + 32 * 36 * 4;
+static_assert(C * LA * 4 <= C * LD * 2, "fp32 A must fit the region it shares");
+static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
+
+__device__ __forceinline__ f32x16 zero16() {
+    f32x16 z;
+#pragma unroll
+    for (int i = 0; i < 16; i++) z[i] = 0.f;
+    return z;
+}
+// rows row0 + lane%32, contraction elements k0 + 8 (lane/32) .. +7, from a tile whose contraction index is contiguous
+__device__ __forceinline__ bf16x8 frag_nt(const __bf16* base, int stride, int row0, int k0, int lane) {
+    return *(const bf16x8*)(base + (row0 + (lane & 31)) * stride + k0 + 8 * (lane >> 5));
+}
+// column n0 + lane%32, contraction rows k0 + 8 (lane/32) .. +7, from a tile whose contraction index is its ROW index
+__device__ __forceinline__ bf16x8 frag_tr(const __bf16* base, int stride, int k0, int n0, int lane) {
+    const int tr_a = lane & 3, tr_j = (lane >> 2) & 3, tr_mb = (lane >> 4) & 1, g = lane >> 5;
+    const __bf16* p = base + (k0 + 8 * g + tr_j) * stride + n0 + 16 * tr_mb + 4 * tr_a;
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p);
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(p + 4 * stride));
+    return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+}
+__device__ __forceinline__ f32x16 mfma(bf16x8 a, bf16x8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+
+}  // namespace
+
+__global__ __launch_bounds__(256) void gdn_chunk_kernel(const GdnParams p) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    __bf16* Ks = (__bf16*)(smem + OFF_K);
+    __bf16* Qs = (__bf16*)(smem + OFF_Q);
+    __bf16* Vs = (__bf16*)(smem + OFF_V);
+    float* As = (float*)(smem + OFF_A);
+    __bf16* Vd = (__bf16*)(smem + OFF_A);
+    __bf16* Tu = (__bf16*)(smem + OFF_TU);
+    __bf16* Tw = (__bf16*)(smem + OFF_TW);
+    __bf16* Pm = (__bf16*)(smem + OFF_P);
+    __bf16* Wn = (__bf16*)(smem + OFF_W);
+    __bf16* St = (__bf16*)(smem + OFF_ST);
+    float* Gs = (float*)(smem + OFF_G);
+    float* Bs = Gs + 64;
+    long* Rs = (long*)(Bs + 64);
+    float* Xs = (float*)(smem + OFF_X);
+
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, n32 = lane & 31, g = lane >> 5;
+    const long seg = blockIdx.x / p.hv;
+    const int hv = (int)(blockIdx.x % p.hv);
+    const int hk = hv / (p.hv / p.h);
+    const long bos = p.cu[seg], eos = p.cu[seg + 1];
+    const int T = (int)(eos - bos);
+
+    // ---- state: S[k][v], wave w owns k rows 32w..32w+31; tile vt covers v columns 32vt..; lane = v column, reg r = k row
+    f32x16 S[4];
+#pragma unroll
+    for (int vt = 0; vt < 4; vt++) S[vt] = zero16();
+    long src = -1;
+    if (p.h0 != nullptr && p.h0_idx != nullptr) src = p.h0_idx[seg];
+    if (src >= 0) {
+        const float* hp = p.h0 + (src * p.hv + hv) * (long)KD * VD;
+#pragma unroll
+        for (int vt = 0; vt < 4; vt++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) S[vt][r] = hp[(long)(32 * w + 8 * (r >> 2) + 4 * g + (r & 3)) * VD + 32 * vt + n32];
+    }
+    // S^T mirror (bf16): St[v][k]
+#pragma unroll
+    for (int vt = 0; vt < 4; vt++)
+#pragma unroll
+        for (int r4 = 0; r4 < 4; r4++) {
+            bf16x4 t;
+#pragma unroll
+            for (int j = 0; j < 4; j++) t[j] = (__bf16)S[vt][4 * r4 + j];
+            *(bf16x4*)(St + (32 * vt + n32) * LD + 32 * w + 8 * r4 + 4 * g) = t;
+        }
+
+    for (int c0 = 0; c0 < T; c0 += C) {
+        const int L = min(C, T - c0);
+        __syncthreads();   // previous chunk fully consumed (and St written)
+        // ---- stage the chunk: rows, g, beta, then K / Q / V tiles (rows >= L are zero)
+        if (tid < 64) {
+            long r = -1;
+            float gv = 0.f, bv = 0.f;
+            if (tid < L) {
+                const long t = bos + c0 + tid;
+                r = p.idx ? p.idx[t] : t;
+                gv = p.g[r * p.g_tok + hv];
+                bv = (float)p.beta[r * p.g_tok + hv];
+            }
+            // inclusive prefix sum of g over the wave
+            float x = gv;
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                const float y = __shfl_up(x, d);
+                if (lane >= d) x += y;
+            }
+            Gs[tid] = x;
+            Bs[tid] = bv;
+            Rs[tid] = r;
+        }
+        __syncthreads();
+        {
+            // 64 rows x 16 chunks of 16 bytes per tile, 3 tiles: thread handles row tid/4, chunks 4(tid%4)..+3
+            const int row = tid >> 2, cb = (tid & 3) * 4;
+            const long r = Rs[row];
+#pragma unroll
+            for (int cc = 0; cc < 4; cc++) {
+                const int col = (cb + cc) * 8;
+                bf16x8 kz, qz, vz;
+#pragma unroll
+                for (int j = 0; j < 8; j++) { kz[j] = (__bf16)0.f; qz[j] = (__bf16)0.f; vz[j] = (__bf16)0.f; }
+                if (r >= 0) {
+                    kz = *(const bf16x8*)(p.k + r * p.q_tok + (long)hk * KD + col);
+                    qz = *(const bf16x8*)(p.q + r * p.q_tok + (long)hk * KD + col);
+                    vz = *(const bf16x8*)(p.v + r * p.v_tok + (long)hv * VD + col);
+                }
+                *(bf16x8*)(Ks + row * LD + col) = kz;
+                *(bf16x8*)(Qs + row * LD + col) = qz;
+                *(bf16x8*)(Vs + row * LD + col) = vz;
+            }
+        }
+        __syncthreads();
+        const float GL = Gs[63];
+
+        // ---- (a) A = -strict_tril(beta_i K_i.K_j D_ij) fp32, (b) P = tril(s Q_i.K_j D_ij) bf16; computed transposed so that
+        // a lane holds row i and 4 consecutive columns j per register group.  Wave w: tile (jt = w>>1, it = w&1).
+        {
+            const int jt = w >> 1, it = w & 1;
+            f32x16 kk = zero16(), qk = zero16();
+#pragma unroll
+            for (int s = 0; s < KD / 16; s++) {
+                const bf16x8 a = frag_nt(Ks, LD, 32 * jt, 16 * s, lane);    // rows j
+                kk = mfma(a, frag_nt(Ks, LD, 32 * it, 16 * s, lane), kk);   // cols i
+                qk = mfma(a, frag_nt(Qs, LD, 32 * it, 16 * s, lane), qk);
+            }
+            const int i = 32 * it + n32;
+            const float Gi = Gs[i], bi = Bs[i];
+#pragma unroll
+            for (int r4 = 0; r4 < 4; r4++) {
+                const int j0 = 32 * jt + 8 * r4 + 4 * g;
+                float4 av;
+                bf16x4 pv;
+                float avv[4];
+#pragma unroll
+                for (int jj = 0; jj < 4; jj++) {
+                    const int j = j0 + jj;
+                    const float d = __expf(Gi - Gs[j]);
+                    avv[jj] = j < i ? -bi * kk[4 * r4 + jj] * d : 0.f;
+                    pv[jj] = (__bf16)(j <= i ? p.scale * qk[4 * r4 + jj] * d : 0.f);
+                }
+                av = make_float4(avv[0], avv[1], avv[2], avv[3]);
+                *(float4*)(As + i * LA + j0) = av;
+                *(bf16x4*)(Pm + i * LT + j0) = pv;
+            }
+        }
+        __syncthreads();
+
+        // ---- T = (I - A)^-1 in place (fp32).  Stage 1: the four 16x16 diagonal blocks by forward substitution, wave b =
+        // block b, lane c < 16 = column c of the block.
+        if (lane < 16) {
+            float t[16];
+            const float* Ab = As + (16 * w) * LA + 16 * w;
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                float acc = (i == lane) ? 1.f : 0.f;
+#pragma unroll
+                for (int j = 0; j < i; j++) acc = __builtin_fmaf(Ab[i * LA + j], t[j], acc);
+                t[i] = acc;
+            }
+            __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): all reads of A done before the block is overwritten
+#pragma unroll
+            for (int i = 0; i < 16; i++) As[(16 * w + i) * LA + 16 * w + lane] = t[i];
+        }
+        __syncthreads();
+        // Stage 2: 32x32 diagonal blocks: T_lo = T_bb A_lo T_aa for (a, b) = (0,1) and (2,3).  256 threads = 2 blocks x 16 x 8;
+        // thread: block q, row i, columns 2c..2c+1
+        {
+            const int qb = tid >> 7, i = (tid >> 3) & 15, c2 = (tid & 7) * 2;
+            const int ra = 32 * qb, rb = ra + 16;
+            float x0 = 0.f, x1 = 0.f;
+#pragma unroll
+            for (int j = 0; j < 16; j++) {            // X = A_lo T_aa
+                const float a = As[(rb + i) * LA + ra + j];
+                x0 = __builtin_fmaf(a, As[(ra + j) * LA + ra + c2], x0);
+                x1 = __builtin_fmaf(a, As[(ra + j) * LA + ra + c2 + 1], x1);
+            }
+            Xs[(16 * qb + i) * 36 + c2] = x0;
+            Xs[(16 * qb + i) * 36 + c2 + 1] = x1;
+            __syncthreads();
+            float y0 = 0.f, y1 = 0.f;
+#pragma unroll
+            for (int j = 0; j < 16; j++) {            // T_lo = T_bb X
+                const float tb = As[(rb + i) * LA + rb + j];
+                y0 = __builtin_fmaf(tb, Xs[(16 * qb + j) * 36 + c2], y0);
+                y1 = __builtin_fmaf(tb, Xs[(16 * qb + j) * 36 + c2 + 1], y1);
+            }
+            As[(rb + i) * LA + ra + c2] = y0;
+            As[(rb + i) * LA + ra + c2 + 1] = y1;
+        }
+        __syncthreads();
+        // Stage 3: the 64x64 matrix: T_lo = T_11 A_lo T_00 with 32x32 blocks.  thread: row i (32), columns 4c..4c+3 (8 groups)
+        {
+            const int i = tid >> 3, c4 = (tid & 7) * 4;
+            float x[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 8
+            for (int j = 0; j < 32; j++) {
+                const float a = As[(32 + i) * LA + j];
+                const float4 t = *(const float4*)(As + j * LA + c4);
+                x[0] = __builtin_fmaf(a, t.x, x[0]); x[1] = __builtin_fmaf(a, t.y, x[1]);
+                x[2] = __builtin_fmaf(a, t.z, x[2]); x[3] = __builtin_fmaf(a, t.w, x[3]);
+            }
+            *(float4*)(Xs + i * 36 + c4) = make_float4(x[0], x[1], x[2], x[3]);
+            __syncthreads();
+            float y[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 8
+            for (int j = 0; j < 32; j++) {
+                const float tb = As[(32 + i) * LA + 32 + j];
+                const float4 t = *(const float4*)(Xs + j * 36 + c4);
+                y[0] = __builtin_fmaf(tb, t.x, y[0]); y[1] = __builtin_fmaf(tb, t.y, y[1]);
+                y[2] = __builtin_fmaf(tb, t.z, y[2]); y[3] = __builtin_fmaf(tb, t.w, y[3]);
+            }
+            __syncthreads();   // every read of the A_lo block is done
+            *(float4*)(As + (32 + i) * LA + c4) = make_float4(y[0], y[1], y[2], y[3]);
+        }
+        __syncthreads();
+        // ---- Tu = T diag(beta), Tw = -T diag(beta e^G) (bf16).  thread: row tid/4, 16 columns
+        {
+            const int i = tid >> 2, jb = (tid & 3) * 16;
+#pragma unroll
+            for (int j4 = 0; j4 < 4; j4++) {
+                const float4 t = *(const float4*)(As + i * LA + jb + 4 * j4);
+                const float tv[4] = {t.x, t.y, t.z, t.w};
+                bf16x4 u, ww;
+#pragma unroll
+                for (int jj = 0; jj < 4; jj++) {
+                    const int j = jb + 4 * j4 + jj;
+                    const float tb = tv[jj] * Bs[j];
+                    u[jj] = (__bf16)tb;
+                    ww[jj] = (__bf16)(-tb * __expf(Gs[j]));
+                }
+                *(bf16x4*)(Tu + i * LT + jb + 4 * j4) = u;
+                *(bf16x4*)(Tw + i * LT + jb + 4 * j4) = ww;
+            }
+        }
+        __syncthreads();
+
+        // ---- (c) U^T[v][i] = sum_j V[j][v] Tu[i][j]  and  -W^T[d][i] = sum_j K[j][d] Tw[i][j]; wave w: rows 32w.. of v / d
+        f32x16 acc[2];      // U^T, later V'^T : tile it = token columns 32 it..
+        {
+            f32x16 wn[2];
+            acc[0] = zero16(); acc[1] = zero16(); wn[0] = zero16(); wn[1] = zero16();
+#pragma unroll
+            for (int s = 0; s < C / 16; s++) {
+                const bf16x8 av = frag_tr(Vs, LD, 16 * s, 32 * w, lane);
+                const bf16x8 ak = frag_tr(Ks, LD, 16 * s, 32 * w, lane);
+#pragma unroll
+                for (int it = 0; it < 2; it++) {
+                    acc[it] = mfma(av, frag_nt(Tu, LT, 32 * it, 16 * s, lane), acc[it]);
+                    wn[it] = mfma(ak, frag_nt(Tw, LT, 32 * it, 16 * s, lane), wn[it]);
+                }
+            }
+#pragma unroll
+            for (int it = 0; it < 2; it++)
+#pragma unroll
+                for (int r4 = 0; r4 < 4; r4++) {
+                    bf16x4 t;
+#pragma unroll
+                    for (int j = 0; j < 4; j++) t[j] = (__bf16)wn[it][4 * r4 + j];
+                    *(bf16x4*)(Wn + (32 * it + n32) * LD + 32 * w + 8 * r4 + 4 * g) = t;
+                }
+        }
+        __syncthreads();   // -W visible; V (Vs) and T (As) are dead from here
+
+        // ---- (d) V'^T = U^T + S^T (-W)^T   and   (e1) QS^T[v][i] = sum_k S^T[v][k] Q[i][k]
+        f32x16 qs[2];
+        qs[0] = zero16(); qs[1] = zero16();
+#pragma unroll
+        for (int s = 0; s < KD / 16; s++) {
+            const bf16x8 a = frag_nt(St, LD, 32 * w, 16 * s, lane);
+#pragma unroll
+            for (int it = 0; it < 2; it++) {
+                acc[it] = mfma(a, frag_nt(Wn, LD, 32 * it, 16 * s, lane), acc[it]);
+                qs[it] = mfma(a, frag_nt(Qs, LD, 32 * it, 16 * s, lane), qs[it]);
+            }
+        }
+        // V' and V' e^{G_L - G_i}, row-major [i][v], bf16
+#pragma unroll
+        for (int it = 0; it < 2; it++) {
+            const int i = 32 * it + n32;
+            const float dec = __expf(GL - Gs[i]);
+#pragma unroll
+            for (int r4 = 0; r4 < 4; r4++) {
+                bf16x4 t, td;
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    t[j] = (__bf16)acc[it][4 * r4 + j];
+                    td[j] = (__bf16)(acc[it][4 * r4 + j] * dec);
+                }
+                *(bf16x4*)(Vs + i * LD + 32 * w + 8 * r4 + 4 * g) = t;
+                *(bf16x4*)(Vd + i * LD + 32 * w + 8 * r4 + 4 * g) = td;
+            }
+        }
+        __syncthreads();
+
+        // ---- (e2) O^T[v][i] = s e^{G_i} QS^T + sum_j V'[j][v] P[i][j]
+        {
+            f32x16 ov[2];
+            ov[0] = zero16(); ov[1] = zero16();
+#pragma unroll
+            for (int s = 0; s < C / 16; s++) {
+                const bf16x8 a = frag_tr(Vs, LD, 16 * s, 32 * w, lane);
+#pragma unroll
+                for (int it = 0; it < 2; it++) ov[it] = mfma(a, frag_nt(Pm, LT, 32 * it, 16 * s, lane), ov[it]);
+            }
+#pragma unroll
+            for (int it = 0; it < 2; it++) {
+                const int i = 32 * it + n32;
+                if (i < L) {
+                    const float sc = p.scale * __expf(Gs[i]);
+                    __bf16* op = p.o + Rs[i] * p.o_tok + (long)hv * VD + 32 * w + 4 * g;
+#pragma unroll
+                    for (int r4 = 0; r4 < 4; r4++) {
+                        bf16x4 t;
+#pragma unroll
+                        for (int j = 0; j < 4; j++) t[j] = (__bf16)(__builtin_fmaf(sc, qs[it][4 * r4 + j], ov[it][4 * r4 + j]));
+                        *(bf16x4*)(op + 8 * r4) = t;
+                    }
+                }
+            }
+        }
+
+        // ---- (f) S[k][v] = e^{G_L} S[k][v] + sum_j K[j][k] (V' e^{G_L - G_j})[j][v]; wave w: k rows 32w.., all four v tiles
+        {
+            const float eg = __expf(GL);
+#pragma unroll
+            for (int vt = 0; vt < 4; vt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) S[vt][r] *= eg;
+#pragma unroll
+            for (int s = 0; s < C / 16; s++) {
+                const bf16x8 a = frag_tr(Ks, LD, 16 * s, 32 * w, lane);
+#pragma unroll
+                for (int vt = 0; vt < 4; vt++) S[vt] = mfma(a, frag_tr(Vd, LD, 16 * s, 32 * vt, lane), S[vt]);
+            }
+        }
+        __syncthreads();   // every wave is done reading S^T (d, e1) before it is replaced
+#pragma unroll
+        for (int vt = 0; vt < 4; vt++)
+#pragma unroll
+            for (int r4 = 0; r4 < 4; r4++) {
+                bf16x4 t;
+#pragma unroll
+                for (int j = 0; j < 4; j++) t[j] = (__bf16)S[vt][4 * r4 + j];
+                *(bf16x4*)(St + (32 * vt + n32) * LD + 32 * w + 8 * r4 + 4 * g) = t;
+            }
+    }
+
+    if (p.ht != nullptr && p.ht_idx != nullptr) {
+        const long dst = p.ht_idx[seg];
+        if (dst >= 0) {
+            float* hp = p.ht + (dst * p.hv + hv) * (long)KD * VD;
+#pragma unroll
+            for (int vt = 0; vt < 4; vt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) hp[(long)(32 * w + 8 * (r >> 2) + 4 * g + (r & 3)) * VD + 32 * vt + n32] = S[vt][r];
+        }
+    }
+}
+
+int gdn_chunked_launch(const GdnParams& p, long max_len, hipStream_t stream) {
+    (void)max_len;
+    if (p.dv != VD) return spinf_fail(SPINF_E_ARG, "gdn chunked: value head dim %d, only 128 is built", p.dv);
+    if (p.v_tok % 8 || p.o_tok % 4) return spinf_fail(SPINF_E_ARG, "gdn chunked: v row stride must be a multiple of 8, o of 4 elements");
+    static bool configured = false;
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute((const void*)gdn_chunk_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+        if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "gdn chunked: hipFuncSetAttribute: %s", hipGetErrorString(e));
+        configured = true;
+    }
+    const long blocks = p.n_seg * p.hv;
+    if (blocks > INT32_MAX) return spinf_fail(SPINF_E_ARG, "gdn chunked: too many segments");
+    hipLaunchKernelGGL(gdn_chunk_kernel, dim3((unsigned)blocks), dim3(256), LDS_BYTES, stream, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "gdn chunked: launch: %s", hipGetErrorString(e));
+    return SPINF_OK;
+}

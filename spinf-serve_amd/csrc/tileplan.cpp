@@ -1,0 +1,179 @@
+// Tile-plan compiler: stream metadata -> per-query-tile list of visible key tiles with 32x32 activity / mask bits.
+// Stands in for block_tables (spinf_serve/packer.py:426-491); the visibility predicate is the one of
+// spinf_serve/scorer.py:173-177.  Host code, no global state.
+#include "spinf_tree.h"
+#include "common.h"
+
+#include <algorithm>
+#include <cstring>
+#include <new>
+#include <unordered_map>
+#include <vector>
+
+struct spinf_tileplan {
+    int64_t n = 0;
+    int32_t window = 0;
+    std::vector<int32_t> qt_ptr, kv_idx, order;
+    std::vector<uint32_t> kv_bits;
+    int64_t active = 0, masked = 0;
+};
+
+namespace {
+
+struct Blk {            // aggregates of one 32-token block
+    int32_t lo, hi;     // token range [lo, hi)
+    bool all_real;      // every token is a real token
+    int32_t job;        // the single job of its tokens, -2 if mixed / pads present
+    int32_t min_end, max_end;   // over all tokens (pads count as -1)
+    int64_t min_pos, max_pos;   // over real tokens
+    bool any_real;
+};
+
+inline bool visible(const int32_t* art, const int32_t* end, const int32_t* pos, int32_t window, int64_t q, int64_t k) {
+    if (q == k) return true;
+    bool v = k <= q && art[q] >= 0 && art[k] == art[q] && q < (int64_t)end[k];
+    if (v && window > 0) v = ((int64_t)pos[q] - (int64_t)pos[k]) < (int64_t)window;
+    return v;
+}
+
+}  // namespace
+
+extern "C" int spinf_tileplan_build(const int32_t* art, const int32_t* end, const int32_t* pos, int64_t n, int32_t window,
+                                    spinf_tileplan** out) {
+    if (!out) return spinf_fail(SPINF_E_ARG, "tileplan_build: out is null");
+    *out = nullptr;
+    if (n < 0 || (n > 0 && (!art || !end || !pos))) return spinf_fail(SPINF_E_ARG, "tileplan_build: null metadata");
+    if (n > (int64_t)1 << 30) return spinf_fail(SPINF_E_ARG, "tileplan_build: stream too long");
+    spinf_tileplan* p = new (std::nothrow) spinf_tileplan;
+    if (!p) return spinf_fail(SPINF_E_NOMEM, "tileplan_build: out of memory");
+    try {
+        p->n = n;
+        p->window = window > 0 ? window : 0;
+        const int32_t W = p->window;
+        const int64_t nqt = (n + SPINF_QTILE - 1) / SPINF_QTILE;
+        const int64_t nb = (n + SPINF_SUB - 1) / SPINF_SUB;
+        std::vector<Blk> blk(nb);
+        for (int64_t b = 0; b < nb; b++) {
+            Blk& B = blk[b];
+            B.lo = (int32_t)(b * SPINF_SUB);
+            B.hi = (int32_t)std::min<int64_t>(n, (b + 1) * SPINF_SUB);
+            B.all_real = true; B.any_real = false; B.job = -3;
+            B.min_end = INT32_MAX; B.max_end = INT32_MIN; B.min_pos = INT64_MAX; B.max_pos = INT64_MIN;
+            for (int32_t i = B.lo; i < B.hi; i++) {
+                const bool real = art[i] >= 0;
+                B.all_real &= real;
+                B.min_end = std::min(B.min_end, end[i]);
+                B.max_end = std::max(B.max_end, end[i]);
+                if (real) {
+                    B.any_real = true;
+                    B.min_pos = std::min<int64_t>(B.min_pos, pos[i]);
+                    B.max_pos = std::max<int64_t>(B.max_pos, pos[i]);
+                    if (B.job == -3) B.job = art[i]; else if (B.job != art[i]) B.job = -2;
+                } else {
+                    B.job = -2;
+                }
+            }
+            if (B.job == -3) B.job = -2;
+        }
+        // first stream position of every job: the lowest key any of its rows may see
+        std::unordered_map<int32_t, int64_t> first;
+        std::vector<int64_t> jfirst(n);
+        for (int64_t i = 0; i < n; i++) {
+            if (art[i] < 0) { jfirst[i] = i; continue; }
+            auto it = first.find(art[i]);
+            if (it == first.end()) it = first.emplace(art[i], i).first;
+            jfirst[i] = it->second;
+        }
+        p->qt_ptr.assign(nqt + 1, 0);
+        std::vector<int64_t> weight(nqt, 0);
+        std::vector<int32_t> group(nqt, -1);
+        for (int64_t t = 0; t < nqt; t++) {
+            const int64_t q0 = t * SPINF_QTILE, q1 = std::min<int64_t>(n, q0 + SPINF_QTILE);
+            int64_t lo_key = q0;
+            for (int64_t q = q0; q < q1; q++) {
+                lo_key = std::min(lo_key, jfirst[q]);
+                if (group[t] < 0 && art[q] >= 0) group[t] = art[q];
+            }
+            for (int64_t j = lo_key / SPINF_KTILE; j * SPINF_KTILE < q1; j++) {
+                uint32_t bits = 0;
+                for (int w = 0; w < SPINF_QTILE / SPINF_SUB; w++) {
+                    const int64_t rb = q0 / SPINF_SUB + w;
+                    if (rb >= nb) break;
+                    const Blk& R = blk[rb];
+                    for (int s = 0; s < SPINF_KTILE / SPINF_SUB; s++) {
+                        const int64_t kb = j * (SPINF_KTILE / SPINF_SUB) + s;
+                        if (kb >= nb) break;
+                        const Blk& K = blk[kb];
+                        if (K.lo > R.hi - 1) continue;                       // every key after every row
+                        const bool below = K.hi - 1 < R.lo;                  // every key strictly before every row
+                        bool any, all;
+                        if (below && K.max_end <= R.lo) { any = false; all = false; }
+                        else if (below && W > 0 && R.any_real && K.any_real && R.min_pos - K.max_pos >= W) { any = false; all = false; }
+                        else if (K.hi - 1 <= R.lo && R.all_real && K.all_real && R.job >= 0 && R.job == K.job && K.min_end >= R.hi &&
+                                 (W == 0 || R.max_pos - K.min_pos < W) && (R.hi - R.lo) == SPINF_SUB && (K.hi - K.lo) == SPINF_SUB) {
+                            any = true; all = true;
+                        } else {
+                            any = false; all = (R.hi - R.lo) == SPINF_SUB && (K.hi - K.lo) == SPINF_SUB;
+                            for (int64_t q = R.lo; q < R.hi; q++)
+                                for (int64_t k = K.lo; k < K.hi; k++) {
+                                    const bool v = visible(art, end, pos, W, q, k);
+                                    any |= v; all &= v;
+                                }
+                        }
+                        if (any) {
+                            bits |= 1u << (2 * w + s);
+                            p->active++;
+                            if (!all) { bits |= 1u << (8 + 2 * w + s); p->masked++; }
+                        }
+                    }
+                }
+                if (bits) {
+                    p->kv_idx.push_back((int32_t)j);
+                    p->kv_bits.push_back(bits);
+                    weight[t] += __builtin_popcount(bits & 0xffu);
+                }
+            }
+            p->qt_ptr[t + 1] = (int32_t)p->kv_idx.size();
+        }
+        // launch order: runs of query tiles of one job stay together (they share keys), heaviest first inside a run
+        p->order.resize(nqt);
+        for (int64_t t = 0; t < nqt; t++) p->order[t] = (int32_t)t;
+        int64_t a = 0;
+        while (a < nqt) {
+            int64_t b = a + 1;
+            while (b < nqt && group[b] == group[a]) b++;
+            std::stable_sort(p->order.begin() + a, p->order.begin() + b, [&](int32_t x, int32_t y) { return weight[x] > weight[y]; });
+            a = b;
+        }
+    } catch (const std::bad_alloc&) {
+        delete p;
+        return spinf_fail(SPINF_E_NOMEM, "tileplan_build: out of memory");
+    }
+    *out = p;
+    return SPINF_OK;
+}
+
+extern "C" int spinf_tileplan_counts(const spinf_tileplan* p, int64_t counts[5]) {
+    if (!p || !counts) return spinf_fail(SPINF_E_ARG, "tileplan_counts: null argument");
+    counts[0] = (int64_t)p->order.size();
+    counts[1] = (int64_t)p->kv_idx.size();
+    counts[2] = p->active;
+    counts[3] = p->masked;
+    counts[4] = p->n;
+    return SPINF_OK;
+}
+
+extern "C" int spinf_tileplan_export(const spinf_tileplan* p, int32_t* qt_ptr, int32_t* kv_idx, uint32_t* kv_bits, int32_t* order) {
+    if (!p || !qt_ptr) return spinf_fail(SPINF_E_ARG, "tileplan_export: null argument");
+    if ((!kv_idx || !kv_bits) && !p->kv_idx.empty()) return spinf_fail(SPINF_E_ARG, "tileplan_export: null entry arrays");
+    if (!order && !p->order.empty()) return spinf_fail(SPINF_E_ARG, "tileplan_export: null order array");
+    std::memcpy(qt_ptr, p->qt_ptr.data(), p->qt_ptr.size() * sizeof(int32_t));
+    if (!p->kv_idx.empty()) {
+        std::memcpy(kv_idx, p->kv_idx.data(), p->kv_idx.size() * sizeof(int32_t));
+        std::memcpy(kv_bits, p->kv_bits.data(), p->kv_bits.size() * sizeof(uint32_t));
+    }
+    if (!p->order.empty()) std::memcpy(order, p->order.data(), p->order.size() * sizeof(int32_t));
+    return SPINF_OK;
+}
+
+extern "C" void spinf_tileplan_free(spinf_tileplan* p) { delete p; }

@@ -1,0 +1,19 @@
+"""MI355X-native tree-mask packed-prefill attention and Gated DeltaNet scan behind the reference's call boundary.
+
+  packer      Tree / GroupedTree / Packer / Batch: the stream metadata producer (spinf_serve/packer.py)
+  masks       TreeMask, block_masks: the mask side of the boundary (spinf_serve/scorer.py:163-238)
+  attention   tree_attn custom op, tree_flex_forward, tree_attention (gemma4.py:98-119, qwen.py:604-623)
+  gdn         recurrent, chunked (spinf_serve/models/qwen35/gdn.py)
+  qwen_plan   tree_plan, gdn_tree (spinf_serve/models/qwen35/qwen.py:158-276, 514-590)
+  synth       seeded synthetic workloads of the benchmark configurations
+
+All device work goes through libspinf_tree.so (HIP, gfx950); there is no CPU or PyTorch fallback: importing the
+compute entry points without the built library raises.
+"""
+
+from ._lib import load_library, library_path  # noqa: F401
+from .packer import BLOCK, Batch, GroupedTree, Owner, Packer, ReadPlan, Tree, build_grouped_tree, build_tree, split_grouped_trees, split_trees, trie_branches  # noqa: F401
+from .masks import TreeMask, TilePlan, block_masks  # noqa: F401
+from .attention import CAPTURE, register_tree_attention, tree_attention, tree_attn, tree_flex_forward  # noqa: F401
+from .gdn import chunked, recurrent  # noqa: F401
+from .qwen_plan import Call, TreePlan, gdn_tree, tree_plan  # noqa: F401

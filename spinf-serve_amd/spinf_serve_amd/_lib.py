@@ -1,0 +1,71 @@
+"""ctypes binding of libspinf_tree.so (the C ABI declared in include/spinf_tree.h)."""
+
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = None
+
+SYMBOLS = (
+    "spinf_last_error", "spinf_version", "spinf_tileplan_build", "spinf_tileplan_counts", "spinf_tileplan_export",
+    "spinf_tileplan_free", "spinf_tree_attn_fwd", "spinf_gdn_fwd",
+)
+
+
+class AttnArgs(C.Structure):
+    _fields_ = [
+        ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("out", C.c_void_p),
+        ("q_tok", C.c_int64), ("q_head", C.c_int64), ("k_tok", C.c_int64), ("k_head", C.c_int64),
+        ("v_tok", C.c_int64), ("v_head", C.c_int64), ("o_tok", C.c_int64), ("o_head", C.c_int64),
+        ("n", C.c_int64), ("hq", C.c_int32), ("hkv", C.c_int32), ("d", C.c_int32), ("scale", C.c_float), ("window", C.c_int32),
+        ("art", C.c_void_p), ("end", C.c_void_p), ("pos", C.c_void_p),
+        ("qt_ptr", C.c_void_p), ("kv_idx", C.c_void_p), ("kv_bits", C.c_void_p), ("order", C.c_void_p),
+        ("n_qtiles", C.c_int64), ("variant", C.c_int32),
+    ]
+
+
+class GdnArgs(C.Structure):
+    _fields_ = [
+        ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("g", C.c_void_p), ("beta", C.c_void_p), ("o", C.c_void_p),
+        ("q_tok", C.c_int64), ("v_tok", C.c_int64), ("g_tok", C.c_int64), ("o_tok", C.c_int64),
+        ("h", C.c_int32), ("hv", C.c_int32), ("dk", C.c_int32), ("dv", C.c_int32), ("scale", C.c_float),
+        ("cu", C.c_void_p), ("idx", C.c_void_p), ("n_seg", C.c_int64), ("max_len", C.c_int64),
+        ("h0", C.c_void_p), ("h0_idx", C.c_void_p), ("ht", C.c_void_p), ("ht_idx", C.c_void_p),
+        ("mode", C.c_int32),
+    ]
+
+
+def library_path() -> str:
+    return os.environ.get("SPINF_TREE_LIB", os.path.join(_HERE, "libspinf_tree.so"))
+
+
+def load_library():
+    """-> the loaded library; raises RuntimeError when it has not been built (python __graft_entry__.py)."""
+    global _LIB
+    if _LIB is not None:
+        return _LIB
+    path = library_path()
+    if not os.path.exists(path):
+        raise RuntimeError(f"{path} is missing: build the HIP library first (python __graft_entry__.py); there is no fallback path")
+    lib = C.CDLL(path)
+    lib.spinf_last_error.restype = C.c_char_p
+    lib.spinf_version.restype = C.c_int
+    lib.spinf_tileplan_build.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.POINTER(C.c_void_p)]
+    lib.spinf_tileplan_counts.argtypes = [C.c_void_p, C.POINTER(C.c_int64)]
+    lib.spinf_tileplan_export.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
+    lib.spinf_tileplan_free.argtypes = [C.c_void_p]
+    lib.spinf_tileplan_free.restype = None
+    lib.spinf_tree_attn_fwd.argtypes = [C.POINTER(AttnArgs), C.c_void_p]
+    lib.spinf_gdn_fwd.argtypes = [C.POINTER(GdnArgs), C.c_void_p]
+    for name in ("spinf_tileplan_build", "spinf_tileplan_counts", "spinf_tileplan_export", "spinf_tree_attn_fwd", "spinf_gdn_fwd"):
+        getattr(lib, name).restype = C.c_int
+    _LIB = lib
+    return lib
+
+
+def check(code: int, what: str) -> None:
+    if code != 0:
+        msg = load_library().spinf_last_error().decode()
+        raise (ValueError if code == -1 else RuntimeError)(f"{what}: {msg} (code {code})")

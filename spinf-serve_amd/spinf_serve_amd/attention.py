@@ -1,0 +1,127 @@
+"""The attention op of the packed forward, with the reference's two call signatures.
+
+  tree_attn(q, k, v, mask, scale)                     the custom op spinf::tree_attn on token-major tensors
+  tree_flex_forward(module, query, key, value, ...)   transformers AttentionInterface callable "tree_flex"
+                                                      (spinf_serve/models/gemma4.py:98-119)
+  tree_attention(q, k, v, mask, scale, sidx, ...)     the Qwen stack's function (spinf_serve/models/qwen35/qwen.py:604-623)
+
+The op is a thin wrapper over spinf_tree_attn_fwd of libspinf_tree.so; it runs on ROCm tensors only.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+
+import torch
+
+from . import _lib
+from .masks import TreeMask
+
+VARIANT = 0  # kernel tuning variant handed to the library (0 = its default choice); results do not depend on it
+
+
+@torch.library.custom_op("spinf::tree_attn", mutates_args=())
+def _tree_attn_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, art: torch.Tensor, end: torch.Tensor, pos: torch.Tensor,
+                  qt_ptr: torch.Tensor, kv_idx: torch.Tensor, kv_bits: torch.Tensor, order: torch.Tensor,
+                  scale: float, window: int, variant: int) -> torch.Tensor:
+    """q [n, hq, d], k / v [n, hkv, d] (any token / head strides, d contiguous) -> out [n, hq, d] contiguous, bf16."""
+    if not q.is_cuda:
+        raise RuntimeError("spinf::tree_attn runs on ROCm device tensors only (no CPU path)")
+    if q.dtype != torch.bfloat16 or k.dtype != torch.bfloat16 or v.dtype != torch.bfloat16:
+        raise ValueError("spinf::tree_attn takes bf16 q, k, v")
+    n, hq, d = q.shape
+    hkv = k.shape[1]
+    if k.shape != (n, hkv, d) or v.shape != (n, hkv, d):
+        raise ValueError(f"k / v shapes {tuple(k.shape)} {tuple(v.shape)} do not match q {tuple(q.shape)}")
+    if q.stride(2) != 1 or k.stride(2) != 1 or v.stride(2) != 1:
+        raise ValueError("the head dimension must be contiguous")
+    if art.numel() < n:
+        raise ValueError(f"mask built for {art.numel()} tokens, stream has {n}")
+    out = torch.empty((n, hq, d), dtype=torch.bfloat16, device=q.device)
+    a = _lib.AttnArgs()
+    a.q, a.k, a.v, a.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
+    a.q_tok, a.q_head = q.stride(0), q.stride(1)
+    a.k_tok, a.k_head = k.stride(0), k.stride(1)
+    a.v_tok, a.v_head = v.stride(0), v.stride(1)
+    a.o_tok, a.o_head = out.stride(0), out.stride(1)
+    a.n, a.hq, a.hkv, a.d, a.scale, a.window = n, hq, hkv, d, scale, window
+    a.art, a.end, a.pos = art.data_ptr(), end.data_ptr(), pos.data_ptr()
+    a.qt_ptr, a.kv_idx, a.kv_bits, a.order = qt_ptr.data_ptr(), kv_idx.data_ptr(), kv_bits.data_ptr(), order.data_ptr()
+    a.n_qtiles = qt_ptr.numel() - 1
+    a.variant = variant
+    lib = _lib.load_library()
+    with torch.cuda.device(q.device):
+        stream = torch.cuda.current_stream(q.device).cuda_stream
+        _lib.check(lib.spinf_tree_attn_fwd(C.byref(a), C.c_void_p(stream)), "spinf_tree_attn_fwd")
+    return out
+
+
+@_tree_attn_op.register_fake
+def _(q, k, v, art, end, pos, qt_ptr, kv_idx, kv_bits, order, scale, window, variant):
+    return torch.empty(q.shape, dtype=torch.bfloat16, device=q.device)
+
+
+def tree_attn(q, k, v, mask: TreeMask, scale=None, variant=None):
+    """q [n, hq, d], k / v [n, hkv, d] bf16 -> [n, hq, d]: softmax(scale q k^T under the tree mask) v."""
+    if not isinstance(mask, TreeMask):
+        raise TypeError("attention_mask must be a TreeMask (masks.block_masks)")
+    if q.shape[0] != mask.n:
+        raise ValueError(f"mask describes {mask.n} tokens, q has {q.shape[0]}")
+    scale = float(q.shape[-1] ** -0.5 if scale is None else scale)
+    return _tree_attn_op(q, k, v, mask.art, mask.end, mask.pos, mask.qt_ptr, mask.kv_idx, mask.kv_bits, mask.order,
+                         scale, int(mask.window), int(VARIANT if variant is None else variant))
+
+
+# K/V capture for extraction, as spinf_serve/models/gemma4.py:66-70: while CAPTURE[device] = {"window", "ranges": [(start, n, key)],
+# "kv": {}} is set, every call keeps the layer's keys / values of the ranges (sliding layers only their last window - 1)
+CAPTURE: dict = {}
+
+
+@torch.compiler.disable
+def tree_flex_forward(module, query, key, value, attention_mask, scaling=None, sliding_window=None, **kw):
+    """transformers attention interface: query [1, Hq, N, D], key / value [1, Hkv, N, D] (views of token-major tensors),
+    attention_mask a TreeMask -> (attn_output [1, N, Hq, D] contiguous, None)   (spinf_serve/models/gemma4.py:98-119)"""
+    cap = CAPTURE.get(query.device)
+    if cap is not None:
+        keep = cap["window"] - 1
+        sliding = module.config.layer_types[module.layer_idx] == "sliding_attention"
+        for start, n, name in cap["ranges"]:
+            a = start + (max(0, n - keep) if sliding else 0)
+            cap["kv"].setdefault(name, {})[module.layer_idx] = (key[:, :, a : start + n].clone(), value[:, :, a : start + n].clone())
+    if query.shape[0] != 1:
+        raise ValueError("the packed stream is one sequence: batch size must be 1")
+    out = tree_attn(query[0].transpose(0, 1), key[0].transpose(0, 1), value[0].transpose(0, 1), attention_mask, scaling)
+    return out[None], None
+
+
+def register_tree_attention(name: str = "tree_flex") -> None:
+    """registers tree_flex_forward with transformers, as spinf_serve/models/gemma4.py:121-122 does"""
+    from transformers import AttentionInterface
+
+    if name not in AttentionInterface._global_mapping:
+        AttentionInterface.register(name, tree_flex_forward)
+
+
+@torch.compiler.disable
+def tree_attention(q, k, v, mask, scale, sidx=None, plan=None, mod=None):
+    """q [1, H, rows, d], k / v [1, Hkv, rows, d] -> [1, H, rows, d]   (spinf_serve/models/qwen35/qwen.py:604-623).
+    sidx (compact rows): stream position of each real row; rows are scattered into the stream layout the mask describes
+    (pads: zero rows attending to themselves) and the output gathered back."""
+    cap = plan.cap if plan is not None else None
+    if cap is not None:
+        for r0, n, name in cap["ranges"]:
+            cap["out"]["kv"].setdefault(name, {})[mod.li] = (k[:, :, r0 : r0 + n].clone(), v[:, :, r0 : r0 + n].clone())
+    if sidx is None:
+        o = tree_attn(q[0].transpose(0, 1), k[0].transpose(0, 1), v[0].transpose(0, 1), mask, scale)
+        return o.transpose(0, 1)[None]
+    T, R = mask.seq_lengths[0], sidx.shape[0]
+
+    def up(t):  # [1, h, rows, d] -> token-major stream layout [T, h, d]
+        s = t.new_zeros(T, t.shape[1], t.shape[3])
+        s.index_copy_(0, sidx, t[0, :, :R].transpose(0, 1))
+        return s
+
+    o = tree_attn(up(q), up(k), up(v), mask, scale)
+    out = q.new_zeros(q.shape)
+    out[0, :, :R] = o.index_select(0, sidx).transpose(0, 1)
+    return out

@@ -1,0 +1,187 @@
+"""GPU parity of the tree-mask attention kernel (through the C ABI) against the CPU oracle.
+
+Bars: max abs error <= 2e-2 for the bf16 kernel against the float64 oracle on the same seeded bf16 inputs; bit-exact
+per-content output alone vs packed vs reversed pack order (the reference's protocol, docs/BATCH_INVARIANCE.md:71-72)."""
+
+import numpy as np
+import pytest
+import torch
+
+import spinf_serve_amd as sa
+from oracle import attention as oattn
+from spinf_serve_amd import synth
+from spinf_serve_amd.packer import GroupedTree
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-2
+
+
+def _oracle(q, k, v, b, scale, window=None):
+    return oattn.tree_attention(q.float().cpu().numpy(), k.float().cpu().numpy(), v.float().cpu().numpy(), b.art, b.end, b.pos,
+                                window=window, scale=scale, spans=oattn.job_spans(b.art))
+
+
+def _pads_selfattend(out, v, b, g):
+    pad = np.flatnonzero(b.art < 0)
+    if len(pad):
+        want = v[pad].repeat_interleave(g, dim=1)
+        assert torch.equal(out[pad], want), "a pad row attends to itself only: its output is its own V row"
+
+
+def _check(cfg, b, dev, window=None, seed=0, variant=None):
+    q, k, v = synth.qkv(cfg, b, seed=seed, device=dev)
+    mask = sa.TreeMask.build(b.art, b.end, b.pos, window=window, device=dev)
+    print(f"case {cfg.name} n={b.length} hq={cfg.hq} hkv={cfg.hkv} d={cfg.d} window={window} variant={variant}", flush=True)
+    out = sa.tree_attn(q, k, v, mask, cfg.scale, variant=variant)
+    torch.cuda.synchronize()
+    ref = _oracle(q, k, v, b, cfg.scale, window)
+    err = float(np.abs(out.float().cpu().numpy() - ref).max())
+    assert np.isfinite(out.float().cpu().numpy()).all()
+    assert err <= TOL, err
+    _pads_selfattend(out, v, b, cfg.hq // cfg.hkv)
+    return out, err
+
+
+@pytest.mark.parametrize("name", ["C1", "smoke"])
+def test_small_configs(dev, name):
+    cfg = synth.attention_config(name)
+    _check(cfg, cfg.batches[0], dev)
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2])
+def test_c2_shape_three_contents(dev, variant):
+    cfg = synth.attention_config("C2", contents=3)
+    _check(cfg, cfg.batches[0], dev, variant=variant)
+
+
+def test_c4_shape_two_level_tree(dev):
+    rng = np.random.default_rng(5)
+    lens, parents = [], []
+    for _ in range(4):
+        node = len(lens)
+        lens.append(32); parents.append(-1)
+        for _ in range(5):
+            lens.append(int(rng.integers(6, 11))); parents.append(node)
+    trees = [synth._tree(rng, 700, lens, parents), synth._tree(rng, 130, lens[:7], parents[:7])]
+    cfg = synth.AttnConfig("C4-small", 32, 16, 128, 128 ** -0.5, 0.5, None, trees)
+    cfg.batches = synth.pack(trees)
+    _check(cfg, cfg.batches[0], dev)
+
+
+@pytest.mark.parametrize("window", [64, 200, 1024])
+def test_sliding_window(dev, window):
+    rng = np.random.default_rng(11)
+    trees = [synth._tree(rng, 1500, rng.integers(4, 25, 12)), synth._tree(rng, 90, [7, 9])]
+    cfg = synth.AttnConfig("C3-small", 16, 8, 256, 1.0 / 16, 0.5, window, trees)
+    cfg.batches = synth.pack(trees)
+    _check(cfg, cfg.batches[0], dev, window=window)
+
+
+def test_odd_group_and_mha(dev):
+    rng = np.random.default_rng(2)
+    trees = [synth._tree(rng, 200, [9, 17, 4])]
+    for hq, hkv in ((6, 2), (4, 4), (3, 1)):
+        cfg = synth.AttnConfig("odd", hq, hkv, 128, 128 ** -0.5, 1.0, None, trees)
+        cfg.batches = synth.pack(trees)
+        _check(cfg, cfg.batches[0], dev)
+
+
+def test_unaligned_packing_and_ragged_length(dev):
+    """jobs packed densely (align off) share tiles; the stream length need not be a multiple of the tile"""
+    rng = np.random.default_rng(3)
+    trees = [synth._tree(rng, 100, [5, 6]), synth._tree(rng, 37, [3]), synth._tree(rng, 260, [11] * 6)]
+    cfg = synth.AttnConfig("dense", 4, 2, 64, 0.125, 1.0, None, trees)
+    b = synth.pack(trees, align=False)[0]
+    _check(cfg, b, dev)
+    # ragged: cut the stream after the last real token
+    n = int(np.flatnonzero(b.art >= 0)[-1]) + 1
+    q, k, v = synth.qkv(cfg, b, device=dev)
+    mask = sa.TreeMask.build(b.art[:n], b.end[:n], b.pos[:n], device=dev)
+    out = sa.tree_attn(q[:n], k[:n], v[:n], mask, cfg.scale)
+    ref = oattn.tree_attention(q[:n].float().cpu().numpy(), k[:n].float().cpu().numpy(), v[:n].float().cpu().numpy(), b.art[:n], b.end[:n], scale=cfg.scale)
+    assert np.abs(out.float().cpu().numpy() - ref).max() <= TOL
+
+
+def test_aligned_query_groups_leave_gaps(dev):
+    """a branch group that starts on a block boundary leaves pads inside the job (spinf_serve/packer.py:390-391)"""
+    rng = np.random.default_rng(4)
+    t = GroupedTree(rng.integers(5, 99, 300).tolist(), [rng.integers(5, 99, n).tolist() for n in (9, 12, 7, 30)], [], [], parents=[-1, -1, -1, -1], aligned=[2])
+    cfg = synth.AttnConfig("gaps", 8, 4, 128, 128 ** -0.5, 1.0, None, [t])
+    b = synth.pack([t])[0]
+    assert (b.art[300:] == -1).any()
+    _check(cfg, b, dev)
+
+
+def test_batch_invariance_bit_exact(dev):
+    """each content's rows are bit-identical alone, packed with the others, and packed in reverse order"""
+    cfg = synth.attention_config("C2", contents=4)
+    trees = cfg.trees
+    rng = np.random.default_rng(0)
+    qs = [torch.from_numpy(rng.standard_normal((t.n_tokens, cfg.hq, cfg.d)).astype(np.float32) * 0.5).to(torch.bfloat16) for t in trees]
+    ks = [torch.from_numpy(rng.standard_normal((t.n_tokens, cfg.hkv, cfg.d)).astype(np.float32) * 0.5).to(torch.bfloat16) for t in trees]
+    vs = [torch.from_numpy(rng.standard_normal((t.n_tokens, cfg.hkv, cfg.d)).astype(np.float32) * 0.5).to(torch.bfloat16) for t in trees]
+
+    def run(order, window=None):
+        b = synth.pack([trees[i] for i in order])[0]
+        n = b.length
+        q = torch.zeros((n, cfg.hq, cfg.d), dtype=torch.bfloat16)
+        k = torch.zeros((n, cfg.hkv, cfg.d), dtype=torch.bfloat16)
+        v = torch.zeros((n, cfg.hkv, cfg.d), dtype=torch.bfloat16)
+        for slot, i in enumerate(order):
+            s0 = b.owners[slot].start
+            q[s0 : s0 + trees[i].n_tokens] = qs[i]
+            k[s0 : s0 + trees[i].n_tokens] = ks[i]
+            v[s0 : s0 + trees[i].n_tokens] = vs[i]
+        mask = sa.TreeMask.build(b.art, b.end, b.pos, window=window, device=dev)
+        out = sa.tree_attn(q.to(dev), k.to(dev), v.to(dev), mask, cfg.scale).cpu()
+        return {i: out[b.owners[slot].start : b.owners[slot].start + trees[i].n_tokens] for slot, i in enumerate(order)}
+
+    for window in (None, 256):
+        packed = run([0, 1, 2, 3], window)
+        rev = run([3, 2, 1, 0], window)
+        for i in range(4):
+            alone = run([i], window)[i]
+            assert torch.equal(alone, packed[i]), (i, window)
+            assert torch.equal(alone, rev[i]), (i, window)
+
+
+def test_reference_call_signatures(dev):
+    """tree_flex_forward (gemma4.py:98-119) and tree_attention (qwen.py:604-623) give the op's result in their layouts"""
+    cfg = synth.attention_config("smoke")
+    b = cfg.batches[0]
+    q, k, v = synth.qkv(cfg, b, device=dev)
+    masks = sa.block_masks(b, sliding_window=None, device=dev)
+    base = sa.tree_attn(q, k, v, masks["full_attention"], cfg.scale)
+    out, none = sa.tree_flex_forward(None, q.transpose(0, 1)[None], k.transpose(0, 1)[None], v.transpose(0, 1)[None], masks["full_attention"], scaling=cfg.scale)
+    assert none is None and out.shape == (1, b.length, cfg.hq, cfg.d) and out.is_contiguous()
+    assert torch.equal(out[0], base)
+    o2 = sa.tree_attention(q.transpose(0, 1)[None], k.transpose(0, 1)[None], v.transpose(0, 1)[None], masks["full_attention"], cfg.scale)
+    assert o2.shape == (1, cfg.hq, b.length, cfg.d) and torch.equal(o2[0].transpose(0, 1), base)
+    # compact rows: real rows first, then zero rows
+    real = np.flatnonzero(b.art >= 0)
+    sidx = torch.from_numpy(real).to(dev)
+    rows = (len(real) + 127) // 128 * 128
+
+    def compact(t):
+        c = t.new_zeros(rows, t.shape[1], t.shape[2])
+        c[: len(real)] = t[sidx]
+        return c.transpose(0, 1)[None]
+
+    o3 = sa.tree_attention(compact(q), compact(k), compact(v), masks["full_attention"], cfg.scale, sidx=sidx)
+    assert torch.equal(o3[0, :, : len(real)].transpose(0, 1), base[sidx])
+    assert (o3[0, :, len(real):] == 0).all()
+
+
+def test_argument_errors(dev):
+    cfg = synth.attention_config("smoke")
+    b = cfg.batches[0]
+    q, k, v = synth.qkv(cfg, b, device=dev)
+    mask = sa.TreeMask.build(b.art, b.end, b.pos, device=dev)
+    with pytest.raises(ValueError):
+        sa.tree_attn(q[:, :3], k, v, mask, cfg.scale)            # 3 query heads over 2 kv heads
+    with pytest.raises(ValueError):
+        sa.tree_attn(q[:100], k[:100], v[:100], mask, cfg.scale)  # mask of another length
+    with pytest.raises(ValueError):
+        sa.tree_attn(q.float(), k, v, mask, cfg.scale)
+    with pytest.raises(RuntimeError):
+        sa.tree_attn(q.cpu(), k.cpu(), v.cpu(), mask, cfg.scale)  # no CPU path
