@@ -1,0 +1,154 @@
+"""Benchmark of the tree-mask packed-prefill attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C2|C3|C4|C5] [--seed S] [--no-cpu]
+
+A step is one pass of the attention op (one layer's call through the C ABI) over one packed synthetic stream already
+resident in HBM; the tile plan is compiled once per stream, outside the timed region, as the reference builds its block
+masks once per forward for all layers.  Prints ONE JSON line: packed query tokens/s, the useful-FLOP roofline fraction of
+the kernel (events on the launch stream around every step) and the CPU baseline (dense-mask attention on the host cores).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "spinf-serve_amd")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA (published)
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E (published)
+
+WORKLOADS = {
+    "C2": "C2: 24 contents x (470-token trunk + 56 branches of U{8..16} tokens) in one varlen pass, 16 query / 8 KV heads, head_dim 256, scale 1/16, Q/K/V ~ 0.5 N(0,1), global layer",
+    "C3": "C3: 512 contents, trunk lognormal(median 800, sigma 0.6) clipped 64..4096, U{8..64} branches of U{4..24}, passes <= 65,536 tokens, 16/8 heads, head_dim 256, one sliding (W=1024) + one global layer per pass",
+    "C4": "C4: contents x (8192-token trunk + 16 nodes x 32 + 192 leaves of U{6..10}), 32/16 heads, head_dim 128, one varlen pass",
+    "C5": "C5: Gated DeltaNet, contents x (2048-token trunk + 32 branches x 12), 16 qk / 32 v heads, 128 x 128 fp32 state, chunk 64",
+}
+
+
+def timed(fn, steps, warmup, torch):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for a, b in ev:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    kern = [a.elapsed_time(b) for a, b in ev]
+    return wall, kern
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="C2", choices=sorted(WORKLOADS))
+    ap.add_argument("--contents", type=int, default=None, help="override the number of contents (C4 / C5 memory)")
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--variant", type=int, default=0)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU's throughput; contents shard across GPUs with no exchange, run one process per GPU (--gpus 1)")
+
+    import numpy as np
+    import torch
+
+    import spinf_serve_amd as sa
+    from spinf_serve_amd import synth
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible (the attention op has no CPU path)")
+    sa.load_library()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    line = {"metric": "packed query tokens/s + % bf16 MFMA peak (useful FLOPs), tree-mask attn", "unit": "tokens/s", "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "data": "synthetic (seeded, numpy default_rng / torch generator)", "seed": args.seed}
+
+    if args.workload == "C5":
+        cfg = synth.gdn_config("C5", seed=args.seed, contents=args.contents)
+        t = synth.gdn_inputs(cfg, seed=args.seed, device=dev)
+        plan = cfg.plan(dev)
+
+        def step():
+            return sa.gdn_tree(t["q"], t["k"], t["v"], t["g"], t["beta"], plan)
+
+        wall, kern = timed(step, args.steps, args.warmup, torch)
+        ms = float(np.mean(kern))
+        gbs = cfg.bytes() / (ms * 1e-3) / 1e9
+        line.update(metric="packed tokens/s, Gated DeltaNet tree scan", value=cfg.n_real * args.steps / wall, ms_per_step=1e3 * wall / args.steps,
+                    dtype="bf16 (fp32 state)", config={"workload": WORKLOADS["C5"], "contents": len(cfg.trees), "tokens": cfg.n_real},
+                    roofline={"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS, "traffic": None,
+                              "kernel_ms": ms, "algorithmic_bytes": cfg.bytes()})
+        if not args.no_cpu:
+            from oracle import cpu_baseline
+
+            tps, n, dt, _ = cpu_baseline.gdn_tokens_per_s(*(t[x].cpu() for x in ("q", "k", "v", "g", "beta")), cfg.batch.prev, cfg.batch.art >= 0)
+            line["cpu_baseline"] = {"value": tps, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+                                    "sample": f"fp32 token-by-token recurrence on the first {n} real tokens of the stream ({dt:.1f} s)"}
+        print(json.dumps(line))
+        return
+
+    cfg = synth.attention_config(args.workload, seed=args.seed, contents=args.contents)
+    layers = [None] if cfg.window is None else [cfg.window, None]   # C3 alternates sliding and global layers
+    t0 = time.perf_counter()
+    work = []
+    for b in cfg.batches:
+        masks = sa.block_masks(b, sliding_window=cfg.window, device=dev)
+        work.append((synth.qkv(cfg, b, seed=args.seed, device=dev), masks))
+    torch.cuda.synchronize()
+    setup_s = time.perf_counter() - t0
+    tp0 = time.perf_counter()
+    for b in cfg.batches:
+        sa.TilePlan.build(b.art, b.end, b.pos, None)
+    plan_ms = 1e3 * (time.perf_counter() - tp0)
+
+    def step():
+        out = None
+        for (q, k, v), masks in work:
+            for w in layers:
+                out = sa.tree_attn(q, k, v, masks["sliding_attention" if w else "full_attention"], cfg.scale, variant=args.variant)
+        return out
+
+    wall, kern = timed(step, args.steps, args.warmup, torch)
+    ms = float(np.mean(kern))
+    flops = sum(cfg.flops(w) for w in layers)
+    tokens = cfg.n_real * len(layers)
+    tfl = flops / (ms * 1e-3) / 1e12
+    line.update(value=tokens * args.steps / wall, ms_per_step=1e3 * wall / args.steps, dtype="bf16",
+                config={"workload": WORKLOADS[args.workload], "contents": len(cfg.trees), "packed_tokens": cfg.n_real,
+                        "stream_tokens": sum(b.length for b in cfg.batches), "passes": len(cfg.batches), "layers_per_step": len(layers),
+                        "visible_pairs": [cfg.pairs(w) for w in layers], "variant": args.variant},
+                roofline={"bound": "mfma", "achieved": tfl, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": tfl / PEAK_BF16_TFLOPS,
+                          "traffic": None, "kernel_ms": ms, "kernel_ms_min": float(np.min(kern)), "useful_flops": flops,
+                          "algorithmic_bytes": cfg.bytes() * len(layers), "hbm_frac_at_algorithmic_bytes": cfg.bytes() * len(layers) / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS},
+                plan_build_ms_host=plan_ms, setup_s=setup_s)
+    if not args.no_cpu:
+        from oracle import cpu_baseline
+
+        (q, k, v), _ = work[0]
+        b = cfg.batches[0]
+        w = layers[0]
+        tps, done, done_tok, dt, outs = cpu_baseline.attention_tokens_per_s(q.cpu(), k.cpu(), v.cpu(), b.art, b.end, b.pos, cfg.scale, window=w)
+        gpu = sa.tree_attn(q, k, v, work[0][1]["sliding_attention" if w else "full_attention"], cfg.scale).float().cpu()
+        err = max(float((gpu[a:bb] - o).abs().max()) for (a, bb), o in outs.items())
+        line["cpu_baseline"] = {"value": tps, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+                                "sample": f"{done} of {len(cfg.trees) if len(cfg.batches) == 1 else 'the first pass'} contents ({done_tok} packed tokens), fp32 torch scaled_dot_product_attention with an explicit dense tree mask per content, {dt:.1f} s; os.cpu_count()={os.cpu_count()}",
+                                "max_abs_err_gpu_vs_cpu_fp32": err}
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
