@@ -1,0 +1,321 @@
+"""Host side of the path (no GPU): the packer mirror, the tile-plan compiler (C ABI, host code), the recurrent-layer planner,
+and that the shared library loads and exports every symbol include/spinf_tree.h declares."""
+
+import ctypes
+import gzip
+import json
+import os
+import re
+
+import numpy as np
+import pytest
+
+import spinf_serve_amd as sa
+from oracle import mask as omask
+from oracle import plan as oplan
+from oracle.layout import Job, pack_stream
+from spinf_serve_amd import synth
+from spinf_serve_amd.packer import BLOCK, GroupedTree, Packer, ReadPlan, build_grouped_tree, build_tree, split_trees, trie_branches
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+
+
+@pytest.fixture(scope="module")
+def golden():
+    with gzip.open(os.path.join(HERE, "golden", "packer_golden.json.gz"), "rt") as f:
+        return json.load(f)
+
+
+# ------------------------------------------------------------------------------------------------ C ABI
+def test_library_exports_every_declared_symbol(lib):
+    header = open(os.path.join(ROOT, "include", "spinf_tree.h")).read()
+    declared = set(re.findall(r"\b(spinf_[a-z0-9_]+)\s*\(", header))
+    assert {"spinf_tileplan_build", "spinf_tree_attn_fwd", "spinf_gdn_fwd", "spinf_last_error"} <= declared
+    raw = ctypes.CDLL(sa.library_path())
+    for name in declared:
+        assert hasattr(raw, name), name
+    assert lib.spinf_version() >= 1
+
+
+def test_c_abi_rejects_bad_arguments(lib):
+    out = ctypes.c_void_p()
+    assert lib.spinf_tileplan_build(None, None, None, 5, 0, ctypes.byref(out)) == -1
+    assert b"null" in lib.spinf_last_error()
+    assert lib.spinf_tileplan_build(None, None, None, 0, 0, None) == -1
+    assert lib.spinf_tree_attn_fwd(None, None) == -1 and lib.spinf_gdn_fwd(None, None) == -1
+    # an empty stream is a valid (empty) plan
+    assert lib.spinf_tileplan_build(None, None, None, 0, 0, ctypes.byref(out)) == 0
+    counts = (ctypes.c_int64 * 5)()
+    assert lib.spinf_tileplan_counts(out, counts) == 0 and list(counts) == [0, 0, 0, 0, 0]
+    lib.spinf_tileplan_free(out)
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    from spinf_serve_amd import _lib
+
+    monkeypatch.setattr(_lib, "_LIB", None)
+    monkeypatch.setenv("SPINF_TREE_LIB", "/nonexistent/libspinf_tree.so")
+    with pytest.raises(RuntimeError, match="no fallback"):
+        _lib.load_library()
+
+
+def test_ops_have_no_cpu_path(lib):
+    import torch
+
+    cfg = synth.attention_config("C1")
+    b = cfg.batches[0]
+    q = torch.zeros((b.length, cfg.hq, cfg.d), dtype=torch.bfloat16)
+    k = torch.zeros((b.length, cfg.hkv, cfg.d), dtype=torch.bfloat16)
+    mask = sa.TreeMask.build(b.art, b.end, b.pos, device="cpu")
+    with pytest.raises(RuntimeError, match="ROCm"):
+        sa.tree_attn(q, k, k, mask, cfg.scale)
+
+
+# ------------------------------------------------------------------------------------------------ packer mirror
+def test_build_tree_and_trie_literals(golden):
+    # spinf_serve/packer.py:38-64 via the reference's tests/test_packer.py:11-39
+    t = build_tree([[1, 5, 6, 7], [1, 5, 6, 8, 9]], [[[10], [11]], [[12], [13]]])
+    assert t.prefix == [1, 5, 6] and t.branches == [[7], [8, 9]]
+    assert t.reads == [(0, 0, 10, 0, 0), (0, 0, 11, 0, 1), (1, 1, 12, 1, 0), (1, 1, 13, 1, 1)] and t.n_tokens == 6
+    t = build_tree([[1, 2, 3], [1, 2, 3]], [[[4]], [[5]]])
+    assert t.prefix == [1, 2] and t.branches == [[3], [3]]
+    t = build_tree([[1, 2, 3]], [[[20], [21, 22], [21, 23]]])
+    assert t.branches == [[3], [3, 21]] and t.n_options == [3]
+    assert sorted(t.reads) == sorted([(0, 0, 20, 0, 0), (0, 0, 21, 0, 1), (1, 1, 22, 0, 1), (0, 0, 21, 0, 2), (1, 1, 23, 0, 2)])
+    with pytest.raises(ValueError):
+        build_tree([[1, 2]], [[[]]])
+    with pytest.raises(ValueError):
+        build_tree([], [])
+    g = golden["build_tree"]
+    t = build_tree([[1, 5, 6, 7], [1, 5, 6, 8, 9]], [[[10], [11]], [[12], [13, 14]]])
+    assert (t.prefix, t.branches, [list(r) for r in t.reads], t.n_options) == (g["prefix"], g["branches"], g["reads"], g["n_options"])
+    # tests/test_packer.py:191-206
+    plans = [ReadPlan.build([[30], [31]]), ReadPlan.build([[30], [31]]), ReadPlan.build([[20], [21, 22], [21, 23]])]
+    t = build_grouped_tree([[1, 2, 5, 6, 7, 8], [1, 2, 5, 6, 7, 9], [1, 2, 4]], plans)
+    gg = golden["build_grouped_tree"]
+    assert (t.prefix, t.branches, t.parents) == (gg["prefix"], gg["branches"], gg["parents"]) == ([1, 2], [[5, 6, 7], [8], [9], [4, 21]], [-1, 0, 0, -1])
+    assert [[list(x) for x in r] for r in t.prompt_rows] == gg["prompt_rows"] and t.n_tokens == 9
+    br, pa, rows = trie_branches([[3], [3]], [ReadPlan.build([[9]]), ReadPlan.build([[4, 5, 6], [4, 5, 7], [4, 8]])])
+    assert br == [[3, 4, 5]] and pa == [-1] and rows == [[(0, 0)], [(0, 0), (0, 1), (0, 2), (0, 1)]]
+
+
+def test_split_trees_halves_until_each_run_fits():
+    prompts = [[1] * 50 + [i] * 30 for i in range(2, 10)]
+    options = [[[100], [101]]] * len(prompts)
+    assert build_tree(prompts, options).n_tokens == 50 + 8 * 30
+    runs = split_trees(prompts, options, 110)
+    assert [a for a, _ in runs] == [0, 2, 4, 6] and all(t.n_tokens <= 110 for _, t in runs)
+    with pytest.raises(ValueError):
+        split_trees(prompts, options, 60)
+
+
+def test_packer_reproduces_reference_streams(golden):
+    """same trees pushed the same way -> the same batches, field by field (Packer.push / _flush / _pack)"""
+    for case in golden["cases"]:
+        trees = [GroupedTree(t["prefix"], t["branches"], [], [], parents=t["parents"], aligned=t["aligned"]) for t in case["trees"]]
+        pk = Packer(case["budget"], case["max_tokens"], align=case["align"], min_stream=case["min_stream"])
+        batches = []
+        for k, t in enumerate(trees):
+            batches += list(pk.push(k, t, window=case["push_window"]))
+        batches += list(pk.flush())
+        assert len(batches) == len(case["batches"])
+        for b, want in zip(batches, case["batches"]):
+            for key in ("ids", "pos", "seg", "art", "end", "prev"):
+                assert getattr(b, key).tolist() == want[key], key
+            assert b.n_tokens == want["n_tokens"]
+            assert [[o.job_id, o.start, o.n_tokens, o.prefix_len] for o in b.owners] == want["owners"]
+
+
+def test_packer_budget_rows_alignment_and_cost():
+    packer = Packer(256)
+    trees = [build_tree([[1] + [i] * n, [1] + [i] * n + [7]], [[[9], [8]], [[9], [8]]]) for i, n in ((2, 100), (3, 90), (4, 80))]
+    batches = [b for i, t in enumerate(trees) for b in packer.push(i, t, window=2)] + list(packer.flush())
+    assert sorted(o.job_id for b in batches for o in b.owners) == [0, 1, 2]
+    for b in batches:
+        assert b.length % BLOCK == 0 and b.length <= 256
+        assert b.n_tokens == sum(o.n_tokens for o in b.owners) and len(b.sel) == sum(o.n_rows for o in b.owners)
+        assert all(len(o.plan) == 4 and o.n_rows == 2 for o in b.owners)
+    with pytest.raises(ValueError):
+        list(Packer(128, 256).push("x", build_tree([[1] * 600], [[[2]]])))
+    (b,) = list(Packer(128, 1024).push("long", build_tree([[1] * 600], [[[2]]])))   # over the budget: runs alone, at once
+    assert b.length == 640
+    # second packing dimension (tests/test_packer.py:262-283)
+    def tree(n, costly):
+        t = build_grouped_tree([list(range(5, 5 + n)) + [3]], [ReadPlan.build([[4]])])
+        if costly:
+            t.xbranches = [(0, object())]
+        return t
+    cost = lambda t: 100 if t.xbranches else 0  # noqa: E731
+    pk = Packer(4096, cost=cost, cost_budget=250)
+    batches = [b for k, t in enumerate([tree(300, True) for _ in range(4)]) for b in pk.push(k, t)] + list(pk.flush())
+    assert sorted(len(b.owners) for b in batches) == [2, 2]
+
+
+def test_reads_see_exactly_their_prompt():
+    """tests/test_packer.py:209-239 with the mirror packer and the oracle mask"""
+    rng = np.random.default_rng(0)
+    for _ in range(10):
+        stem = [1] + rng.integers(2, 6, 3).tolist()
+        prompts = [stem + rng.integers(2, 6, int(rng.integers(1, 6))).tolist() for _ in range(int(rng.integers(1, 9)))]
+        plans = [ReadPlan.build([rng.integers(6, 9, int(rng.integers(1, 4))).tolist() for _ in range(int(rng.integers(1, 6)))]) for _ in prompts]
+        t = build_grouped_tree(prompts, plans)
+        pk = Packer(1024)
+        list(pk.push("o", build_grouped_tree([[1, 7, 7, 2], [1, 7, 7, 3]], [ReadPlan.build([[9]])] * 2)))
+        list(pk.push("t", t))
+        (b,) = list(pk.flush())
+        o = next(o for o in b.owners if o.job_id == "t")
+        k0 = sum(x.n_rows for x in b.owners[: b.owners.index(o)])
+        m = omask.dense_tree_mask(b.art, b.end)
+        for c, (x, plan) in enumerate(zip(prompts, plans)):
+            want = [x] + [x + list(lead[:j]) for lead in plan.leadins for j in range(1, len(lead) + 1)]
+            for r, wseq in enumerate(want):
+                qpos = int(b.sel[k0 + o.row_start[c] + r])
+                ks = np.flatnonzero(m[qpos])
+                assert b.ids[ks].tolist() == wseq and b.pos[ks].tolist() == list(range(len(wseq)))
+
+
+# ------------------------------------------------------------------------------------------------ tile plan
+def _check_plan(art, end, pos, window):
+    """exactness of the compiled plan against the dense mask at 32 x 32 granularity: a set bit <=> some pair visible,
+    a clear mask bit <=> every pair visible, unlisted tiles <=> nothing visible; key tiles ascending"""
+    plan = sa.TilePlan.build(art, end, pos, window)
+    n = len(art)
+    m = omask.dense_tree_mask(art, end, pos, window)
+    nqt = -(-n // 128)
+    assert plan.n_qtiles == nqt and sorted(plan.order.tolist()) == list(range(nqt))
+    active = masked = 0
+    for t in range(nqt):
+        ents = range(plan.qt_ptr[t], plan.qt_ptr[t + 1])
+        kts = [int(plan.kv_idx[e]) for e in ents]
+        assert kts == sorted(set(kts))
+        listed = dict(zip(kts, (int(plan.kv_bits[e]) for e in ents)))
+        for j in range(-(-n // 64)):
+            bits = listed.get(j, 0)
+            for w in range(4):
+                for s in range(2):
+                    blk = m[128 * t + 32 * w : 128 * t + 32 * w + 32, 64 * j + 32 * s : 64 * j + 32 * s + 32]
+                    on = bool(bits >> (2 * w + s) & 1)
+                    assert on == bool(blk.size and blk.any()), (t, j, w, s)
+                    if on:
+                        active += 1
+                        need = bool(bits >> (8 + 2 * w + s) & 1)
+                        assert need == (not (blk.all() and blk.shape == (32, 32))), (t, j, w, s)
+                        masked += need
+                    else:
+                        assert not (bits >> (8 + 2 * w + s) & 1)
+    assert (active, masked) == (plan.active_blocks, plan.masked_blocks)
+    return plan
+
+
+def test_tileplan_is_exact_on_golden_streams(golden):
+    for case in golden["cases"]:
+        for b in case["batches"]:
+            art, end, pos = (np.array(b[k], np.int32) for k in ("art", "end", "pos"))
+            _check_plan(art, end, pos, None)
+            _check_plan(art, end, pos, b["window"])
+
+
+def test_tileplan_edge_cases():
+    # all pads; a single token; ragged length; dense (unaligned) packing with jobs sharing tiles
+    _check_plan(np.full(130, -1, np.int32), np.full(130, -1, np.int32), np.zeros(130, np.int32), None)
+    _check_plan(np.zeros(1, np.int32), np.ones(1, np.int32), np.zeros(1, np.int32), None)
+    s = pack_stream([Job([1] * 100, [[2] * 5, [3] * 6]), Job([4] * 37, [[5] * 3]), Job([6] * 260, [[7] * 11] * 6)], align=False)
+    n = int(np.flatnonzero(s.art >= 0)[-1]) + 1
+    _check_plan(s.art[:n], np.minimum(s.end[:n], n), s.pos[:n], None)
+    _check_plan(s.art[:n], np.minimum(s.end[:n], n), s.pos[:n], 50)
+    # the reference's literal: 2000-token trunk at window 512, query block 14 needs exactly key blocks 10..14
+    s = pack_stream([Job([1] * 2000, [[2]])], length=2048)
+    plan = sa.TilePlan.build(s.art, s.end, s.pos, 512)
+    assert sorted({int(k) // 2 for k in plan.kv_idx[plan.qt_ptr[14] : plan.qt_ptr[15]]}) == [10, 11, 12, 13, 14]
+    # finished sibling branches are skipped (tests/test_packer.py:251-259)
+    s = pack_stream([Job([1] * 200, [[2] * 300, [3] * 300])], length=1024)
+    plan = sa.TilePlan.build(s.art, s.end, s.pos, None)
+    blocks = {int(k) // 2 for k in plan.kv_idx[plan.qt_ptr[5] : plan.qt_ptr[6]]}
+    assert 2 not in blocks and {0, 1, 3, 4, 5} <= blocks
+
+
+def test_a_jobs_plan_does_not_depend_on_its_neighbours():
+    """aligned jobs: a job's tile lists, relative to its first tile, are the same alone and packed (the host half of batch
+    invariance, tests/test_packer.py:115-134)"""
+    cfg = synth.attention_config("C2", contents=3)
+
+    def rel(trees, which, window):
+        b = synth.pack(trees)[0]
+        plan = sa.TilePlan.build(b.art, b.end, b.pos, window)
+        o = b.owners[which]
+        t0, t1 = o.start // 128, -(-(o.start + o.n_tokens) // 128)
+        return [[(int(plan.kv_idx[e]) - 2 * t0, int(plan.kv_bits[e])) for e in range(plan.qt_ptr[t], plan.qt_ptr[t + 1])] for t in range(t0, t1)]
+
+    for window in (None, 256):
+        for i, t in enumerate(cfg.trees):
+            assert rel([t], 0, window) == rel(cfg.trees, i, window) == rel(cfg.trees[::-1], 2 - i, window)
+
+
+def test_config_workloads_match_their_closed_forms():
+    c1 = synth.attention_config("C1")
+    assert (c1.n_real, c1.pairs(), c1.flops()) == (192, 8544, 8749056.0) and c1.batches[0].length == 256
+    # P = T(T+1)/2 + sum_b (L_b * ancestors + L_b (L_b + 1) / 2), here against the dense mask
+    c2 = synth.attention_config("C2", contents=2)
+    b = c2.batches[0]
+    m = omask.dense_tree_mask(b.art, b.end)
+    assert c2.pairs() == int(m[b.art >= 0].sum())
+    assert c2.pairs(100) == int(omask.dense_tree_mask(b.art, b.end, b.pos, 100)[b.art >= 0].sum())
+
+
+# ------------------------------------------------------------------------------------------------ recurrent-layer plan
+def test_tree_plan_matches_reference_and_oracle(golden):
+    for case in golden["cases"]:
+        for b in case["batches"]:
+            prev, real = np.array(b["prev"]), np.array(b["art"]) >= 0
+            for short, ct in ((64, 8192), (4, 300)):
+                want = b[f"plan_short{short}_ct{ct}"]
+                plan = sa.tree_plan(prev, real, "cpu", path="indexed", short=short, call_tokens=ct)
+                assert plan.n_keep == want["n_keep"] and plan.n_segments == want["n_segments"]
+                assert plan.conv.tolist() == want["conv"]
+                for lv, wl in zip(plan.levels, want["levels"]):
+                    assert len(lv) == len(wl)
+                    for c, wc in zip(lv, wl):
+                        assert c.kind == wc["kind"] and c.idx.tolist() == wc["idx"] and c.cu.tolist() == wc["cu"]
+                        assert (None if c.h0_idx is None else c.h0_idx.tolist()) == wc["h0_idx"]
+                        assert (None if c.ht_idx is None else c.ht_idx.tolist()) == wc["ht_idx"]
+
+
+def test_tree_plan_compact_rows_keep_and_levels():
+    """tests/test_qwen_plan.py:102-164 and tests/test_stacks.py:67-75 against the mirror"""
+    plan = sa.tree_plan(np.array([-1, 0, 1, 1, 3]), np.ones(5, bool), "cpu")
+    assert plan.n_segments == 3
+    rng = np.random.default_rng(1)
+    job = Job(list(rng.integers(5, 50, 150)), [list(rng.integers(5, 50, n)) for n in (6, 70, 3, 2, 9)], [-1, 0, 0, 2, -1])
+    s = pack_stream([job, Job([9] * 5, [[1], [2]])], align=True)
+    real = s.art >= 0
+    R = int(real.sum())
+    rows = (R + 127) // 128 * 128
+    cp = sa.tree_plan(s.prev, real, "cpu", short=4, rows=rows)
+    ip = sa.tree_plan(s.prev, real, "cpu", short=4)
+    sidx = cp.sidx.numpy()
+    assert (sidx == np.flatnonzero(real)).all()
+    for lc, ls in zip(cp.levels, ip.levels):
+        for c, d in zip(lc, ls):
+            assert (sidx[c.idx.numpy()] == d.idx.numpy()).all() and (c.cu.numpy() == d.cu.numpy()).all()
+    T = len(s.prev)
+    back = np.full(rows + 1, T, np.int64)
+    back[:R] = sidx
+    assert (back[cp.conv.numpy()[:R]] == ip.conv.numpy()[sidx]).all() and (cp.conv.numpy()[R:] == rows).all()
+    assert (cp.seg_of_row[R:] == -1).all() and (cp.seg_of_row[:R] >= 0).all()
+    # a leaf keeps no state unless asked to
+    leaf = [i for i in np.flatnonzero(real) if not (s.prev == i).any()][0]
+    c_of = np.cumsum(real) - 1
+    sg = cp.seg_of_row[c_of[leaf]]
+    assert cp.seg_slot[sg] == -1
+    kept = sa.tree_plan(s.prev, real, "cpu", short=4, rows=rows, keep=[leaf])
+    assert kept.seg_slot[sg] >= 0 and kept.n_keep[kept.seg_level[sg]] == cp.n_keep[cp.seg_level[sg]] + 1
+    # the levels path covers every real token once
+    lp = sa.tree_plan(s.prev, real, "cpu", max_init=3, path="levels")
+    seen = np.concatenate([c.idx.numpy() for lv in lp.levels for c in lv])
+    assert sorted(seen.tolist()) == np.flatnonzero(real).tolist()
+    with pytest.raises(ValueError):
+        sa.tree_plan(s.prev, real, "cpu", rows=R - 1)
+    # the oracle's restatement agrees
+    levels, n_keep, _ = oplan.tree_plan(s.prev, real, short=4)
+    assert n_keep == ip.n_keep and [[c["kind"] for c in lv] for lv in levels] == [[c.kind for c in lv] for lv in ip.levels]
