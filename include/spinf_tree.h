@@ -39,7 +39,13 @@ int spinf_version(void);
  * Entry e of query tile t (qt_ptr[t] <= e < qt_ptr[t+1]) names key tile kv_idx[e]; kv_bits[e] bit (2*w + s) says that
  * rows 32w..32w+31 of the query tile see at least one key of keys 32s..32s+31 of the key tile, bit 8 + (2*w + s) that
  * some pair of that 32 x 32 block is masked (the kernel then evaluates spinf_serve/scorer.py:173-177 per element).
- * order[] lists the query tiles job by job, heaviest first inside a job (a launch order, it does not change results).
+ * order[] lists the query tiles job by job, heaviest first inside a job.
+ *
+ * spinf_tileplan_schedule turns the plan into the kernel's work lists for a given number of head groups (query heads /
+ * heads per work item, see spinf_attn_heads_per_item): items[4*i..4*i+3] = {query tile, first entry, entries | head
+ * group << 20, first key tile}; list_ptr[0..8] delimits eight lists of roughly equal weight (one per XCD), inside a list
+ * the items of a job stay together, head group by head group, heaviest query tile first.  The order of the items never
+ * changes a result.
  */
 typedef struct spinf_tileplan spinf_tileplan;
 
@@ -49,6 +55,8 @@ int spinf_tileplan_build(const int32_t* art, const int32_t* end, const int32_t* 
 int spinf_tileplan_counts(const spinf_tileplan* plan, int64_t counts[5]);
 /* qt_ptr [n_qtiles+1], kv_idx [entries], kv_bits [entries], order [n_qtiles]: caller-allocated host arrays */
 int spinf_tileplan_export(const spinf_tileplan* plan, int32_t* qt_ptr, int32_t* kv_idx, uint32_t* kv_bits, int32_t* order);
+/* items [4 * n_qtiles * head_groups], list_ptr [9]: caller-allocated host arrays */
+int spinf_tileplan_schedule(const spinf_tileplan* plan, int32_t head_groups, int32_t* items, int32_t* list_ptr);
 void spinf_tileplan_free(spinf_tileplan* plan);
 
 /* ------------------------------------------------------------------------------------------------ attention
@@ -58,19 +66,25 @@ void spinf_tileplan_free(spinf_tileplan* plan);
  *
  *   q [n, hq, d], k / v [n, hkv, d], out [n, hq, d]: bf16 device tensors, d contiguous; *_tok / *_head are the token
  *   and head strides in elements (multiples of 8).  d is 64, 128 or 256.
- *   art, end, pos, qt_ptr, kv_idx, kv_bits, order: device copies of the metadata and of the exported plan
+ *   art, end, pos, kv_idx, kv_bits: device copies of the metadata and of the exported plan; items, list_ptr: device copy of
+ *   the schedule for hq / spinf_attn_heads_per_item(hq, hkv, d, variant) head groups, n_items = query tiles x head groups
  *   window: the window the plan was built with (<= 0 global)
+ *
+ * The kernel is persistent (one workgroup per CU pulling items from the lists) and keeps its list cursors in a small
+ * per-device buffer of the library: launches that overlap on one device (different streams) are not supported.
  */
 typedef struct spinf_attn_args {
     const void* q; const void* k; const void* v; void* out;
     int64_t q_tok, q_head, k_tok, k_head, v_tok, v_head, o_tok, o_head;
     int64_t n; int32_t hq, hkv, d; float scale; int32_t window;
     const int32_t* art; const int32_t* end; const int32_t* pos;
-    const int32_t* qt_ptr; const int32_t* kv_idx; const uint32_t* kv_bits; const int32_t* order;
-    int64_t n_qtiles;
-    int32_t variant;   /* 0 = default kernel choice; other values select a tuning variant (same results) */
+    const int32_t* kv_idx; const uint32_t* kv_bits; const int32_t* items; const int32_t* list_ptr;
+    int64_t n_items;
+    int32_t variant;   /* 0 = default kernel choice; 1 = one head per work item even where two would fit */
 } spinf_attn_args;
 
+/* query heads one work item covers for this geometry (1 or 2); 0 for an invalid geometry */
+int spinf_attn_heads_per_item(int32_t hq, int32_t hkv, int32_t d, int32_t variant);
 int spinf_tree_attn_fwd(const spinf_attn_args* args, void* stream);
 
 /* ------------------------------------------------------------------------------------------------ Gated DeltaNet

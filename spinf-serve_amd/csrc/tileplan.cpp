@@ -15,6 +15,8 @@ struct spinf_tileplan {
     int32_t window = 0;
     std::vector<int32_t> qt_ptr, kv_idx, order;
     std::vector<uint32_t> kv_bits;
+    std::vector<int64_t> weight;     // active 32 x 32 blocks per query tile
+    std::vector<int32_t> group;      // job of the tile's first real row (-1: pads only)
     int64_t active = 0, masked = 0;
 };
 
@@ -85,8 +87,10 @@ extern "C" int spinf_tileplan_build(const int32_t* art, const int32_t* end, cons
             jfirst[i] = it->second;
         }
         p->qt_ptr.assign(nqt + 1, 0);
-        std::vector<int64_t> weight(nqt, 0);
-        std::vector<int32_t> group(nqt, -1);
+        std::vector<int64_t>& weight = p->weight;
+        std::vector<int32_t>& group = p->group;
+        weight.assign(nqt, 0);
+        group.assign(nqt, -1);
         for (int64_t t = 0; t < nqt; t++) {
             const int64_t q0 = t * SPINF_QTILE, q1 = std::min<int64_t>(n, q0 + SPINF_QTILE);
             int64_t lo_key = q0;
@@ -173,6 +177,46 @@ extern "C" int spinf_tileplan_export(const spinf_tileplan* p, int32_t* qt_ptr, i
         std::memcpy(kv_bits, p->kv_bits.data(), p->kv_bits.size() * sizeof(uint32_t));
     }
     if (!p->order.empty()) std::memcpy(order, p->order.data(), p->order.size() * sizeof(int32_t));
+    return SPINF_OK;
+}
+
+extern "C" int spinf_tileplan_schedule(const spinf_tileplan* p, int32_t head_groups, int32_t* items, int32_t* list_ptr) {
+    if (!p || !list_ptr) return spinf_fail(SPINF_E_ARG, "tileplan_schedule: null argument");
+    if (head_groups <= 0 || head_groups >= 4096) return spinf_fail(SPINF_E_ARG, "tileplan_schedule: head groups %d out of range", head_groups);
+    const int64_t nqt = (int64_t)p->order.size();
+    if (nqt && !items) return spinf_fail(SPINF_E_ARG, "tileplan_schedule: null items");
+    if (nqt * head_groups > (int64_t)1 << 30) return spinf_fail(SPINF_E_ARG, "tileplan_schedule: too many items");
+    // items: job run by job run (tiles that share keys), head group by head group, heaviest tile first
+    std::vector<int64_t> cum;
+    cum.reserve(nqt * head_groups + 1);
+    cum.push_back(0);
+    int64_t k = 0;
+    int64_t a = 0;
+    while (a < nqt) {
+        int64_t b = a + 1;
+        while (b < nqt && p->group[p->order[b]] == p->group[p->order[a]]) b++;
+        for (int32_t hp = 0; hp < head_groups; hp++)
+            for (int64_t pos = a; pos < b; pos++) {
+                const int32_t t = p->order[pos];
+                const int32_t e0 = p->qt_ptr[t], ne = p->qt_ptr[t + 1] - e0;
+                items[4 * k + 0] = t;
+                items[4 * k + 1] = e0;
+                items[4 * k + 2] = (ne & 0xfffff) | (hp << 20);
+                items[4 * k + 3] = ne > 0 ? p->kv_idx[e0] : 0;
+                cum.push_back(cum.back() + p->weight[t] + 6);   // + a fixed cost per item (prologue, output)
+                k++;
+            }
+        a = b;
+    }
+    // eight contiguous lists of about equal weight
+    const int64_t total = cum.back();
+    list_ptr[0] = 0;
+    for (int l = 1; l < 8; l++) {
+        const int64_t want = total * l / 8;
+        const int64_t at = std::lower_bound(cum.begin(), cum.end(), want) - cum.begin();
+        list_ptr[l] = (int32_t)std::max<int64_t>(list_ptr[l - 1], std::min<int64_t>(at, k));
+    }
+    list_ptr[8] = (int32_t)k;
     return SPINF_OK;
 }
 

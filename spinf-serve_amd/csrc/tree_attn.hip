@@ -3,22 +3,29 @@
 // Replaces the flex_attention call of spinf_serve/models/gemma4.py:107-118 and spinf_serve/models/qwen35/qwen.py:614,620;
 // the per-element visibility test is the predicate of spinf_serve/scorer.py:173-177.
 //
-// Work decomposition.  One workgroup (4 waves) = one 128-token query tile x RT query heads of one GQA group; wave w owns
+// Work decomposition.  A work item = one 128-token query tile x RT query heads of one GQA group; 4 waves, wave w owns
 // tokens 32w..32w+31 of the tile for all RT heads, so a K or V fragment read from LDS feeds RT MFMAs and the mask of a
 // 32x32 block is evaluated once for all RT heads.  Scores are computed transposed, S^T = K Q^T, with
 // v_mfma_f32_32x32x16_bf16: a lane then owns ONE query row (column lane%32 of the 32x32 result) and 16 of the 32 keys,
 // so the softmax row reductions are in-lane plus one exchange with lane^32.  O^T = V^T P^T reuses the score registers
 // as the B operand without any shuffle; V^T fragments come from row-major V in LDS through ds_read_b64_tr_b16.
 //
-// K/V tiles (64 keys) are copied global -> LDS by the DMA path (global_load_lds_dwordx4), double-buffered, with an XOR
-// swizzle of the 16-byte chunks that keeps both the b128 reads of K and the transposing reads of V free of bank
-// conflicts.  The key tile's art/end/pos ride along so that masked blocks never touch global memory in the loop.
+// Persistent workgroups.  One workgroup per CU pulls work items from eight lists (one per XCD, so that the tiles sharing
+// K/V meet in one L2; a workgroup that exhausts its list continues with the next one).  While an item is computed the
+// next item's descriptor, plan entries and query fragments are fetched, and the K/V tile pipeline runs straight across
+// the item boundary, so the fixed cost of an item is its epilogue only.
+//
+// K/V tiles (64 keys) are copied global -> LDS by the DMA path (global_load_lds_dwordx4), double-buffered, in a padded
+// layout that keeps both the b128 reads of K and the transposing reads of V free of bank conflicts.  The key tile's
+// art/end/pos ride along so that masked blocks never touch global memory in the loop.
 //
 // Reduction order.  A row's keys are visited in ascending 32-key blocks that depend only on the row's own job (jobs start
 // on 128-token boundaries), masked entries contribute exact zeros, and a skipped block equals a fully masked one bit for
-// bit; the running maximum is updated per row from that row's scores only.  A job's output is therefore bit-identical
-// whatever it is packed with.
+// bit; the softmax reference point of a row is taken from that row's scores only.  A job's output is therefore
+// bit-identical whatever it is packed with, and whichever workgroup happens to compute it.
 #include <hip/hip_runtime.h>
+
+#include <mutex>
 
 #include "spinf_tree.h"
 #include "common.h"
@@ -32,6 +39,9 @@ typedef __attribute__((ext_vector_type(2))) unsigned u32x2;
 typedef __attribute__((address_space(3))) void lds_void;
 typedef const __attribute__((address_space(1))) void gbl_void;
 
+constexpr int NLIST = 8;       // work lists (XCDs of an MI355X)
+constexpr int ENT_CAP = 256;   // plan entries of a query tile kept in LDS at a time
+
 struct AttnParams {
     const __bf16* q; const __bf16* k; const __bf16* v; __bf16* o;
     long q_tok, q_head, k_tok, k_head, v_tok, v_head, o_tok, o_head;
@@ -39,10 +49,22 @@ struct AttnParams {
     float c;              // scale * log2(e)
     int window;
     const int* art; const int* end; const int* pos;
-    const int* qt_ptr; const int* kv_idx; const unsigned* kv_bits; const int* order;
-    int nqt, total, per_xcd;
+    const int* kv_idx; const unsigned* kv_bits;
+    const int4* items;    // work items {query tile, first entry, entries | head group << 20, first key tile}, list by list
+    const int* list_ptr;  // [NLIST + 1] offsets of the lists in items
+    int* counters;        // [0..NLIST) next item of each list, [NLIST] workgroups done, [NLIST+1] items awaiting the exact pass,
+                          // [NLIST+2] exact-pass workgroups done; each kernel's last workgroup resets what it used
+    int* redo;            // indices (into items) of the work items the fast pass handed to the exact pass
 };
 
+// Softmax reference point.  The fast pass fixes each row's reference at the maximum of the first 32-key block in which
+// the row sees a key and never rescales the accumulators: probabilities are exp2(t - ref) and stay below 2^TAU_FAST, well
+// inside fp32 / bf16 range.  If any row of a tile meets a score more than TAU_FAST above its reference, the whole tile is
+// recomputed by the exact pass: classic online softmax, reference raised and accumulators rescaled whenever a block
+// maximum exceeds the reference by more than TAU_LAZY.  Which pass produced a row depends on the rows of its own
+// 128-token tile only, so it does not depend on what the job is packed with.
+constexpr float TAU_FAST = 60.f;
+constexpr float TAU_LAZY = 8.f;
 
 __device__ __forceinline__ float lane32_max(float x) {
     u32x2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
@@ -69,16 +91,41 @@ struct Geo {
     static constexpr int KTILEB = NREG * KRS, VTILEB = NREG * VRS;
     static constexpr int METAB = 3 * 64 * 4;
     static constexpr int BUFB = KTILEB + VTILEB + METAB;   // K tile | V tile | art,end,pos of the keys
+    static constexpr int SUBB = (32 / NREG) * ROWB;        // byte offset of rows 32.. relative to rows 0.. (same regions)
     __host__ __device__ static constexpr int k_off(int row) { return (row % NREG) * KRS + (row / NREG) * ROWB; }
     __host__ __device__ static constexpr int v_off(int row) { return (row % NREG) * VRS + (row / NREG) * ROWB; }
 };
 
-// Starts the DMA of key tile kt (64 keys of kv head kvh) into an LDS buffer.  Wave w copies regions w*IPW .. w*IPW+IPW-1;
-// lane -> (slot = which row of the region, 16-byte chunk of the row).  For a tile that lies fully inside the stream every
-// address is a wave-uniform base plus a per-lane constant (lane_k / lane_v, bytes), so the loop spends no vector ALU on
-// addressing; the last, partial tile clamps its rows per lane.
+// One wave-wide DMA instruction: 64 lanes x `16` (or 4) bytes from global memory straight into 1 KiB (256 B) of contiguous
+// LDS at byte address `lds`.  Written as inline assembly on purpose: the compiler then does not track these LDS writes, so
+// it never makes the fragment reads of the OTHER tile buffer wait for them (it cannot tell the two buffers apart once the
+// buffer is chosen at run time); the kernel orders them itself with s_waitcnt vmcnt(0) + a barrier before a buffer is read.
+__device__ __forceinline__ const char* uniform_ptr(const char* p) {   // a wave-uniform pointer, pinned to scalar registers
+    const unsigned long long v = (unsigned long long)p;
+    const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)v), hi = __builtin_amdgcn_readfirstlane((unsigned)(v >> 32));
+    return (const char*)(((unsigned long long)hi << 32) | lo);
+}
+__device__ __forceinline__ void dma16_uniform(const char* base, unsigned lane_off, unsigned lds) {   // base is wave-uniform
+    base = uniform_ptr(base);
+    lds = __builtin_amdgcn_readfirstlane(lds);
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0" ::"s"(base), "v"(lane_off), "s"(lds) : "memory");
+}
+__device__ __forceinline__ void dma16_lane(const char* addr, unsigned lds) {
+    lds = __builtin_amdgcn_readfirstlane(lds);
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(addr), "s"(lds) : "memory");
+}
+__device__ __forceinline__ void dma4_lane(const int* addr, unsigned lds) {
+    lds = __builtin_amdgcn_readfirstlane(lds);
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(addr), "s"(lds) : "memory");
+}
+__device__ __forceinline__ unsigned lds_addr(const void* p) { return (unsigned)(size_t)(const __attribute__((address_space(3))) char*)p; }
+
+// Starts the DMA of key tile kt (64 keys of kv head kvh) into the LDS buffer at byte address `buf`.  Wave w copies regions
+// w*IPW .. w*IPW+IPW-1; lane -> (slot = which row of the region, 16-byte chunk of the row).  For a tile that lies fully inside
+// the stream every address is a wave-uniform base plus a per-lane constant (lane_k / lane_v, bytes), so the loop spends no
+// vector ALU on addressing; the last, partial tile clamps its rows per lane.
 template <int D>
-__device__ __forceinline__ void issue_tile(const AttnParams& p, char* buf, int kt, int kvh, int w, int lane, unsigned lane_k, unsigned lane_v) {
+__device__ __forceinline__ void issue_tile(const AttnParams& p, unsigned buf, int kt, int kvh, int w, int lane, unsigned lane_k, unsigned lane_v) {
     using G = Geo<D>;
     const char* kbase = (const char*)(p.k + (long)kvh * p.k_head);
     const char* vbase = (const char*)(p.v + (long)kvh * p.v_head);
@@ -87,12 +134,12 @@ __device__ __forceinline__ void issue_tile(const AttnParams& p, char* buf, int k
         for (int i = 0; i < G::IPW; i++) {
             const int reg = w * G::IPW + i;
             const long row = (long)kt * 64 + reg;
-            __builtin_amdgcn_global_load_lds((gbl_void*)(kbase + row * p.k_tok * 2 + lane_k), (lds_void*)(buf + reg * G::KRS), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((gbl_void*)(vbase + row * p.v_tok * 2 + lane_v), (lds_void*)(buf + G::KTILEB + reg * G::VRS), 16, 0, 0);
+            dma16_uniform(kbase + row * p.k_tok * 2, lane_k, buf + reg * G::KRS);
+            dma16_uniform(vbase + row * p.v_tok * 2, lane_v, buf + G::KTILEB + reg * G::VRS);
         }
         if (w < 3) {   // wave 0: art, wave 1: end, wave 2: pos of the 64 keys
             const int* src = (w == 0 ? p.art : w == 1 ? p.end : p.pos) + (long)kt * 64;
-            __builtin_amdgcn_global_load_lds((gbl_void*)(src + lane), (lds_void*)(buf + G::KTILEB + G::VTILEB + w * 256), 4, 0, 0);
+            dma4_lane(src + lane, buf + G::KTILEB + G::VTILEB + w * 256);
         }
     } else {
         const int slot = lane / G::CPR, chunk = lane % G::CPR;
@@ -101,174 +148,178 @@ __device__ __forceinline__ void issue_tile(const AttnParams& p, char* buf, int k
             const int reg = w * G::IPW + i;
             long grow = (long)kt * 64 + reg + G::NREG * slot;
             grow = grow < p.n ? grow : p.n - 1;
-            __builtin_amdgcn_global_load_lds((gbl_void*)(kbase + grow * p.k_tok * 2 + chunk * 16), (lds_void*)(buf + reg * G::KRS), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((gbl_void*)(vbase + grow * p.v_tok * 2 + chunk * 16), (lds_void*)(buf + G::KTILEB + reg * G::VRS), 16, 0, 0);
+            dma16_lane(kbase + grow * p.k_tok * 2 + chunk * 16, buf + reg * G::KRS);
+            dma16_lane(vbase + grow * p.v_tok * 2 + chunk * 16, buf + G::KTILEB + reg * G::VRS);
         }
         if (w < 3) {
             long gk = (long)kt * 64 + lane;
             gk = gk < p.n ? gk : p.n - 1;
-            const int* src = (w == 0 ? p.art : w == 1 ? p.end : p.pos) + gk;
-            __builtin_amdgcn_global_load_lds((gbl_void*)src, (lds_void*)(buf + G::KTILEB + G::VTILEB + w * 256), 4, 0, 0);
+            dma4_lane((w == 0 ? p.art : w == 1 ? p.end : p.pos) + gk, buf + G::KTILEB + G::VTILEB + w * 256);
         }
     }
 }
 
-#ifndef SPINF_ABL
-#define SPINF_ABL 0   // measurement builds only: 1 = no tile DMA after the first, 2 = no block compute
-#endif
-#ifdef SPINF_TRACE
-__device__ long g_trace[16 * 16384];
-extern "C" int spinf_debug_trace(long* out, int n) { return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_trace), sizeof(long) * n, 0, hipMemcpyDeviceToHost); }
-#define TRACE(slot, val) do { if (threadIdx.x == 0 && blockIdx.x < 16384) g_trace[blockIdx.x * 16 + (slot)] = (val); } while (0)
-#define PH_DECL long ph_t = 0, ph_acc[4] = {0, 0, 0, 0};
-#define PH_START do { ph_t = clock64(); } while (0)
-#define PH_MARK(k) do { const long ph_n = clock64(); ph_acc[k] += ph_n - ph_t; ph_t = ph_n; } while (0)
-#else
-#define TRACE(slot, val) do { } while (0)
-#define PH_DECL
-#define PH_START do { } while (0)
-#define PH_MARK(k) do { } while (0)
-#endif
-constexpr int ENT_CAP = 256;   // plan entries of the current query tile kept in LDS at a time
-
-// Softmax reference point.  The first pass over a query tile fixes each row's reference at the maximum of the first 32-key
-// block in which the row sees a key and never rescales the accumulators: probabilities are exp2(t - ref) and stay below
-// 2^TAU_FAST in fp32 / bf16 range.  If any row of the tile meets a score more than TAU_FAST above its reference, the
-// whole tile is recomputed by the second, classic online-softmax pass (reference raised, accumulators rescaled, whenever a
-// block maximum exceeds it by more than TAU_LAZY).  Which pass produced a row depends on the rows of its own 128-token tile
-// only, so it does not depend on what the job is packed with.
-constexpr float TAU_FAST = 60.f;
-constexpr float TAU_LAZY = 8.f;
-
-// One workgroup's whole job: load the query fragments, walk the tile's key list, normalise and store.  EXACT = false is the
-// fast pass (returns true, without storing, when some row needs the exact pass); EXACT = true the classic online softmax.
-template <int D, int RT, bool WIN, int KPF, int VPF, bool EXACT>
-__device__ __forceinline__ bool attn_tile(const AttnParams& p, char* buf0, char* buf1, int2* ent) {
+// Everything a wave needs to know about its place in the workgroup and its LDS fragment addresses.
+template <int D>
+struct Lane {
     using G = Geo<D>;
-    constexpr int NS = D / 16;    // contraction steps of K Q^T
-    constexpr int NDT = D / 32;   // 32-wide slices of the head dimension in O^T
+    int lane, m, g, w;
+    int k_lane, v_lane;          // byte offsets of this lane's K fragment row / V^T fragment address inside a tile
+    unsigned lane_k, lane_v;     // per-lane part of the DMA source addresses
+    __device__ __forceinline__ Lane(const AttnParams& p) {
+        lane = threadIdx.x & 63;
+        m = lane & 31;
+        g = lane >> 5;
+        w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+        // K fragment: row m of the 32-key block, 16-byte chunk g of each 32-byte step.  V^T fragment
+        // (ds_read_b64_tr_b16): inside its 16-lane group a lane supplies the address of key row 4g + tr_j, head dims
+        // 16 tr_mb + 4 tr_a .. +3 of the 32-wide slice, and receives head dim lane%32 of 4 consecutive keys.
+        const int tr_a = lane & 3, tr_j = (lane >> 2) & 3, tr_mb = (lane >> 4) & 1;
+        k_lane = G::k_off(m) + 16 * g;
+        v_lane = G::v_off(4 * g + tr_j) + 32 * tr_mb + 8 * tr_a;
+        lane_k = (unsigned)((lane / G::CPR) * G::NREG * p.k_tok * 2 + (lane % G::CPR) * 16);
+        lane_v = (unsigned)((lane / G::CPR) * G::NREG * p.v_tok * 2 + (lane % G::CPR) * 16);
+    }
+};
 
-    const int lane = threadIdx.x & 63, m = lane & 31, g = lane >> 5;
-    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    // consecutive workgroups go round-robin over the 8 XCDs; give every XCD a contiguous range of the
-    // (head group major, job by job) work list so that the tiles sharing K/V meet in one L2
-    const int L = (blockIdx.x & 7) * p.per_xcd + (blockIdx.x >> 3);
-    if (L >= p.total) return false;
-    TRACE(0, (long)__builtin_amdgcn_s_memrealtime());
-    TRACE(1, (long)clock64());
-    const int hp = L / p.nqt;
-    const int t = p.order[L - hp * p.nqt];
+// mask of one 32-key block: register i of the S^T tile holds key 8*(i/4) + 4g + i%4 of the block
+template <int RT, bool WIN>
+__device__ __forceinline__ void apply_mask(f32x16 (&s_acc)[RT], const int* meta, int kt, int sub, int g, int tok, int art_q, int pos_q, int window) {
+#pragma unroll
+    for (int i4 = 0; i4 < 4; i4++) {
+        const int ko = 32 * sub + 8 * i4 + 4 * g;
+        const int4 ka = *(const int4*)(meta + ko);
+        const int4 ke = *(const int4*)(meta + 64 + ko);
+        int4 kp = make_int4(0, 0, 0, 0);
+        if (WIN) kp = *(const int4*)(meta + 128 + ko);
+        const int kg = kt * 64 + ko;
+        const int kav[4] = {ka.x, ka.y, ka.z, ka.w};
+        const int kev[4] = {ke.x, ke.y, ke.z, ke.w};
+        const int kpv[4] = {kp.x, kp.y, kp.z, kp.w};
+#pragma unroll
+        for (int jj = 0; jj < 4; jj++) {
+            const int kk = kg + jj;
+            bool vis = (kk <= tok) & (art_q >= 0) & (kav[jj] == art_q) & (tok < kev[jj]);
+            vis = vis | (kk == tok);
+            if (WIN) vis = vis & ((pos_q - kpv[jj]) < window);
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++) s_acc[rt][4 * i4 + jj] = vis ? s_acc[rt][4 * i4 + jj] : -INFINITY;
+        }
+    }
+}
+
+// normalise O^T and store it as rows: each wave stages 32 rows x 64 head dims at a time in its own LDS slice (144-byte
+// rows) and writes them out as 16-byte pieces, 8 lanes per 128-byte row segment
+template <int D, int RT>
+__device__ __forceinline__ void store_rows(const AttnParams& p, const Lane<D>& L, char* stage, const f32x16 (&o)[RT][D / 32], const float (&l)[RT],
+                                           int t, int h0) {
+    constexpr int NDT = D / 32;
+    constexpr int SROW = 128 + 16;
+    const int tok0 = t * SPINF_QTILE + 32 * L.w;
+#pragma unroll
+    for (int rt = 0; rt < RT; rt++) {
+        const float inv = 1.0f / lane32_sum(l[rt]);
+        __bf16* ob = p.o + (long)(h0 + rt) * p.o_head;
+#pragma unroll
+        for (int qd = 0; qd < NDT / 2; qd++) {
+#pragma unroll
+            for (int dd = 0; dd < 2; dd++)
+#pragma unroll
+                for (int i4 = 0; i4 < 4; i4++) {
+                    bf16x4 r;
+#pragma unroll
+                    for (int jj = 0; jj < 4; jj++) r[jj] = (__bf16)(o[rt][2 * qd + dd][4 * i4 + jj] * inv);
+                    *(bf16x4*)(stage + L.m * SROW + (32 * dd + 8 * i4 + 4 * L.g) * 2) = r;
+                }
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int c = j * 64 + L.lane, row = c >> 3, col = c & 7;
+                const bf16x8 val = *(const bf16x8*)(stage + row * SROW + col * 16);
+                if (tok0 + row < p.n) *(bf16x8*)(ob + (long)(tok0 + row) * p.o_tok + 64 * qd + col * 8) = val;
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ exact pass
+// Classic online softmax over one work item, one 32-key block at a time, nothing overlapped: the rare fallback, in a
+// kernel of its own because its accumulator rescaling (vector ALU on all of O) would cost the fast pass its register
+// allocation.
+template <int D, int RT, bool WIN>
+__device__ __forceinline__ void attn_item_exact(const AttnParams& p, const int4 item, char* buf0, int2* ent, char* stage) {
+    using G = Geo<D>;
+    constexpr int NS = D / 16, NDT = D / 32;
+    const Lane<D> L(p);
+    const int t = item.x, e0 = item.y, ne = item.z & 0xfffff, hp = (unsigned)item.z >> 20;
     const int h0 = hp * RT, kvh = h0 / p.group;
-    const int tok = t * SPINF_QTILE + 32 * w + m;
+    const int tok = t * SPINF_QTILE + 32 * L.w + L.m;
     const int tok_c = tok < p.n ? tok : p.n - 1;
-
-    // per-lane part of the DMA source addresses (bytes): row slot of the region and 16-byte chunk
-    const unsigned lane_k = (unsigned)((lane / G::CPR) * G::NREG * p.k_tok * 2 + (lane % G::CPR) * 16);
-    const unsigned lane_v = (unsigned)((lane / G::CPR) * G::NREG * p.v_tok * 2 + (lane % G::CPR) * 16);
-
-    const int e0 = p.qt_ptr[t], e1 = p.qt_ptr[t + 1];
-    const int ne = e1 - e0;
-
     bf16x8 qf[RT][NS];
 #pragma unroll
     for (int rt = 0; rt < RT; rt++) {
-        const __bf16* qp = p.q + (long)tok_c * p.q_tok + (long)(h0 + rt) * p.q_head + 8 * g;
+        const __bf16* qp = p.q + (long)tok_c * p.q_tok + (long)(h0 + rt) * p.q_head + 8 * L.g;
 #pragma unroll
         for (int s = 0; s < NS; s++) qf[rt][s] = *(const bf16x8*)(qp + 16 * s);
     }
     const int art_q = tok < p.n ? p.art[tok_c] : -1;
     const int pos_q = WIN ? p.pos[tok_c] : 0;
-
     f32x16 o[RT][NDT];
     float M[RT], l[RT];
-    bool viol = false;
-    PH_DECL
-
-    // lane parts of the LDS addresses.  K fragment: row m of the 32-key block, 16-byte chunk g of each 32-byte step.
-    // V^T fragment (ds_read_b64_tr_b16): inside its 16-lane group a lane supplies the address of key row 4g + tr_j,
-    // head dims 16 tr_mb + 4 tr_a .. +3 of the 32-wide slice, and receives head dim lane%32 of 4 consecutive keys.
-    const int tr_a = lane & 3, tr_j = (lane >> 2) & 3, tr_mb = (lane >> 4) & 1;
-    const int k_lane = G::k_off(m) + 16 * g;
-    const int v_lane = G::v_off(4 * g + tr_j) + 32 * tr_mb + 8 * tr_a;
-
-    // ---- one 32-key block of the current tile against this wave's 32 query rows (x RT heads)
-    auto block = [&](const char* kb, const char* vb, const int* meta, const int kt, const int sub, const bool needmask)
-                     __attribute__((always_inline)) {
-        // rows 32 sub .. 32 sub + 31 of the tile sit in region slot(s) sub * 32 / NREG: a runtime byte offset
-        const char* krow = kb + k_lane + sub * (32 / G::NREG) * G::ROWB;
-        const char* vrow = vb + v_lane + sub * (32 / G::NREG) * G::ROWB;
-
-        // S^T = K Q^T : rows = 32 keys, columns = this wave's 32 query rows; K fragments run PF reads ahead of the MFMAs
-        f32x16 s_acc[RT];
 #pragma unroll
-        for (int rt = 0; rt < RT; rt++)
+    for (int rt = 0; rt < RT; rt++) {
+        M[rt] = -INFINITY;
+        l[rt] = 0.f;
 #pragma unroll
-            for (int i2 = 0; i2 < 16; i2++) s_acc[rt][i2] = 0.f;
-        {
-            constexpr int PF = KPF < NS ? KPF : NS;
-            bf16x8 kf[PF];
+        for (int dt = 0; dt < NDT; dt++)
 #pragma unroll
-            for (int s = 0; s < PF; s++) kf[s] = *(const bf16x8*)(krow + 32 * s);
-            __builtin_amdgcn_sched_barrier(0);
+            for (int i = 0; i < 16; i++) o[rt][dt][i] = 0.f;
+    }
+    int base = 0;
+    __syncthreads();
+    if ((int)threadIdx.x < ne) ent[threadIdx.x] = make_int2(p.kv_idx[e0 + threadIdx.x], (int)p.kv_bits[e0 + threadIdx.x]);
+    __syncthreads();
+    for (int i = 0; i < ne; i++) {
+        if (i - base >= ENT_CAP) {
+            __syncthreads();
+            base = i;
+            if (i + (int)threadIdx.x < ne) ent[threadIdx.x] = make_int2(p.kv_idx[e0 + i + threadIdx.x], (int)p.kv_bits[e0 + i + threadIdx.x]);
+            __syncthreads();
+        }
+        const int2 en = ent[i - base];
+        const int kt = __builtin_amdgcn_readfirstlane(en.x);
+        const unsigned bits = (unsigned)__builtin_amdgcn_readfirstlane(en.y) >> (2 * L.w);
+        __syncthreads();   // everyone is done with the buffer
+        issue_tile<D>(p, lds_addr(buf0), kt, kvh, L.w, L.lane, L.lane_k, L.lane_v);
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        __syncthreads();
+        const char* kb = buf0;
+        const char* vb = buf0 + G::KTILEB;
+        const int* meta = (const int*)(buf0 + G::KTILEB + G::VTILEB);
+#pragma unroll 1
+        for (int sub = 0; sub < 2; sub++) {
+            if (!((bits >> sub) & 1u)) continue;
+            const char* krow = kb + L.k_lane + sub * G::SUBB;
+            const char* vrow = vb + L.v_lane + sub * G::SUBB;
+            f32x16 s_acc[RT];
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++)
+#pragma unroll
+                for (int i2 = 0; i2 < 16; i2++) s_acc[rt][i2] = 0.f;
 #pragma unroll
             for (int s = 0; s < NS; s++) {
+                const bf16x8 kf = *(const bf16x8*)(krow + 32 * s);
 #pragma unroll
-                for (int rt = 0; rt < RT; rt++)
-                    s_acc[rt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[s % PF], qf[rt][s], s_acc[rt], 0, 0, 0);
-                if (s + PF < NS) kf[s % PF] = *(const bf16x8*)(krow + 32 * (s + PF));
-                __builtin_amdgcn_sched_barrier(0);
+                for (int rt = 0; rt < RT; rt++) s_acc[rt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[rt][s], s_acc[rt], 0, 0, 0);
             }
-        }
-        PH_MARK(1);
-        // V^T fragments (fragment f = 16-key half f / NDT, head-dim slice f % NDT): the first VPF are in flight while the
-        // softmax runs, the rest replace them as they are consumed
-        constexpr int NVF = 2 * NDT;
-        constexpr int VPF_ = VPF < NVF ? VPF : NVF;
-        s16x4 vlo[VPF_], vhi[VPF_];
-        auto vload = [&](const int f, const int slot) __attribute__((always_inline)) {
-            const char* vp = vrow + G::v_off(16 * (f / NDT)) + 64 * (f % NDT);
-            vlo[slot] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)vp);
-            vhi[slot] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vp + G::v_off(8)));
-        };
+            if ((bits >> (8 + sub)) & 1u) apply_mask<RT, WIN>(s_acc, meta, kt, sub, L.g, tok, art_q, pos_q, p.window);
+            bf16x8 pb[RT][2];
 #pragma unroll
-        for (int f = 0; f < VPF_; f++) vload(f, f);
-        __builtin_amdgcn_sched_barrier(0);
-
-        // mask (register i of the result holds key 8*(i/4) + 4g + i%4 of the block)
-        if (needmask) {
+            for (int rt = 0; rt < RT; rt++) {
+                float mx = s_acc[rt][0];
 #pragma unroll
-            for (int i4 = 0; i4 < 4; i4++) {
-                const int ko = 32 * sub + 8 * i4 + 4 * g;
-                const int4 ka = *(const int4*)(meta + ko);
-                const int4 ke = *(const int4*)(meta + 64 + ko);
-                int4 kp = make_int4(0, 0, 0, 0);
-                if (WIN) kp = *(const int4*)(meta + 128 + ko);
-                const int kg = kt * 64 + ko;
-                const int kav[4] = {ka.x, ka.y, ka.z, ka.w};
-                const int kev[4] = {ke.x, ke.y, ke.z, ke.w};
-                const int kpv[4] = {kp.x, kp.y, kp.z, kp.w};
-#pragma unroll
-                for (int jj = 0; jj < 4; jj++) {
-                    const int kk = kg + jj;
-                    bool vis = (kk <= tok) & (art_q >= 0) & (kav[jj] == art_q) & (tok < kev[jj]);
-                    vis = vis | (kk == tok);
-                    if (WIN) vis = vis & ((pos_q - kpv[jj]) < p.window);
-#pragma unroll
-                    for (int rt = 0; rt < RT; rt++) s_acc[rt][4 * i4 + jj] = vis ? s_acc[rt][4 * i4 + jj] : -INFINITY;
-                }
-            }
-        }
-
-        // softmax numerators, one query row per lane pair (lane, lane^32)
-        bf16x8 pb[RT][2];
-#pragma unroll
-        for (int rt = 0; rt < RT; rt++) {
-            float mx = s_acc[rt][0];
-#pragma unroll
-            for (int i2 = 1; i2 < 16; i2++) mx = fmaxf(mx, s_acc[rt][i2]);
-            mx = lane32_max(mx);
-            const float tm = mx * p.c;
-            if (EXACT) {
+                for (int i2 = 1; i2 < 16; i2++) mx = fmaxf(mx, s_acc[rt][i2]);
+                mx = lane32_max(mx);
+                const float tm = mx * p.c;
                 const bool up = tm > M[rt] + TAU_LAZY;
                 const float mn = up ? tm : M[rt];
                 const float alpha = up ? __builtin_amdgcn_exp2f(M[rt] - mn) : 1.0f;
@@ -280,45 +331,144 @@ __device__ __forceinline__ bool attn_tile(const AttnParams& p, char* buf0, char*
                 }
                 l[rt] *= alpha;
                 M[rt] = mn;
-            } else {
-                const bool first = M[rt] == -INFINITY;
-                viol = viol | (!first & (tm > M[rt] + TAU_FAST));
-                M[rt] = first ? tm : M[rt];
-            }
-            const float ms = M[rt] == -INFINITY ? 0.f : M[rt];
-            float sum = 0.f;
-            float pv[16];
+                const float ms = mn == -INFINITY ? 0.f : mn;
+                float sum = 0.f;
 #pragma unroll
-            for (int i2 = 0; i2 < 16; i2++) {
-                pv[i2] = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[rt][i2], p.c, -ms));
-                sum += pv[i2];
+                for (int i2 = 0; i2 < 16; i2++) {
+                    const float pr = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[rt][i2], p.c, -ms));
+                    sum += pr;
+                    pb[rt][i2 >> 3][i2 & 7] = (__bf16)pr;
+                }
+                l[rt] += sum;
             }
-            l[rt] += sum;
 #pragma unroll
-            for (int i2 = 0; i2 < 8; i2++) {
-                pb[rt][0][i2] = (__bf16)pv[i2];
-                pb[rt][1][i2] = (__bf16)pv[8 + i2];
+            for (int f = 0; f < 2 * NDT; f++) {
+                const char* vp = vrow + G::v_off(16 * (f / NDT)) + 64 * (f % NDT);
+                const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)vp);
+                const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vp + G::v_off(8)));
+                const bf16x8 a = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+#pragma unroll
+                for (int rt = 0; rt < RT; rt++) o[rt][f % NDT] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[rt][f / NDT], o[rt][f % NDT], 0, 0, 0);
             }
         }
-        __builtin_amdgcn_sched_barrier(0);
+    }
+    store_rows<D, RT>(p, L, stage, o, l, t, h0);
+}
 
-        PH_MARK(2);
-        // O^T += V^T P^T : rows = 32 head dims, columns = query rows, contraction = 16 keys per MFMA
-#pragma unroll
-        for (int f = 0; f < NVF; f++) {
-            const s16x8 av = __builtin_shufflevector(vlo[f % VPF_], vhi[f % VPF_], 0, 1, 2, 3, 4, 5, 6, 7);
-            const bf16x8 a = __builtin_bit_cast(bf16x8, av);
-#pragma unroll
-            for (int rt = 0; rt < RT; rt++)
-                o[rt][f % NDT] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[rt][f / NDT], o[rt][f % NDT], 0, 0, 0);
-            if (f + VPF_ < NVF) vload(f + VPF_, f % VPF_);
-            __builtin_amdgcn_sched_barrier(0);
+template <int D, int RT, bool WIN>
+__global__ __launch_bounds__(256) void tree_attn_exact_kernel(const AttnParams p) {
+    using G = Geo<D>;
+    __shared__ __attribute__((aligned(16))) char buf0[G::BUFB];
+    __shared__ int2 ent[ENT_CAP];
+    __shared__ __attribute__((aligned(16))) char stage_all[4 * 32 * 144];
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n_redo = p.counters[NLIST + 1];
+    for (int j = blockIdx.x; j < n_redo; j += gridDim.x) {
+        const int4 it = p.items[p.redo[j]];
+        const int4 item = make_int4(__builtin_amdgcn_readfirstlane(it.x), __builtin_amdgcn_readfirstlane(it.y),
+                                    __builtin_amdgcn_readfirstlane(it.z), __builtin_amdgcn_readfirstlane(it.w));
+        attn_item_exact<D, RT, WIN>(p, item, buf0, ent, stage_all + w * 32 * 144);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0f70);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        __threadfence();
+        if (atomicAdd(&p.counters[NLIST + 2], 1) == (int)gridDim.x - 1) {
+            p.counters[NLIST + 1] = 0;
+            p.counters[NLIST + 2] = 0;
+            __threadfence();
         }
-        PH_MARK(3);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ fast pass, persistent
+#ifdef SPINF_TRACE
+__device__ long g_trace[16 * 4096];
+extern "C" int spinf_debug_trace(long* out, int n) { return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_trace), sizeof(long) * n, 0, hipMemcpyDeviceToHost); }
+#define TRACE_ADD(slot, val) do { if (threadIdx.x == 64 && blockIdx.x < 4096) g_trace[blockIdx.x * 16 + (slot)] += (val); } while (0)
+#define TRACE_CLK(var) const long var = clock64()
+#else
+#define TRACE_ADD(slot, val) do { } while (0)
+#define TRACE_CLK(var) do { } while (0)
+#endif
+
+template <int D, int RT, bool WIN>
+__global__ __launch_bounds__(256) void tree_attn_kernel(const AttnParams p) {
+    using G = Geo<D>;
+    constexpr int NS = D / 16;     // contraction steps of K Q^T
+    constexpr int NDT = D / 32;    // 32-wide slices of the head dimension in O^T
+    constexpr int NVF = 2 * NDT;   // V^T fragments of one 32-key block
+    constexpr int PFD = D >= 256 ? 4 : 8;   // fragment read-ahead depth: the vector register file (256) is the tight one at head dim 256
+    constexpr int PF = NS < PFD ? NS : PFD;     // K fragments read ahead of the MFMAs
+    constexpr int VPF = NVF < PFD ? NVF : PFD;  // V^T fragments read ahead
+    constexpr int EK = 16 / NS;    // softmax elements folded into one K Q^T step
+    constexpr int EV = (16 + NVF - 1) / NVF;   // ... into one P V step
+    __shared__ __attribute__((aligned(16))) char bufs[2 * G::BUFB];   // the two tile buffers
+    __shared__ int2 ent_a[ENT_CAP];   // (key tile, bits) of the current item's plan entries base .. base + ENT_CAP - 1
+    __shared__ int2 ent_b[ENT_CAP];   // first entries of the next item
+    __shared__ __attribute__((aligned(16))) char stage_all[4 * 32 * 144];
+    __shared__ int s_next[2];         // item grabbed by thread 0 for the whole workgroup, double buffered
+
+    const Lane<D> L(p);
+    char* stage = stage_all + L.w * 32 * 144;
+
+    // ---- work lists: start with the list of this workgroup's XCD, continue with the following ones
+    unsigned xcc;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+    int my_list = (int)(xcc & 7u), lists_done = 0;    // thread 0 only
+    auto grab = [&](const int slot) __attribute__((always_inline)) {   // thread 0: next item index into s_next[slot], -1 when all lists are empty
+        if (threadIdx.x == 0) {
+            int idx = -1;
+            while (lists_done < NLIST) {
+                const int lo = p.list_ptr[my_list], hi = p.list_ptr[my_list + 1];
+                const int j = lo + atomicAdd(&p.counters[my_list], 1);
+                if (j < hi) { idx = j; break; }
+                my_list = (my_list + 1) & (NLIST - 1);
+                lists_done++;
+            }
+            s_next[slot] = idx;
+        }
     };
 
-    // ---- one pass over the tile's key list
-    {
+    // ---- per-item state
+    int4 cur = make_int4(0, 0, 0, 0), nxt = make_int4(0, 0, 0, 0);
+    int cur_idx = -1, nxt_idx = -1;
+    bool cur_ok = false, nxt_ok = false;
+    bf16x8 qf[RT][NS];
+    int art_q = -1, pos_q = 0;
+    f32x16 o[RT][NDT];
+    float M[RT], l[RT];
+    bool viol = false;
+    int2* ent_cur = ent_a;
+    int2* ent_nxt = ent_b;
+
+    auto uniform4 = [](const int4 v) __attribute__((always_inline)) {   // the same value in every lane: keep it in scalar registers
+        return make_int4(__builtin_amdgcn_readfirstlane(v.x), __builtin_amdgcn_readfirstlane(v.y), __builtin_amdgcn_readfirstlane(v.z),
+                         __builtin_amdgcn_readfirstlane(v.w));
+    };
+    auto item_t = [](const int4& it) { return it.x; };
+    auto item_ne = [](const int4& it) { return it.z & 0xfffff; };
+    auto item_hp = [](const int4& it) { return (int)((unsigned)it.z >> 20); };
+
+    auto load_q = [&](const int4& it, bf16x8 (&dst)[RT][NS], int& a_q, int& p_q) __attribute__((always_inline)) {
+        const int tok = item_t(it) * SPINF_QTILE + 32 * L.w + L.m;
+        const int tok_c = tok < p.n ? tok : p.n - 1;
+        const int h0 = item_hp(it) * RT;
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++) {
+            const __bf16* qp = p.q + (long)tok_c * p.q_tok + (long)(h0 + rt) * p.q_head + 8 * L.g;
+#pragma unroll
+            for (int s = 0; s < NS; s++) dst[rt][s] = *(const bf16x8*)(qp + 16 * s);
+        }
+        a_q = tok < p.n ? p.art[tok_c] : -1;
+        p_q = WIN ? p.pos[tok_c] : 0;
+    };
+    auto load_ent = [&](const int4& it, int2* dst, const int from) __attribute__((always_inline)) {
+        const int ne = item_ne(it);
+        if (from + (int)threadIdx.x < ne)
+            dst[threadIdx.x] = make_int2(p.kv_idx[it.y + from + threadIdx.x], (int)p.kv_bits[it.y + from + threadIdx.x]);
+    };
+    auto reset_acc = [&]() __attribute__((always_inline)) {
 #pragma unroll
         for (int rt = 0; rt < RT; rt++) {
             M[rt] = -INFINITY;
@@ -326,177 +476,342 @@ __device__ __forceinline__ bool attn_tile(const AttnParams& p, char* buf0, char*
 #pragma unroll
             for (int dt = 0; dt < NDT; dt++)
 #pragma unroll
-                for (int i2 = 0; i2 < 16; i2++) o[rt][dt][i2] = 0.f;
+                for (int i = 0; i < 16; i++) o[rt][dt][i] = 0.f;
         }
-        int base = 0;
-        __syncthreads();   // nobody still reads the entry window or the buffers of the fast pass
-        if ((int)threadIdx.x < ne) ent[threadIdx.x] = make_int2(p.kv_idx[e0 + threadIdx.x], (int)p.kv_bits[e0 + threadIdx.x]);
-        __syncthreads();
-        if (ne > 0) issue_tile<D>(p, buf0, __builtin_amdgcn_readfirstlane(ent[0].x), kvh, w, lane, lane_k, lane_v);
-        TRACE(2, (long)clock64());
-        PH_START;
-        auto step = [&](char* buf, char* nxt, const int i) __attribute__((always_inline)) {
-            __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's DMA into buf has landed
-            __syncthreads();                     // ... and everyone's; the other buffer is free again
-            if (i + 1 - base >= ENT_CAP) {       // slide the window of plan entries (uniform; rare)
+        viol = false;
+    };
+
+    // ---- compute pieces
+    auto sm_head = [&](const int rt, const f32x16& sv) __attribute__((always_inline)) -> float {
+        float mx = sv[0];
+#pragma unroll
+        for (int i2 = 1; i2 < 16; i2++) mx = fmaxf(mx, sv[i2]);
+        mx = lane32_max(mx);
+        const float tm = mx * p.c;
+        const bool first = M[rt] == -INFINITY;
+        viol = viol | (!first & (tm > M[rt] + TAU_FAST));
+        M[rt] = first ? tm : M[rt];
+        return M[rt] == -INFINITY ? 0.f : M[rt];
+    };
+    auto sm_elem = [&](const f32x16& sv, const int i2, const float ms, float& sum, bf16x8 (&pb)[2]) __attribute__((always_inline)) {
+        const float pr = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[i2], p.c, -ms));
+        sum += pr;
+        pb[i2 >> 3][i2 & 7] = (__bf16)pr;
+    };
+    // S^T = K Q^T for one 32-key block; `shadow(s)` is vector-ALU work of another block slotted in after step s
+    auto qk_phase = [&](const char* krow, f32x16 (&s_acc)[RT], auto shadow) __attribute__((always_inline)) {
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++)
+#pragma unroll
+            for (int i2 = 0; i2 < 16; i2++) s_acc[rt][i2] = 0.f;
+        bf16x8 kf[PF];
+#pragma unroll
+        for (int s = 0; s < PF; s++) kf[s] = *(const bf16x8*)(krow + 32 * s);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < NS; s++) {
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++)
+                s_acc[rt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[s % PF], qf[rt][s], s_acc[rt], 0, 0, 0);
+            if (s + PF < NS) kf[s % PF] = *(const bf16x8*)(krow + 32 * (s + PF));
+            shadow(s);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    // O^T += V^T P^T for one 32-key block
+    auto pv_phase = [&](const char* vrow, const bf16x8 (&pb)[RT][2], auto shadow) __attribute__((always_inline)) {
+        s16x4 vlo[VPF], vhi[VPF];
+        auto vload = [&](const int f, const int slot) __attribute__((always_inline)) {
+            const char* vp = vrow + G::v_off(16 * (f / NDT)) + 64 * (f % NDT);
+            vlo[slot] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)vp);
+            vhi[slot] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vp + G::v_off(8)));
+        };
+#pragma unroll
+        for (int f = 0; f < VPF; f++) vload(f, f);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int f = 0; f < NVF; f++) {
+            const bf16x8 a = __builtin_bit_cast(bf16x8, __builtin_shufflevector(vlo[f % VPF], vhi[f % VPF], 0, 1, 2, 3, 4, 5, 6, 7));
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++)
+                o[rt][f % NDT] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[rt][f / NDT], o[rt][f % NDT], 0, 0, 0);
+            if (f + VPF < NVF) vload(f + VPF, f % VPF);
+            shadow(f);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    auto no_shadow = [](const int) __attribute__((always_inline)) {};
+    // softmax of a whole block spread over `steps` shadow slots, `per` elements each
+    auto compute_tile = [&](const char* buf, const int kt, const unsigned bits) __attribute__((always_inline)) {
+        const bool a0 = bits & 1u, a1 = bits & 2u;
+        if (!a0 && !a1) return;   // wave-uniform: no row of this wave sees a key of the tile
+        const char* kb = buf + L.k_lane;
+        const char* vb = buf + G::KTILEB + L.v_lane;
+        const int* meta = (const int*)(buf + G::KTILEB + G::VTILEB);
+        const int tok = item_t(cur) * SPINF_QTILE + 32 * L.w + L.m;
+        if (a0 && a1) {
+            // both blocks: K Q^T(0) | K Q^T(1) with softmax(0) in its shadow | P V(0) with softmax(1) in its shadow | P V(1)
+            f32x16 sa[RT], sb[RT];
+            bf16x8 pa[RT][2], pb[RT][2];
+            float ms[RT], sum[RT];
+            qk_phase(kb, sa, no_shadow);
+            if ((bits >> 8) & 1u) apply_mask<RT, WIN>(sa, meta, kt, 0, L.g, tok, art_q, pos_q, p.window);
+            qk_phase(kb + G::SUBB, sb, [&](const int s) __attribute__((always_inline)) {
+                if (s == 0) {
+#pragma unroll
+                    for (int rt = 0; rt < RT; rt++) { ms[rt] = sm_head(rt, sa[rt]); sum[rt] = 0.f; }
+                }
+#pragma unroll
+                for (int rt = 0; rt < RT; rt++)
+#pragma unroll
+                    for (int e = 0; e < EK; e++) sm_elem(sa[rt], s * EK + e, ms[rt], sum[rt], pa[rt]);
+            });
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++) l[rt] += sum[rt];
+            if ((bits >> 9) & 1u) apply_mask<RT, WIN>(sb, meta, kt, 1, L.g, tok, art_q, pos_q, p.window);
+            pv_phase(vb, pa, [&](const int f) __attribute__((always_inline)) {
+                if (f == 0) {
+#pragma unroll
+                    for (int rt = 0; rt < RT; rt++) { ms[rt] = sm_head(rt, sb[rt]); sum[rt] = 0.f; }
+                }
+#pragma unroll
+                for (int rt = 0; rt < RT; rt++)
+#pragma unroll
+                    for (int e = 0; e < EV; e++)
+                        if (f * EV + e < 16) sm_elem(sb[rt], f * EV + e, ms[rt], sum[rt], pb[rt]);
+            });
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++) l[rt] += sum[rt];
+            pv_phase(vb + G::SUBB, pb, no_shadow);
+        } else {
+            const int sub = a0 ? 0 : 1;
+            f32x16 sa[RT];
+            bf16x8 pa[RT][2];
+            qk_phase(kb + sub * G::SUBB, sa, no_shadow);
+            if ((bits >> (8 + sub)) & 1u) apply_mask<RT, WIN>(sa, meta, kt, sub, L.g, tok, art_q, pos_q, p.window);
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++) {
+                const float ms = sm_head(rt, sa[rt]);
+                float sum = 0.f;
+#pragma unroll
+                for (int i2 = 0; i2 < 16; i2++) sm_elem(sa[rt], i2, ms, sum, pa[rt]);
+                l[rt] += sum;
+            }
+            pv_phase(vb + sub * G::SUBB, pa, no_shadow);
+        }
+    };
+
+    // ---- prologue: first item, its queries, entries and first tile; the second item is grabbed right away
+    grab(0);
+    __syncthreads();
+    {
+        cur_idx = __builtin_amdgcn_readfirstlane(s_next[0]);
+        cur_ok = cur_idx >= 0;
+        if (cur_ok) cur = uniform4(p.items[cur_idx]);
+    }
+    if (cur_ok) {
+        load_q(cur, qf, art_q, pos_q);
+        load_ent(cur, ent_cur, 0);
+        issue_tile<D>(p, lds_addr(bufs), cur.w, item_hp(cur) * RT / p.group, L.w, L.lane, L.lane_k, L.lane_v);
+    }
+    grab(1);
+    int gslot = 1;      // slot of s_next that holds the item after `cur`
+    int i = 0;          // tile step inside the current item
+    int base = 0;       // first plan entry held in ent_cur
+    int pstage = 0;     // next-item prefetch: 0 nothing, 1 descriptor known, 2 entries requested, 3 first tile requested
+
+    // Item loop around a tile loop (two real loop levels on purpose: the accumulators are touched by the vector ALU only
+    // outside the tile loop, so inside it they stay in the MFMA accumulator registers).
+    // One tile step = one key tile of the current item from buffer `par`, the next tile (of this item or of the next one)
+    // requested into the other buffer.
+    int par = 0;
+    while (cur_ok) {
+        const int ne = item_ne(cur);
+        const int kvh = item_hp(cur) * RT / p.group;
+        reset_acc();
+        base = 0;
+        pstage = 0;
+        for (i = 0; i < ne; i++, par ^= 1) {
+            const char* buf = bufs + par * G::BUFB;
+            const unsigned oth = lds_addr(bufs + (par ^ 1) * G::BUFB);
+            TRACE_CLK(tc0);
+            __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's DMA into buf (and its other loads) have landed
+            __syncthreads();                     // ... and everyone's; the other buffer is free; s_next[gslot] is visible
+            TRACE_CLK(tc1);
+            TRACE_ADD(8, tc1 - tc0);
+            // next-item prefetch, one stage per step
+            if (pstage == 0) {
+                nxt_idx = __builtin_amdgcn_readfirstlane(s_next[gslot]);
+                nxt_ok = nxt_idx >= 0;
+                if (nxt_ok) nxt = uniform4(p.items[nxt_idx]);
+                pstage = 1;
+            } else if (pstage == 1) {
+                if (nxt_ok) load_ent(nxt, ent_nxt, 0);
+                pstage = 2;
+            }
+            if (i + 1 - base >= ENT_CAP) {       // slide the window of plan entries (uniform; long key lists only)
                 base = i;
-                if (i + (int)threadIdx.x < ne) ent[threadIdx.x] = make_int2(p.kv_idx[e0 + i + threadIdx.x], (int)p.kv_bits[e0 + i + threadIdx.x]);
+                load_ent(cur, ent_cur, i);
                 __syncthreads();
             }
-#if SPINF_ABL != 1
-            if (i + 1 < ne) issue_tile<D>(p, nxt, __builtin_amdgcn_readfirstlane(ent[i + 1 - base].x), kvh, w, lane, lane_k, lane_v);
-#endif
-            const int2 en = ent[i - base];
-            const int kt = __builtin_amdgcn_readfirstlane(en.x);
-            const unsigned bits = (unsigned)__builtin_amdgcn_readfirstlane(en.y) >> (2 * w);
-            const char* kb = buf;
-            const char* vb = buf + G::KTILEB;
-            const int* meta = (const int*)(buf + G::KTILEB + G::VTILEB);
-            PH_MARK(0);
-#pragma unroll 1
-            for (int sub = 0; sub < 2; sub++) {
-                if (!((bits >> sub) & 1u)) continue;   // wave-uniform: no row of this wave sees these 32 keys
-#if SPINF_ABL != 2
-                block(kb, vb, meta, kt, sub, (bits >> (8 + sub)) & 1u);
-#endif
+            if (i + 1 < ne) {
+                issue_tile<D>(p, oth, __builtin_amdgcn_readfirstlane(ent_cur[i + 1 - base].x), kvh, L.w, L.lane, L.lane_k, L.lane_v);
+            } else if (nxt_ok) {
+                issue_tile<D>(p, oth, nxt.w, item_hp(nxt) * RT / p.group, L.w, L.lane, L.lane_k, L.lane_v);
+                pstage = pstage == 2 ? 3 : -1;   // -1: tile requested before the entries (one-tile items)
             }
-        };
-        for (int i = 0; i < ne; i += 2) {
-            step(buf0, buf1, i);
-            if (i + 1 < ne) step(buf1, buf0, i + 1);
+            const int2 en = ent_cur[i - base];
+            compute_tile(buf, __builtin_amdgcn_readfirstlane(en.x), (unsigned)__builtin_amdgcn_readfirstlane(en.y) >> (2 * L.w));
+            TRACE_CLK(tc2);
+            TRACE_ADD(9, tc2 - tc1);
+        }
+        // ---- item finished: output (or hand the item to the exact pass), switch to the next item
+        TRACE_CLK(tc3);
+        if (__builtin_amdgcn_readfirstlane(__syncthreads_or(viol))) {
+            if (threadIdx.x == 0) p.redo[atomicAdd(&p.counters[NLIST + 1], 1)] = cur_idx;
+        } else {
+            store_rows<D, RT>(p, L, stage, o, l, item_t(cur), item_hp(cur) * RT);
+        }
+        TRACE_CLK(tc4);
+        TRACE_ADD(10, tc4 - tc3);
+        TRACE_ADD(11, 1);
+        cur_ok = nxt_ok;
+        if (!cur_ok) break;
+        // finish whatever of the next item's prefetch has not happened yet (one-tile items), then switch
+        if (pstage == -1) load_ent(nxt, ent_nxt, 0);
+        cur = nxt;
+        cur_idx = nxt_idx;
+        load_q(cur, qf, art_q, pos_q);
+        { int2* tmp = ent_cur; ent_cur = ent_nxt; ent_nxt = tmp; }
+        gslot ^= 1;
+        grab(gslot);     // the item after the new current one; read at the next tile step's barrier
+    }
+    // ---- the last workgroup to finish resets the counters for the next launch
+    __builtin_amdgcn_s_waitcnt(0x0f70);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        __threadfence();
+        const int done = atomicAdd(&p.counters[NLIST], 1);
+        if (done == (int)gridDim.x - 1) {
+            for (int k = 0; k < NLIST; k++) p.counters[k] = 0;
+            p.counters[NLIST] = 0;
+            __threadfence();
         }
     }
-    TRACE(3, (long)clock64());
-    TRACE(6, (long)ne);
-    if (!EXACT && __syncthreads_or(viol)) return true;
+}
 
-    // ---- epilogue: normalise, transpose through LDS and store whole rows.  Register i of O^T[dt] is head dim
-    // 32dt + 8(i/4) + 4g + i%4 of row `tok`; each wave stages its 32 rows in its own slice of the (now idle) tile buffers
-    // and writes them out as 16-byte pieces, 32 lanes per row.
-    __syncthreads();   // every wave is done with the tile buffers
-    {
-        constexpr int SROW = G::ROWB + 16;
-        static_assert(2 * 32 * SROW <= G::BUFB, "output staging must fit the tile buffers");
-        char* stage = ((w & 2) ? buf1 : buf0) + (w & 1) * 32 * SROW;
-        const int tok0 = t * SPINF_QTILE + 32 * w;
-#pragma unroll
-        for (int rt = 0; rt < RT; rt++) {
-            const float inv = 1.0f / lane32_sum(l[rt]);
-#pragma unroll
-            for (int dt = 0; dt < NDT; dt++)
-#pragma unroll
-                for (int i4 = 0; i4 < 4; i4++) {
-                    bf16x4 r;
-#pragma unroll
-                    for (int jj = 0; jj < 4; jj++) r[jj] = (__bf16)(o[rt][dt][4 * i4 + jj] * inv);
-                    *(bf16x4*)(stage + m * SROW + (32 * dt + 8 * i4 + 4 * g) * 2) = r;
-                }
-            __bf16* ob = p.o + (long)(h0 + rt) * p.o_head;
-#pragma unroll
-            for (int j = 0; j < 32 * G::CPR / 64; j++) {
-                const int c = j * 64 + lane, row = c / G::CPR, col = c % G::CPR;
-                const bf16x8 val = *(const bf16x8*)(stage + row * SROW + col * 16);
-                if (tok0 + row < p.n) *(bf16x8*)(ob + (long)(tok0 + row) * p.o_tok + col * 8) = val;
-            }
+// ------------------------------------------------------------------------------------------------ host side
+namespace {
+
+struct DeviceState {
+    int* counters = nullptr;   // 64 ints of cursors and counts, then the redo list
+    long redo_cap = 0;
+    int cus = 0;
+};
+std::mutex g_mu;
+DeviceState g_dev[64];
+
+int device_state(DeviceState** out, long n_items) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= 64) return spinf_fail(SPINF_E_HIP, "tree_attn: hipGetDevice: %s", hipGetErrorString(e));
+    std::lock_guard<std::mutex> lock(g_mu);
+    DeviceState& s = g_dev[dev];
+    if (!s.cus) {
+        hipDeviceProp_t prop;
+        e = hipGetDeviceProperties(&prop, dev);
+        if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: hipGetDeviceProperties: %s", hipGetErrorString(e));
+        s.cus = prop.multiProcessorCount;
+    }
+    if (!s.counters || n_items > s.redo_cap) {   // first call on this device, or a bigger schedule than ever before
+        if (s.counters) {
+            e = hipFree(s.counters);   // waits for the device to drain
+            if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: hipFree: %s", hipGetErrorString(e));
+            s.counters = nullptr;
         }
+        const long cap = n_items < (1 << 16) ? (1 << 16) : 2 * n_items;
+        e = hipMalloc((void**)&s.counters, (64 + cap) * sizeof(int));
+        if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: hipMalloc: %s", hipGetErrorString(e));
+        e = hipMemset(s.counters, 0, 64 * sizeof(int));
+        if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: hipMemset: %s", hipGetErrorString(e));
+        s.redo_cap = cap;
     }
-    TRACE(4, (long)clock64());
-    TRACE(5, (long)__builtin_amdgcn_s_memrealtime());
-    {
-        unsigned hwid;
-        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
-        unsigned xcc;
-        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
-        TRACE(7, (long)hwid | ((long)xcc << 32));
-    }
-#ifdef SPINF_TRACE
-    if (threadIdx.x == 64 && blockIdx.x < 16384) {   // wave 1: time spent waiting (0), in K Q^T (1), softmax (2), P V (3)
-        g_trace[blockIdx.x * 16 + 8] = ph_acc[0]; g_trace[blockIdx.x * 16 + 9] = ph_acc[1];
-        g_trace[blockIdx.x * 16 + 10] = ph_acc[2]; g_trace[blockIdx.x * 16 + 11] = ph_acc[3];
-    }
-#endif
-    return false;
-}
-
-// the exact pass lives in its own, never inlined function: its accumulator rescaling (vector ALU on all of O) would
-// otherwise cost the fast pass its register allocation
-template <int D, int RT, bool WIN, int KPF, int VPF>
-__device__ __attribute__((noinline)) void attn_tile_exact(const AttnParams p, char* buf0, char* buf1, int2* ent) {   // by value: a reference would pin the kernel arguments in scratch
-    (void)attn_tile<D, RT, WIN, KPF, VPF, true>(p, buf0, buf1, ent);
-}
-
-template <int D, int RT, bool WIN, int KPF, int VPF>
-__global__ __launch_bounds__(256) void tree_attn_kernel(const AttnParams p) {
-    using G = Geo<D>;
-    // two tile buffers as DISTINCT LDS objects: the compiler then knows that the DMA writes into one of them cannot
-    // alias the fragment reads of the other, and does not make those reads wait for the DMA
-    __shared__ __attribute__((aligned(16))) char buf0[G::BUFB];
-    __shared__ __attribute__((aligned(16))) char buf1[G::BUFB];
-    __shared__ int2 ent[ENT_CAP];   // (key tile, bits) of plan entries base .. base + ENT_CAP - 1
-    if (attn_tile<D, RT, WIN, KPF, VPF, false>(p, buf0, buf1, ent)) attn_tile_exact<D, RT, WIN, KPF, VPF>(p, buf0, buf1, ent);
+    *out = &s;
+    return SPINF_OK;
 }
 
 template <int D, int RT, bool WIN>
-static int launch(const AttnParams& p, hipStream_t stream) {
+int launch(const AttnParams& p, int blocks, hipStream_t stream) {
     using G = Geo<D>;
-    static_assert(2 * G::BUFB + ENT_CAP * 8 <= 160 * 1024, "LDS budget");
-    // fragment prefetch depths: at head dim 256 with two heads per wave the accumulators and query fragments take 416 of the
-    // 512 registers, which leaves room for two fragments in flight; elsewhere eight
-    constexpr int KPF = (D == 256 && RT == 2) ? 2 : 8;
-    constexpr int VPF = (D == 256 && RT == 2) ? 2 : 8;
-    hipLaunchKernelGGL((tree_attn_kernel<D, RT, WIN, KPF, VPF>), dim3(8 * p.per_xcd), dim3(256), 0, stream, p);
+    static_assert(2 * G::BUFB + 2 * ENT_CAP * 8 + 4 * 32 * 144 + 64 <= 160 * 1024, "LDS budget");
+    hipLaunchKernelGGL((tree_attn_kernel<D, RT, WIN>), dim3(blocks), dim3(256), 0, stream, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: launch: %s", hipGetErrorString(e));
+    // the exact pass over whatever the fast pass handed on (normally nothing: its workgroups read a zero count and leave)
+    hipLaunchKernelGGL((tree_attn_exact_kernel<D, RT, WIN>), dim3(blocks), dim3(256), 0, stream, p);
+    e = hipGetLastError();
+    if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: launch (exact pass): %s", hipGetErrorString(e));
     return SPINF_OK;
 }
 
 template <int D>
-static int launch_d(const AttnParams& p, int rt, bool win, hipStream_t s) {
-    if (rt == 2) return win ? launch<D, 2, true>(p, s) : launch<D, 2, false>(p, s);
-    return win ? launch<D, 1, true>(p, s) : launch<D, 1, false>(p, s);
+int launch_d(const AttnParams& p, int rt, bool win, int blocks, hipStream_t s) {
+    if (rt == 2) return win ? launch<D, 2, true>(p, blocks, s) : launch<D, 2, false>(p, blocks, s);
+    return win ? launch<D, 1, true>(p, blocks, s) : launch<D, 1, false>(p, blocks, s);
+}
+
+}  // namespace
+
+extern "C" int spinf_attn_heads_per_item(int32_t hq, int32_t hkv, int32_t d, int32_t variant) {
+    if (hq <= 0 || hkv <= 0 || hq % hkv) return 0;
+    const int group = hq / hkv;
+    // two heads of a GQA group per wave halve the LDS and L2 traffic per MFMA; at head dim 256 their accumulators and
+    // query fragments (384 registers, 512 with the next item's queries) do not fit, so that size runs one head per wave
+    int rt = (group % 2 == 0 && d <= 128) ? 2 : 1;
+    if (variant == 1) rt = 1;
+    return rt;
 }
 
 extern "C" int spinf_tree_attn_fwd(const spinf_attn_args* a, void* stream) {
     if (!a) return spinf_fail(SPINF_E_ARG, "tree_attn: null args");
-    if (a->n <= 0 || a->n_qtiles <= 0) return SPINF_OK;
-    if (!a->q || !a->k || !a->v || !a->out || !a->art || !a->end || !a->pos || !a->qt_ptr || !a->order)
+    if (a->n <= 0 || a->n_items <= 0) return SPINF_OK;
+    if (!a->q || !a->k || !a->v || !a->out || !a->art || !a->end || !a->pos || !a->kv_idx || !a->kv_bits || !a->items || !a->list_ptr)
         return spinf_fail(SPINF_E_ARG, "tree_attn: null pointer");
     if (a->d != 64 && a->d != 128 && a->d != 256) return spinf_fail(SPINF_E_ARG, "tree_attn: head dim %d not in {64,128,256}", a->d);
     if (a->hq <= 0 || a->hkv <= 0 || a->hq % a->hkv) return spinf_fail(SPINF_E_ARG, "tree_attn: hq %d not a multiple of hkv %d", a->hq, a->hkv);
     if (a->n > INT32_MAX / 2) return spinf_fail(SPINF_E_ARG, "tree_attn: stream too long");
-    if (a->n_qtiles != (a->n + SPINF_QTILE - 1) / SPINF_QTILE) return spinf_fail(SPINF_E_ARG, "tree_attn: plan has %lld query tiles, stream needs %lld", (long long)a->n_qtiles, (long long)((a->n + SPINF_QTILE - 1) / SPINF_QTILE));
     if (!(a->scale > 0.f)) return spinf_fail(SPINF_E_ARG, "tree_attn: scale must be positive");
+    const int rt = spinf_attn_heads_per_item(a->hq, a->hkv, a->d, a->variant);
+    const int64_t nqt = (a->n + SPINF_QTILE - 1) / SPINF_QTILE;
+    if (a->n_items != nqt * (a->hq / rt))
+        return spinf_fail(SPINF_E_ARG, "tree_attn: schedule has %lld items, %lld query tiles x %d head groups need %lld", (long long)a->n_items,
+                          (long long)nqt, a->hq / rt, (long long)(nqt * (a->hq / rt)));
     const int64_t strides[8] = {a->q_tok, a->q_head, a->k_tok, a->k_head, a->v_tok, a->v_head, a->o_tok, a->o_head};
     for (int i = 0; i < 8; i++)
         if (strides[i] % 8) return spinf_fail(SPINF_E_ARG, "tree_attn: strides must be multiples of 8 elements");
     const uintptr_t ptrs[4] = {(uintptr_t)a->q, (uintptr_t)a->k, (uintptr_t)a->v, (uintptr_t)a->out};
     for (int i = 0; i < 4; i++)
         if (ptrs[i] % 16) return spinf_fail(SPINF_E_ARG, "tree_attn: tensors must be 16-byte aligned");
-    const int group = a->hq / a->hkv;
-    // two heads of a GQA group per wave halve the LDS traffic per MFMA; at head dim 256 their accumulators and query
-    // fragments (384 registers) leave too little room, so that size runs one head per wave
-    int rt = (group % 2 == 0 && a->d <= 128) ? 2 : 1;
-    if (a->variant == 1) rt = 1;
-    if (a->variant == 2 && group % 2 == 0) rt = 2;
+    DeviceState* st = nullptr;
+    if (int rc = device_state(&st, (long)a->n_items)) return rc;
     AttnParams p;
     p.q = (const __bf16*)a->q; p.k = (const __bf16*)a->k; p.v = (const __bf16*)a->v; p.o = (__bf16*)a->out;
     p.q_tok = a->q_tok; p.q_head = a->q_head; p.k_tok = a->k_tok; p.k_head = a->k_head;
     p.v_tok = a->v_tok; p.v_head = a->v_head; p.o_tok = a->o_tok; p.o_head = a->o_head;
-    p.n = (int)a->n; p.group = group;
+    p.n = (int)a->n; p.group = a->hq / a->hkv;
     p.c = a->scale * 1.4426950408889634f;
     p.window = a->window > 0 ? a->window : 0;
     p.art = a->art; p.end = a->end; p.pos = a->pos;
-    p.qt_ptr = a->qt_ptr; p.kv_idx = a->kv_idx; p.kv_bits = a->kv_bits; p.order = a->order;
-    p.nqt = (int)a->n_qtiles;
-    const int64_t total = a->n_qtiles * (a->hq / rt);
-    if (total > INT32_MAX / 2) return spinf_fail(SPINF_E_ARG, "tree_attn: too many work items");
-    p.total = (int)total;
-    p.per_xcd = (int)((total + 7) / 8);
+    p.kv_idx = a->kv_idx; p.kv_bits = a->kv_bits;
+    p.items = (const int4*)a->items; p.list_ptr = a->list_ptr;
+    p.counters = st->counters;
+    p.redo = st->counters + 64;
+    const int blocks = (int)(a->n_items < st->cus ? a->n_items : st->cus);
     const bool win = p.window > 0;
     hipStream_t s = (hipStream_t)stream;
     switch (a->d) {
-        case 64: return launch_d<64>(p, rt, win, s);
-        case 128: return launch_d<128>(p, rt, win, s);
-        default: return launch_d<256>(p, rt, win, s);
+        case 64: return launch_d<64>(p, rt, win, blocks, s);
+        case 128: return launch_d<128>(p, rt, win, blocks, s);
+        default: return launch_d<256>(p, rt, win, blocks, s);
     }
 }

@@ -10,7 +10,7 @@ _LIB = None
 
 SYMBOLS = (
     "spinf_last_error", "spinf_version", "spinf_tileplan_build", "spinf_tileplan_counts", "spinf_tileplan_export",
-    "spinf_tileplan_free", "spinf_tree_attn_fwd", "spinf_gdn_fwd",
+    "spinf_tileplan_schedule", "spinf_tileplan_free", "spinf_attn_heads_per_item", "spinf_tree_attn_fwd", "spinf_gdn_fwd",
 )
 
 
@@ -21,8 +21,8 @@ class AttnArgs(C.Structure):
         ("v_tok", C.c_int64), ("v_head", C.c_int64), ("o_tok", C.c_int64), ("o_head", C.c_int64),
         ("n", C.c_int64), ("hq", C.c_int32), ("hkv", C.c_int32), ("d", C.c_int32), ("scale", C.c_float), ("window", C.c_int32),
         ("art", C.c_void_p), ("end", C.c_void_p), ("pos", C.c_void_p),
-        ("qt_ptr", C.c_void_p), ("kv_idx", C.c_void_p), ("kv_bits", C.c_void_p), ("order", C.c_void_p),
-        ("n_qtiles", C.c_int64), ("variant", C.c_int32),
+        ("kv_idx", C.c_void_p), ("kv_bits", C.c_void_p), ("items", C.c_void_p), ("list_ptr", C.c_void_p),
+        ("n_items", C.c_int64), ("variant", C.c_int32),
     ]
 
 
@@ -55,11 +55,14 @@ def load_library():
     lib.spinf_tileplan_build.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.POINTER(C.c_void_p)]
     lib.spinf_tileplan_counts.argtypes = [C.c_void_p, C.POINTER(C.c_int64)]
     lib.spinf_tileplan_export.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
+    lib.spinf_tileplan_schedule.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p]
+    lib.spinf_attn_heads_per_item.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_int32]
+    lib.spinf_attn_heads_per_item.restype = C.c_int
     lib.spinf_tileplan_free.argtypes = [C.c_void_p]
     lib.spinf_tileplan_free.restype = None
     lib.spinf_tree_attn_fwd.argtypes = [C.POINTER(AttnArgs), C.c_void_p]
     lib.spinf_gdn_fwd.argtypes = [C.POINTER(GdnArgs), C.c_void_p]
-    for name in ("spinf_tileplan_build", "spinf_tileplan_counts", "spinf_tileplan_export", "spinf_tree_attn_fwd", "spinf_gdn_fwd"):
+    for name in ("spinf_tileplan_build", "spinf_tileplan_counts", "spinf_tileplan_export", "spinf_tileplan_schedule", "spinf_tree_attn_fwd", "spinf_gdn_fwd"):
         getattr(lib, name).restype = C.c_int
     _LIB = lib
     return lib

@@ -22,7 +22,7 @@ VARIANT = 0  # kernel tuning variant handed to the library (0 = its default choi
 
 @torch.library.custom_op("spinf::tree_attn", mutates_args=())
 def _tree_attn_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, art: torch.Tensor, end: torch.Tensor, pos: torch.Tensor,
-                  qt_ptr: torch.Tensor, kv_idx: torch.Tensor, kv_bits: torch.Tensor, order: torch.Tensor,
+                  kv_idx: torch.Tensor, kv_bits: torch.Tensor, items: torch.Tensor, list_ptr: torch.Tensor, n_items: int,
                   scale: float, window: int, variant: int) -> torch.Tensor:
     """q [n, hq, d], k / v [n, hkv, d] (any token / head strides, d contiguous) -> out [n, hq, d] contiguous, bf16."""
     if not q.is_cuda:
@@ -46,8 +46,8 @@ def _tree_attn_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, art: torch.
     a.o_tok, a.o_head = out.stride(0), out.stride(1)
     a.n, a.hq, a.hkv, a.d, a.scale, a.window = n, hq, hkv, d, scale, window
     a.art, a.end, a.pos = art.data_ptr(), end.data_ptr(), pos.data_ptr()
-    a.qt_ptr, a.kv_idx, a.kv_bits, a.order = qt_ptr.data_ptr(), kv_idx.data_ptr(), kv_bits.data_ptr(), order.data_ptr()
-    a.n_qtiles = qt_ptr.numel() - 1
+    a.kv_idx, a.kv_bits, a.items, a.list_ptr = kv_idx.data_ptr(), kv_bits.data_ptr(), items.data_ptr(), list_ptr.data_ptr()
+    a.n_items = n_items
     a.variant = variant
     lib = _lib.load_library()
     with torch.cuda.device(q.device):
@@ -57,7 +57,7 @@ def _tree_attn_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, art: torch.
 
 
 @_tree_attn_op.register_fake
-def _(q, k, v, art, end, pos, qt_ptr, kv_idx, kv_bits, order, scale, window, variant):
+def _(q, k, v, art, end, pos, kv_idx, kv_bits, items, list_ptr, n_items, scale, window, variant):
     return torch.empty(q.shape, dtype=torch.bfloat16, device=q.device)
 
 
@@ -68,8 +68,14 @@ def tree_attn(q, k, v, mask: TreeMask, scale=None, variant=None):
     if q.shape[0] != mask.n:
         raise ValueError(f"mask describes {mask.n} tokens, q has {q.shape[0]}")
     scale = float(q.shape[-1] ** -0.5 if scale is None else scale)
-    return _tree_attn_op(q, k, v, mask.art, mask.end, mask.pos, mask.qt_ptr, mask.kv_idx, mask.kv_bits, mask.order,
-                         scale, int(mask.window), int(VARIANT if variant is None else variant))
+    variant = int(VARIANT if variant is None else variant)
+    hq, hkv, d = q.shape[1], k.shape[1], q.shape[2]
+    per_item = _lib.load_library().spinf_attn_heads_per_item(hq, hkv, d, variant)
+    if per_item <= 0:
+        raise ValueError(f"{hq} query heads do not group over {hkv} key / value heads")
+    items, list_ptr, n_items = mask.schedule(hq // per_item)
+    return _tree_attn_op(q, k, v, mask.art, mask.end, mask.pos, mask.kv_idx, mask.kv_bits, items, list_ptr, n_items,
+                         scale, int(mask.window), variant)
 
 
 # K/V capture for extraction, as spinf_serve/models/gemma4.py:66-70: while CAPTURE[device] = {"window", "ranges": [(start, n, key)],

@@ -9,25 +9,28 @@ library's tile-plan compiler.  No dense mask is built anywhere.
 from __future__ import annotations
 
 import ctypes as C
-from dataclasses import dataclass
-
 import numpy as np
 
 from . import _lib
 
 
-@dataclass
 class TilePlan:
-    """host arrays of a compiled plan (see include/spinf_tree.h)"""
+    """host arrays of a compiled plan (see include/spinf_tree.h) and the native handle that makes its work lists"""
 
-    qt_ptr: np.ndarray
-    kv_idx: np.ndarray
-    kv_bits: np.ndarray
-    order: np.ndarray
-    n: int
-    window: int
-    active_blocks: int
-    masked_blocks: int
+    def __init__(self, handle, qt_ptr, kv_idx, kv_bits, order, n, window, active_blocks, masked_blocks):
+        self._handle = handle
+        self.qt_ptr, self.kv_idx, self.kv_bits, self.order = qt_ptr, kv_idx, kv_bits, order
+        self.n, self.window = n, window
+        self.active_blocks, self.masked_blocks = active_blocks, masked_blocks
+        self._schedules = {}
+
+    def __del__(self):
+        h, self._handle = getattr(self, "_handle", None), None
+        if h:
+            try:
+                _lib.load_library().spinf_tileplan_free(h)
+            except Exception:  # noqa: BLE001  (interpreter shutdown)
+                pass
 
     @classmethod
     def build(cls, art, end, pos, window=None) -> "TilePlan":
@@ -50,13 +53,24 @@ class TilePlan:
             kv_bits = np.zeros(max(nent, 1), np.uint32)
             order = np.zeros(max(nqt, 1), np.int32)
             _lib.check(lib.spinf_tileplan_export(h, qt_ptr.ctypes.data, kv_idx.ctypes.data, kv_bits.ctypes.data, order.ctypes.data), "tileplan_export")
-        finally:
+        except Exception:
             lib.spinf_tileplan_free(h)
-        return cls(qt_ptr, kv_idx[:nent], kv_bits[:nent], order[:nqt], n, w, int(counts[2]), int(counts[3]))
+            raise
+        return cls(h, qt_ptr, kv_idx[:nent], kv_bits[:nent], order[:nqt], n, w, int(counts[2]), int(counts[3]))
 
     @property
     def n_qtiles(self) -> int:
         return len(self.order)
+
+    def schedule(self, head_groups: int):
+        """-> (items [n_qtiles * head_groups, 4] int32, list_ptr [9] int32): the kernel's work lists"""
+        got = self._schedules.get(head_groups)
+        if got is None:
+            items = np.zeros((max(self.n_qtiles * head_groups, 1), 4), np.int32)
+            list_ptr = np.zeros(9, np.int32)
+            _lib.check(_lib.load_library().spinf_tileplan_schedule(self._handle, head_groups, items.ctypes.data, list_ptr.ctypes.data), "tileplan_schedule")
+            got = self._schedules[head_groups] = (items[: self.n_qtiles * head_groups], list_ptr)
+        return got
 
 
 def _upload(a, dtype, device):
@@ -80,10 +94,19 @@ class TreeMask:
         self.device = device
         self.art, self.end, self.pos = meta
         one = np.zeros(1, np.int32)
-        self.qt_ptr = _upload(plan.qt_ptr, np.int32, device)
         self.kv_idx = _upload(plan.kv_idx if len(plan.kv_idx) else one, np.int32, device)
         self.kv_bits = _upload((plan.kv_bits if len(plan.kv_bits) else one.view(np.uint32)).view(np.int32), np.int32, device)
-        self.order = _upload(plan.order if len(plan.order) else one, np.int32, device)
+        self._sched = {}
+
+    def schedule(self, head_groups: int):
+        """device copy of the work lists for this many head groups (built on first use, then kept)"""
+        got = self._sched.get(head_groups)
+        if got is None:
+            items, list_ptr = self.plan.schedule(head_groups)
+            if not len(items):
+                items = np.zeros((1, 4), np.int32)
+            got = self._sched[head_groups] = (_upload(items, np.int32, self.device), _upload(list_ptr, np.int32, self.device), self.plan.n_qtiles * head_groups)
+        return got
 
     @classmethod
     def build(cls, art, end, pos, window=None, device="cuda", meta=None):
