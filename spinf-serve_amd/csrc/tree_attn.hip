@@ -541,7 +541,6 @@ __global__ __launch_bounds__(256) void tree_attn_kernel(const AttnParams p) {
         }
     };
     auto no_shadow = [](const int) __attribute__((always_inline)) {};
-    // softmax of a whole block spread over `steps` shadow slots, `per` elements each
     auto compute_tile = [&](const char* buf, const int kt, const unsigned bits) __attribute__((always_inline)) {
         const bool a0 = bits & 1u, a1 = bits & 2u;
         if (!a0 && !a1) return;   // wave-uniform: no row of this wave sees a key of the tile
@@ -549,6 +548,27 @@ __global__ __launch_bounds__(256) void tree_attn_kernel(const AttnParams p) {
         const char* vb = buf + G::KTILEB + L.v_lane;
         const int* meta = (const int*)(buf + G::KTILEB + G::VTILEB);
         const int tok = item_t(cur) * SPINF_QTILE + 32 * L.w + L.m;
+        // one 32-key block on its own: K Q^T, softmax, P V in sequence
+        auto one_block = [&](const int sub) __attribute__((always_inline)) {
+            f32x16 sa[RT];
+            bf16x8 pa[RT][2];
+            qk_phase(kb + sub * G::SUBB, sa, no_shadow);
+            if ((bits >> (8 + sub)) & 1u) apply_mask<RT, WIN>(sa, meta, kt, sub, L.g, tok, art_q, pos_q, p.window);
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++) {
+                const float ms = sm_head(rt, sa[rt]);
+                float sum = 0.f;
+#pragma unroll
+                for (int i2 = 0; i2 < 16; i2++) sm_elem(sa[rt], i2, ms, sum, pa[rt]);
+                l[rt] += sum;
+            }
+            pv_phase(vb + sub * G::SUBB, pa, no_shadow);
+        };
+#ifndef SPINF_FUSE   // measured faster than the variant below, which hides each softmax behind the other block's MFMAs
+        if (a0) one_block(0);
+        if (a1) one_block(1);
+        return;
+#endif
         if (a0 && a1) {
             // both blocks: K Q^T(0) | K Q^T(1) with softmax(0) in its shadow | P V(0) with softmax(1) in its shadow | P V(1)
             f32x16 sa[RT], sb[RT];
@@ -584,20 +604,7 @@ __global__ __launch_bounds__(256) void tree_attn_kernel(const AttnParams p) {
             for (int rt = 0; rt < RT; rt++) l[rt] += sum[rt];
             pv_phase(vb + G::SUBB, pb, no_shadow);
         } else {
-            const int sub = a0 ? 0 : 1;
-            f32x16 sa[RT];
-            bf16x8 pa[RT][2];
-            qk_phase(kb + sub * G::SUBB, sa, no_shadow);
-            if ((bits >> (8 + sub)) & 1u) apply_mask<RT, WIN>(sa, meta, kt, sub, L.g, tok, art_q, pos_q, p.window);
-#pragma unroll
-            for (int rt = 0; rt < RT; rt++) {
-                const float ms = sm_head(rt, sa[rt]);
-                float sum = 0.f;
-#pragma unroll
-                for (int i2 = 0; i2 < 16; i2++) sm_elem(sa[rt], i2, ms, sum, pa[rt]);
-                l[rt] += sum;
-            }
-            pv_phase(vb + sub * G::SUBB, pa, no_shadow);
+            one_block(a0 ? 0 : 1);
         }
     };
 
