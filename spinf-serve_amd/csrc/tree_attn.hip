@@ -363,6 +363,7 @@ __global__ __launch_bounds__(256) void tree_attn_exact_kernel(const AttnParams p
     __shared__ __attribute__((aligned(16))) char stage_all[4 * 32 * 144];
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int n_redo = p.counters[NLIST + 1];
+    if (n_redo == 0) return;   // the normal case: the fast pass handed nothing on (every workgroup reads the same count)
     for (int j = blockIdx.x; j < n_redo; j += gridDim.x) {
         const int4 it = p.items[p.redo[j]];
         const int4 item = make_int4(__builtin_amdgcn_readfirstlane(it.x), __builtin_amdgcn_readfirstlane(it.y),
@@ -755,7 +756,7 @@ int launch(const AttnParams& p, int blocks, hipStream_t stream) {
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: launch: %s", hipGetErrorString(e));
     // the exact pass over whatever the fast pass handed on (normally nothing: its workgroups read a zero count and leave)
-    hipLaunchKernelGGL((tree_attn_exact_kernel<D, RT, WIN>), dim3(blocks), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((tree_attn_exact_kernel<D, RT, WIN>), dim3(blocks < 64 ? blocks : 64), dim3(256), 0, stream, p);
     e = hipGetLastError();
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: launch (exact pass): %s", hipGetErrorString(e));
     return SPINF_OK;

@@ -148,8 +148,12 @@ class GdnConfig:
     batch: object = None
 
     def plan(self, device, **kw):
+        """the recurrent-layer plan of the stream.  call_tokens (the reference's cap on a chunked call, there to bound its
+        per-chunk state snapshots, spinf_serve/models/qwen35/qwen.py:228-236) is lifted by default: the fused kernel writes
+        no snapshots, so one launch per level and kind serves the whole stream"""
         from .qwen_plan import tree_plan
 
+        kw.setdefault("call_tokens", 1 << 40)
         return tree_plan(self.batch.prev, self.batch.art >= 0, device, path="indexed", **kw)
 
     @property
