@@ -235,6 +235,37 @@ def test_tileplan_edge_cases():
     assert 2 not in blocks and {0, 1, 3, 4, 5} <= blocks
 
 
+def test_schedule_covers_every_tile_and_head_group_once():
+    """the kernel's work lists: every (query tile, head group) appears in exactly one list, with its own entry range and
+    first key tile; lists are contiguous and ordered job by job (items of one job and head group are neighbours, so that
+    the workgroups that take them share K/V in one L2)"""
+    cfg = synth.attention_config("C2", contents=5)
+    b = cfg.batches[0]
+    plan = sa.TilePlan.build(b.art, b.end, b.pos, None)
+    for head_groups in (1, 3, 16):
+        items, list_ptr = plan.schedule(head_groups)
+        assert items.shape == (plan.n_qtiles * head_groups, 4)
+        assert list_ptr[0] == 0 and list_ptr[8] == len(items) and (np.diff(list_ptr) >= 0).all()
+        seen = set()
+        for t, e0, z, kt0 in items.tolist():
+            ne, hp = z & 0xFFFFF, (z & 0xFFFFFFFF) >> 20
+            assert 0 <= t < plan.n_qtiles and 0 <= hp < head_groups and (t, hp) not in seen
+            seen.add((t, hp))
+            assert e0 == plan.qt_ptr[t] and ne == plan.qt_ptr[t + 1] - plan.qt_ptr[t] and ne >= 1
+            assert kt0 == plan.kv_idx[e0]
+        assert len(seen) == plan.n_qtiles * head_groups
+        # a list never splits the head groups of one query tile's job across lists more than necessary: within a list the
+        # items of one (job, head group) are contiguous
+        job_of_tile = {}
+        for o in b.owners:
+            for t in range(o.start // 128, -(-(o.start + o.n_tokens) // 128)):
+                job_of_tile[t] = o.job_id
+        for l in range(8):
+            runs = [(job_of_tile.get(t, -1), ((z & 0xFFFFFFFF) >> 20)) for t, _, z, _ in items[list_ptr[l] : list_ptr[l + 1]].tolist()]
+            compact = [r for i, r in enumerate(runs) if i == 0 or r != runs[i - 1]]
+            assert len(compact) == len(set(compact))
+
+
 def test_a_jobs_plan_does_not_depend_on_its_neighbours():
     """aligned jobs: a job's tile lists, relative to its first tile, are the same alone and packed (the host half of batch
     invariance, tests/test_packer.py:115-134)"""
