@@ -86,6 +86,10 @@ typedef struct spinf_attn_args {
 /* query heads one work item covers for this geometry (1 or 2); 0 for an invalid geometry */
 int spinf_attn_heads_per_item(int32_t hq, int32_t hkv, int32_t d, int32_t variant);
 int spinf_tree_attn_fwd(const spinf_attn_args* args, void* stream);
+/* Diagnostics (no counterpart in the reference): *total = work items that the exact (rescaling) pass has recomputed on the
+ * current device since the library was loaded, i.e. query tiles whose scores ranged too widely for the fast pass.
+ * Synchronises the device. */
+int spinf_attn_exact_items(int64_t* total);
 
 /* ------------------------------------------------------------------------------------------------ Gated DeltaNet
  * Replaces gdn.recurrent / gdn.chunked (spinf_serve/models/qwen35/gdn.py:197-235 and :109-133): the gated delta rule

@@ -375,6 +375,7 @@ __global__ __launch_bounds__(256) void tree_attn_exact_kernel(const AttnParams p
     if (threadIdx.x == 0) {
         __threadfence();
         if (atomicAdd(&p.counters[NLIST + 2], 1) == (int)gridDim.x - 1) {
+            p.counters[NLIST + 3] += n_redo;   // running total, for spinf_attn_exact_items
             p.counters[NLIST + 1] = 0;
             p.counters[NLIST + 2] = 0;
             __threadfence();
@@ -769,6 +770,21 @@ int launch_d(const AttnParams& p, int rt, bool win, int blocks, hipStream_t s) {
 }
 
 }  // namespace
+
+extern "C" int spinf_attn_exact_items(int64_t* total) {
+    if (!total) return spinf_fail(SPINF_E_ARG, "attn_exact_items: null pointer");
+    *total = 0;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= 64) return spinf_fail(SPINF_E_HIP, "attn_exact_items: hipGetDevice: %s", hipGetErrorString(e));
+    std::lock_guard<std::mutex> lock(g_mu);
+    if (!g_dev[dev].counters) return SPINF_OK;   // no attention launch on this device yet
+    int v = 0;
+    e = hipMemcpy(&v, g_dev[dev].counters + NLIST + 3, sizeof(int), hipMemcpyDeviceToHost);
+    if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "attn_exact_items: hipMemcpy: %s", hipGetErrorString(e));
+    *total = v;
+    return SPINF_OK;
+}
 
 extern "C" int spinf_attn_heads_per_item(int32_t hq, int32_t hkv, int32_t d, int32_t variant) {
     if (hq <= 0 || hkv <= 0 || hq % hkv) return 0;

@@ -10,7 +10,7 @@ _LIB = None
 
 SYMBOLS = (
     "spinf_last_error", "spinf_version", "spinf_tileplan_build", "spinf_tileplan_counts", "spinf_tileplan_export",
-    "spinf_tileplan_schedule", "spinf_tileplan_free", "spinf_attn_heads_per_item", "spinf_tree_attn_fwd", "spinf_gdn_fwd",
+    "spinf_tileplan_schedule", "spinf_tileplan_free", "spinf_attn_heads_per_item", "spinf_tree_attn_fwd", "spinf_attn_exact_items", "spinf_gdn_fwd",
 )
 
 
@@ -61,8 +61,9 @@ def load_library():
     lib.spinf_tileplan_free.argtypes = [C.c_void_p]
     lib.spinf_tileplan_free.restype = None
     lib.spinf_tree_attn_fwd.argtypes = [C.POINTER(AttnArgs), C.c_void_p]
+    lib.spinf_attn_exact_items.argtypes = [C.POINTER(C.c_int64)]
     lib.spinf_gdn_fwd.argtypes = [C.POINTER(GdnArgs), C.c_void_p]
-    for name in ("spinf_tileplan_build", "spinf_tileplan_counts", "spinf_tileplan_export", "spinf_tileplan_schedule", "spinf_tree_attn_fwd", "spinf_gdn_fwd"):
+    for name in ("spinf_tileplan_build", "spinf_tileplan_counts", "spinf_tileplan_export", "spinf_tileplan_schedule", "spinf_tree_attn_fwd", "spinf_attn_exact_items", "spinf_gdn_fwd"):
         getattr(lib, name).restype = C.c_int
     _LIB = lib
     return lib

@@ -54,6 +54,44 @@ def test_c2_shape_three_contents(dev, variant):
     _check(cfg, cfg.batches[0], dev, variant=variant)
 
 
+def _exact_items():
+    import ctypes
+
+    total = ctypes.c_int64(0)
+    assert sa.load_library().spinf_attn_exact_items(ctypes.byref(total)) == 0
+    return total.value
+
+
+@pytest.mark.parametrize("d,hq,hkv", [(64, 4, 2), (128, 4, 2), (256, 2, 1), (128, 3, 3)])
+def test_wide_score_range_takes_the_exact_pass(dev, d, hq, hkv):
+    """scores that grow by far more than the fast pass allows for (2^60 above a row's first block maximum) send the query tile
+    to the exact pass, which rescales its accumulators like a classic online softmax; the result must still match"""
+    rng = np.random.default_rng(11)
+    trees = [synth._tree(rng, 300, [20, 9]), synth._tree(rng, 90, [7])]
+    cfg = synth.AttnConfig("wide", hq, hkv, d, d ** -0.5, 1.0, None, trees)
+    b = synth.pack(trees)[0]
+    q, k, v = synth.qkv(cfg, b, seed=3, device=dev)
+    k = k.clone()
+    k[96:] *= 60.0        # keys from the fourth 32-key block on: scores 60 times wider than in the blocks before
+    mask = sa.TreeMask.build(b.art, b.end, b.pos, device=dev)
+    before = _exact_items()
+    out = sa.tree_attn(q, k, v, mask, cfg.scale)
+    torch.cuda.synchronize()
+    assert _exact_items() > before, "the exact pass did not run"
+    ref = _oracle(q, k, v, b, cfg.scale)
+    got = out.float().cpu().numpy()
+    assert np.isfinite(got).all()
+    assert float(np.abs(got - ref).max()) <= TOL
+    _pads_selfattend(out, v, b, hq // hkv)
+    # and an ordinary launch afterwards leaves the count alone
+    k2 = synth.qkv(cfg, b, seed=3, device=dev)[1]
+    mid = _exact_items()
+    out2 = sa.tree_attn(q, k2, v, mask, cfg.scale)
+    torch.cuda.synchronize()
+    assert _exact_items() == mid
+    assert float(np.abs(out2.float().cpu().numpy() - _oracle(q, k2, v, b, cfg.scale)).max()) <= TOL
+
+
 def test_c4_shape_two_level_tree(dev):
     rng = np.random.default_rng(5)
     lens, parents = [], []
