@@ -20,6 +20,7 @@
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((ext_vector_type(8))) short s16x8;
 
@@ -30,6 +31,16 @@ struct GdnParams {
     const long* cu; const long* idx; long n_seg;
     const float* h0; const long* h0_idx; float* ht; const long* ht_idx;
 };
+
+#ifdef SPINF_TRACE
+__device__ long g_gdn_trace[16];
+extern "C" int spinf_debug_gdn_trace(long* out) { return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_gdn_trace), sizeof(long) * 16, 0, hipMemcpyDeviceToHost); }
+#define GT_CLK(v) const long v = clock64()
+#define GT_ADD(slot, val) do { if (threadIdx.x == 64 && blockIdx.x == 7) g_gdn_trace[slot] += (val); } while (0)
+#else
+#define GT_CLK(v) do { } while (0)
+#define GT_ADD(slot, val) do { } while (0)
+#endif
 
 namespace {
 
@@ -73,6 +84,14 @@ __device__ __forceinline__ bf16x8 frag_tr(const __bf16* base, int stride, int k0
     const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p);
     const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(p + 4 * stride));
     return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+}
+// Workgroup barrier for LDS traffic only: waits for this wave's LDS operations, not for its global loads.  __syncthreads()
+// carries a memory fence in front of which the compiler drains every load in flight, the next chunk's prefetch included.
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
 }
 __device__ __forceinline__ f32x16 mfma(bf16x8 a, bf16x8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
 
@@ -126,53 +145,86 @@ __global__ __launch_bounds__(256) void gdn_chunk_kernel(const GdnParams p) {
             *(bf16x4*)(St + (32 * vt + n32) * LD + 32 * w + 8 * r4 + 4 * g) = t;
         }
 
+    // The next chunk's rows are fetched into registers while the current chunk is computed (global latency would otherwise
+    // be exposed in front of every chunk: a workgroup walks its chunks strictly in order), and the stream rows of the chunk
+    // after that (idx) one chunk earlier still, so that no load ever waits for the load of its own address.
+    // Thread -> row tid/4 of the chunk, 16-byte pieces 4(tid%4)..+3 of its K, Q and V rows; threads 0..63 also -> g, beta and
+    // the stream row of chunk row tid.
+    bf16x8 pk[4], pq[4], pv[4];
+    long pr64 = -1;
+    float pg = 0.f;
+    __bf16 pbeta = (__bf16)0.f;   // (kept as loaded: converting here would make the wave wait for the load at once)
+    long ra = -1, rb = -1;     // stream rows (thread's K/Q/V row; chunk row tid) of the chunk whose data is fetched next
+    auto fetch_rows = [&](const int c0) __attribute__((always_inline)) {
+        const int L = min(C, T - c0);      // <= 0: there is no such chunk
+        const int row = tid >> 2;
+        ra = -1;
+        if (row < L) {
+            const long t = bos + c0 + row;
+            ra = p.idx ? p.idx[t] : t;
+        }
+        rb = -1;
+        if (tid < 64 && tid < L) {
+            const long t = bos + c0 + tid;
+            rb = p.idx ? p.idx[t] : t;
+        }
+    };
+    auto fetch_data = [&]() __attribute__((always_inline)) {
+        const int cb = (tid & 3) * 4;
+#pragma unroll
+        for (int cc = 0; cc < 4; cc++) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) { pk[cc][j] = (__bf16)0.f; pq[cc][j] = (__bf16)0.f; pv[cc][j] = (__bf16)0.f; }
+            if (ra >= 0) {
+                const int col = (cb + cc) * 8;
+                pk[cc] = *(const bf16x8*)(p.k + ra * p.q_tok + (long)hk * KD + col);
+                pq[cc] = *(const bf16x8*)(p.q + ra * p.q_tok + (long)hk * KD + col);
+                pv[cc] = *(const bf16x8*)(p.v + ra * p.v_tok + (long)hv * VD + col);
+            }
+        }
+        pr64 = rb;
+        pg = 0.f;
+        pbeta = (__bf16)0.f;
+        if (rb >= 0) {
+            pg = p.g[rb * p.g_tok + hv];
+            pbeta = p.beta[rb * p.g_tok + hv];
+        }
+    };
+    fetch_rows(0);
+    fetch_data();
+    fetch_rows(C);
+
     for (int c0 = 0; c0 < T; c0 += C) {
         const int L = min(C, T - c0);
-        __syncthreads();   // previous chunk fully consumed (and St written)
-        // ---- stage the chunk: rows, g, beta, then K / Q / V tiles (rows >= L are zero)
+        GT_CLK(g0);
+        lds_barrier();   // previous chunk fully consumed (and St written)
+        // ---- stage the chunk from the prefetch registers: rows, cumulative g, beta, then K / Q / V tiles (rows >= L are zero)
         if (tid < 64) {
-            long r = -1;
-            float gv = 0.f, bv = 0.f;
-            if (tid < L) {
-                const long t = bos + c0 + tid;
-                r = p.idx ? p.idx[t] : t;
-                gv = p.g[r * p.g_tok + hv];
-                bv = (float)p.beta[r * p.g_tok + hv];
-            }
-            // inclusive prefix sum of g over the wave
-            float x = gv;
+            float x = pg;      // inclusive prefix sum of g over the wave
 #pragma unroll
             for (int d = 1; d < 64; d <<= 1) {
                 const float y = __shfl_up(x, d);
                 if (lane >= d) x += y;
             }
             Gs[tid] = x;
-            Bs[tid] = bv;
-            Rs[tid] = r;
+            Bs[tid] = (float)pbeta;
+            Rs[tid] = pr64;
         }
-        __syncthreads();
         {
-            // 64 rows x 16 chunks of 16 bytes per tile, 3 tiles: thread handles row tid/4, chunks 4(tid%4)..+3
             const int row = tid >> 2, cb = (tid & 3) * 4;
-            const long r = Rs[row];
 #pragma unroll
             for (int cc = 0; cc < 4; cc++) {
                 const int col = (cb + cc) * 8;
-                bf16x8 kz, qz, vz;
-#pragma unroll
-                for (int j = 0; j < 8; j++) { kz[j] = (__bf16)0.f; qz[j] = (__bf16)0.f; vz[j] = (__bf16)0.f; }
-                if (r >= 0) {
-                    kz = *(const bf16x8*)(p.k + r * p.q_tok + (long)hk * KD + col);
-                    qz = *(const bf16x8*)(p.q + r * p.q_tok + (long)hk * KD + col);
-                    vz = *(const bf16x8*)(p.v + r * p.v_tok + (long)hv * VD + col);
-                }
-                *(bf16x8*)(Ks + row * LD + col) = kz;
-                *(bf16x8*)(Qs + row * LD + col) = qz;
-                *(bf16x8*)(Vs + row * LD + col) = vz;
+                *(bf16x8*)(Ks + row * LD + col) = pk[cc];
+                *(bf16x8*)(Qs + row * LD + col) = pq[cc];
+                *(bf16x8*)(Vs + row * LD + col) = pv[cc];
             }
         }
-        __syncthreads();
+        fetch_data();          // chunk c0 + C, whose rows are known since the previous chunk
+        fetch_rows(c0 + 2 * C);
+        lds_barrier();
         const float GL = Gs[63];
+        GT_CLK(g1);
 
         // ---- (a) A = -strict_tril(beta_i K_i.K_j D_ij) fp32, (b) P = tril(s Q_i.K_j D_ij) bf16; computed transposed so that
         // a lane holds row i and 4 consecutive columns j per register group.  Wave w: tile (jt = w>>1, it = w&1).
@@ -205,8 +257,9 @@ __global__ __launch_bounds__(256) void gdn_chunk_kernel(const GdnParams p) {
                 *(bf16x4*)(Pm + i * LT + j0) = pv;
             }
         }
-        __syncthreads();
+        lds_barrier();
 
+        GT_CLK(g2);
         // ---- T = (I - A)^-1 in place (fp32).  Stage 1: the four 16x16 diagonal blocks by forward substitution, wave b =
         // block b, lane c < 16 = column c of the block.
         if (lane < 16) {
@@ -223,58 +276,51 @@ __global__ __launch_bounds__(256) void gdn_chunk_kernel(const GdnParams p) {
 #pragma unroll
             for (int i = 0; i < 16; i++) As[(16 * w + i) * LA + 16 * w + lane] = t[i];
         }
-        __syncthreads();
-        // Stage 2: 32x32 diagonal blocks: T_lo = T_bb A_lo T_aa for (a, b) = (0,1) and (2,3).  256 threads = 2 blocks x 16 x 8;
-        // thread: block q, row i, columns 2c..2c+1
+        lds_barrier();
+        // Stages 2 and 3 are products of 16x16 / 32x32 fp32 blocks, done with v_mfma_f32_16x16x4_f32 (operands: lane l gives
+        // A[l%16][l/16] and B[l/16][l%16] of a 16x4 by 4x16 step; result: lane l holds rows 4(l/16)..+3 of column l%16).
+        // Stage 2: 32x32 diagonal blocks: T_lo = T_bb A_lo T_aa for (a, b) = (0,1) and (2,3); wave q < 2 does block q.
         {
-            const int qb = tid >> 7, i = (tid >> 3) & 15, c2 = (tid & 7) * 2;
-            const int ra = 32 * qb, rb = ra + 16;
-            float x0 = 0.f, x1 = 0.f;
+            const int c16 = lane & 15, g4 = lane >> 4;
+            if (w < 2) {
+                const int ra = 32 * w, rb = ra + 16;
+                f32x4 x = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int j = 0; j < 16; j++) {            // X = A_lo T_aa
-                const float a = As[(rb + i) * LA + ra + j];
-                x0 = __builtin_fmaf(a, As[(ra + j) * LA + ra + c2], x0);
-                x1 = __builtin_fmaf(a, As[(ra + j) * LA + ra + c2 + 1], x1);
-            }
-            Xs[(16 * qb + i) * 36 + c2] = x0;
-            Xs[(16 * qb + i) * 36 + c2 + 1] = x1;
-            __syncthreads();
-            float y0 = 0.f, y1 = 0.f;
+                for (int s4 = 0; s4 < 4; s4++)        // X = A_lo T_aa
+                    x = __builtin_amdgcn_mfma_f32_16x16x4f32(As[(rb + c16) * LA + ra + 4 * s4 + g4], As[(ra + 4 * s4 + g4) * LA + ra + c16], x, 0, 0, 0);
 #pragma unroll
-            for (int j = 0; j < 16; j++) {            // T_lo = T_bb X
-                const float tb = As[(rb + i) * LA + rb + j];
-                y0 = __builtin_fmaf(tb, Xs[(16 * qb + j) * 36 + c2], y0);
-                y1 = __builtin_fmaf(tb, Xs[(16 * qb + j) * 36 + c2 + 1], y1);
+                for (int i = 0; i < 4; i++) Xs[(16 * w + 4 * g4 + i) * 36 + c16] = x[i];
+                __builtin_amdgcn_s_waitcnt(0xc07f);   // this wave's own X is in LDS (nobody else reads it)
+                f32x4 y = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int s4 = 0; s4 < 4; s4++)        // T_lo = T_bb X
+                    y = __builtin_amdgcn_mfma_f32_16x16x4f32(As[(rb + c16) * LA + rb + 4 * s4 + g4], Xs[(16 * w + 4 * s4 + g4) * 36 + c16], y, 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < 4; i++) As[(rb + 4 * g4 + i) * LA + ra + c16] = y[i];
             }
-            As[(rb + i) * LA + ra + c2] = y0;
-            As[(rb + i) * LA + ra + c2 + 1] = y1;
         }
-        __syncthreads();
-        // Stage 3: the 64x64 matrix: T_lo = T_11 A_lo T_00 with 32x32 blocks.  thread: row i (32), columns 4c..4c+3 (8 groups)
+        lds_barrier();
+        // Stage 3: the 64x64 matrix: T_lo = T_11 A_lo T_00 with 32x32 blocks; wave w does the 16x16 tile (w>>1, w&1) of both products
         {
-            const int i = tid >> 3, c4 = (tid & 7) * 4;
-            float x[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 8
-            for (int j = 0; j < 32; j++) {
-                const float a = As[(32 + i) * LA + j];
-                const float4 t = *(const float4*)(As + j * LA + c4);
-                x[0] = __builtin_fmaf(a, t.x, x[0]); x[1] = __builtin_fmaf(a, t.y, x[1]);
-                x[2] = __builtin_fmaf(a, t.z, x[2]); x[3] = __builtin_fmaf(a, t.w, x[3]);
-            }
-            *(float4*)(Xs + i * 36 + c4) = make_float4(x[0], x[1], x[2], x[3]);
-            __syncthreads();
-            float y[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 8
-            for (int j = 0; j < 32; j++) {
-                const float tb = As[(32 + i) * LA + 32 + j];
-                const float4 t = *(const float4*)(Xs + j * 36 + c4);
-                y[0] = __builtin_fmaf(tb, t.x, y[0]); y[1] = __builtin_fmaf(tb, t.y, y[1]);
-                y[2] = __builtin_fmaf(tb, t.z, y[2]); y[3] = __builtin_fmaf(tb, t.w, y[3]);
-            }
-            __syncthreads();   // every read of the A_lo block is done
-            *(float4*)(As + (32 + i) * LA + c4) = make_float4(y[0], y[1], y[2], y[3]);
+            const int c16 = lane & 15, g4 = lane >> 4;
+            const int ti = 16 * (w >> 1), tj = 16 * (w & 1);
+            f32x4 x = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s4 = 0; s4 < 8; s4++)            // X = A_lo T_00
+                x = __builtin_amdgcn_mfma_f32_16x16x4f32(As[(32 + ti + c16) * LA + 4 * s4 + g4], As[(4 * s4 + g4) * LA + tj + c16], x, 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < 4; i++) Xs[(ti + 4 * g4 + i) * 36 + tj + c16] = x[i];
+            lds_barrier();
+            f32x4 y = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s4 = 0; s4 < 8; s4++)            // T_lo = T_11 X
+                y = __builtin_amdgcn_mfma_f32_16x16x4f32(As[(32 + ti + c16) * LA + 32 + 4 * s4 + g4], Xs[(4 * s4 + g4) * 36 + tj + c16], y, 0, 0, 0);
+            lds_barrier();   // every read of the A_lo block is done
+#pragma unroll
+            for (int i = 0; i < 4; i++) As[(32 + ti + 4 * g4 + i) * LA + tj + c16] = y[i];
         }
-        __syncthreads();
+        lds_barrier();
+        GT_CLK(g3);
         // ---- Tu = T diag(beta), Tw = -T diag(beta e^G) (bf16).  thread: row tid/4, 16 columns
         {
             const int i = tid >> 2, jb = (tid & 3) * 16;
@@ -294,8 +340,9 @@ __global__ __launch_bounds__(256) void gdn_chunk_kernel(const GdnParams p) {
                 *(bf16x4*)(Tw + i * LT + jb + 4 * j4) = ww;
             }
         }
-        __syncthreads();
+        lds_barrier();
 
+        GT_CLK(g4);
         // ---- (c) U^T[v][i] = sum_j V[j][v] Tu[i][j]  and  -W^T[d][i] = sum_j K[j][d] Tw[i][j]; wave w: rows 32w.. of v / d
         f32x16 acc[2];      // U^T, later V'^T : tile it = token columns 32 it..
         {
@@ -321,8 +368,9 @@ __global__ __launch_bounds__(256) void gdn_chunk_kernel(const GdnParams p) {
                     *(bf16x4*)(Wn + (32 * it + n32) * LD + 32 * w + 8 * r4 + 4 * g) = t;
                 }
         }
-        __syncthreads();   // -W visible; V (Vs) and T (As) are dead from here
+        lds_barrier();   // -W visible; V (Vs) and T (As) are dead from here
 
+        GT_CLK(g5);
         // ---- (d) V'^T = U^T + S^T (-W)^T   and   (e1) QS^T[v][i] = sum_k S^T[v][k] Q[i][k]
         f32x16 qs[2];
         qs[0] = zero16(); qs[1] = zero16();
@@ -352,8 +400,9 @@ __global__ __launch_bounds__(256) void gdn_chunk_kernel(const GdnParams p) {
                 *(bf16x4*)(Vd + i * LD + 32 * w + 8 * r4 + 4 * g) = td;
             }
         }
-        __syncthreads();
+        lds_barrier();
 
+        GT_CLK(g6);
         // ---- (e2) O^T[v][i] = s e^{G_i} QS^T + sum_j V'[j][v] P[i][j]
         {
             f32x16 ov[2];
@@ -381,6 +430,7 @@ __global__ __launch_bounds__(256) void gdn_chunk_kernel(const GdnParams p) {
             }
         }
 
+        GT_CLK(g7);
         // ---- (f) S[k][v] = e^{G_L} S[k][v] + sum_j K[j][k] (V' e^{G_L - G_j})[j][v]; wave w: k rows 32w.., all four v tiles
         {
             const float eg = __expf(GL);
@@ -395,7 +445,7 @@ __global__ __launch_bounds__(256) void gdn_chunk_kernel(const GdnParams p) {
                 for (int vt = 0; vt < 4; vt++) S[vt] = mfma(a, frag_tr(Vd, LD, 16 * s, 32 * vt, lane), S[vt]);
             }
         }
-        __syncthreads();   // every wave is done reading S^T (d, e1) before it is replaced
+        lds_barrier();   // every wave is done reading S^T (d, e1) before it is replaced
 #pragma unroll
         for (int vt = 0; vt < 4; vt++)
 #pragma unroll
@@ -405,6 +455,8 @@ __global__ __launch_bounds__(256) void gdn_chunk_kernel(const GdnParams p) {
                 for (int j = 0; j < 4; j++) t[j] = (__bf16)S[vt][4 * r4 + j];
                 *(bf16x4*)(St + (32 * vt + n32) * LD + 32 * w + 8 * r4 + 4 * g) = t;
             }
+        GT_CLK(g8);
+        GT_ADD(0, g1 - g0); GT_ADD(1, g2 - g1); GT_ADD(2, g3 - g2); GT_ADD(3, g4 - g3); GT_ADD(4, g5 - g4); GT_ADD(5, g6 - g5); GT_ADD(6, g7 - g6); GT_ADD(7, g8 - g7); GT_ADD(8, 1);
     }
 
     if (p.ht != nullptr && p.ht_idx != nullptr) {
