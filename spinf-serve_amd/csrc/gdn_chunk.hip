@@ -148,20 +148,23 @@ __global__ __launch_bounds__(256) void gdn_chunk_kernel(const GdnParams p) {
     // The next chunk's rows are fetched into registers while the current chunk is computed (global latency would otherwise
     // be exposed in front of every chunk: a workgroup walks its chunks strictly in order), and the stream rows of the chunk
     // after that (idx) one chunk earlier still, so that no load ever waits for the load of its own address.
-    // Thread -> row tid/4 of the chunk, 16-byte pieces 4(tid%4)..+3 of its K, Q and V rows; threads 0..63 also -> g, beta and
-    // the stream row of chunk row tid.
+    // Thread -> 16-byte piece tid%16 of chunk rows tid/16 + 16 cc, cc = 0..3 (one load instruction of a wave then covers four
+    // whole rows); threads 0..63 also -> g, beta and the stream row of chunk row tid.
     bf16x8 pk[4], pq[4], pv[4];
     long pr64 = -1;
     float pg = 0.f;
     __bf16 pbeta = (__bf16)0.f;   // (kept as loaded: converting here would make the wave wait for the load at once)
-    long ra = -1, rb = -1;     // stream rows (thread's K/Q/V row; chunk row tid) of the chunk whose data is fetched next
+    long ra[4] = {-1, -1, -1, -1}, rb = -1;     // stream rows (the thread's four K/Q/V rows; chunk row tid) of the chunk fetched next
     auto fetch_rows = [&](const int c0) __attribute__((always_inline)) {
         const int L = min(C, T - c0);      // <= 0: there is no such chunk
-        const int row = tid >> 2;
-        ra = -1;
-        if (row < L) {
-            const long t = bos + c0 + row;
-            ra = p.idx ? p.idx[t] : t;
+#pragma unroll
+        for (int cc = 0; cc < 4; cc++) {
+            const int row = (tid >> 4) + 16 * cc;
+            ra[cc] = -1;
+            if (row < L) {
+                const long t = bos + c0 + row;
+                ra[cc] = p.idx ? p.idx[t] : t;
+            }
         }
         rb = -1;
         if (tid < 64 && tid < L) {
@@ -170,16 +173,15 @@ __global__ __launch_bounds__(256) void gdn_chunk_kernel(const GdnParams p) {
         }
     };
     auto fetch_data = [&]() __attribute__((always_inline)) {
-        const int cb = (tid & 3) * 4;
+        const int col = (tid & 15) * 8;
 #pragma unroll
         for (int cc = 0; cc < 4; cc++) {
 #pragma unroll
             for (int j = 0; j < 8; j++) { pk[cc][j] = (__bf16)0.f; pq[cc][j] = (__bf16)0.f; pv[cc][j] = (__bf16)0.f; }
-            if (ra >= 0) {
-                const int col = (cb + cc) * 8;
-                pk[cc] = *(const bf16x8*)(p.k + ra * p.q_tok + (long)hk * KD + col);
-                pq[cc] = *(const bf16x8*)(p.q + ra * p.q_tok + (long)hk * KD + col);
-                pv[cc] = *(const bf16x8*)(p.v + ra * p.v_tok + (long)hv * VD + col);
+            if (ra[cc] >= 0) {
+                pk[cc] = *(const bf16x8*)(p.k + ra[cc] * p.q_tok + (long)hk * KD + col);
+                pq[cc] = *(const bf16x8*)(p.q + ra[cc] * p.q_tok + (long)hk * KD + col);
+                pv[cc] = *(const bf16x8*)(p.v + ra[cc] * p.v_tok + (long)hv * VD + col);
             }
         }
         pr64 = rb;
@@ -198,31 +200,37 @@ __global__ __launch_bounds__(256) void gdn_chunk_kernel(const GdnParams p) {
         const int L = min(C, T - c0);
         GT_CLK(g0);
         lds_barrier();   // previous chunk fully consumed (and St written)
+        GT_CLK(h0);
         // ---- stage the chunk from the prefetch registers: rows, cumulative g, beta, then K / Q / V tiles (rows >= L are zero)
         if (tid < 64) {
-            float x = pg;      // inclusive prefix sum of g over the wave
-#pragma unroll
-            for (int d = 1; d < 64; d <<= 1) {
-                const float y = __shfl_up(x, d);
-                if (lane >= d) x += y;
-            }
+            // inclusive prefix sum of g over the wave: within rows of 16 lanes by shifts, then across rows by broadcasts
+            float x = pg;
+            x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x111, 0xf, 0xf, true));   // row_shr:1
+            x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x112, 0xf, 0xf, true));   // row_shr:2
+            x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x114, 0xf, 0xf, true));   // row_shr:4
+            x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x118, 0xf, 0xf, true));   // row_shr:8
+            x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x142, 0xa, 0xf, false));  // row_bcast:15 -> rows 1, 3
+            x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x143, 0xc, 0xf, false));  // row_bcast:31 -> rows 2, 3
             Gs[tid] = x;
             Bs[tid] = (float)pbeta;
             Rs[tid] = pr64;
         }
         {
-            const int row = tid >> 2, cb = (tid & 3) * 4;
+            const int col = (tid & 15) * 8;
 #pragma unroll
             for (int cc = 0; cc < 4; cc++) {
-                const int col = (cb + cc) * 8;
+                const int row = (tid >> 4) + 16 * cc;
                 *(bf16x8*)(Ks + row * LD + col) = pk[cc];
                 *(bf16x8*)(Qs + row * LD + col) = pq[cc];
                 *(bf16x8*)(Vs + row * LD + col) = pv[cc];
             }
         }
+        GT_CLK(h1);
         fetch_data();          // chunk c0 + C, whose rows are known since the previous chunk
         fetch_rows(c0 + 2 * C);
+        GT_CLK(h2);
         lds_barrier();
+        GT_ADD(9, h0 - g0); GT_ADD(10, h1 - h0); GT_ADD(11, h2 - h1);
         const float GL = Gs[63];
         GT_CLK(g1);
 
