@@ -2,8 +2,8 @@
 // i.e. for fla's cumsum -> intra-chunk WY solve -> state recurrence (gdn.py:21-106) -> output pipeline, without writing
 // the per-chunk state snapshots or the w / u / v_new intermediates to memory.
 //
-// One workgroup (4 waves) owns one (segment, value head) and walks its 64-token chunks in order.  The state S [K=128, V=128]
-// lives in fp32 MFMA accumulators (wave w owns key rows 32w..32w+31) and is mirrored once per chunk as bf16 S^T in LDS,
+// One workgroup (8 waves) owns one (segment, value head) and walks its 64-token chunks in order.  The state S [K=128, V=128]
+// lives in fp32 MFMA accumulators (a wave owns 32 key rows x 64 value columns) and is mirrored once per chunk as bf16 S^T in LDS,
 // where it serves as an MFMA operand.  Per chunk, with G = cumsum(g), D_ij = exp(G_i - G_j):
 //     A   = -strict_tril(beta_i (K K^T)_ij D_ij)         T = (I - A)^-1        (fp32, blocked forward substitution)
 //     U   = T diag(beta) V          W = T diag(beta e^G) K                     (bf16 MFMA, fp32 accumulate)
@@ -97,7 +97,7 @@ __device__ __forceinline__ f32x16 mfma(bf16x8 a, bf16x8 b, f32x16 c) { return __
 
 }  // namespace
 
-__global__ __launch_bounds__(256) void gdn_chunk_kernel(const GdnParams p) {
+__global__ __launch_bounds__(512) void gdn_chunk_kernel(const GdnParams p) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     __bf16* Ks = (__bf16*)(smem + OFF_K);
     __bf16* Qs = (__bf16*)(smem + OFF_Q);
@@ -114,52 +114,59 @@ __global__ __launch_bounds__(256) void gdn_chunk_kernel(const GdnParams p) {
     long* Rs = (long*)(Bs + 64);
     float* Xs = (float*)(smem + OFF_X);
 
-    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, n32 = lane & 31, g = lane >> 5;
+    // Eight waves, two per SIMD: every phase below is a short dependent chain (LDS reads -> MFMAs -> conversions -> LDS
+    // writes -> barrier), and a second wave on the SIMD is what fills the gaps of the first.  Wave w = (wq, wh): quarter
+    // wq = w % 4 of whatever a phase splits four ways (32 of 128 rows, a 32x32 tile of a 64x64 matrix), half wh = w / 4.
+    const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6), wq = w & 3, wh = w >> 2, n32 = lane & 31, g = lane >> 5;
     const long seg = blockIdx.x / p.hv;
     const int hv = (int)(blockIdx.x % p.hv);
     const int hk = hv / (p.hv / p.h);
     const long bos = p.cu[seg], eos = p.cu[seg + 1];
     const int T = (int)(eos - bos);
 
-    // ---- state: S[k][v], wave w owns k rows 32w..32w+31; tile vt covers v columns 32vt..; lane = v column, reg r = k row
-    f32x16 S[4];
+    // ---- state: S[k][v]; wave (wq, wh) owns k rows 32wq..32wq+31 of v columns 64wh..64wh+63 as two 32x32 tiles (tile j:
+    // v columns 64wh + 32j ..); lane = v column, reg r = k row
+    f32x16 S[2];
 #pragma unroll
-    for (int vt = 0; vt < 4; vt++) S[vt] = zero16();
+    for (int j = 0; j < 2; j++) S[j] = zero16();
     long src = -1;
     if (p.h0 != nullptr && p.h0_idx != nullptr) src = p.h0_idx[seg];
     if (src >= 0) {
         const float* hp = p.h0 + (src * p.hv + hv) * (long)KD * VD;
 #pragma unroll
-        for (int vt = 0; vt < 4; vt++)
+        for (int j = 0; j < 2; j++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) S[vt][r] = hp[(long)(32 * w + 8 * (r >> 2) + 4 * g + (r & 3)) * VD + 32 * vt + n32];
+            for (int r = 0; r < 16; r++) S[j][r] = hp[(long)(32 * wq + 8 * (r >> 2) + 4 * g + (r & 3)) * VD + 64 * wh + 32 * j + n32];
     }
     // S^T mirror (bf16): St[v][k]
+    auto mirror = [&]() __attribute__((always_inline)) {
 #pragma unroll
-    for (int vt = 0; vt < 4; vt++)
+        for (int j = 0; j < 2; j++)
 #pragma unroll
-        for (int r4 = 0; r4 < 4; r4++) {
-            bf16x4 t;
+            for (int r4 = 0; r4 < 4; r4++) {
+                bf16x4 t;
 #pragma unroll
-            for (int j = 0; j < 4; j++) t[j] = (__bf16)S[vt][4 * r4 + j];
-            *(bf16x4*)(St + (32 * vt + n32) * LD + 32 * w + 8 * r4 + 4 * g) = t;
-        }
+                for (int jj = 0; jj < 4; jj++) t[jj] = (__bf16)S[j][4 * r4 + jj];
+                *(bf16x4*)(St + (64 * wh + 32 * j + n32) * LD + 32 * wq + 8 * r4 + 4 * g) = t;
+            }
+    };
+    mirror();
 
     // The next chunk's rows are fetched into registers while the current chunk is computed (global latency would otherwise
     // be exposed in front of every chunk: a workgroup walks its chunks strictly in order), and the stream rows of the chunk
     // after that (idx) one chunk earlier still, so that no load ever waits for the load of its own address.
-    // Thread -> 16-byte piece tid%16 of chunk rows tid/16 + 16 cc, cc = 0..3 (one load instruction of a wave then covers four
-    // whole rows); threads 0..63 also -> g, beta and the stream row of chunk row tid.
-    bf16x8 pk[4], pq[4], pv[4];
+    // Thread -> 16-byte piece tid%16 of chunk rows tid/16 and tid/16 + 32 (one load instruction of a wave covers four whole
+    // rows); threads 0..63 also -> g, beta and the stream row of chunk row tid.
+    bf16x8 pk[2], pq[2], pv[2];
     long pr64 = -1;
     float pg = 0.f;
     __bf16 pbeta = (__bf16)0.f;   // (kept as loaded: converting here would make the wave wait for the load at once)
-    long ra[4] = {-1, -1, -1, -1}, rb = -1;     // stream rows (the thread's four K/Q/V rows; chunk row tid) of the chunk fetched next
+    long ra[2] = {-1, -1}, rb = -1;     // stream rows (the thread's two K/Q/V rows; chunk row tid) of the chunk fetched next
     auto fetch_rows = [&](const int c0) __attribute__((always_inline)) {
         const int L = min(C, T - c0);      // <= 0: there is no such chunk
 #pragma unroll
-        for (int cc = 0; cc < 4; cc++) {
-            const int row = (tid >> 4) + 16 * cc;
+        for (int cc = 0; cc < 2; cc++) {
+            const int row = (tid >> 4) + 32 * cc;
             ra[cc] = -1;
             if (row < L) {
                 const long t = bos + c0 + row;
@@ -175,7 +182,7 @@ __global__ __launch_bounds__(256) void gdn_chunk_kernel(const GdnParams p) {
     auto fetch_data = [&]() __attribute__((always_inline)) {
         const int col = (tid & 15) * 8;
 #pragma unroll
-        for (int cc = 0; cc < 4; cc++) {
+        for (int cc = 0; cc < 2; cc++) {
 #pragma unroll
             for (int j = 0; j < 8; j++) { pk[cc][j] = (__bf16)0.f; pq[cc][j] = (__bf16)0.f; pv[cc][j] = (__bf16)0.f; }
             if (ra[cc] >= 0) {
@@ -200,7 +207,6 @@ __global__ __launch_bounds__(256) void gdn_chunk_kernel(const GdnParams p) {
         const int L = min(C, T - c0);
         GT_CLK(g0);
         lds_barrier();   // previous chunk fully consumed (and St written)
-        GT_CLK(h0);
         // ---- stage the chunk from the prefetch registers: rows, cumulative g, beta, then K / Q / V tiles (rows >= L are zero)
         if (tid < 64) {
             // inclusive prefix sum of g over the wave: within rows of 16 lanes by shifts, then across rows by broadcasts
@@ -218,59 +224,51 @@ __global__ __launch_bounds__(256) void gdn_chunk_kernel(const GdnParams p) {
         {
             const int col = (tid & 15) * 8;
 #pragma unroll
-            for (int cc = 0; cc < 4; cc++) {
-                const int row = (tid >> 4) + 16 * cc;
+            for (int cc = 0; cc < 2; cc++) {
+                const int row = (tid >> 4) + 32 * cc;
                 *(bf16x8*)(Ks + row * LD + col) = pk[cc];
                 *(bf16x8*)(Qs + row * LD + col) = pq[cc];
                 *(bf16x8*)(Vs + row * LD + col) = pv[cc];
             }
         }
-        GT_CLK(h1);
         fetch_data();          // chunk c0 + C, whose rows are known since the previous chunk
         fetch_rows(c0 + 2 * C);
-        GT_CLK(h2);
         lds_barrier();
-        GT_ADD(9, h0 - g0); GT_ADD(10, h1 - h0); GT_ADD(11, h2 - h1);
         const float GL = Gs[63];
         GT_CLK(g1);
 
-        // ---- (a) A = -strict_tril(beta_i K_i.K_j D_ij) fp32, (b) P = tril(s Q_i.K_j D_ij) bf16; computed transposed so that
-        // a lane holds row i and 4 consecutive columns j per register group.  Wave w: tile (jt = w>>1, it = w&1).
+        // ---- (a) A = -strict_tril(beta_i K_i.K_j D_ij) fp32 (waves with wh = 0), (b) P = tril(s Q_i.K_j D_ij) bf16 (wh = 1);
+        // computed transposed so that a lane holds row i and 4 consecutive columns j per register group.  Tile (jt, it) = wq.
         {
-            const int jt = w >> 1, it = w & 1;
-            f32x16 kk = zero16(), qk = zero16();
+            const int jt = wq >> 1, it = wq & 1;
+            const __bf16* rhs = wh ? Qs : Ks;
+            f32x16 acc = zero16();
 #pragma unroll
-            for (int s = 0; s < KD / 16; s++) {
-                const bf16x8 a = frag_nt(Ks, LD, 32 * jt, 16 * s, lane);    // rows j
-                kk = mfma(a, frag_nt(Ks, LD, 32 * it, 16 * s, lane), kk);   // cols i
-                qk = mfma(a, frag_nt(Qs, LD, 32 * it, 16 * s, lane), qk);
-            }
+            for (int s = 0; s < KD / 16; s++) acc = mfma(frag_nt(Ks, LD, 32 * jt, 16 * s, lane), frag_nt(rhs, LD, 32 * it, 16 * s, lane), acc);
             const int i = 32 * it + n32;
             const float Gi = Gs[i], bi = Bs[i];
 #pragma unroll
             for (int r4 = 0; r4 < 4; r4++) {
                 const int j0 = 32 * jt + 8 * r4 + 4 * g;
-                float4 av;
-                bf16x4 pv;
+                bf16x4 pv4;
                 float avv[4];
 #pragma unroll
                 for (int jj = 0; jj < 4; jj++) {
                     const int j = j0 + jj;
                     const float d = __expf(Gi - Gs[j]);
-                    avv[jj] = j < i ? -bi * kk[4 * r4 + jj] * d : 0.f;
-                    pv[jj] = (__bf16)(j <= i ? p.scale * qk[4 * r4 + jj] * d : 0.f);
+                    avv[jj] = j < i ? -bi * acc[4 * r4 + jj] * d : 0.f;
+                    pv4[jj] = (__bf16)(j <= i ? p.scale * acc[4 * r4 + jj] * d : 0.f);
                 }
-                av = make_float4(avv[0], avv[1], avv[2], avv[3]);
-                *(float4*)(As + i * LA + j0) = av;
-                *(bf16x4*)(Pm + i * LT + j0) = pv;
+                if (wh == 0) *(float4*)(As + i * LA + j0) = make_float4(avv[0], avv[1], avv[2], avv[3]);
+                else *(bf16x4*)(Pm + i * LT + j0) = pv4;
             }
         }
         lds_barrier();
-
         GT_CLK(g2);
-        // ---- T = (I - A)^-1 in place (fp32).  Stage 1: the four 16x16 diagonal blocks by forward substitution, wave b =
+
+        // ---- T = (I - A)^-1 in place (fp32).  Stage 1: the four 16x16 diagonal blocks by forward substitution, wave b < 4 =
         // block b, lane c < 16 = column c of the block.
-        if (lane < 16) {
+        if (w < 4 && lane < 16) {
             float t[16];
             const float* Ab = As + (16 * w) * LA + 16 * w;
 #pragma unroll
@@ -291,49 +289,55 @@ __global__ __launch_bounds__(256) void gdn_chunk_kernel(const GdnParams p) {
         {
             const int c16 = lane & 15, g4 = lane >> 4;
             if (w < 2) {
-                const int ra = 32 * w, rb = ra + 16;
+                const int rA = 32 * w, rB = rA + 16;
                 f32x4 x = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int s4 = 0; s4 < 4; s4++)        // X = A_lo T_aa
-                    x = __builtin_amdgcn_mfma_f32_16x16x4f32(As[(rb + c16) * LA + ra + 4 * s4 + g4], As[(ra + 4 * s4 + g4) * LA + ra + c16], x, 0, 0, 0);
+                    x = __builtin_amdgcn_mfma_f32_16x16x4f32(As[(rB + c16) * LA + rA + 4 * s4 + g4], As[(rA + 4 * s4 + g4) * LA + rA + c16], x, 0, 0, 0);
 #pragma unroll
                 for (int i = 0; i < 4; i++) Xs[(16 * w + 4 * g4 + i) * 36 + c16] = x[i];
                 __builtin_amdgcn_s_waitcnt(0xc07f);   // this wave's own X is in LDS (nobody else reads it)
                 f32x4 y = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int s4 = 0; s4 < 4; s4++)        // T_lo = T_bb X
-                    y = __builtin_amdgcn_mfma_f32_16x16x4f32(As[(rb + c16) * LA + rb + 4 * s4 + g4], Xs[(16 * w + 4 * s4 + g4) * 36 + c16], y, 0, 0, 0);
+                    y = __builtin_amdgcn_mfma_f32_16x16x4f32(As[(rB + c16) * LA + rB + 4 * s4 + g4], Xs[(16 * w + 4 * s4 + g4) * 36 + c16], y, 0, 0, 0);
 #pragma unroll
-                for (int i = 0; i < 4; i++) As[(rb + 4 * g4 + i) * LA + ra + c16] = y[i];
+                for (int i = 0; i < 4; i++) As[(rB + 4 * g4 + i) * LA + rA + c16] = y[i];
             }
         }
         lds_barrier();
-        // Stage 3: the 64x64 matrix: T_lo = T_11 A_lo T_00 with 32x32 blocks; wave w does the 16x16 tile (w>>1, w&1) of both products
+        // Stage 3: the 64x64 matrix: T_lo = T_11 A_lo T_00 with 32x32 blocks; wave w < 4 does the 16x16 tile (w>>1, w&1) of both products
         {
             const int c16 = lane & 15, g4 = lane >> 4;
-            const int ti = 16 * (w >> 1), tj = 16 * (w & 1);
-            f32x4 x = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int s4 = 0; s4 < 8; s4++)            // X = A_lo T_00
-                x = __builtin_amdgcn_mfma_f32_16x16x4f32(As[(32 + ti + c16) * LA + 4 * s4 + g4], As[(4 * s4 + g4) * LA + tj + c16], x, 0, 0, 0);
-#pragma unroll
-            for (int i = 0; i < 4; i++) Xs[(ti + 4 * g4 + i) * 36 + tj + c16] = x[i];
-            lds_barrier();
+            const int ti = 16 * ((w >> 1) & 1), tj = 16 * (w & 1);
             f32x4 y = {0.f, 0.f, 0.f, 0.f};
+            if (w < 4) {
+                f32x4 x = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int s4 = 0; s4 < 8; s4++)            // T_lo = T_11 X
-                y = __builtin_amdgcn_mfma_f32_16x16x4f32(As[(32 + ti + c16) * LA + 32 + 4 * s4 + g4], Xs[(4 * s4 + g4) * 36 + tj + c16], y, 0, 0, 0);
+                for (int s4 = 0; s4 < 8; s4++)            // X = A_lo T_00
+                    x = __builtin_amdgcn_mfma_f32_16x16x4f32(As[(32 + ti + c16) * LA + 4 * s4 + g4], As[(4 * s4 + g4) * LA + tj + c16], x, 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < 4; i++) Xs[(ti + 4 * g4 + i) * 36 + tj + c16] = x[i];
+            }
+            lds_barrier();
+            if (w < 4) {
+#pragma unroll
+                for (int s4 = 0; s4 < 8; s4++)            // T_lo = T_11 X
+                    y = __builtin_amdgcn_mfma_f32_16x16x4f32(As[(32 + ti + c16) * LA + 32 + 4 * s4 + g4], Xs[(4 * s4 + g4) * 36 + tj + c16], y, 0, 0, 0);
+            }
             lds_barrier();   // every read of the A_lo block is done
+            if (w < 4) {
 #pragma unroll
-            for (int i = 0; i < 4; i++) As[(32 + ti + 4 * g4 + i) * LA + tj + c16] = y[i];
+                for (int i = 0; i < 4; i++) As[(32 + ti + 4 * g4 + i) * LA + tj + c16] = y[i];
+            }
         }
         lds_barrier();
         GT_CLK(g3);
-        // ---- Tu = T diag(beta), Tw = -T diag(beta e^G) (bf16).  thread: row tid/4, 16 columns
+        // ---- Tu = T diag(beta), Tw = -T diag(beta e^G) (bf16).  thread: row tid/8, 8 columns
         {
-            const int i = tid >> 2, jb = (tid & 3) * 16;
+            const int i = tid >> 3, jb = (tid & 7) * 8;
 #pragma unroll
-            for (int j4 = 0; j4 < 4; j4++) {
+            for (int j4 = 0; j4 < 2; j4++) {
                 const float4 t = *(const float4*)(As + i * LA + jb + 4 * j4);
                 const float tv[4] = {t.x, t.y, t.z, t.w};
                 bf16x4 u, ww;
@@ -349,75 +353,78 @@ __global__ __launch_bounds__(256) void gdn_chunk_kernel(const GdnParams p) {
             }
         }
         lds_barrier();
-
         GT_CLK(g4);
-        // ---- (c) U^T[v][i] = sum_j V[j][v] Tu[i][j]  and  -W^T[d][i] = sum_j K[j][d] Tw[i][j]; wave w: rows 32w.. of v / d
-        f32x16 acc[2];      // U^T, later V'^T : tile it = token columns 32 it..
+
+        // ---- (c) U^T[v][i] = sum_j V[j][v] Tu[i][j] (waves wh = 0, kept in registers) and -W^T[d][i] = sum_j K[j][d] Tw[i][j]
+        // (waves wh = 1, written to LDS); wave: rows 32wq.. of v / d, both token tiles
+        f32x16 acc[2];      // wh = 0: U^T, later V'^T; wh = 1: -W^T, later (Q S)^T.  Tile it = token columns 32 it..
+        acc[0] = zero16();
+        acc[1] = zero16();
         {
-            f32x16 wn[2];
-            acc[0] = zero16(); acc[1] = zero16(); wn[0] = zero16(); wn[1] = zero16();
+            const __bf16* lhs = wh ? Ks : Vs;
+            const __bf16* rhs = wh ? Tw : Tu;
 #pragma unroll
             for (int s = 0; s < C / 16; s++) {
-                const bf16x8 av = frag_tr(Vs, LD, 16 * s, 32 * w, lane);
-                const bf16x8 ak = frag_tr(Ks, LD, 16 * s, 32 * w, lane);
+                const bf16x8 a = frag_tr(lhs, LD, 16 * s, 32 * wq, lane);
 #pragma unroll
-                for (int it = 0; it < 2; it++) {
-                    acc[it] = mfma(av, frag_nt(Tu, LT, 32 * it, 16 * s, lane), acc[it]);
-                    wn[it] = mfma(ak, frag_nt(Tw, LT, 32 * it, 16 * s, lane), wn[it]);
-                }
+                for (int it = 0; it < 2; it++) acc[it] = mfma(a, frag_nt(rhs, LT, 32 * it, 16 * s, lane), acc[it]);
             }
+            if (wh) {
 #pragma unroll
-            for (int it = 0; it < 2; it++)
+                for (int it = 0; it < 2; it++)
 #pragma unroll
-                for (int r4 = 0; r4 < 4; r4++) {
-                    bf16x4 t;
+                    for (int r4 = 0; r4 < 4; r4++) {
+                        bf16x4 t;
 #pragma unroll
-                    for (int j = 0; j < 4; j++) t[j] = (__bf16)wn[it][4 * r4 + j];
-                    *(bf16x4*)(Wn + (32 * it + n32) * LD + 32 * w + 8 * r4 + 4 * g) = t;
-                }
+                        for (int j = 0; j < 4; j++) t[j] = (__bf16)acc[it][4 * r4 + j];
+                        *(bf16x4*)(Wn + (32 * it + n32) * LD + 32 * wq + 8 * r4 + 4 * g) = t;
+                    }
+                acc[0] = zero16();
+                acc[1] = zero16();
+            }
         }
         lds_barrier();   // -W visible; V (Vs) and T (As) are dead from here
-
         GT_CLK(g5);
-        // ---- (d) V'^T = U^T + S^T (-W)^T   and   (e1) QS^T[v][i] = sum_k S^T[v][k] Q[i][k]
-        f32x16 qs[2];
-        qs[0] = zero16(); qs[1] = zero16();
+
+        // ---- (d) wh = 0: V'^T = U^T + S^T (-W)^T;  (e1) wh = 1: QS^T[v][i] = sum_k S^T[v][k] Q[i][k]
+        {
+            const __bf16* rhs = wh ? Qs : Wn;
 #pragma unroll
-        for (int s = 0; s < KD / 16; s++) {
-            const bf16x8 a = frag_nt(St, LD, 32 * w, 16 * s, lane);
+            for (int s = 0; s < KD / 16; s++) {
+                const bf16x8 a = frag_nt(St, LD, 32 * wq, 16 * s, lane);
 #pragma unroll
-            for (int it = 0; it < 2; it++) {
-                acc[it] = mfma(a, frag_nt(Wn, LD, 32 * it, 16 * s, lane), acc[it]);
-                qs[it] = mfma(a, frag_nt(Qs, LD, 32 * it, 16 * s, lane), qs[it]);
+                for (int it = 0; it < 2; it++) acc[it] = mfma(a, frag_nt(rhs, LD, 32 * it, 16 * s, lane), acc[it]);
             }
         }
         // V' and V' e^{G_L - G_i}, row-major [i][v], bf16
+        if (wh == 0) {
 #pragma unroll
-        for (int it = 0; it < 2; it++) {
-            const int i = 32 * it + n32;
-            const float dec = __expf(GL - Gs[i]);
+            for (int it = 0; it < 2; it++) {
+                const int i = 32 * it + n32;
+                const float dec = __expf(GL - Gs[i]);
 #pragma unroll
-            for (int r4 = 0; r4 < 4; r4++) {
-                bf16x4 t, td;
+                for (int r4 = 0; r4 < 4; r4++) {
+                    bf16x4 t, td;
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    t[j] = (__bf16)acc[it][4 * r4 + j];
-                    td[j] = (__bf16)(acc[it][4 * r4 + j] * dec);
+                    for (int j = 0; j < 4; j++) {
+                        t[j] = (__bf16)acc[it][4 * r4 + j];
+                        td[j] = (__bf16)(acc[it][4 * r4 + j] * dec);
+                    }
+                    *(bf16x4*)(Vs + i * LD + 32 * wq + 8 * r4 + 4 * g) = t;
+                    *(bf16x4*)(Vd + i * LD + 32 * wq + 8 * r4 + 4 * g) = td;
                 }
-                *(bf16x4*)(Vs + i * LD + 32 * w + 8 * r4 + 4 * g) = t;
-                *(bf16x4*)(Vd + i * LD + 32 * w + 8 * r4 + 4 * g) = td;
             }
         }
         lds_barrier();
-
         GT_CLK(g6);
-        // ---- (e2) O^T[v][i] = s e^{G_i} QS^T + sum_j V'[j][v] P[i][j]
-        {
+
+        // ---- (e2) wh = 1: O^T[v][i] = s e^{G_i} QS^T + sum_j V'[j][v] P[i][j]
+        if (wh) {
             f32x16 ov[2];
             ov[0] = zero16(); ov[1] = zero16();
 #pragma unroll
             for (int s = 0; s < C / 16; s++) {
-                const bf16x8 a = frag_tr(Vs, LD, 16 * s, 32 * w, lane);
+                const bf16x8 a = frag_tr(Vs, LD, 16 * s, 32 * wq, lane);
 #pragma unroll
                 for (int it = 0; it < 2; it++) ov[it] = mfma(a, frag_nt(Pm, LT, 32 * it, 16 * s, lane), ov[it]);
             }
@@ -426,43 +433,35 @@ __global__ __launch_bounds__(256) void gdn_chunk_kernel(const GdnParams p) {
                 const int i = 32 * it + n32;
                 if (i < L) {
                     const float sc = p.scale * __expf(Gs[i]);
-                    __bf16* op = p.o + Rs[i] * p.o_tok + (long)hv * VD + 32 * w + 4 * g;
+                    __bf16* op = p.o + Rs[i] * p.o_tok + (long)hv * VD + 32 * wq + 4 * g;
 #pragma unroll
                     for (int r4 = 0; r4 < 4; r4++) {
                         bf16x4 t;
 #pragma unroll
-                        for (int j = 0; j < 4; j++) t[j] = (__bf16)(__builtin_fmaf(sc, qs[it][4 * r4 + j], ov[it][4 * r4 + j]));
+                        for (int j = 0; j < 4; j++) t[j] = (__bf16)(__builtin_fmaf(sc, acc[it][4 * r4 + j], ov[it][4 * r4 + j]));
                         *(bf16x4*)(op + 8 * r4) = t;
                     }
                 }
             }
         }
-
         GT_CLK(g7);
-        // ---- (f) S[k][v] = e^{G_L} S[k][v] + sum_j K[j][k] (V' e^{G_L - G_j})[j][v]; wave w: k rows 32w.., all four v tiles
+
+        // ---- (f) S[k][v] = e^{G_L} S[k][v] + sum_j K[j][k] (V' e^{G_L - G_j})[j][v]; wave: k rows 32wq.., v tiles 2wh, 2wh + 1
         {
             const float eg = __expf(GL);
 #pragma unroll
-            for (int vt = 0; vt < 4; vt++)
+            for (int j = 0; j < 2; j++)
 #pragma unroll
-                for (int r = 0; r < 16; r++) S[vt][r] *= eg;
+                for (int r = 0; r < 16; r++) S[j][r] *= eg;
 #pragma unroll
             for (int s = 0; s < C / 16; s++) {
-                const bf16x8 a = frag_tr(Ks, LD, 16 * s, 32 * w, lane);
+                const bf16x8 a = frag_tr(Ks, LD, 16 * s, 32 * wq, lane);
 #pragma unroll
-                for (int vt = 0; vt < 4; vt++) S[vt] = mfma(a, frag_tr(Vd, LD, 16 * s, 32 * vt, lane), S[vt]);
+                for (int j = 0; j < 2; j++) S[j] = mfma(a, frag_tr(Vd, LD, 16 * s, 64 * wh + 32 * j, lane), S[j]);
             }
         }
         lds_barrier();   // every wave is done reading S^T (d, e1) before it is replaced
-#pragma unroll
-        for (int vt = 0; vt < 4; vt++)
-#pragma unroll
-            for (int r4 = 0; r4 < 4; r4++) {
-                bf16x4 t;
-#pragma unroll
-                for (int j = 0; j < 4; j++) t[j] = (__bf16)S[vt][4 * r4 + j];
-                *(bf16x4*)(St + (32 * vt + n32) * LD + 32 * w + 8 * r4 + 4 * g) = t;
-            }
+        mirror();
         GT_CLK(g8);
         GT_ADD(0, g1 - g0); GT_ADD(1, g2 - g1); GT_ADD(2, g3 - g2); GT_ADD(3, g4 - g3); GT_ADD(4, g5 - g4); GT_ADD(5, g6 - g5); GT_ADD(6, g7 - g6); GT_ADD(7, g8 - g7); GT_ADD(8, 1);
     }
@@ -472,9 +471,9 @@ __global__ __launch_bounds__(256) void gdn_chunk_kernel(const GdnParams p) {
         if (dst >= 0) {
             float* hp = p.ht + (dst * p.hv + hv) * (long)KD * VD;
 #pragma unroll
-            for (int vt = 0; vt < 4; vt++)
+            for (int j = 0; j < 2; j++)
 #pragma unroll
-                for (int r = 0; r < 16; r++) hp[(long)(32 * w + 8 * (r >> 2) + 4 * g + (r & 3)) * VD + 32 * vt + n32] = S[vt][r];
+                for (int r = 0; r < 16; r++) hp[(long)(32 * wq + 8 * (r >> 2) + 4 * g + (r & 3)) * VD + 64 * wh + 32 * j + n32] = S[j][r];
         }
     }
 }
@@ -491,7 +490,7 @@ int gdn_chunked_launch(const GdnParams& p, long max_len, hipStream_t stream) {
     }
     const long blocks = p.n_seg * p.hv;
     if (blocks > INT32_MAX) return spinf_fail(SPINF_E_ARG, "gdn chunked: too many segments");
-    hipLaunchKernelGGL(gdn_chunk_kernel, dim3((unsigned)blocks), dim3(256), LDS_BYTES, stream, p);
+    hipLaunchKernelGGL(gdn_chunk_kernel, dim3((unsigned)blocks), dim3(512), LDS_BYTES, stream, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "gdn chunked: launch: %s", hipGetErrorString(e));
     return SPINF_OK;
