@@ -20,11 +20,60 @@ struct GdnParams {
     const float* h0; const long* h0_idx; float* ht; const long* ht_idx;
 };
 
-// ---------------------------------------------------------------------------------------------- token by token
-// One wave per (segment, value head, 32 values): lane (v = lane%32, half = lane/32) keeps rows 64 half .. 64 half + 63
-// of column v of the state in registers.  Meant for the short segments of a trie (a handful of tokens after a fork).
-__global__ __launch_bounds__(64) void gdn_recurrent_kernel(const GdnParams p) {
+// ---------------------------------------------------------------------------------------------- short segments
+// The recurrent entry point: meant for the short segments of a trie (a handful of tokens after a fork), thousands per call.
+// One wave per (segment, value head, 32 value columns) and no workgroup barrier anywhere.  The wave walks its segment in
+// mini-chunks of 16 tokens with the same WY algebra as the chunk-64 kernel (A = -strict_tril(beta_i K_i.K_j e^{G_i-G_j}),
+// T = (I - A)^-1, U = T diag(beta) V, -W = -T diag(beta e^G) K, V' = U - W S, O = s e^G Q S + P V', S <- e^{G_L} S +
+// K^T (V' e^{G_L-G})), on 16x16 MFMA tiles laid out so that every product's result is already the next product's operand:
+//   * the state slice S[128][32] stays in fp32 accumulator layout (lane = value column, 4 consecutive key rows per tile): two
+//     key tiles side by side are the B operand of a 16x16x32 product over a permuted contraction index, and K and Q rows are
+//     fetched in that same permutation, so S is never moved, only rounded to bf16 on the way into the matrix core;
+//   * Q.K^T and K.K^T are computed transposed (lane = row i, registers = columns j), which is the A operand layout of P in
+//     O = P V' and the row layout (I - A)^-1 is solved in; every lane solves row i = lane % 16 by substitution in registers;
+//   * -W^T and V' come out of their products as the A and B operands of the products that consume them.
+// The state is kept and accumulated in fp32; products take bf16 operands, as in the chunk-64 kernel.
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+namespace {
+constexpr int MC = 16;      // tokens per mini-chunk
+constexpr int LDK = 136;    // row stride (elements) of the K tile in LDS
+constexpr int LDV = 40;     // row stride of the V and O tiles
+constexpr int LDA = 20;     // row stride (floats) of A
+
+__device__ __forceinline__ f32x4 mfma32(bf16x8 a, bf16x8 b, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); }
+__device__ __forceinline__ f32x4 mfma16(bf16x4 a, bf16x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, a), __builtin_bit_cast(s16x4, b), c, 0, 0, 0);
+}
+// Operand of a 16x16x16 product whose contraction index is the ROW index of a row-major LDS tile: lane gets column
+// col0 + lane%16 of rows row0 + 4 (lane/16) .. +3 (each group of 16 lanes transposes a 4 x 16 block).
+__device__ __forceinline__ bf16x4 frag_tr4(const __bf16* base, int stride, int row0, int col0, int lane) {
+    const int t = lane & 15;
+    const __bf16* p = base + (row0 + 4 * (lane >> 4) + (t >> 2)) * stride + col0 + 4 * (t & 3);
+    return __builtin_bit_cast(bf16x4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p));
+}
+__device__ __forceinline__ bf16x8 join(bf16x4 lo, bf16x4 hi) { return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7); }
+__device__ __forceinline__ bf16x4 round4(f32x4 x) {
+    bf16x4 r;
+#pragma unroll
+    for (int i = 0; i < 4; i++) r[i] = (__bf16)x[i];
+    return r;
+}
+// Orders this wave's LDS writes before its later LDS reads for the compiler; the hardware runs one wave's LDS operations in order.
+__device__ __forceinline__ void wave_lds_order() { asm volatile("" ::: "memory"); }
+}  // namespace
+
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void gdn_short_kernel(const GdnParams p) {
     constexpr int K = 128;
+    __shared__ __attribute__((aligned(16))) __bf16 Ksm[MC * LDK];
+    __shared__ __attribute__((aligned(16))) __bf16 Vsm[MC * LDV];
+    __shared__ __attribute__((aligned(16))) __bf16 Osm[MC * LDV];
+    __shared__ __attribute__((aligned(16))) float As[MC * LDA];
+    __shared__ __attribute__((aligned(16))) float Gs[MC];
+    __shared__ __attribute__((aligned(16))) float Bs[MC];
+
     const int nvb = p.dv / 32;
     const long b = blockIdx.x;
     const int iv = (int)(b % nvb);
@@ -32,57 +81,186 @@ __global__ __launch_bounds__(64) void gdn_recurrent_kernel(const GdnParams p) {
     const long n = nh / p.hv;
     const int hv = (int)(nh % p.hv);
     const int hk = hv / (p.hv / p.h);
-    const int lane = threadIdx.x, vv = iv * 32 + (lane & 31), half = lane >> 5;
-    float S[64];
+    const int lane = threadIdx.x, c = lane & 15, q4 = lane >> 4;
+    const int vrow = lane >> 2, vcol = (lane & 3) * 8;      // this lane's 16-byte piece of the V and O tiles
+
+    // state: S[kt][vt][r] = S[16 kt + 4 q4 + r][32 iv + 16 vt + c]
+    f32x4 S[8][2];
 #pragma unroll
-    for (int i = 0; i < 64; i++) S[i] = 0.f;
+    for (int kt = 0; kt < 8; kt++)
+#pragma unroll
+        for (int vt = 0; vt < 2; vt++) S[kt][vt] = f32x4{0.f, 0.f, 0.f, 0.f};
     if (p.h0 != nullptr && p.h0_idx != nullptr) {
         const long src = p.h0_idx[n];
         if (src >= 0) {
-            const float* hp = p.h0 + ((src * p.hv + hv) * K + 64 * half) * p.dv + vv;
+            const float* hp = p.h0 + ((src * p.hv + hv) * K + 4 * q4) * p.dv + 32 * iv + c;
 #pragma unroll
-            for (int i = 0; i < 64; i++) S[i] = hp[(long)i * p.dv];
+            for (int kt = 0; kt < 8; kt++)
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+#pragma unroll
+                    for (int vt = 0; vt < 2; vt++) S[kt][vt][r] = hp[(long)(16 * kt + r) * p.dv + 16 * vt];
         }
     }
+    const bool keep = p.ht != nullptr && p.ht_idx != nullptr && p.ht_idx[n] >= 0;
     const long bos = p.cu[n], eos = p.cu[n + 1];
-    for (long t = bos; t < eos; t++) {
-        const long r = p.idx ? p.idx[t] : t;
-        const __bf16* kp = p.k + r * p.q_tok + (long)hk * K + 64 * half;
-        const __bf16* qp = p.q + r * p.q_tok + (long)hk * K + 64 * half;
-        bf16x8 kr[8], qr[8];
+    const int T = (int)(eos - bos);
+
+    for (int c0 = 0; c0 < T; c0 += MC) {
+        const int L = min(MC, T - c0);
+        // ---- fetch: lane (c, q4) takes row c of K and Q in the contraction order of the state operand (per 32 columns: 4 q4 ..+3
+        // and 16 + 4 q4 ..+3), g and beta of row c; lane (vrow, vcol) a 16-byte piece of V.  Rows >= L are zero.
+        long rc = -1, rv = -1;
+        if (c < L) { const long t = bos + c0 + c; rc = p.idx ? p.idx[t] : t; }
+        if (vrow < L) { const long t = bos + c0 + vrow; rv = p.idx ? p.idx[t] : t; }
+        bf16x4 klo[4], khi[4], qlo[4], qhi[4];
 #pragma unroll
-        for (int c = 0; c < 8; c++) {
-            kr[c] = *(const bf16x8*)(kp + 8 * c);
-            qr[c] = *(const bf16x8*)(qp + 8 * c);
-        }
-        const float vt = (float)p.v[r * p.v_tok + (long)hv * p.dv + vv];
-        const float gt = p.g[r * p.g_tok + hv];
-        const float bt = (float)p.beta[r * p.g_tok + hv];
-        const float eg = __expf(gt);
-        float dot = 0.f;
+        for (int s = 0; s < 4; s++)
 #pragma unroll
-        for (int i = 0; i < 64; i++) {
-            S[i] *= eg;
-            dot = __builtin_fmaf(S[i], (float)kr[i >> 3][i & 7], dot);
-        }
-        dot += __shfl_xor(dot, 32);
-        const float dl = (vt - dot) * bt;
-        float od = 0.f;
+            for (int j = 0; j < 4; j++) { klo[s][j] = (__bf16)0.f; khi[s][j] = (__bf16)0.f; qlo[s][j] = (__bf16)0.f; qhi[s][j] = (__bf16)0.f; }
+        float gv = 0.f, bv = 0.f;
+        if (rc >= 0) {
+            const __bf16* kp = p.k + rc * p.q_tok + (long)hk * K + 4 * q4;
+            const __bf16* qp = p.q + rc * p.q_tok + (long)hk * K + 4 * q4;
 #pragma unroll
-        for (int i = 0; i < 64; i++) {
-            S[i] = __builtin_fmaf((float)kr[i >> 3][i & 7], dl, S[i]);
-            od = __builtin_fmaf(S[i], (float)qr[i >> 3][i & 7] * p.scale, od);
+            for (int s = 0; s < 4; s++) {
+                klo[s] = *(const bf16x4*)(kp + 32 * s);
+                khi[s] = *(const bf16x4*)(kp + 32 * s + 16);
+                qlo[s] = *(const bf16x4*)(qp + 32 * s);
+                qhi[s] = *(const bf16x4*)(qp + 32 * s + 16);
+            }
+            gv = p.g[rc * p.g_tok + hv];
+            bv = (float)p.beta[rc * p.g_tok + hv];
         }
-        od += __shfl_xor(od, 32);
-        if (half == 0) p.o[r * p.o_tok + (long)hv * p.dv + vv] = (__bf16)od;
+        bf16x8 vv;
+#pragma unroll
+        for (int j = 0; j < 8; j++) vv[j] = (__bf16)0.f;
+        if (rv >= 0) vv = *(const bf16x8*)(p.v + rv * p.v_tok + (long)hv * p.dv + 32 * iv + vcol);
+
+        wave_lds_order();   // the previous mini-chunk's reads come first
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+            *(bf16x4*)(Ksm + c * LDK + 32 * s + 4 * q4) = klo[s];
+            *(bf16x4*)(Ksm + c * LDK + 32 * s + 16 + 4 * q4) = khi[s];
+        }
+        *(bf16x8*)(Vsm + vrow * LDV + vcol) = vv;
+        // G_c = g_0 + .. + g_c: every group of 16 lanes holds the same 16 values
+        float Gi = gv;
+        Gi += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, Gi), 0x111, 0xf, 0xf, true));   // row_shr:1
+        Gi += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, Gi), 0x112, 0xf, 0xf, true));   // row_shr:2
+        Gi += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, Gi), 0x114, 0xf, 0xf, true));   // row_shr:4
+        Gi += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, Gi), 0x118, 0xf, 0xf, true));   // row_shr:8
+        Gs[c] = Gi;
+        Bs[c] = bv;
+        wave_lds_order();
+        const f32x4 Gj = *(const f32x4*)(Gs + 4 * q4), Bj = *(const f32x4*)(Bs + 4 * q4);
+        const float GL = Gs[MC - 1];
+
+        // ---- (K K^T)^T and (Q K^T)^T: lane = row i = c, registers = columns j = 4 q4 + r
+        f32x4 kk = {0.f, 0.f, 0.f, 0.f}, qk = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+            const bf16x8 kf = join(klo[s], khi[s]);
+            kk = mfma32(kf, kf, kk);
+            qk = mfma32(kf, join(qlo[s], qhi[s]), qk);
+        }
+        bf16x4 pA;     // P[i][j] = s Q_i.K_j e^{G_i - G_j}, j <= i
+        {
+            f32x4 a4;
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int j = 4 * q4 + r;
+                const float d = __expf(Gi - Gj[r]);
+                a4[r] = j < c ? -bv * kk[r] * d : 0.f;
+                pA[r] = (__bf16)(j <= c ? p.scale * qk[r] * d : 0.f);
+            }
+            *(f32x4*)(As + c * LDA + 4 * q4) = a4;
+        }
+        wave_lds_order();
+        // ---- row c of T = (I - A)^-1 (T = I + T A): t[j] = [j == c] + sum_{m > j} t[m] A[m][j], highest m first
+        float t[MC];
+#pragma unroll
+        for (int j = 0; j < MC; j++) t[j] = (j == c) ? 1.f : 0.f;
+#pragma unroll
+        for (int m = MC - 1; m >= 1; m--) {
+#pragma unroll
+            for (int j4 = 0; 4 * j4 < m; j4++) {
+                const f32x4 am = *(const f32x4*)(As + m * LDA + 4 * j4);
+#pragma unroll
+                for (int jj = 0; jj < 4; jj++)
+                    if (4 * j4 + jj < m) t[4 * j4 + jj] = __builtin_fmaf(t[m], am[jj], t[4 * j4 + jj]);
+            }
+        }
+        // T diag(beta) and -T diag(beta e^G), columns 4 q4 + r of row c
+        bf16x4 tuA, twB;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const float tv = q4 == 0 ? t[r] : q4 == 1 ? t[4 + r] : q4 == 2 ? t[8 + r] : t[12 + r];
+            const float tb = tv * Bj[r];
+            tuA[r] = (__bf16)tb;
+            twB[r] = (__bf16)(-tb * __expf(Gj[r]));
+        }
+        // ---- U[i][v] = sum_j Tu[i][j] V[j][v]   (lane = column v, registers = rows i)
+        f32x4 vp[2], qs[2];
+#pragma unroll
+        for (int vt = 0; vt < 2; vt++) {
+            vp[vt] = mfma16(tuA, frag_tr4(Vsm, LDV, 0, 16 * vt, lane), f32x4{0.f, 0.f, 0.f, 0.f});
+            qs[vt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+        // ---- -W^T[k][i] = sum_j K[j][k] Tw[i][j]; then V' = U + (-W) S and Q S over the 128 key rows, 32 at a time
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+            const f32x4 w0 = mfma16(frag_tr4(Ksm, LDK, 0, 32 * s, lane), twB, f32x4{0.f, 0.f, 0.f, 0.f});
+            const f32x4 w1 = mfma16(frag_tr4(Ksm, LDK, 0, 32 * s + 16, lane), twB, f32x4{0.f, 0.f, 0.f, 0.f});
+            const bf16x8 wA = join(round4(w0), round4(w1));
+            const bf16x8 qA = join(qlo[s], qhi[s]);
+#pragma unroll
+            for (int vt = 0; vt < 2; vt++) {
+                const bf16x8 sb = join(round4(S[2 * s][vt]), round4(S[2 * s + 1][vt]));
+                vp[vt] = mfma32(wA, sb, vp[vt]);
+                qs[vt] = mfma32(qA, sb, qs[vt]);
+            }
+        }
+        // ---- O[i][v] = s e^{G_i} (Q S)[i][v] + sum_j P[i][j] V'[j][v], rows i = 4 q4 + r; through LDS for 16-byte stores
+        bf16x4 vb[2];
+#pragma unroll
+        for (int vt = 0; vt < 2; vt++) {
+            vb[vt] = round4(vp[vt]);
+            const f32x4 o = mfma16(pA, vb[vt], f32x4{0.f, 0.f, 0.f, 0.f});
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                Osm[(4 * q4 + r) * LDV + 16 * vt + c] = (__bf16)__builtin_fmaf(p.scale * __expf(Gj[r]), qs[vt][r], o[r]);
+        }
+        wave_lds_order();
+        if (rv >= 0) *(bf16x8*)(p.o + rv * p.o_tok + (long)hv * p.dv + 32 * iv + vcol) = *(const bf16x8*)(Osm + vrow * LDV + vcol);
+        // ---- S[k][v] = e^{G_L} S[k][v] + sum_j K[j][k] (V' e^{G_L - G_j})[j][v]; skipped when nothing reads the state again
+        if (c0 + MC < T || keep) {
+            const float eg = __expf(GL);
+            bf16x4 vd[2];
+#pragma unroll
+            for (int vt = 0; vt < 2; vt++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) vd[vt][r] = (__bf16)(vp[vt][r] * __expf(GL - Gj[r]));
+#pragma unroll
+            for (int kt = 0; kt < 8; kt++) {
+                const bf16x4 kT = frag_tr4(Ksm, LDK, 0, 16 * kt, lane);
+#pragma unroll
+                for (int vt = 0; vt < 2; vt++) {
+#pragma unroll
+                    for (int r = 0; r < 4; r++) S[kt][vt][r] *= eg;
+                    S[kt][vt] = mfma16(kT, vd[vt], S[kt][vt]);
+                }
+            }
+        }
     }
-    if (p.ht != nullptr && p.ht_idx != nullptr) {
-        const long dst = p.ht_idx[n];
-        if (dst >= 0) {
-            float* hp = p.ht + ((dst * p.hv + hv) * K + 64 * half) * p.dv + vv;
+    if (keep) {
+        float* hp = p.ht + ((p.ht_idx[n] * p.hv + hv) * K + 4 * q4) * p.dv + 32 * iv + c;
 #pragma unroll
-            for (int i = 0; i < 64; i++) hp[(long)i * p.dv] = S[i];
-        }
+        for (int kt = 0; kt < 8; kt++)
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+#pragma unroll
+                for (int vt = 0; vt < 2; vt++) hp[(long)(16 * kt + r) * p.dv + 16 * vt] = S[kt][vt][r];
     }
 }
 
@@ -109,9 +287,11 @@ extern "C" int spinf_gdn_fwd(const spinf_gdn_args* a, void* stream) {
     hipStream_t s = (hipStream_t)stream;
     if (a->mode == 1) return gdn_chunked_launch(p, a->max_len, s);
     if (a->mode != 0) return spinf_fail(SPINF_E_ARG, "gdn: unknown mode %d", a->mode);
+    if (a->v_tok % 8 || a->o_tok % 8) return spinf_fail(SPINF_E_ARG, "gdn: v/o row stride must be a multiple of 8 elements");
+    if (((uintptr_t)a->v | (uintptr_t)a->o) % 16) return spinf_fail(SPINF_E_ARG, "gdn: v/o must be 16-byte aligned");
     const long blocks = a->n_seg * a->hv * (a->dv / 32);
     if (blocks > INT32_MAX) return spinf_fail(SPINF_E_ARG, "gdn: too many segments");
-    hipLaunchKernelGGL(gdn_recurrent_kernel, dim3((unsigned)blocks), dim3(64), 0, s, p);
+    hipLaunchKernelGGL(gdn_short_kernel, dim3((unsigned)blocks), dim3(64), 0, s, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "gdn: launch: %s", hipGetErrorString(e));
     return SPINF_OK;
