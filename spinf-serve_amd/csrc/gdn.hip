@@ -10,15 +10,9 @@
 #include "spinf_tree.h"
 #include "common.h"
 
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+#include "gdn_tiles.h"
 
-struct GdnParams {
-    const __bf16* q; const __bf16* k; const __bf16* v; const float* g; const __bf16* beta; __bf16* o;
-    long q_tok, v_tok, g_tok, o_tok;
-    int h, hv, dk, dv; float scale;
-    const long* cu; const long* idx; long n_seg;
-    const float* h0; const long* h0_idx; float* ht; const long* ht_idx;
-};
+using namespace gdn_tiles;
 
 // ---------------------------------------------------------------------------------------------- short segments
 // The recurrent entry point: meant for the short segments of a trie (a handful of tokens after a fork), thousands per call.
@@ -33,36 +27,11 @@ struct GdnParams {
 //     O = P V' and the row layout (I - A)^-1 is solved in; every lane solves row i = lane % 16 by substitution in registers;
 //   * -W^T and V' come out of their products as the A and B operands of the products that consume them.
 // The state is kept and accumulated in fp32; products take bf16 operands, as in the chunk-64 kernel.
-typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
-typedef __attribute__((ext_vector_type(4))) short s16x4;
-typedef __attribute__((ext_vector_type(4))) float f32x4;
-
 namespace {
 constexpr int MC = 16;      // tokens per mini-chunk
 constexpr int LDK = 136;    // row stride (elements) of the K tile in LDS
 constexpr int LDV = 40;     // row stride of the V and O tiles
 constexpr int LDA = 20;     // row stride (floats) of A
-
-__device__ __forceinline__ f32x4 mfma32(bf16x8 a, bf16x8 b, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); }
-__device__ __forceinline__ f32x4 mfma16(bf16x4 a, bf16x4 b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, a), __builtin_bit_cast(s16x4, b), c, 0, 0, 0);
-}
-// Operand of a 16x16x16 product whose contraction index is the ROW index of a row-major LDS tile: lane gets column
-// col0 + lane%16 of rows row0 + 4 (lane/16) .. +3 (each group of 16 lanes transposes a 4 x 16 block).
-__device__ __forceinline__ bf16x4 frag_tr4(const __bf16* base, int stride, int row0, int col0, int lane) {
-    const int t = lane & 15;
-    const __bf16* p = base + (row0 + 4 * (lane >> 4) + (t >> 2)) * stride + col0 + 4 * (t & 3);
-    return __builtin_bit_cast(bf16x4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p));
-}
-__device__ __forceinline__ bf16x8 join(bf16x4 lo, bf16x4 hi) { return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7); }
-__device__ __forceinline__ bf16x4 round4(f32x4 x) {
-    bf16x4 r;
-#pragma unroll
-    for (int i = 0; i < 4; i++) r[i] = (__bf16)x[i];
-    return r;
-}
-// Orders this wave's LDS writes before its later LDS reads for the compiler; the hardware runs one wave's LDS operations in order.
-__device__ __forceinline__ void wave_lds_order() { asm volatile("" ::: "memory"); }
 }  // namespace
 
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void gdn_short_kernel(const GdnParams p) {
@@ -89,7 +58,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void
 #pragma unroll
     for (int kt = 0; kt < 8; kt++)
 #pragma unroll
-        for (int vt = 0; vt < 2; vt++) S[kt][vt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int vt = 0; vt < 2; vt++) S[kt][vt] = zero4();
     if (p.h0 != nullptr && p.h0_idx != nullptr) {
         const long src = p.h0_idx[n];
         if (src >= 0) {
@@ -145,11 +114,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void
         }
         *(bf16x8*)(Vsm + vrow * LDV + vcol) = vv;
         // G_c = g_0 + .. + g_c: every group of 16 lanes holds the same 16 values
-        float Gi = gv;
-        Gi += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, Gi), 0x111, 0xf, 0xf, true));   // row_shr:1
-        Gi += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, Gi), 0x112, 0xf, 0xf, true));   // row_shr:2
-        Gi += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, Gi), 0x114, 0xf, 0xf, true));   // row_shr:4
-        Gi += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, Gi), 0x118, 0xf, 0xf, true));   // row_shr:8
+        const float Gi = row_prefix_sum(gv);
         Gs[c] = Gi;
         Bs[c] = bv;
         wave_lds_order();
@@ -177,26 +142,15 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void
             *(f32x4*)(As + c * LDA + 4 * q4) = a4;
         }
         wave_lds_order();
-        // ---- row c of T = (I - A)^-1 (T = I + T A): t[j] = [j == c] + sum_{m > j} t[m] A[m][j], highest m first
+        // ---- row c of T = (I - A)^-1, solved by every group of 16 lanes alike
         float t[MC];
-#pragma unroll
-        for (int j = 0; j < MC; j++) t[j] = (j == c) ? 1.f : 0.f;
-#pragma unroll
-        for (int m = MC - 1; m >= 1; m--) {
-#pragma unroll
-            for (int j4 = 0; 4 * j4 < m; j4++) {
-                const f32x4 am = *(const f32x4*)(As + m * LDA + 4 * j4);
-#pragma unroll
-                for (int jj = 0; jj < 4; jj++)
-                    if (4 * j4 + jj < m) t[4 * j4 + jj] = __builtin_fmaf(t[m], am[jj], t[4 * j4 + jj]);
-            }
-        }
+        unit_lower_inverse_row(As, LDA, c, t);
         // T diag(beta) and -T diag(beta e^G), columns 4 q4 + r of row c
         bf16x4 tuA, twB;
+        const f32x4 tq = pick4(t, q4);
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-            const float tv = q4 == 0 ? t[r] : q4 == 1 ? t[4 + r] : q4 == 2 ? t[8 + r] : t[12 + r];
-            const float tb = tv * Bj[r];
+            const float tb = tq[r] * Bj[r];
             tuA[r] = (__bf16)tb;
             twB[r] = (__bf16)(-tb * __expf(Gj[r]));
         }
@@ -204,14 +158,14 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void
         f32x4 vp[2], qs[2];
 #pragma unroll
         for (int vt = 0; vt < 2; vt++) {
-            vp[vt] = mfma16(tuA, frag_tr4(Vsm, LDV, 0, 16 * vt, lane), f32x4{0.f, 0.f, 0.f, 0.f});
-            qs[vt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            vp[vt] = mfma16(tuA, frag_tr4(Vsm, LDV, 0, 16 * vt, lane), zero4());
+            qs[vt] = zero4();
         }
         // ---- -W^T[k][i] = sum_j K[j][k] Tw[i][j]; then V' = U + (-W) S and Q S over the 128 key rows, 32 at a time
 #pragma unroll
         for (int s = 0; s < 4; s++) {
-            const f32x4 w0 = mfma16(frag_tr4(Ksm, LDK, 0, 32 * s, lane), twB, f32x4{0.f, 0.f, 0.f, 0.f});
-            const f32x4 w1 = mfma16(frag_tr4(Ksm, LDK, 0, 32 * s + 16, lane), twB, f32x4{0.f, 0.f, 0.f, 0.f});
+            const f32x4 w0 = mfma16(frag_tr4(Ksm, LDK, 0, 32 * s, lane), twB, zero4());
+            const f32x4 w1 = mfma16(frag_tr4(Ksm, LDK, 0, 32 * s + 16, lane), twB, zero4());
             const bf16x8 wA = join(round4(w0), round4(w1));
             const bf16x8 qA = join(qlo[s], qhi[s]);
 #pragma unroll
@@ -226,7 +180,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void
 #pragma unroll
         for (int vt = 0; vt < 2; vt++) {
             vb[vt] = round4(vp[vt]);
-            const f32x4 o = mfma16(pA, vb[vt], f32x4{0.f, 0.f, 0.f, 0.f});
+            const f32x4 o = mfma16(pA, vb[vt], zero4());
 #pragma unroll
             for (int r = 0; r < 4; r++)
                 Osm[(4 * q4 + r) * LDV + 16 * vt + c] = (__bf16)__builtin_fmaf(p.scale * __expf(Gj[r]), qs[vt][r], o[r]);
@@ -277,6 +231,8 @@ extern "C" int spinf_gdn_fwd(const spinf_gdn_args* a, void* stream) {
     if (((uintptr_t)a->q | (uintptr_t)a->k) % 16) return spinf_fail(SPINF_E_ARG, "gdn: q/k must be 16-byte aligned");
     if ((a->h0 == nullptr) != (a->h0_idx == nullptr) && a->h0 == nullptr) return spinf_fail(SPINF_E_ARG, "gdn: h0_idx without h0");
     if (a->ht_idx != nullptr && a->ht == nullptr) return spinf_fail(SPINF_E_ARG, "gdn: ht_idx without ht");
+    if (a->v_tok % 8 || a->o_tok % 8) return spinf_fail(SPINF_E_ARG, "gdn: v/o row stride must be a multiple of 8 elements");
+    if (((uintptr_t)a->v | (uintptr_t)a->o) % 16) return spinf_fail(SPINF_E_ARG, "gdn: v/o must be 16-byte aligned");
     GdnParams p;
     p.q = (const __bf16*)a->q; p.k = (const __bf16*)a->k; p.v = (const __bf16*)a->v; p.g = a->g; p.beta = (const __bf16*)a->beta;
     p.o = (__bf16*)a->o;
@@ -287,8 +243,6 @@ extern "C" int spinf_gdn_fwd(const spinf_gdn_args* a, void* stream) {
     hipStream_t s = (hipStream_t)stream;
     if (a->mode == 1) return gdn_chunked_launch(p, a->max_len, s);
     if (a->mode != 0) return spinf_fail(SPINF_E_ARG, "gdn: unknown mode %d", a->mode);
-    if (a->v_tok % 8 || a->o_tok % 8) return spinf_fail(SPINF_E_ARG, "gdn: v/o row stride must be a multiple of 8 elements");
-    if (((uintptr_t)a->v | (uintptr_t)a->o) % 16) return spinf_fail(SPINF_E_ARG, "gdn: v/o must be 16-byte aligned");
     const long blocks = a->n_seg * a->hv * (a->dv / 32);
     if (blocks > INT32_MAX) return spinf_fail(SPINF_E_ARG, "gdn: too many segments");
     hipLaunchKernelGGL(gdn_short_kernel, dim3((unsigned)blocks), dim3(64), 0, s, p);

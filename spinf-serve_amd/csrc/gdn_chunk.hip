@@ -1,36 +1,26 @@
-// Gated DeltaNet, chunk-64 WY form, one fused kernel: stands in for gdn.chunked (spinf_serve/models/qwen35/gdn.py:109-133),
+// Gated DeltaNet, chunked WY form, one fused kernel: stands in for gdn.chunked (spinf_serve/models/qwen35/gdn.py:109-133),
 // i.e. for fla's cumsum -> intra-chunk WY solve -> state recurrence (gdn.py:21-106) -> output pipeline, without writing
 // the per-chunk state snapshots or the w / u / v_new intermediates to memory.
 //
-// One workgroup (8 waves) owns one (segment, value head) and walks its 64-token chunks in order.  The state S [K=128, V=128]
-// lives in fp32 MFMA accumulators (a wave owns 32 key rows x 64 value columns) and is mirrored once per chunk as bf16 S^T in LDS,
-// where it serves as an MFMA operand.  Per chunk, with G = cumsum(g), D_ij = exp(G_i - G_j):
-//     A   = -strict_tril(beta_i (K K^T)_ij D_ij)         T = (I - A)^-1        (fp32, blocked forward substitution)
-//     U   = T diag(beta) V          W = T diag(beta e^G) K                     (bf16 MFMA, fp32 accumulate)
+// One workgroup (4 waves) owns one (segment, value head) and walks its 32-token chunks in order; wave w owns value columns
+// 32w .. 32w+31 of the state S [K=128, V=128], which never leaves its fp32 accumulator registers.  The four waves share
+// only the staged K / Q / V rows of the chunk: each wave forms the (small) token x token quantities itself, so between two
+// chunks there are two workgroup barriers (rows consumed, rows staged) and none inside a chunk, and three workgroups fit a
+// compute unit (44 KB of LDS, <= 168 registers) and fill each other's latencies.  Per chunk, G = cumsum(g), D_ij = e^{G_i - G_j}:
+//     A   = -strict_tril(beta_i (K K^T)_ij D_ij)         T = (I - A)^-1      (fp32: two 16 x 16 blocks solved by substitution
+//                                                                             in registers, merged with fp32 MFMAs)
+//     U   = T diag(beta) V          -W = -T diag(beta e^G) K                 (bf16 MFMA, fp32 accumulate)
 //     V'  = U - W S                 O = s e^{G_i} (Q S)_i + tril(s (Q K^T) D) V'
 //     S  <- e^{G_L} S + (K e^{G_L - G})^T V'
-// Every product is computed in the orientation whose result has the token index on the lanes, so results go to LDS or to
-// memory as 8-byte row-major vectors; operands whose contraction index is their row index are read with
-// ds_read_b64_tr_b16.
+// Every product leaves its result in the register layout the next product takes as an operand (see gdn_tiles.h), so only
+// the output rows pass through LDS again (for 16-byte stores).
 #include <hip/hip_runtime.h>
 
 #include "spinf_tree.h"
 #include "common.h"
+#include "gdn_tiles.h"
 
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
-typedef __attribute__((ext_vector_type(16))) float f32x16;
-typedef __attribute__((ext_vector_type(4))) float f32x4;
-typedef __attribute__((ext_vector_type(4))) short s16x4;
-typedef __attribute__((ext_vector_type(8))) short s16x8;
-
-struct GdnParams {
-    const __bf16* q; const __bf16* k; const __bf16* v; const float* g; const __bf16* beta; __bf16* o;
-    long q_tok, v_tok, g_tok, o_tok;
-    int h, hv, dk, dv; float scale;
-    const long* cu; const long* idx; long n_seg;
-    const float* h0; const long* h0_idx; float* ht; const long* ht_idx;
-};
+using namespace gdn_tiles;
 
 #ifdef SPINF_TRACE
 __device__ long g_gdn_trace[16];
@@ -44,129 +34,72 @@ extern "C" int spinf_debug_gdn_trace(long* out) { return (int)hipMemcpyFromSymbo
 
 namespace {
 
-constexpr int C = 64;          // chunk
+constexpr int CH = 32;         // chunk
 constexpr int KD = 128;        // key head dim
 constexpr int VD = 128;        // value head dim
-constexpr int LD = 136;        // row stride (elements) of the [*, 128] bf16 tiles: 272 B, b128 row reads hit 16 distinct bank groups
-constexpr int LT = 72;         // row stride of the [64, 64] bf16 tiles
-constexpr int LA = 68;         // row stride (floats) of the fp32 [64, 64] matrix
-
-// LDS map (bytes)
-constexpr int OFF_K = 0;                         // K   [64][LD] bf16
-constexpr int OFF_Q = OFF_K + C * LD * 2;        // Q   [64][LD]
-constexpr int OFF_V = OFF_Q + C * LD * 2;        // V, later V' [64][LD]
-constexpr int OFF_A = OFF_V + C * LD * 2;        // A / T fp32 [64][LA]; later V' e^{G_L - G} bf16 [64][LD] (same size)
-constexpr int OFF_TU = OFF_A + C * LD * 2;       // T diag(beta)            bf16 [64][LT]
-constexpr int OFF_TW = OFF_TU + C * LT * 2;      // -T diag(beta e^G)       bf16 [64][LT]
-constexpr int OFF_P = OFF_TW + C * LT * 2;       // tril(s Q K^T D)         bf16 [64][LT]
-constexpr int OFF_W = OFF_P + C * LT * 2;        // -W  [64][LD] bf16
-constexpr int OFF_ST = OFF_W + C * LD * 2;       // S^T [128][LD] bf16
-constexpr int OFF_G = OFF_ST + VD * LD * 2;      // G [64] fp32, beta [64] fp32, idx rows [64] int64
-constexpr int OFF_X = OFF_G + 64 * 4 * 2 + 64 * 8;   // scratch fp32 [32][36] for the block merges
-constexpr int LDS_BYTES = OFF_X + 32 * 36 * 4;
-static_assert(C * LA * 4 <= C * LD * 2, "fp32 A must fit the region it shares");
-static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
-
-__device__ __forceinline__ f32x16 zero16() {
-    f32x16 z;
-#pragma unroll
-    for (int i = 0; i < 16; i++) z[i] = 0.f;
-    return z;
-}
-// rows row0 + lane%32, contraction elements k0 + 8 (lane/32) .. +7, from a tile whose contraction index is contiguous
-__device__ __forceinline__ bf16x8 frag_nt(const __bf16* base, int stride, int row0, int k0, int lane) {
-    return *(const bf16x8*)(base + (row0 + (lane & 31)) * stride + k0 + 8 * (lane >> 5));
-}
-// column n0 + lane%32, contraction rows k0 + 8 (lane/32) .. +7, from a tile whose contraction index is its ROW index
-__device__ __forceinline__ bf16x8 frag_tr(const __bf16* base, int stride, int k0, int n0, int lane) {
-    const int tr_a = lane & 3, tr_j = (lane >> 2) & 3, tr_mb = (lane >> 4) & 1, g = lane >> 5;
-    const __bf16* p = base + (k0 + 8 * g + tr_j) * stride + n0 + 16 * tr_mb + 4 * tr_a;
-    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p);
-    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(p + 4 * stride));
-    return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-}
-// Workgroup barrier for LDS traffic only: waits for this wave's LDS operations, not for its global loads.  __syncthreads()
-// carries a memory fence in front of which the compiler drains every load in flight, the next chunk's prefetch included.
-__device__ __forceinline__ void lds_barrier() {
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0)
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-}
-__device__ __forceinline__ f32x16 mfma(bf16x8 a, bf16x8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+constexpr int LD = 136;        // row stride (elements) of the [32, 128] bf16 tiles
+constexpr int LA = 36;         // row stride (floats) of the fp32 [32, 32] matrix A
+constexpr int LX = 20;         // row stride (floats) of the 16 x 16 merge scratch
+constexpr int LO = 40;         // row stride (elements) of a wave's [32, 32] output tile
 
 }  // namespace
 
-__global__ __launch_bounds__(512) void gdn_chunk_kernel(const GdnParams p) {
-    extern __shared__ __attribute__((aligned(16))) char smem[];
-    __bf16* Ks = (__bf16*)(smem + OFF_K);
-    __bf16* Qs = (__bf16*)(smem + OFF_Q);
-    __bf16* Vs = (__bf16*)(smem + OFF_V);
-    float* As = (float*)(smem + OFF_A);
-    __bf16* Vd = (__bf16*)(smem + OFF_A);
-    __bf16* Tu = (__bf16*)(smem + OFF_TU);
-    __bf16* Tw = (__bf16*)(smem + OFF_TW);
-    __bf16* Pm = (__bf16*)(smem + OFF_P);
-    __bf16* Wn = (__bf16*)(smem + OFF_W);
-    __bf16* St = (__bf16*)(smem + OFF_ST);
-    float* Gs = (float*)(smem + OFF_G);
-    float* Bs = Gs + 64;
-    long* Rs = (long*)(Bs + 64);
-    float* Xs = (float*)(smem + OFF_X);
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gdn_chunk_kernel(const GdnParams p) {
+    __shared__ __attribute__((aligned(16))) __bf16 Ks[CH * LD];
+    __shared__ __attribute__((aligned(16))) __bf16 Qs[CH * LD];
+    __shared__ __attribute__((aligned(16))) __bf16 Vs[CH * LD];
+    // A, the upper-left block of T and the merge intermediate are written by all four waves with identical values (each
+    // wave reads back what it wrote itself or the same number from another wave)
+    __shared__ __attribute__((aligned(16))) float As[CH * LA];
+    __shared__ __attribute__((aligned(16))) float Ts[32 * LX];     // T_00 (rows 0..15) and T_11 (rows 16..31)
+    __shared__ __attribute__((aligned(16))) float Xs[16 * LX];
+    __shared__ __attribute__((aligned(16))) __bf16 Os[4 * CH * LO];
+    __shared__ __attribute__((aligned(16))) float Gs[CH];
+    __shared__ __attribute__((aligned(16))) float Bs[CH];
+    __shared__ long Rs[CH];
 
-    // Eight waves, two per SIMD: every phase below is a short dependent chain (LDS reads -> MFMAs -> conversions -> LDS
-    // writes -> barrier), and a second wave on the SIMD is what fills the gaps of the first.  Wave w = (wq, wh): quarter
-    // wq = w % 4 of whatever a phase splits four ways (32 of 128 rows, a 32x32 tile of a 64x64 matrix), half wh = w / 4.
-    const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6), wq = w & 3, wh = w >> 2, n32 = lane & 31, g = lane >> 5;
+    const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6), c = lane & 15, q4 = lane >> 4;
     const long seg = blockIdx.x / p.hv;
     const int hv = (int)(blockIdx.x % p.hv);
     const int hk = hv / (p.hv / p.h);
     const long bos = p.cu[seg], eos = p.cu[seg + 1];
     const int T = (int)(eos - bos);
+    __bf16* Ow = Os + w * CH * LO;
 
-    // ---- state: S[k][v]; wave (wq, wh) owns k rows 32wq..32wq+31 of v columns 64wh..64wh+63 as two 32x32 tiles (tile j:
-    // v columns 64wh + 32j ..); lane = v column, reg r = k row
-    f32x16 S[2];
+    // ---- state: S[kt][vt][r] = S[16 kt + 4 q4 + r][32 w + 16 vt + c]
+    f32x4 S[8][2];
 #pragma unroll
-    for (int j = 0; j < 2; j++) S[j] = zero16();
-    long src = -1;
-    if (p.h0 != nullptr && p.h0_idx != nullptr) src = p.h0_idx[seg];
-    if (src >= 0) {
-        const float* hp = p.h0 + (src * p.hv + hv) * (long)KD * VD;
+    for (int kt = 0; kt < 8; kt++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+        for (int vt = 0; vt < 2; vt++) S[kt][vt] = zero4();
+    if (p.h0 != nullptr && p.h0_idx != nullptr) {
+        const long src = p.h0_idx[seg];
+        if (src >= 0) {
+            const float* hp = p.h0 + ((src * p.hv + hv) * KD + 4 * q4) * VD + 32 * w + c;
 #pragma unroll
-            for (int r = 0; r < 16; r++) S[j][r] = hp[(long)(32 * wq + 8 * (r >> 2) + 4 * g + (r & 3)) * VD + 64 * wh + 32 * j + n32];
+            for (int kt = 0; kt < 8; kt++)
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+#pragma unroll
+                    for (int vt = 0; vt < 2; vt++) S[kt][vt][r] = hp[(long)(16 * kt + r) * VD + 16 * vt];
+        }
     }
-    // S^T mirror (bf16): St[v][k]
-    auto mirror = [&]() __attribute__((always_inline)) {
-#pragma unroll
-        for (int j = 0; j < 2; j++)
-#pragma unroll
-            for (int r4 = 0; r4 < 4; r4++) {
-                bf16x4 t;
-#pragma unroll
-                for (int jj = 0; jj < 4; jj++) t[jj] = (__bf16)S[j][4 * r4 + jj];
-                *(bf16x4*)(St + (64 * wh + 32 * j + n32) * LD + 32 * wq + 8 * r4 + 4 * g) = t;
-            }
-    };
-    mirror();
+    const bool keep = p.ht != nullptr && p.ht_idx != nullptr && p.ht_idx[seg] >= 0;
 
-    // The next chunk's rows are fetched into registers while the current chunk is computed (global latency would otherwise
-    // be exposed in front of every chunk: a workgroup walks its chunks strictly in order), and the stream rows of the chunk
-    // after that (idx) one chunk earlier still, so that no load ever waits for the load of its own address.
-    // Thread -> 16-byte piece tid%16 of chunk rows tid/16 and tid/16 + 32 (one load instruction of a wave covers four whole
-    // rows); threads 0..63 also -> g, beta and the stream row of chunk row tid.
+    // The next chunk's rows are fetched into registers while the current chunk is computed, and the stream rows (idx) of
+    // the chunk after that one chunk earlier still, so that no load ever waits for the load of its own address.
+    // Thread -> 16-byte piece tid%16 of chunk rows tid/16 and tid/16 + 16 (one load instruction of a wave covers four whole
+    // rows); threads 0..31 also -> g, beta and the stream row of chunk row tid.
     bf16x8 pk[2], pq[2], pv[2];
     long pr64 = -1;
     float pg = 0.f;
     __bf16 pbeta = (__bf16)0.f;   // (kept as loaded: converting here would make the wave wait for the load at once)
-    long ra[2] = {-1, -1}, rb = -1;     // stream rows (the thread's two K/Q/V rows; chunk row tid) of the chunk fetched next
+    long ra[2] = {-1, -1}, rb = -1;
     auto fetch_rows = [&](const int c0) __attribute__((always_inline)) {
-        const int L = min(C, T - c0);      // <= 0: there is no such chunk
+        const int L = min(CH, T - c0);      // <= 0: there is no such chunk
 #pragma unroll
         for (int cc = 0; cc < 2; cc++) {
-            const int row = (tid >> 4) + 32 * cc;
+            const int row = (tid >> 4) + 16 * cc;
             ra[cc] = -1;
             if (row < L) {
                 const long t = bos + c0 + row;
@@ -174,7 +107,7 @@ __global__ __launch_bounds__(512) void gdn_chunk_kernel(const GdnParams p) {
             }
         }
         rb = -1;
-        if (tid < 64 && tid < L) {
+        if (tid < CH && tid < L) {
             const long t = bos + c0 + tid;
             rb = p.idx ? p.idx[t] : t;
         }
@@ -201,22 +134,16 @@ __global__ __launch_bounds__(512) void gdn_chunk_kernel(const GdnParams p) {
     };
     fetch_rows(0);
     fetch_data();
-    fetch_rows(C);
+    fetch_rows(CH);
 
-    for (int c0 = 0; c0 < T; c0 += C) {
-        const int L = min(C, T - c0);
+    for (int c0 = 0; c0 < T; c0 += CH) {
+        const int L = min(CH, T - c0);
         GT_CLK(g0);
-        lds_barrier();   // previous chunk fully consumed (and St written)
-        // ---- stage the chunk from the prefetch registers: rows, cumulative g, beta, then K / Q / V tiles (rows >= L are zero)
-        if (tid < 64) {
-            // inclusive prefix sum of g over the wave: within rows of 16 lanes by shifts, then across rows by broadcasts
-            float x = pg;
-            x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x111, 0xf, 0xf, true));   // row_shr:1
-            x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x112, 0xf, 0xf, true));   // row_shr:2
-            x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x114, 0xf, 0xf, true));   // row_shr:4
-            x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x118, 0xf, 0xf, true));   // row_shr:8
-            x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x142, 0xa, 0xf, false));  // row_bcast:15 -> rows 1, 3
-            x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x143, 0xc, 0xf, false));  // row_bcast:31 -> rows 2, 3
+        lds_barrier();   // every wave is done with the previous chunk's rows
+        // ---- stage the chunk from the prefetch registers (rows >= L are zero): cumulative g, beta, stream rows, K / Q / V
+        if (tid < CH) {
+            float x = row_prefix_sum(pg);
+            x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x142, 0xa, 0xf, false));  // row_bcast:15 -> lanes 16..31
             Gs[tid] = x;
             Bs[tid] = (float)pbeta;
             Rs[tid] = pr64;
@@ -225,272 +152,224 @@ __global__ __launch_bounds__(512) void gdn_chunk_kernel(const GdnParams p) {
             const int col = (tid & 15) * 8;
 #pragma unroll
             for (int cc = 0; cc < 2; cc++) {
-                const int row = (tid >> 4) + 32 * cc;
+                const int row = (tid >> 4) + 16 * cc;
                 *(bf16x8*)(Ks + row * LD + col) = pk[cc];
                 *(bf16x8*)(Qs + row * LD + col) = pq[cc];
                 *(bf16x8*)(Vs + row * LD + col) = pv[cc];
             }
         }
-        fetch_data();          // chunk c0 + C, whose rows are known since the previous chunk
-        fetch_rows(c0 + 2 * C);
         lds_barrier();
-        const float GL = Gs[63];
         GT_CLK(g1);
 
-        // ---- (a) A = -strict_tril(beta_i K_i.K_j D_ij) fp32 (waves with wh = 0), (b) P = tril(s Q_i.K_j D_ij) bf16 (wh = 1);
-        // computed transposed so that a lane holds row i and 4 consecutive columns j per register group.  Tile (jt, it) = wq.
-        {
-            const int jt = wq >> 1, it = wq & 1;
-            const __bf16* rhs = wh ? Qs : Ks;
-            f32x16 acc = zero16();
+        // Token tiles: tile 0 = chunk rows 0..15, tile 1 = rows 16..31.  Index [it] = tile of the row i = 16 it + c this lane
+        // owns in a transposed result, [jt] = tile of the columns j = 16 jt + 4 q4 + r its registers hold.
+        const float GL = Gs[CH - 1];
+        float Gi[2], bi[2];
+        f32x4 Gj[2], Bj[2];
 #pragma unroll
-            for (int s = 0; s < KD / 16; s++) acc = mfma(frag_nt(Ks, LD, 32 * jt, 16 * s, lane), frag_nt(rhs, LD, 32 * it, 16 * s, lane), acc);
-            const int i = 32 * it + n32;
-            const float Gi = Gs[i], bi = Bs[i];
-#pragma unroll
-            for (int r4 = 0; r4 < 4; r4++) {
-                const int j0 = 32 * jt + 8 * r4 + 4 * g;
-                bf16x4 pv4;
-                float avv[4];
-#pragma unroll
-                for (int jj = 0; jj < 4; jj++) {
-                    const int j = j0 + jj;
-                    const float d = __expf(Gi - Gs[j]);
-                    avv[jj] = j < i ? -bi * acc[4 * r4 + jj] * d : 0.f;
-                    pv4[jj] = (__bf16)(j <= i ? p.scale * acc[4 * r4 + jj] * d : 0.f);
-                }
-                if (wh == 0) *(float4*)(As + i * LA + j0) = make_float4(avv[0], avv[1], avv[2], avv[3]);
-                else *(bf16x4*)(Pm + i * LT + j0) = pv4;
-            }
+        for (int t = 0; t < 2; t++) {
+            Gi[t] = Gs[16 * t + c];
+            bi[t] = Bs[16 * t + c];
+            Gj[t] = *(const f32x4*)(Gs + 16 * t + 4 * q4);
+            Bj[t] = *(const f32x4*)(Bs + 16 * t + 4 * q4);
         }
-        lds_barrier();
+        // ---- (K K^T)^T and (Q K^T)^T, tiles (jt, it) = (0,0), (0,1), (1,1); (1,0) lies above the diagonal
+        f32x4 kk[3], qk[3];
+#pragma unroll
+        for (int x = 0; x < 3; x++) { kk[x] = zero4(); qk[x] = zero4(); }
+#pragma unroll
+        for (int s = 0; s < KD / 32; s++) {
+            const bf16x8 k0 = *(const bf16x8*)(Ks + c * LD + 32 * s + 8 * q4);
+            const bf16x8 k1 = *(const bf16x8*)(Ks + (16 + c) * LD + 32 * s + 8 * q4);
+            const bf16x8 q0 = *(const bf16x8*)(Qs + c * LD + 32 * s + 8 * q4);
+            const bf16x8 q1 = *(const bf16x8*)(Qs + (16 + c) * LD + 32 * s + 8 * q4);
+            kk[0] = mfma32(k0, k0, kk[0]);
+            kk[1] = mfma32(k0, k1, kk[1]);
+            kk[2] = mfma32(k1, k1, kk[2]);
+            qk[0] = mfma32(k0, q0, qk[0]);
+            qk[1] = mfma32(k0, q1, qk[1]);
+            qk[2] = mfma32(k1, q1, qk[2]);
+        }
+        // A[i][j] (fp32, to LDS) and P[i][j] = s Q_i.K_j e^{G_i - G_j}, j <= i (kept as the A operand of O = P V')
+        bf16x8 pA[2];
+        {
+            bf16x4 pT[3];
+#pragma unroll
+            for (int x = 0; x < 3; x++) {
+                const int jt = x >> 1, it = (x + 1) >> 1;     // (0,0), (0,1), (1,1)
+                const int i = 16 * it + c;
+                f32x4 a4;
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int j = 16 * jt + 4 * q4 + r;
+                    const float d = __expf(Gi[it] - Gj[jt][r]);
+                    a4[r] = j < i ? -bi[it] * kk[x][r] * d : 0.f;
+                    pT[x][r] = (__bf16)(j <= i ? p.scale * qk[x][r] * d : 0.f);
+                }
+                *(f32x4*)(As + i * LA + 16 * jt + 4 * q4) = a4;
+            }
+            bf16x4 z;
+#pragma unroll
+            for (int r = 0; r < 4; r++) z[r] = (__bf16)0.f;
+            pA[0] = join(pT[0], z);
+            pA[1] = join(pT[1], pT[2]);
+        }
+        wave_lds_order();
         GT_CLK(g2);
 
-        // ---- T = (I - A)^-1 in place (fp32).  Stage 1: the four 16x16 diagonal blocks by forward substitution, wave b < 4 =
-        // block b, lane c < 16 = column c of the block.
-        if (w < 4 && lane < 16) {
+        // ---- T = (I - A)^-1: rows c of the two diagonal blocks in registers, then the lower-left block
+        // T_lo = T_11 A_lo T_00, computed transposed (T_lo^T = T_00^T (A_lo^T T_11^T)) so that the lane again holds row 16 + c.
+        f32x4 t00, t11, tlo;
+        {
+            const float* T1s = Ts + 16 * LX;
+            // the rows pass through LDS to reach the lanes in operand order (row c, columns 4 q4 ..+3; single elements for the
+            // fp32 products); all four groups of 16 lanes write the same values
+            // lane groups 0 and 2 solve the upper-left block, groups 1 and 3 the lower-right one, in the same instructions
             float t[16];
-            const float* Ab = As + (16 * w) * LA + 16 * w;
+            const int blk = q4 & 1;
+            unit_lower_inverse_row(As + blk * (16 * LA + 16), LA, c, t);
 #pragma unroll
-            for (int i = 0; i < 16; i++) {
-                float acc = (i == lane) ? 1.f : 0.f;
+            for (int j4 = 0; j4 < 4; j4++) *(f32x4*)(Ts + (16 * blk + c) * LX + 4 * j4) = f32x4{t[4 * j4], t[4 * j4 + 1], t[4 * j4 + 2], t[4 * j4 + 3]};
+            wave_lds_order();
+            t00 = *(const f32x4*)(Ts + c * LX + 4 * q4);
+            t11 = *(const f32x4*)(T1s + c * LX + 4 * q4);
+            f32x4 x = zero4();
 #pragma unroll
-                for (int j = 0; j < i; j++) acc = __builtin_fmaf(Ab[i * LA + j], t[j], acc);
-                t[i] = acc;
-            }
-            __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): all reads of A done before the block is overwritten
+            for (int s4 = 0; s4 < 4; s4++)        // X[j][i] = sum_m A_lo[m][j] T_11[i][m]
+                x = mfma4(As[(16 + 4 * s4 + q4) * LA + c], T1s[c * LX + 4 * s4 + q4], x);
 #pragma unroll
-            for (int i = 0; i < 16; i++) As[(16 * w + i) * LA + 16 * w + lane] = t[i];
+            for (int r = 0; r < 4; r++) Xs[(4 * q4 + r) * LX + c] = x[r];
+            wave_lds_order();
+            tlo = zero4();
+#pragma unroll
+            for (int s4 = 0; s4 < 4; s4++)        // T_lo[16 + i][j'] = sum_j T_00[j][j'] X[j][i]
+                tlo = mfma4(Ts[(4 * s4 + q4) * LX + c], Xs[(4 * s4 + q4) * LX + c], tlo);
         }
-        lds_barrier();
-        // Stages 2 and 3 are products of 16x16 / 32x32 fp32 blocks, done with v_mfma_f32_16x16x4_f32 (operands: lane l gives
-        // A[l%16][l/16] and B[l/16][l%16] of a 16x4 by 4x16 step; result: lane l holds rows 4(l/16)..+3 of column l%16).
-        // Stage 2: 32x32 diagonal blocks: T_lo = T_bb A_lo T_aa for (a, b) = (0,1) and (2,3); wave q < 2 does block q.
+        // T diag(beta) and -T diag(beta e^G): row 16 it + c, columns in the order of the contraction slots
+        bf16x8 tu[2], tw[2];
         {
-            const int c16 = lane & 15, g4 = lane >> 4;
-            if (w < 2) {
-                const int rA = 32 * w, rB = rA + 16;
-                f32x4 x = {0.f, 0.f, 0.f, 0.f};
+            bf16x4 u00, w00, u10, w10, u11, w11, z;
 #pragma unroll
-                for (int s4 = 0; s4 < 4; s4++)        // X = A_lo T_aa
-                    x = __builtin_amdgcn_mfma_f32_16x16x4f32(As[(rB + c16) * LA + rA + 4 * s4 + g4], As[(rA + 4 * s4 + g4) * LA + rA + c16], x, 0, 0, 0);
-#pragma unroll
-                for (int i = 0; i < 4; i++) Xs[(16 * w + 4 * g4 + i) * 36 + c16] = x[i];
-                __builtin_amdgcn_s_waitcnt(0xc07f);   // this wave's own X is in LDS (nobody else reads it)
-                f32x4 y = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int s4 = 0; s4 < 4; s4++)        // T_lo = T_bb X
-                    y = __builtin_amdgcn_mfma_f32_16x16x4f32(As[(rB + c16) * LA + rB + 4 * s4 + g4], Xs[(16 * w + 4 * s4 + g4) * 36 + c16], y, 0, 0, 0);
-#pragma unroll
-                for (int i = 0; i < 4; i++) As[(rB + 4 * g4 + i) * LA + rA + c16] = y[i];
+            for (int r = 0; r < 4; r++) {
+                const float e0 = Bj[0][r] * __expf(Gj[0][r]), e1 = Bj[1][r] * __expf(Gj[1][r]);
+                u00[r] = (__bf16)(t00[r] * Bj[0][r]);
+                w00[r] = (__bf16)(-t00[r] * e0);
+                u10[r] = (__bf16)(tlo[r] * Bj[0][r]);
+                w10[r] = (__bf16)(-tlo[r] * e0);
+                u11[r] = (__bf16)(t11[r] * Bj[1][r]);
+                w11[r] = (__bf16)(-t11[r] * e1);
+                z[r] = (__bf16)0.f;
             }
+            tu[0] = join(u00, z);
+            tw[0] = join(w00, z);
+            tu[1] = join(u10, u11);
+            tw[1] = join(w10, w11);
         }
-        lds_barrier();
-        // Stage 3: the 64x64 matrix: T_lo = T_11 A_lo T_00 with 32x32 blocks; wave w < 4 does the 16x16 tile (w>>1, w&1) of both products
-        {
-            const int c16 = lane & 15, g4 = lane >> 4;
-            const int ti = 16 * ((w >> 1) & 1), tj = 16 * (w & 1);
-            f32x4 y = {0.f, 0.f, 0.f, 0.f};
-            if (w < 4) {
-                f32x4 x = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int s4 = 0; s4 < 8; s4++)            // X = A_lo T_00
-                    x = __builtin_amdgcn_mfma_f32_16x16x4f32(As[(32 + ti + c16) * LA + 4 * s4 + g4], As[(4 * s4 + g4) * LA + tj + c16], x, 0, 0, 0);
-#pragma unroll
-                for (int i = 0; i < 4; i++) Xs[(ti + 4 * g4 + i) * 36 + tj + c16] = x[i];
-            }
-            lds_barrier();
-            if (w < 4) {
-#pragma unroll
-                for (int s4 = 0; s4 < 8; s4++)            // T_lo = T_11 X
-                    y = __builtin_amdgcn_mfma_f32_16x16x4f32(As[(32 + ti + c16) * LA + 32 + 4 * s4 + g4], Xs[(4 * s4 + g4) * 36 + tj + c16], y, 0, 0, 0);
-            }
-            lds_barrier();   // every read of the A_lo block is done
-            if (w < 4) {
-#pragma unroll
-                for (int i = 0; i < 4; i++) As[(32 + ti + 4 * g4 + i) * LA + tj + c16] = y[i];
-            }
-        }
-        lds_barrier();
         GT_CLK(g3);
-        // ---- Tu = T diag(beta), Tw = -T diag(beta e^G) (bf16).  thread: row tid/8, 8 columns
-        {
-            const int i = tid >> 3, jb = (tid & 7) * 8;
+
+        // ---- U[i][v] = sum_j Tu[i][j] V[j][v]   (lane = column v, registers = rows i)
+        f32x4 vp[2][2], qs[2][2];
 #pragma unroll
-            for (int j4 = 0; j4 < 2; j4++) {
-                const float4 t = *(const float4*)(As + i * LA + jb + 4 * j4);
-                const float tv[4] = {t.x, t.y, t.z, t.w};
-                bf16x4 u, ww;
+        for (int vt = 0; vt < 2; vt++) {
+            const bf16x8 vB = join(frag_tr4(Vs, LD, 0, 32 * w + 16 * vt, lane), frag_tr4(Vs, LD, 16, 32 * w + 16 * vt, lane));
 #pragma unroll
-                for (int jj = 0; jj < 4; jj++) {
-                    const int j = jb + 4 * j4 + jj;
-                    const float tb = tv[jj] * Bs[j];
-                    u[jj] = (__bf16)tb;
-                    ww[jj] = (__bf16)(-tb * __expf(Gs[j]));
-                }
-                *(bf16x4*)(Tu + i * LT + jb + 4 * j4) = u;
-                *(bf16x4*)(Tw + i * LT + jb + 4 * j4) = ww;
+            for (int it = 0; it < 2; it++) {
+                vp[it][vt] = mfma32(tu[it], vB, zero4());
+                qs[it][vt] = zero4();
             }
         }
-        lds_barrier();
+        // ---- -W^T[k][i] = sum_j K[j][k] Tw[i][j]; then V' = U + (-W) S and Q S over the 128 key rows, 32 at a time
+#pragma unroll
+        for (int s = 0; s < KD / 32; s++) {
+            const bf16x8 kT0 = join(frag_tr4(Ks, LD, 0, 32 * s, lane), frag_tr4(Ks, LD, 16, 32 * s, lane));
+            const bf16x8 kT1 = join(frag_tr4(Ks, LD, 0, 32 * s + 16, lane), frag_tr4(Ks, LD, 16, 32 * s + 16, lane));
+            bf16x8 wA[2], qA[2];
+#pragma unroll
+            for (int it = 0; it < 2; it++) {
+                wA[it] = join(round4(mfma32(kT0, tw[it], zero4())), round4(mfma32(kT1, tw[it], zero4())));
+                const __bf16* qp = Qs + (16 * it + c) * LD + 32 * s + 4 * q4;
+                qA[it] = join(*(const bf16x4*)qp, *(const bf16x4*)(qp + 16));
+            }
+#pragma unroll
+            for (int vt = 0; vt < 2; vt++) {
+                const bf16x8 sb = join(round4(S[2 * s][vt]), round4(S[2 * s + 1][vt]));
+#pragma unroll
+                for (int it = 0; it < 2; it++) {
+                    vp[it][vt] = mfma32(wA[it], sb, vp[it][vt]);
+                    qs[it][vt] = mfma32(qA[it], sb, qs[it][vt]);
+                }
+            }
+        }
         GT_CLK(g4);
-
-        // ---- (c) U^T[v][i] = sum_j V[j][v] Tu[i][j] (waves wh = 0, kept in registers) and -W^T[d][i] = sum_j K[j][d] Tw[i][j]
-        // (waves wh = 1, written to LDS); wave: rows 32wq.. of v / d, both token tiles
-        f32x16 acc[2];      // wh = 0: U^T, later V'^T; wh = 1: -W^T, later (Q S)^T.  Tile it = token columns 32 it..
-        acc[0] = zero16();
-        acc[1] = zero16();
-        {
-            const __bf16* lhs = wh ? Ks : Vs;
-            const __bf16* rhs = wh ? Tw : Tu;
+        // the next chunk's rows are requested here, where few registers are live; they arrive during the state update
+        fetch_data();          // chunk c0 + CH, whose rows are known since the previous chunk
+        fetch_rows(c0 + 2 * CH);
+        // ---- O[i][v] = s e^{G_i} (Q S)[i][v] + sum_j P[i][j] V'[j][v], rows i = 16 it + 4 q4 + r; through LDS for 16-byte stores
+        bf16x8 vb[2];
 #pragma unroll
-            for (int s = 0; s < C / 16; s++) {
-                const bf16x8 a = frag_tr(lhs, LD, 16 * s, 32 * wq, lane);
+        for (int vt = 0; vt < 2; vt++) {
+            vb[vt] = join(round4(vp[0][vt]), round4(vp[1][vt]));
 #pragma unroll
-                for (int it = 0; it < 2; it++) acc[it] = mfma(a, frag_nt(rhs, LT, 32 * it, 16 * s, lane), acc[it]);
-            }
-            if (wh) {
+            for (int it = 0; it < 2; it++) {
+                const f32x4 o = mfma32(pA[it], vb[vt], zero4());
 #pragma unroll
-                for (int it = 0; it < 2; it++)
-#pragma unroll
-                    for (int r4 = 0; r4 < 4; r4++) {
-                        bf16x4 t;
-#pragma unroll
-                        for (int j = 0; j < 4; j++) t[j] = (__bf16)acc[it][4 * r4 + j];
-                        *(bf16x4*)(Wn + (32 * it + n32) * LD + 32 * wq + 8 * r4 + 4 * g) = t;
-                    }
-                acc[0] = zero16();
-                acc[1] = zero16();
+                for (int r = 0; r < 4; r++)
+                    Ow[(16 * it + 4 * q4 + r) * LO + 16 * vt + c] = (__bf16)__builtin_fmaf(p.scale * __expf(Gj[it][r]), qs[it][vt][r], o[r]);
             }
         }
-        lds_barrier();   // -W visible; V (Vs) and T (As) are dead from here
+        wave_lds_order();
+#pragma unroll
+        for (int cc = 0; cc < 2; cc++) {
+            const int row = (lane >> 2) + 16 * cc;
+            if (row < L) *(bf16x8*)(p.o + Rs[row] * p.o_tok + (long)hv * VD + 32 * w + (lane & 3) * 8) = *(const bf16x8*)(Ow + row * LO + (lane & 3) * 8);
+        }
         GT_CLK(g5);
-
-        // ---- (d) wh = 0: V'^T = U^T + S^T (-W)^T;  (e1) wh = 1: QS^T[v][i] = sum_k S^T[v][k] Q[i][k]
-        {
-            const __bf16* rhs = wh ? Qs : Wn;
-#pragma unroll
-            for (int s = 0; s < KD / 16; s++) {
-                const bf16x8 a = frag_nt(St, LD, 32 * wq, 16 * s, lane);
-#pragma unroll
-                for (int it = 0; it < 2; it++) acc[it] = mfma(a, frag_nt(rhs, LD, 32 * it, 16 * s, lane), acc[it]);
-            }
-        }
-        // V' and V' e^{G_L - G_i}, row-major [i][v], bf16
-        if (wh == 0) {
-#pragma unroll
-            for (int it = 0; it < 2; it++) {
-                const int i = 32 * it + n32;
-                const float dec = __expf(GL - Gs[i]);
-#pragma unroll
-                for (int r4 = 0; r4 < 4; r4++) {
-                    bf16x4 t, td;
-#pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        t[j] = (__bf16)acc[it][4 * r4 + j];
-                        td[j] = (__bf16)(acc[it][4 * r4 + j] * dec);
-                    }
-                    *(bf16x4*)(Vs + i * LD + 32 * wq + 8 * r4 + 4 * g) = t;
-                    *(bf16x4*)(Vd + i * LD + 32 * wq + 8 * r4 + 4 * g) = td;
-                }
-            }
-        }
-        lds_barrier();
-        GT_CLK(g6);
-
-        // ---- (e2) wh = 1: O^T[v][i] = s e^{G_i} QS^T + sum_j V'[j][v] P[i][j]
-        if (wh) {
-            f32x16 ov[2];
-            ov[0] = zero16(); ov[1] = zero16();
-#pragma unroll
-            for (int s = 0; s < C / 16; s++) {
-                const bf16x8 a = frag_tr(Vs, LD, 16 * s, 32 * wq, lane);
-#pragma unroll
-                for (int it = 0; it < 2; it++) ov[it] = mfma(a, frag_nt(Pm, LT, 32 * it, 16 * s, lane), ov[it]);
-            }
-#pragma unroll
-            for (int it = 0; it < 2; it++) {
-                const int i = 32 * it + n32;
-                if (i < L) {
-                    const float sc = p.scale * __expf(Gs[i]);
-                    __bf16* op = p.o + Rs[i] * p.o_tok + (long)hv * VD + 32 * wq + 4 * g;
-#pragma unroll
-                    for (int r4 = 0; r4 < 4; r4++) {
-                        bf16x4 t;
-#pragma unroll
-                        for (int j = 0; j < 4; j++) t[j] = (__bf16)(__builtin_fmaf(sc, acc[it][4 * r4 + j], ov[it][4 * r4 + j]));
-                        *(bf16x4*)(op + 8 * r4) = t;
-                    }
-                }
-            }
-        }
-        GT_CLK(g7);
-
-        // ---- (f) S[k][v] = e^{G_L} S[k][v] + sum_j K[j][k] (V' e^{G_L - G_j})[j][v]; wave: k rows 32wq.., v tiles 2wh, 2wh + 1
-        {
+        // ---- S[k][v] = e^{G_L} S[k][v] + sum_j K[j][k] (V' e^{G_L - G_j})[j][v]; skipped when nothing reads the state again
+        if (c0 + CH < T || keep) {
             const float eg = __expf(GL);
+            bf16x8 vd[2];
 #pragma unroll
-            for (int j = 0; j < 2; j++)
+            for (int vt = 0; vt < 2; vt++) {
+                bf16x4 d0, d1;
 #pragma unroll
-                for (int r = 0; r < 16; r++) S[j][r] *= eg;
+                for (int r = 0; r < 4; r++) {
+                    d0[r] = (__bf16)(vp[0][vt][r] * __expf(GL - Gj[0][r]));
+                    d1[r] = (__bf16)(vp[1][vt][r] * __expf(GL - Gj[1][r]));
+                }
+                vd[vt] = join(d0, d1);
+            }
 #pragma unroll
-            for (int s = 0; s < C / 16; s++) {
-                const bf16x8 a = frag_tr(Ks, LD, 16 * s, 32 * wq, lane);
+            for (int kt = 0; kt < 8; kt++) {
+                const bf16x8 kT = join(frag_tr4(Ks, LD, 0, 16 * kt, lane), frag_tr4(Ks, LD, 16, 16 * kt, lane));
 #pragma unroll
-                for (int j = 0; j < 2; j++) S[j] = mfma(a, frag_tr(Vd, LD, 16 * s, 64 * wh + 32 * j, lane), S[j]);
+                for (int vt = 0; vt < 2; vt++) {
+#pragma unroll
+                    for (int r = 0; r < 4; r++) S[kt][vt][r] *= eg;
+                    S[kt][vt] = mfma32(kT, vd[vt], S[kt][vt]);
+                }
             }
         }
-        lds_barrier();   // every wave is done reading S^T (d, e1) before it is replaced
-        mirror();
-        GT_CLK(g8);
-        GT_ADD(0, g1 - g0); GT_ADD(1, g2 - g1); GT_ADD(2, g3 - g2); GT_ADD(3, g4 - g3); GT_ADD(4, g5 - g4); GT_ADD(5, g6 - g5); GT_ADD(6, g7 - g6); GT_ADD(7, g8 - g7); GT_ADD(8, 1);
+        GT_CLK(g6);
+        GT_ADD(0, g1 - g0); GT_ADD(1, g2 - g1); GT_ADD(2, g3 - g2); GT_ADD(3, g4 - g3); GT_ADD(4, g5 - g4); GT_ADD(5, g6 - g5); GT_ADD(8, 1);
     }
 
-    if (p.ht != nullptr && p.ht_idx != nullptr) {
-        const long dst = p.ht_idx[seg];
-        if (dst >= 0) {
-            float* hp = p.ht + (dst * p.hv + hv) * (long)KD * VD;
+    if (keep) {
+        float* hp = p.ht + ((p.ht_idx[seg] * p.hv + hv) * KD + 4 * q4) * VD + 32 * w + c;
 #pragma unroll
-            for (int j = 0; j < 2; j++)
+        for (int kt = 0; kt < 8; kt++)
 #pragma unroll
-                for (int r = 0; r < 16; r++) hp[(long)(32 * wq + 8 * (r >> 2) + 4 * g + (r & 3)) * VD + 64 * wh + 32 * j + n32] = S[j][r];
-        }
+            for (int r = 0; r < 4; r++)
+#pragma unroll
+                for (int vt = 0; vt < 2; vt++) hp[(long)(16 * kt + r) * VD + 16 * vt] = S[kt][vt][r];
     }
 }
 
 int gdn_chunked_launch(const GdnParams& p, long max_len, hipStream_t stream) {
     (void)max_len;
     if (p.dv != VD) return spinf_fail(SPINF_E_ARG, "gdn chunked: value head dim %d, only 128 is built", p.dv);
-    if (p.v_tok % 8 || p.o_tok % 4) return spinf_fail(SPINF_E_ARG, "gdn chunked: v row stride must be a multiple of 8, o of 4 elements");
-    static bool configured = false;
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute((const void*)gdn_chunk_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
-        if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "gdn chunked: hipFuncSetAttribute: %s", hipGetErrorString(e));
-        configured = true;
-    }
     const long blocks = p.n_seg * p.hv;
     if (blocks > INT32_MAX) return spinf_fail(SPINF_E_ARG, "gdn chunked: too many segments");
-    hipLaunchKernelGGL(gdn_chunk_kernel, dim3((unsigned)blocks), dim3(512), LDS_BYTES, stream, p);
+    hipLaunchKernelGGL(gdn_chunk_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "gdn chunked: launch: %s", hipGetErrorString(e));
     return SPINF_OK;
