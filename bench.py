@@ -1,6 +1,6 @@
 """Benchmark of the tree-mask packed-prefill attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C2|C3|C4|C5] [--seed S] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C2|C3|C4|C5|copy] [--seed S] [--no-cpu]
 
 A step is one pass of the attention op (one layer's call through the C ABI) over one packed synthetic stream already
 resident in HBM; the tile plan is compiled once per stream, outside the timed region, as the reference builds its block
@@ -28,8 +28,15 @@ WORKLOADS = {
     "C2": "C2: 24 contents x (470-token trunk + 56 branches of U{8..16} tokens) in one varlen pass, 16 query / 8 KV heads, head_dim 256, scale 1/16, Q/K/V ~ 0.5 N(0,1), global layer",
     "C3": "C3: 512 contents, trunk lognormal(median 800, sigma 0.6) clipped 64..4096, U{8..64} branches of U{4..24}, passes <= 65,536 tokens, 16/8 heads, head_dim 256, one sliding (W=1024) + one global layer per pass",
     "C4": "C4: contents x (8192-token trunk + 16 nodes x 32 + 192 leaves of U{6..10}), 32/16 heads, head_dim 128, one varlen pass",
-    "C5": "C5: Gated DeltaNet, contents x (2048-token trunk + 32 branches x 12), 16 qk / 32 v heads, 128 x 128 fp32 state, chunk 64",
+    "copy": "plain device copy of 1 GiB (reads 1 GiB, writes 1 GiB per launch): the yardstick the FETCH_SIZE / WRITE_SIZE counters are scaled by",
+    "C5": "C5: Gated DeltaNet, contents x (2048-token trunk + 32 branches x 12), 16 qk / 32 v heads, 128 x 128 fp32 state",
 }
+
+
+# HBM bytes per launch of the dominant kernel(s), from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE runs of this file (KiB per
+# dispatch), each scaled by what the same counter reads for `--workload copy` (whose traffic is known).  The figures and the
+# commands are in profiles/*_counters.md; a workload without a counter run has None.
+TRAFFIC_BYTES = {"C2": None, "C5": None}
 
 
 def timed(fn, steps, warmup, torch):
@@ -77,6 +84,19 @@ def main():
             "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
             "data": "synthetic (seeded, numpy default_rng / torch generator)", "seed": args.seed}
 
+    if args.workload == "copy":
+        n = 1 << 30
+        src = torch.arange(n // 4, dtype=torch.int32, device=dev)
+        dst = torch.empty_like(src)
+        wall, kern = timed(lambda: dst.copy_(src), args.steps, args.warmup, torch)
+        ms = float(np.mean(kern))
+        line.update(metric="device copy", unit="GB/s", value=2 * n / (ms * 1e-3) / 1e9, ms_per_step=1e3 * wall / args.steps, dtype="u8",
+                    config={"workload": WORKLOADS["copy"], "bytes_read": n, "bytes_written": n},
+                    roofline={"bound": "hbm", "achieved": 2 * n / (ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                              "frac": 2 * n / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": 2 * n, "kernel_ms": ms})
+        print(json.dumps(line))
+        return
+
     if args.workload == "C5":
         cfg = synth.gdn_config("C5", seed=args.seed, contents=args.contents)
         t = synth.gdn_inputs(cfg, seed=args.seed, device=dev)
@@ -90,8 +110,8 @@ def main():
         gbs = cfg.bytes() / (ms * 1e-3) / 1e9
         line.update(metric="packed tokens/s, Gated DeltaNet tree scan", value=cfg.n_real * args.steps / wall, ms_per_step=1e3 * wall / args.steps,
                     dtype="bf16 (fp32 state)", config={"workload": WORKLOADS["C5"], "contents": len(cfg.trees), "tokens": cfg.n_real},
-                    roofline={"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS, "traffic": None,
-                              "kernel_ms": ms, "algorithmic_bytes": cfg.bytes()})
+                    roofline={"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
+                              "traffic": TRAFFIC_BYTES["C5"] if args.contents is None else None, "kernel_ms": ms, "algorithmic_bytes": cfg.bytes()})
         if not args.no_cpu:
             from oracle import cpu_baseline
 
@@ -132,7 +152,8 @@ def main():
                         "stream_tokens": sum(b.length for b in cfg.batches), "passes": len(cfg.batches), "layers_per_step": len(layers),
                         "visible_pairs": [cfg.pairs(w) for w in layers], "variant": args.variant},
                 roofline={"bound": "mfma", "achieved": tfl, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": tfl / PEAK_BF16_TFLOPS,
-                          "traffic": None, "kernel_ms": ms, "kernel_ms_min": float(np.min(kern)), "useful_flops": flops,
+                          "traffic": TRAFFIC_BYTES.get(args.workload) if args.contents is None else None, "kernel_ms": ms,
+                          "kernel_ms_min": float(np.min(kern)), "useful_flops": flops,
                           "algorithmic_bytes": cfg.bytes() * len(layers), "hbm_frac_at_algorithmic_bytes": cfg.bytes() * len(layers) / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS},
                 plan_build_ms_host=plan_ms, setup_s=setup_s)
     if not args.no_cpu:

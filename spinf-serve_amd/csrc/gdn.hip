@@ -15,7 +15,8 @@
 using namespace gdn_tiles;
 
 // ---------------------------------------------------------------------------------------------- short segments
-// The recurrent entry point: meant for the short segments of a trie (a handful of tokens after a fork), thousands per call.
+// The recurrent entry point for value head dims other than 128 (128 runs the workgroup kernel of gdn_chunk.hip on 16-token
+// chunks): meant for the short segments of a trie (a handful of tokens after a fork), thousands per call.
 // One wave per (segment, value head, 32 value columns) and no workgroup barrier anywhere.  The wave walks its segment in
 // mini-chunks of 16 tokens with the same WY algebra as the chunk-64 kernel (A = -strict_tril(beta_i K_i.K_j e^{G_i-G_j}),
 // T = (I - A)^-1, U = T diag(beta) V, -W = -T diag(beta e^G) K, V' = U - W S, O = s e^G Q S + P V', S <- e^{G_L} S +
@@ -218,7 +219,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void
     }
 }
 
-int gdn_chunked_launch(const GdnParams& p, long max_len, hipStream_t stream);   // gdn_chunk.hip
+int gdn_wy_launch(const GdnParams& p, int tokens_per_chunk, hipStream_t stream);   // gdn_chunk.hip
 
 extern "C" int spinf_gdn_fwd(const spinf_gdn_args* a, void* stream) {
     if (!a) return spinf_fail(SPINF_E_ARG, "gdn: null args");
@@ -241,8 +242,9 @@ extern "C" int spinf_gdn_fwd(const spinf_gdn_args* a, void* stream) {
     p.cu = (const long*)a->cu; p.idx = (const long*)a->idx; p.n_seg = a->n_seg;
     p.h0 = a->h0; p.h0_idx = (const long*)a->h0_idx; p.ht = a->ht; p.ht_idx = (const long*)a->ht_idx;
     hipStream_t s = (hipStream_t)stream;
-    if (a->mode == 1) return gdn_chunked_launch(p, a->max_len, s);
+    if (a->mode == 1) return gdn_wy_launch(p, 32, s);
     if (a->mode != 0) return spinf_fail(SPINF_E_ARG, "gdn: unknown mode %d", a->mode);
+    if (a->dv == 128) return gdn_wy_launch(p, 16, s);   // the workgroup kernel shares the per-head work of the four 32-column waves
     const long blocks = a->n_seg * a->hv * (a->dv / 32);
     if (blocks > INT32_MAX) return spinf_fail(SPINF_E_ARG, "gdn: too many segments");
     hipLaunchKernelGGL(gdn_short_kernel, dim3((unsigned)blocks), dim3(64), 0, s, p);

@@ -1,6 +1,7 @@
 """Gated DeltaNet over trie segments with the reference's two entry points (spinf_serve/models/qwen35/gdn.py:109-133, 197-235).
 
-Both run in libspinf_tree.so: `recurrent` token by token (short segments), `chunked` the fused chunk-64 WY kernel (long
+Both run in libspinf_tree.so as fused WY-form kernels: `recurrent` one wave per (segment, head, 32 values) on 16-token
+mini-chunks (short segments), `chunked` one workgroup per (segment, head) on 32-token chunks (long
 segments).  Unlike the reference's chunked(), the kernel reads and writes the stream rows through `idx` itself, so callers
 need no gather / scatter around it, and it writes no per-chunk state snapshots.
 
@@ -67,8 +68,8 @@ def chunked(q, k, v, g, beta, scale, cu, cu_cpu, h0=None, h0_idx=None, ht=None, 
     """gdn.chunked's contract (spinf_serve/models/qwen35/gdn.py:109-112): sequence n = call rows cu[n] .. cu[n+1]-1 starts from
     h0[h0_idx[n]] (zero when absent or negative) and leaves its final state in ht[ht_idx[n]] where that is >= 0.
     idx / o: optional row indirection as in `recurrent` (not in the reference, which gathers before and scatters after)."""
-    if chunk_size != 64:
-        raise ValueError("the fused kernel is built for 64-token chunks")
+    if chunk_size <= 0:
+        raise ValueError("chunk_size must be positive")  # the result does not depend on it: the kernel chunks by 32 internally
     if k.shape[-1] != 128:
         raise ValueError("the state kernel is written for K = 128")  # gdn.py:120
     n = len(cu_cpu) - 1

@@ -40,6 +40,7 @@ class TreePlan:
     seg_level: object | None = None
     seg_slot: object | None = None
     cap: dict | None = None
+    pad_rows: object | None = None   # [pads] int64 (device): rows of the tensors no segment covers; their outputs are zero
 
 
 def _segments(prev, real):
@@ -157,7 +158,8 @@ def tree_plan(prev, real, device, max_init: int = 96, path: str = "indexed", sho
         sidx = put(real_idx)
         seg_rows = np.full(rows, -1, np.int64)
         seg_rows[: len(real_idx)] = seg[real_idx]
-    return TreePlan(put(conv), levels, n, path, n_keep if path == "indexed" else None, rows, sidx, seg_rows, depth, slot)
+    return TreePlan(put(conv), levels, n, path, n_keep if path == "indexed" else None, rows, sidx, seg_rows, depth, slot,
+                    pad_rows=put(np.flatnonzero(seg_rows < 0)))
 
 
 @torch.compiler.disable
@@ -171,7 +173,12 @@ def gdn_tree(q, k, v, g, beta, plan: TreePlan, mod=None):
         for r0, n, name in cap["tok"]:
             cap["out"]["gdn"].setdefault(name, {})[li] = tuple(t[r0 : r0 + n].clone() for t in (q, k, v, g, beta))
     scale = q.shape[-1] ** -0.5
-    o = torch.zeros_like(v)
+    if plan.pad_rows is not None and len(plan.seg_of_row) == v.shape[0]:
+        o = torch.empty_like(v)      # every covered row is written by a kernel; only the pads need the zero fill
+        if plan.pad_rows.numel():
+            o.index_fill_(0, plan.pad_rows, 0)
+    else:
+        o = torch.zeros_like(v)
     g32 = g if g.dtype == torch.float32 else g.float()
     b16 = beta if beta.dtype == torch.bfloat16 else beta.to(torch.bfloat16)
     want = []

@@ -83,6 +83,34 @@ def test_rows_by_index_and_skipped_states(dev):
             assert np.abs(_np(o[0, r]) - want).max() <= TOL, mode
 
 
+def test_segments_forked_from_one_state(dev):
+    """many short segments that start from the same stored state (what a trunk's leaves look like), mixed with segments that
+    are longer than a mini-chunk, keep their final state or start from another state: each must equal its own recurrence"""
+    H, HV = 2, 4
+    lens = [5, 12, 16, 17, 3, 3, 40, 2, 9, 9, 9, 9, 9, 9, 9, 9, 9, 9, 1, 16, 16, 7]
+    src = [0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 1, 1, 1, -1]
+    kept = {2, 6, 12}
+    n, T = len(lens), sum(lens)
+    t = _inputs(T, H, HV, dev, seed=21)
+    cu_cpu = np.concatenate([[0], np.cumsum(lens)])
+    cu = torch.from_numpy(cu_cpu).to(dev)
+    h0 = (torch.randn((2, HV, 128, 128), device=dev) * 0.1).contiguous()
+    h0_idx = torch.tensor(src, device=dev)
+    ht = torch.full((n, HV, 128, 128), float("nan"), device=dev)
+    ht_idx = torch.tensor([i if i in kept else -1 for i in range(n)], device=dev)
+    args = [t[x][None] for x in ("q", "k", "v", "g", "beta")]
+    o = sa.recurrent(*args, 128 ** -0.5, cu, n, h0=h0, h0_idx=h0_idx, ht=ht, ht_idx=ht_idx)
+    torch.cuda.synchronize()
+    for s in range(n):
+        a, b = int(cu_cpu[s]), int(cu_cpu[s + 1])
+        want, S = ogdn.recurrent(*(_np(t[x][a:b]) for x in ("q", "k", "v", "g", "beta")), h0=_np(h0[src[s]]) if src[s] >= 0 else None)
+        assert float(np.abs(_np(o[0, a:b]) - want).max()) <= TOL, s
+        if s in kept:
+            assert float(np.abs(_np(ht[s]) - S).max()) <= STATE_TOL, s
+        else:
+            assert torch.isnan(ht[s]).all(), s
+
+
 def test_tree_scan_forks_from_trunk_state(dev):
     """C5's shape scaled down: every branch continues from its trunk's final state == one sequence trunk||branch"""
     cfg = synth.gdn_config("C5", contents=2)
