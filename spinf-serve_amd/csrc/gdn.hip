@@ -145,7 +145,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void
         wave_lds_order();
         // ---- row c of T = (I - A)^-1, solved by every group of 16 lanes alike
         float t[MC];
-        unit_lower_inverse_row(As, LDA, c, t);
+        unit_lower_inverse_row<false>(As, LDA, c, t);
         // T diag(beta) and -T diag(beta e^G), columns 4 q4 + r of row c
         bf16x4 tuA, twB;
         const f32x4 tq = pick4(t, q4);
@@ -232,6 +232,8 @@ extern "C" int spinf_gdn_fwd(const spinf_gdn_args* a, void* stream) {
     if (((uintptr_t)a->q | (uintptr_t)a->k) % 16) return spinf_fail(SPINF_E_ARG, "gdn: q/k must be 16-byte aligned");
     if ((a->h0 == nullptr) != (a->h0_idx == nullptr) && a->h0 == nullptr) return spinf_fail(SPINF_E_ARG, "gdn: h0_idx without h0");
     if (a->ht_idx != nullptr && a->ht == nullptr) return spinf_fail(SPINF_E_ARG, "gdn: ht_idx without ht");
+    if (a->q_tok <= 0 || a->v_tok <= 0 || a->g_tok <= 0 || a->o_tok <= 0 || (a->q_tok | a->v_tok | a->g_tok | a->o_tok) >> 31)
+        return spinf_fail(SPINF_E_ARG, "gdn: row strides must be positive and below 2^31 elements");
     if (a->v_tok % 8 || a->o_tok % 8) return spinf_fail(SPINF_E_ARG, "gdn: v/o row stride must be a multiple of 8 elements");
     if (((uintptr_t)a->v | (uintptr_t)a->o) % 16) return spinf_fail(SPINF_E_ARG, "gdn: v/o must be 16-byte aligned");
     GdnParams p;

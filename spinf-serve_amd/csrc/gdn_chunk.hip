@@ -46,8 +46,9 @@ constexpr int LW = 132;        // row stride of the -W tile
 constexpr int LP = 40;         // row stride of the token x token bf16 tiles (P, T diag(beta), -T diag(beta e^G))
 constexpr int LA = 36;         // row stride (floats) of A
 constexpr int LX = 20;         // row stride (floats) of the 16 x 16 blocks of T and of the merge scratch
-constexpr int LO = 32;         // row stride (elements) of a wave's output tile
 
+// element offset of a row: one 32 x 32 -> 64 bit multiply (rows and strides are below 2^31; the launch checks the strides)
+__device__ __forceinline__ long row_offset(int row, long stride) { return (long)((unsigned long)(unsigned)row * (unsigned)stride); }
 __device__ __forceinline__ bf16x4 zero_bf4() {
     bf16x4 z;
 #pragma unroll
@@ -74,8 +75,9 @@ struct Tok<1> {
 }  // namespace
 
 template <int NT>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gdn_wy_kernel(const GdnParams p) {
+__device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
     constexpr int CH = 16 * NT;
+    constexpr int LO = CH;                          // row stride (elements) of a wave's transposed output tile [32 values][CH tokens]
     constexpr int NTILES = NT * (NT + 1) / 2;       // 16 x 16 tiles of A / P on or below the diagonal
     typedef typename Tok<NT>::op tok_op;            // operand of a product that contracts over the chunk's tokens
     __shared__ __attribute__((aligned(16))) __bf16 Ks[CH * LD];
@@ -87,13 +89,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     __shared__ __attribute__((aligned(16))) __bf16 Tws[CH * LP];
     __shared__ __attribute__((aligned(16))) float Gs[CH];
     __shared__ __attribute__((aligned(16))) float Bs[CH];
-    __shared__ long Rs[CH];
+    __shared__ int Rs[CH];
     float* As = (float*)solve;
     float* Ts = As + 32 * LA;          // T_00 in rows 0..15, T_11 in rows 16..31
     float* Xs = Ts + 32 * LX;
     __bf16* Wn = (__bf16*)solve;       // -W [CH][LW], written when A and T are dead
     static_assert(32 * LW * 2 <= (int)sizeof(solve), "-W must fit the region it shares");
-    static_assert(4 * CH * LO <= CH * LD, "the output tiles must fit the V tile");
+    static_assert(4 * 32 * LO <= CH * LD, "the output tiles must fit the V tile");
 
     const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6), c = lane & 15, q4 = lane >> 4;
     const long seg = blockIdx.x / p.hv;
@@ -101,7 +103,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int hk = hv / (p.hv / p.h);
     const long bos = p.cu[seg], eos = p.cu[seg + 1];
     const int T = (int)(eos - bos);
-    __bf16* Ow = Vs + w * CH * LO;
+    __bf16* Ow = Vs + w * 32 * LO;
 
     // ---- state: S[kt][vt][r] = S[16 kt + 4 q4 + r][32 w + 16 vt + c]
     f32x4 S[8][2];
@@ -128,10 +130,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // Thread -> 16-byte piece tid%16 of chunk rows tid/16 (+ 16); threads 0..CH-1 also -> g, beta and the stream row of chunk
     // row tid.
     bf16x8 pk[NT], pq[NT], pv[NT];
-    long pr64 = -1;
+    int pr32 = -1;
     float pg = 0.f;
     __bf16 pbeta = (__bf16)0.f;   // (kept as loaded: converting here would make the wave wait for the load at once)
-    long ra[NT], rb = -1;
+    int ra[NT], rb = -1;          // stream rows (< 2^31) of the chunk fetched next: this thread's K / Q / V rows; chunk row tid
+    // Only the low half of an index is loaded: the register of an unused high half would be handed out again at once, and
+    // whoever writes it first has to wait for the load (and with it for every load in flight).
+    const int* idx_lo = (const int*)p.idx;
     auto fetch_rows = [&](const int c0) __attribute__((always_inline)) {
         const int L = min(CH, T - c0);      // <= 0: there is no such chunk
 #pragma unroll
@@ -140,13 +145,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             ra[cc] = -1;
             if (row < L) {
                 const long t = bos + c0 + row;
-                ra[cc] = p.idx ? p.idx[t] : t;
+                ra[cc] = p.idx ? idx_lo[2 * t] : (int)t;
             }
         }
         rb = -1;
         if (tid < CH && tid < L) {
             const long t = bos + c0 + tid;
-            rb = p.idx ? p.idx[t] : t;
+            rb = p.idx ? idx_lo[2 * t] : (int)t;
         }
     };
     auto fetch_data = [&]() __attribute__((always_inline)) {
@@ -156,17 +161,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
             for (int j = 0; j < 8; j++) { pk[cc][j] = (__bf16)0.f; pq[cc][j] = (__bf16)0.f; pv[cc][j] = (__bf16)0.f; }
             if (ra[cc] >= 0) {
-                pk[cc] = *(const bf16x8*)(p.k + ra[cc] * p.q_tok + (long)hk * KD + col);
-                pq[cc] = *(const bf16x8*)(p.q + ra[cc] * p.q_tok + (long)hk * KD + col);
-                pv[cc] = *(const bf16x8*)(p.v + ra[cc] * p.v_tok + (long)hv * VD + col);
+                pk[cc] = *(const bf16x8*)(p.k + row_offset(ra[cc], p.q_tok) + hk * KD + col);
+                pq[cc] = *(const bf16x8*)(p.q + row_offset(ra[cc], p.q_tok) + hk * KD + col);
+                pv[cc] = *(const bf16x8*)(p.v + row_offset(ra[cc], p.v_tok) + hv * VD + col);
             }
         }
-        pr64 = rb;
+        pr32 = rb;
         pg = 0.f;
         pbeta = (__bf16)0.f;
         if (rb >= 0) {
-            pg = p.g[rb * p.g_tok + hv];
-            pbeta = p.beta[rb * p.g_tok + hv];
+            pg = p.g[row_offset(rb, p.g_tok) + hv];
+            pbeta = p.beta[row_offset(rb, p.g_tok) + hv];
         }
     };
     fetch_rows(0);
@@ -183,7 +188,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             if (NT == 2) x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x142, 0xa, 0xf, false));  // row_bcast:15 -> lanes 16..31
             Gs[tid] = x;
             Bs[tid] = (float)pbeta;
-            Rs[tid] = pr64;
+            Rs[tid] = pr32;
         }
         {
             const int col = (tid & 15) * 8;
@@ -238,7 +243,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         if (w == 0) {
             float t[16];
             const int blk = NT == 2 ? (q4 & 1) : 0;
-            unit_lower_inverse_row(As + blk * (16 * LA + 16), LA, c, t);
+            unit_lower_inverse_row<NT == 2>(As + blk * (16 * LA + 16), LA, c, t);
             // the rows pass through LDS to reach the lanes in operand order (row c, columns 4 q4 ..+3)
 #pragma unroll
             for (int j4 = 0; j4 < 4; j4++) *(f32x4*)(Ts + (16 * blk + c) * LX + 4 * j4) = f32x4{t[4 * j4], t[4 * j4 + 1], t[4 * j4 + 2], t[4 * j4 + 3]};
@@ -346,6 +351,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         // the next chunk's rows are requested here, where few registers are live; they arrive during the state update
         fetch_data();          // chunk c0 + CH, whose rows are known since the previous chunk
         fetch_rows(c0 + 2 * CH);
+        GT_CLK(g5a);
         // ---- O[i][v] = s e^{G_i} (Q S)[i][v] + sum_j P[i][j] V'[j][v], rows i = 16 it + 4 q4 + r; through LDS for 16-byte stores
         f32x4 Gj[NT];
 #pragma unroll
@@ -362,18 +368,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 const tok_op vb = Tok<NT>::make(round4(vp[0][vt]), round4(vp[NT - 1][vt]));
 #pragma unroll
                 for (int it = 0; it < NT; it++) {
-                    const f32x4 o = mm(pA[it], vb, zero4());
+                    f32x4 o = mm(pA[it], vb, zero4());
 #pragma unroll
-                    for (int r = 0; r < 4; r++)
-                        Ow[(16 * it + 4 * q4 + r) * LO + 16 * vt + c] = (__bf16)__builtin_fmaf(p.scale * __expf(Gj[it][r]), qs[it][vt][r], o[r]);
+                    for (int r = 0; r < 4; r++) o[r] = __builtin_fmaf(p.scale * __expf(Gj[it][r]), qs[it][vt][r], o[r]);
+                    *(bf16x4*)(Ow + (16 * vt + c) * LO + 16 * it + 4 * q4) = round4(o);      // O^T[v][i]
                 }
             }
         }
         wave_lds_order();
+        GT_CLK(g5b);
+        // row i = 16 it + lane%16, values 8 (lane/16) ..+7 of this wave's 32: two transposing reads, one 16-byte store
 #pragma unroll
-        for (int cc = 0; cc < NT; cc++) {
-            const int row = (lane >> 2) + 16 * cc;
-            if (row < L) *(bf16x8*)(p.o + Rs[row] * p.o_tok + (long)hv * VD + 32 * w + (lane & 3) * 8) = *(const bf16x8*)(Ow + row * LO + (lane & 3) * 8);
+        for (int it = 0; it < NT; it++) {
+            const int row = 16 * it + c;
+            const __bf16* op = Ow + (8 * q4 + (c >> 2)) * LO + 16 * it + 4 * (c & 3);
+            const bf16x4 lo = __builtin_bit_cast(bf16x4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)op));
+            const bf16x4 hi = __builtin_bit_cast(bf16x4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(op + 4 * LO)));
+            if (row < L) *(bf16x8*)(p.o + row_offset(Rs[row], p.o_tok) + hv * VD + 32 * w + 8 * q4) = join(lo, hi);
         }
         GT_CLK(g6);
         // ---- S[k][v] = e^{G_L} S[k][v] + sum_j K[j][k] (V' e^{G_L - G_j})[j][v]; skipped when nothing reads the state again
@@ -402,7 +413,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             }
         }
         GT_CLK(g7);
-        GT_ADD(0, g1 - g0); GT_ADD(1, g2 - g1); GT_ADD(2, g3 - g2); GT_ADD(3, g4 - g3); GT_ADD(4, g5 - g4); GT_ADD(5, g6 - g5); GT_ADD(6, g7 - g6); GT_ADD(8, 1);
+        GT_ADD(0, g1 - g0); GT_ADD(1, g2 - g1); GT_ADD(2, g3 - g2); GT_ADD(3, g4 - g3); GT_ADD(4, g5 - g4); GT_ADD(5, g6 - g5); GT_ADD(6, g7 - g6); GT_ADD(8, 1); GT_ADD(9, g5a - g5); GT_ADD(10, g5b - g5a); GT_ADD(11, g6 - g5b);
     }
 
     if (keep) {
@@ -416,13 +427,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 }
 
+// 32-token chunks: 254 registers (the solve's preloaded triangle), two workgroups per compute unit.  16-token chunks: 168
+// registers, three workgroups per compute unit.
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gdn_wy32_kernel(const GdnParams p) { gdn_wy_body<2>(p); }
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void gdn_wy16_kernel(const GdnParams p) { gdn_wy_body<1>(p); }
+
 // tokens_per_chunk: 32 (long segments) or 16 (short segments)
 int gdn_wy_launch(const GdnParams& p, int tokens_per_chunk, hipStream_t stream) {
     if (p.dv != VD) return spinf_fail(SPINF_E_ARG, "gdn: value head dim %d, the chunked kernel is built for 128", p.dv);
     const long blocks = p.n_seg * p.hv;
     if (blocks > INT32_MAX) return spinf_fail(SPINF_E_ARG, "gdn: too many segments");
-    if (tokens_per_chunk == 32) hipLaunchKernelGGL(gdn_wy_kernel<2>, dim3((unsigned)blocks), dim3(256), 0, stream, p);
-    else hipLaunchKernelGGL(gdn_wy_kernel<1>, dim3((unsigned)blocks), dim3(256), 0, stream, p);
+    if (tokens_per_chunk == 32) hipLaunchKernelGGL(gdn_wy32_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL(gdn_wy16_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "gdn: launch: %s", hipGetErrorString(e));
     return SPINF_OK;

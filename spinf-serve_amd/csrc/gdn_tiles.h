@@ -60,18 +60,34 @@ __device__ __forceinline__ float row_prefix_sum(float x) {
 }
 // Row c of (I - A)^-1 for a strictly lower triangular 16 x 16 block A (row stride lda floats, in LDS), c = this lane's row:
 // T = I + T A, so t[j] = [j == c] + sum_{m > j} t[m] A[m][j]; the highest m goes first and every step updates all j < m.
+// PRELOAD: read A's rows in two batches (rows 15..8, then 7..1) ahead of the steps that use them instead of row by row: the
+// steps form a chain of 15 dependent multiply-adds, and an LDS round trip inside every link is what such a solve otherwise
+// waits for.
+template <bool PRELOAD>
 __device__ __forceinline__ void unit_lower_inverse_row(const float* A, int lda, int c, float (&t)[16]) {
+    f32x4 a[16][4];
 #pragma unroll
     for (int j = 0; j < 16; j++) t[j] = (j == c) ? 1.f : 0.f;
 #pragma unroll
-    for (int m = 15; m >= 1; m--) {
+    for (int half = 1; half >= 0; half--) {
+        if (PRELOAD) {
 #pragma unroll
-        for (int j4 = 0; 4 * j4 < m; j4++) {
-            const f32x4 am = *(const f32x4*)(A + m * lda + 4 * j4);
+            for (int m = 8 * half + 7; m >= 8 * half; m--)
 #pragma unroll
-            for (int jj = 0; jj < 4; jj++)
-                if (4 * j4 + jj < m) t[4 * j4 + jj] = __builtin_fmaf(t[m], am[jj], t[4 * j4 + jj]);
+                for (int j4 = 0; 4 * j4 < m; j4++) a[m][j4] = *(const f32x4*)(A + m * lda + 4 * j4);
+            __builtin_amdgcn_sched_barrier(0);
         }
+#pragma unroll
+        for (int m = 8 * half + 7; m >= 8 * half; m--) {
+#pragma unroll
+            for (int j4 = 0; 4 * j4 < m; j4++) {
+                const f32x4 am = PRELOAD ? a[m][j4] : *(const f32x4*)(A + m * lda + 4 * j4);
+#pragma unroll
+                for (int jj = 0; jj < 4; jj++)
+                    if (4 * j4 + jj < m) t[4 * j4 + jj] = __builtin_fmaf(t[m], am[jj], t[4 * j4 + jj]);
+            }
+        }
+        if (PRELOAD) __builtin_amdgcn_sched_barrier(0);
     }
 }
 // t[4 q + r], r = 0..3, without indexing registers by a lane-dependent value
