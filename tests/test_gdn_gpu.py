@@ -111,6 +111,32 @@ def test_segments_forked_from_one_state(dev):
             assert torch.isnan(ht[s]).all(), s
 
 
+@pytest.mark.parametrize("V", [64, 256])
+def test_recurrent_other_value_dims(dev, V):
+    """value head dims other than 128 take the one-wave-per-32-columns kernel of the recurrent entry point"""
+    H, HV = 2, 4
+    lens = [5, 20, 33, 16]
+    n, T = len(lens), sum(lens)
+    t = _inputs(T, H, HV, dev, seed=5, V=V)
+    cu_cpu = np.concatenate([[0], np.cumsum(lens)])
+    cu = torch.from_numpy(cu_cpu).to(dev)
+    h0 = (torch.randn((n, HV, 128, V), device=dev) * 0.1).contiguous()
+    h0_idx = torch.tensor([0, -1, 2, 3], device=dev)
+    ht = torch.full((n, HV, 128, V), float("nan"), device=dev)
+    ht_idx = torch.tensor([0, 1, -1, 3], device=dev)
+    args = [t[x][None] for x in ("q", "k", "v", "g", "beta")]
+    o = sa.recurrent(*args, 128 ** -0.5, cu, n, h0=h0, h0_idx=h0_idx, ht=ht, ht_idx=ht_idx)
+    torch.cuda.synchronize()
+    for s in range(n):
+        a, b = int(cu_cpu[s]), int(cu_cpu[s + 1])
+        want, S = ogdn.recurrent(*(_np(t[x][a:b]) for x in ("q", "k", "v", "g", "beta")), h0=_np(h0[s]) if int(h0_idx[s]) >= 0 else None)
+        assert float(np.abs(_np(o[0, a:b]) - want).max()) <= TOL, s
+        if int(ht_idx[s]) >= 0:
+            assert float(np.abs(_np(ht[s]) - S).max()) <= STATE_TOL, s
+        else:
+            assert torch.isnan(ht[s]).all(), s
+
+
 def test_tree_scan_forks_from_trunk_state(dev):
     """C5's shape scaled down: every branch continues from its trunk's final state == one sequence trunk||branch"""
     cfg = synth.gdn_config("C5", contents=2)
