@@ -1,0 +1,83 @@
+"""The two headline workloads at their full sizes (C2: 24 contents in one pass; C5: 128 contents, 311,296 tokens), checked
+through properties that do not need the oracle to process the whole stream: a content's rows are bit-identical alone and
+inside the full pack, the delta rule is exactly linear under a power-of-two scaling of v, and one content of the pack is
+compared with the float64 oracle."""
+
+import numpy as np
+import pytest
+import torch
+
+import spinf_serve_amd as sa
+from oracle import attention as oattn
+from oracle import gdn as ogdn
+from spinf_serve_amd import synth
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-2
+
+
+def _np(t):
+    return t.float().cpu().numpy()
+
+
+def test_c2_full_pack_is_invariant_and_matches_the_oracle(dev):
+    cfg = synth.attention_config("C2")
+    assert len(cfg.trees) == 24 and len(cfg.batches) == 1
+    b = cfg.batches[0]
+    q, k, v = synth.qkv(cfg, b, seed=0, device=dev)
+    masks = sa.block_masks(b, sliding_window=None, device=dev)
+    out = sa.tree_attn(q, k, v, masks["full_attention"], cfg.scale)
+    torch.cuda.synchronize()
+    for slot in (0, 11, 23):
+        s0, n = b.owners[slot].start, cfg.trees[slot].n_tokens
+        one = synth.pack([cfg.trees[slot]])[0]
+        m1 = sa.TreeMask.build(one.art, one.end, one.pos, window=None, device=dev)
+        pad = one.length - n
+
+        def z(t):
+            t = t[s0 : s0 + n]
+            return torch.cat([t, torch.zeros((pad, *t.shape[1:]), dtype=t.dtype, device=dev)]) if pad else t.contiguous()
+
+        alone = sa.tree_attn(z(q), z(k), z(v), m1, cfg.scale)
+        assert torch.equal(alone[:n], out[s0 : s0 + n]), slot
+    # one content against the dense float64 oracle
+    s0 = b.owners[5].start
+    one = synth.pack([cfg.trees[5]])[0]
+    n = cfg.trees[5].n_tokens
+    want = oattn.tree_attention(_np(q[s0 : s0 + n]), _np(k[s0 : s0 + n]), _np(v[s0 : s0 + n]), one.art[:n], one.end[:n], pos=one.pos[:n], scale=cfg.scale)
+    real = one.art[:n] >= 0
+    err = float(np.abs(_np(out[s0 : s0 + n])[real] - want[real]).max())
+    print(f"C2 full pack, content 5: max abs err {err:.3e}", flush=True)
+    assert err <= TOL
+
+
+def test_c5_full_stream_properties(dev):
+    cfg = synth.gdn_config("C5")
+    assert len(cfg.trees) == 128
+    t = synth.gdn_inputs(cfg, seed=0, device=dev)
+    plan = cfg.plan(dev)
+    o = sa.gdn_tree(t["q"], t["k"], t["v"], t["g"], t["beta"], plan)
+    # exact linearity in v under a power-of-two scale: every product and rounding commutes with it
+    o2 = sa.gdn_tree(t["q"], t["k"], t["v"] * 2, t["g"], t["beta"], plan)
+    torch.cuda.synchronize()
+    assert torch.equal(o2, o * 2)
+    del o2
+    b = cfg.batch
+    for slot in (0, 77, 127):
+        s0 = b.owners[slot].start
+        n = cfg.trees[slot].n_tokens
+        one = synth.GdnConfig("one", cfg.h, cfg.hv, cfg.dk, cfg.dv, [cfg.trees[slot]])
+        one.batch = synth.pack([cfg.trees[slot]])[0]
+        pad = one.batch.length - n
+
+        def z(x):
+            x = x[s0 : s0 + n]
+            return torch.cat([x, torch.zeros((pad, *x.shape[1:]), dtype=x.dtype, device=dev)]) if pad else x.contiguous()
+
+        alone = sa.gdn_tree(z(t["q"]), z(t["k"]), z(t["v"]), z(t["g"]), z(t["beta"]), one.plan(dev))
+        assert torch.equal(alone[:n], o[s0 : s0 + n]), slot
+        if slot == 77:
+            want = ogdn.tree_scan(*(_np(z(t[x])) for x in ("q", "k", "v", "g", "beta")), one.batch.prev, one.batch.art >= 0)
+            err = float(np.abs(_np(alone) - want).max())
+            print(f"C5 full stream, content 77: max abs err {err:.3e}", flush=True)
+            assert err <= TOL
