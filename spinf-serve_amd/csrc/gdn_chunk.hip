@@ -98,8 +98,12 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
     static_assert(4 * 32 * LO <= CH * LD, "the output tiles must fit the V tile");
 
     const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6), c = lane & 15, q4 = lane >> 4;
-    const long seg = blockIdx.x / p.hv;
-    const int hv = (int)(blockIdx.x % p.hv);
+    // Workgroups go round the 8 XCDs (each with its own L2) in launch order.  Two value heads that share a key head read the
+    // same q and k rows: they get launch slots 8 apart, i.e. the same XCD at about the same time, so the second read hits L2.
+    long slot = blockIdx.x;
+    if (p.hv == 2 * p.h && gridDim.x % 16 == 0) slot = (slot / 16) * 16 + (slot % 8) * 2 + (slot % 16) / 8;
+    const long seg = slot / p.hv;
+    const int hv = (int)(slot % p.hv);
     const int hk = hv / (p.hv / p.h);
     const long bos = p.cu[seg], eos = p.cu[seg + 1];
     const int T = (int)(eos - bos);
