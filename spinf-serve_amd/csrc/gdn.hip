@@ -18,7 +18,7 @@ using namespace gdn_tiles;
 // The recurrent entry point for value head dims other than 128 (128 runs the workgroup kernel of gdn_chunk.hip on 16-token
 // chunks): meant for the short segments of a trie (a handful of tokens after a fork), thousands per call.
 // One wave per (segment, value head, 32 value columns) and no workgroup barrier anywhere.  The wave walks its segment in
-// mini-chunks of 16 tokens with the same WY algebra as the chunk-64 kernel (A = -strict_tril(beta_i K_i.K_j e^{G_i-G_j}),
+// mini-chunks of 16 tokens with the same WY algebra as the workgroup kernel of gdn_chunk.hip (A = -strict_tril(beta_i K_i.K_j e^{G_i-G_j}),
 // T = (I - A)^-1, U = T diag(beta) V, -W = -T diag(beta e^G) K, V' = U - W S, O = s e^G Q S + P V', S <- e^{G_L} S +
 // K^T (V' e^{G_L-G})), on 16x16 MFMA tiles laid out so that every product's result is already the next product's operand:
 //   * the state slice S[128][32] stays in fp32 accumulator layout (lane = value column, 4 consecutive key rows per tile): two
@@ -27,7 +27,7 @@ using namespace gdn_tiles;
 //   * Q.K^T and K.K^T are computed transposed (lane = row i, registers = columns j), which is the A operand layout of P in
 //     O = P V' and the row layout (I - A)^-1 is solved in; every lane solves row i = lane % 16 by substitution in registers;
 //   * -W^T and V' come out of their products as the A and B operands of the products that consume them.
-// The state is kept and accumulated in fp32; products take bf16 operands, as in the chunk-64 kernel.
+// The state is kept and accumulated in fp32; products take bf16 operands, as in the workgroup kernel.
 namespace {
 constexpr int MC = 16;      // tokens per mini-chunk
 constexpr int LDK = 136;    // row stride (elements) of the K tile in LDS
