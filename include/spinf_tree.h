@@ -80,7 +80,8 @@ typedef struct spinf_attn_args {
     const int32_t* art; const int32_t* end; const int32_t* pos;
     const int32_t* kv_idx; const uint32_t* kv_bits; const int32_t* items; const int32_t* list_ptr;
     int64_t n_items;
-    int32_t variant;   /* 0 = default kernel choice; 1 = one head per work item even where two would fit */
+    int32_t variant;   /* 0 = default kernel choice (eight waves, two heads of a GQA group per work item, where the group is even);
+                          1 = one head per work item, four waves; 2 = four waves with two heads each (head dim <= 128) */
 } spinf_attn_args;
 
 /* query heads one work item covers for this geometry (1 or 2); 0 for an invalid geometry */

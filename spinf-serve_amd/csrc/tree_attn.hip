@@ -86,7 +86,6 @@ struct Geo {
     static constexpr int CPR = ROWB / 16;              // 16-byte chunks per row
     static constexpr int RPI = 1024 / ROWB;            // rows per region
     static constexpr int NREG = 64 / RPI;              // regions per tile
-    static constexpr int IPW = NREG / 4;               // DMA instructions per wave and tile
     static constexpr int KRS = 1024 + 16, VRS = 1024 + 64;
     static constexpr int KTILEB = NREG * KRS, VTILEB = NREG * VRS;
     static constexpr int METAB = 3 * 64 * 4;
@@ -120,19 +119,21 @@ __device__ __forceinline__ void dma4_lane(const int* addr, unsigned lds) {
 }
 __device__ __forceinline__ unsigned lds_addr(const void* p) { return (unsigned)(size_t)(const __attribute__((address_space(3))) char*)p; }
 
-// Starts the DMA of key tile kt (64 keys of kv head kvh) into the LDS buffer at byte address `buf`.  Wave w copies regions
+// Starts the DMA of key tile kt (64 keys of kv head kvh) into the LDS buffer at byte address `buf`.  Wave w of NW copies regions
 // w*IPW .. w*IPW+IPW-1; lane -> (slot = which row of the region, 16-byte chunk of the row).  For a tile that lies fully inside
 // the stream every address is a wave-uniform base plus a per-lane constant (lane_k / lane_v, bytes), so the loop spends no
 // vector ALU on addressing; the last, partial tile clamps its rows per lane.
-template <int D>
+template <int D, int NW = 4>
 __device__ __forceinline__ void issue_tile(const AttnParams& p, unsigned buf, int kt, int kvh, int w, int lane, unsigned lane_k, unsigned lane_v) {
     using G = Geo<D>;
+    constexpr int IPW = G::NREG / NW;   // DMA instructions per wave and tile
+    static_assert(IPW >= 1 && IPW * NW == G::NREG, "the tile's regions must divide among the waves");
     const char* kbase = (const char*)(p.k + (long)kvh * p.k_head);
     const char* vbase = (const char*)(p.v + (long)kvh * p.v_head);
     if (kt * 64 + 64 <= p.n) {
 #pragma unroll
-        for (int i = 0; i < G::IPW; i++) {
-            const int reg = w * G::IPW + i;
+        for (int i = 0; i < IPW; i++) {
+            const int reg = w * IPW + i;
             const long row = (long)kt * 64 + reg;
             dma16_uniform(kbase + row * p.k_tok * 2, lane_k, buf + reg * G::KRS);
             dma16_uniform(vbase + row * p.v_tok * 2, lane_v, buf + G::KTILEB + reg * G::VRS);
@@ -144,8 +145,8 @@ __device__ __forceinline__ void issue_tile(const AttnParams& p, unsigned buf, in
     } else {
         const int slot = lane / G::CPR, chunk = lane % G::CPR;
 #pragma unroll
-        for (int i = 0; i < G::IPW; i++) {
-            const int reg = w * G::IPW + i;
+        for (int i = 0; i < IPW; i++) {
+            const int reg = w * IPW + i;
             long grow = (long)kt * 64 + reg + G::NREG * slot;
             grow = grow < p.n ? grow : p.n - 1;
             dma16_lane(kbase + grow * p.k_tok * 2 + chunk * 16, buf + reg * G::KRS);
@@ -164,6 +165,7 @@ template <int D>
 struct Lane {
     using G = Geo<D>;
     int lane, m, g, w;
+    int wr, wh;                  // row group (tokens 32 wr ..) and head slot of this wave: w = 4 wh + wr
     int k_lane, v_lane;          // byte offsets of this lane's K fragment row / V^T fragment address inside a tile
     unsigned lane_k, lane_v;     // per-lane part of the DMA source addresses
     __device__ __forceinline__ Lane(const AttnParams& p) {
@@ -171,6 +173,8 @@ struct Lane {
         m = lane & 31;
         g = lane >> 5;
         w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+        wr = w & 3;
+        wh = w >> 2;
         // K fragment: row m of the 32-key block, 16-byte chunk g of each 32-byte step.  V^T fragment
         // (ds_read_b64_tr_b16): inside its 16-lane group a lane supplies the address of key row 4g + tr_j, head dims
         // 16 tr_mb + 4 tr_a .. +3 of the 32-wide slice, and receives head dim lane%32 of 4 consecutive keys.
@@ -215,7 +219,7 @@ __device__ __forceinline__ void store_rows(const AttnParams& p, const Lane<D>& L
                                            int t, int h0) {
     constexpr int NDT = D / 32;
     constexpr int SROW = 128 + 16;
-    const int tok0 = t * SPINF_QTILE + 32 * L.w;
+    const int tok0 = t * SPINF_QTILE + 32 * L.wr;
 #pragma unroll
     for (int rt = 0; rt < RT; rt++) {
         const float inv = 1.0f / lane32_sum(l[rt]);
@@ -246,12 +250,12 @@ __device__ __forceinline__ void store_rows(const AttnParams& p, const Lane<D>& L
 // kernel of its own because its accumulator rescaling (vector ALU on all of O) would cost the fast pass its register
 // allocation.
 template <int D, int RT, bool WIN>
-__device__ __forceinline__ void attn_item_exact(const AttnParams& p, const int4 item, char* buf0, int2* ent, char* stage) {
+__device__ __forceinline__ void attn_item_exact(const AttnParams& p, const int4 item, const int h0, char* buf0, int2* ent, char* stage) {
     using G = Geo<D>;
     constexpr int NS = D / 16, NDT = D / 32;
     const Lane<D> L(p);
-    const int t = item.x, e0 = item.y, ne = item.z & 0xfffff, hp = (unsigned)item.z >> 20;
-    const int h0 = hp * RT, kvh = h0 / p.group;
+    const int t = item.x, e0 = item.y, ne = item.z & 0xfffff;   // heads h0 .. h0 + RT - 1 of the item
+    const int kvh = h0 / p.group;
     const int tok = t * SPINF_QTILE + 32 * L.w + L.m;
     const int tok_c = tok < p.n ? tok : p.n - 1;
     bf16x8 qf[RT][NS];
@@ -355,7 +359,8 @@ __device__ __forceinline__ void attn_item_exact(const AttnParams& p, const int4 
     store_rows<D, RT>(p, L, stage, o, l, t, h0);
 }
 
-template <int D, int RT, bool WIN>
+// An item of HPI heads is recomputed RT heads at a time.
+template <int D, int RT, bool WIN, int HPI>
 __global__ __launch_bounds__(256) void tree_attn_exact_kernel(const AttnParams p) {
     using G = Geo<D>;
     __shared__ __attribute__((aligned(16))) char buf0[G::BUFB];
@@ -368,7 +373,8 @@ __global__ __launch_bounds__(256) void tree_attn_exact_kernel(const AttnParams p
         const int4 it = p.items[p.redo[j]];
         const int4 item = make_int4(__builtin_amdgcn_readfirstlane(it.x), __builtin_amdgcn_readfirstlane(it.y),
                                     __builtin_amdgcn_readfirstlane(it.z), __builtin_amdgcn_readfirstlane(it.w));
-        attn_item_exact<D, RT, WIN>(p, item, buf0, ent, stage_all + w * 32 * 144);
+        const int hp = (int)((unsigned)item.z >> 20);
+        for (int sub = 0; sub < HPI; sub += RT) attn_item_exact<D, RT, WIN>(p, item, hp * HPI + sub, buf0, ent, stage_all + w * 32 * 144);
     }
     __builtin_amdgcn_s_waitcnt(0x0f70);
     __syncthreads();
@@ -394,9 +400,12 @@ extern "C" int spinf_debug_trace(long* out, int n) { return (int)hipMemcpyFromSy
 #define TRACE_CLK(var) do { } while (0)
 #endif
 
-template <int D, int RT, bool WIN>
-__global__ __launch_bounds__(256) void tree_attn_kernel(const AttnParams p) {
+// NHW = 1: four waves, each with RT heads of the item.  NHW = 2: eight waves, waves 4..7 take the item's second set of RT heads
+// on the same K / V tiles (two waves per SIMD: one wave's softmax runs under the other's MFMAs).
+template <int D, int RT, bool WIN, int NHW>
+__global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p) {
     using G = Geo<D>;
+    constexpr int HPI = RT * NHW;  // heads per work item
     constexpr int NS = D / 16;     // contraction steps of K Q^T
     constexpr int NDT = D / 32;    // 32-wide slices of the head dimension in O^T
     constexpr int NVF = 2 * NDT;   // V^T fragments of one 32-key block
@@ -408,11 +417,16 @@ __global__ __launch_bounds__(256) void tree_attn_kernel(const AttnParams p) {
     __shared__ __attribute__((aligned(16))) char bufs[2 * G::BUFB];   // the two tile buffers
     __shared__ int2 ent_a[ENT_CAP];   // (key tile, bits) of the current item's plan entries base .. base + ENT_CAP - 1
     __shared__ int2 ent_b[ENT_CAP];   // first entries of the next item
-    __shared__ __attribute__((aligned(16))) char stage_all[4 * 32 * 144];
+    // output staging, one slice per wave; with eight waves at head dim 256 there is no room left for it and the slices lie in
+    // the tile buffer the item's last tile was computed from (free from the barrier after the tile loop until the next
+    // item's first tile step requests a tile into it, which comes after that step's barrier)
+    constexpr bool STAGE_IN_TILE = NHW == 2 && D == 256;
+    static_assert(!STAGE_IN_TILE || 8 * 32 * 144 <= G::BUFB, "the staging slices must fit a tile buffer");
+    __shared__ __attribute__((aligned(16))) char stage_all[STAGE_IN_TILE ? 16 : 4 * NHW * 32 * 144];
     __shared__ int s_next[2];         // item grabbed by thread 0 for the whole workgroup, double buffered
 
     const Lane<D> L(p);
-    char* stage = stage_all + L.w * 32 * 144;
+    char* const stage_own = stage_all + (STAGE_IN_TILE ? 0 : L.w * 32 * 144);
 
     // ---- work lists: start with the list of this workgroup's XCD, continue with the following ones
     unsigned xcc;
@@ -453,9 +467,9 @@ __global__ __launch_bounds__(256) void tree_attn_kernel(const AttnParams p) {
     auto item_hp = [](const int4& it) { return (int)((unsigned)it.z >> 20); };
 
     auto load_q = [&](const int4& it, bf16x8 (&dst)[RT][NS], int& a_q, int& p_q) __attribute__((always_inline)) {
-        const int tok = item_t(it) * SPINF_QTILE + 32 * L.w + L.m;
+        const int tok = item_t(it) * SPINF_QTILE + 32 * L.wr + L.m;
         const int tok_c = tok < p.n ? tok : p.n - 1;
-        const int h0 = item_hp(it) * RT;
+        const int h0 = item_hp(it) * HPI + L.wh * RT;
 #pragma unroll
         for (int rt = 0; rt < RT; rt++) {
             const __bf16* qp = p.q + (long)tok_c * p.q_tok + (long)(h0 + rt) * p.q_head + 8 * L.g;
@@ -467,7 +481,7 @@ __global__ __launch_bounds__(256) void tree_attn_kernel(const AttnParams p) {
     };
     auto load_ent = [&](const int4& it, int2* dst, const int from) __attribute__((always_inline)) {
         const int ne = item_ne(it);
-        if (from + (int)threadIdx.x < ne)
+        if ((int)threadIdx.x < ENT_CAP && from + (int)threadIdx.x < ne)
             dst[threadIdx.x] = make_int2(p.kv_idx[it.y + from + threadIdx.x], (int)p.kv_bits[it.y + from + threadIdx.x]);
     };
     auto reset_acc = [&]() __attribute__((always_inline)) {
@@ -549,7 +563,7 @@ __global__ __launch_bounds__(256) void tree_attn_kernel(const AttnParams p) {
         const char* kb = buf + L.k_lane;
         const char* vb = buf + G::KTILEB + L.v_lane;
         const int* meta = (const int*)(buf + G::KTILEB + G::VTILEB);
-        const int tok = item_t(cur) * SPINF_QTILE + 32 * L.w + L.m;
+        const int tok = item_t(cur) * SPINF_QTILE + 32 * L.wr + L.m;
         // one 32-key block on its own: K Q^T, softmax, P V in sequence
         auto one_block = [&](const int sub) __attribute__((always_inline)) {
             f32x16 sa[RT];
@@ -621,7 +635,7 @@ __global__ __launch_bounds__(256) void tree_attn_kernel(const AttnParams p) {
     if (cur_ok) {
         load_q(cur, qf, art_q, pos_q);
         load_ent(cur, ent_cur, 0);
-        issue_tile<D>(p, lds_addr(bufs), cur.w, item_hp(cur) * RT / p.group, L.w, L.lane, L.lane_k, L.lane_v);
+        issue_tile<D, 4 * NHW>(p, lds_addr(bufs), cur.w, item_hp(cur) * HPI / p.group, L.w, L.lane, L.lane_k, L.lane_v);
     }
     grab(1);
     int gslot = 1;      // slot of s_next that holds the item after `cur`
@@ -636,7 +650,7 @@ __global__ __launch_bounds__(256) void tree_attn_kernel(const AttnParams p) {
     int par = 0;
     while (cur_ok) {
         const int ne = item_ne(cur);
-        const int kvh = item_hp(cur) * RT / p.group;
+        const int kvh = item_hp(cur) * HPI / p.group;
         reset_acc();
         base = 0;
         pstage = 0;
@@ -664,13 +678,13 @@ __global__ __launch_bounds__(256) void tree_attn_kernel(const AttnParams p) {
                 __syncthreads();
             }
             if (i + 1 < ne) {
-                issue_tile<D>(p, oth, __builtin_amdgcn_readfirstlane(ent_cur[i + 1 - base].x), kvh, L.w, L.lane, L.lane_k, L.lane_v);
+                issue_tile<D, 4 * NHW>(p, oth, __builtin_amdgcn_readfirstlane(ent_cur[i + 1 - base].x), kvh, L.w, L.lane, L.lane_k, L.lane_v);
             } else if (nxt_ok) {
-                issue_tile<D>(p, oth, nxt.w, item_hp(nxt) * RT / p.group, L.w, L.lane, L.lane_k, L.lane_v);
+                issue_tile<D, 4 * NHW>(p, oth, nxt.w, item_hp(nxt) * HPI / p.group, L.w, L.lane, L.lane_k, L.lane_v);
                 pstage = pstage == 2 ? 3 : -1;   // -1: tile requested before the entries (one-tile items)
             }
             const int2 en = ent_cur[i - base];
-            compute_tile(buf, __builtin_amdgcn_readfirstlane(en.x), (unsigned)__builtin_amdgcn_readfirstlane(en.y) >> (2 * L.w));
+            compute_tile(buf, __builtin_amdgcn_readfirstlane(en.x), (unsigned)__builtin_amdgcn_readfirstlane(en.y) >> (2 * L.wr));
             TRACE_CLK(tc2);
             TRACE_ADD(9, tc2 - tc1);
         }
@@ -679,7 +693,9 @@ __global__ __launch_bounds__(256) void tree_attn_kernel(const AttnParams p) {
         if (__builtin_amdgcn_readfirstlane(__syncthreads_or(viol))) {
             if (threadIdx.x == 0) p.redo[atomicAdd(&p.counters[NLIST + 1], 1)] = cur_idx;
         } else {
-            store_rows<D, RT>(p, L, stage, o, l, item_t(cur), item_hp(cur) * RT);
+            // (the loop has already flipped par: the last tile came from buffer par ^ 1)
+            char* const stage = STAGE_IN_TILE ? bufs + (par ^ 1) * G::BUFB + L.w * 32 * 144 : stage_own;
+            store_rows<D, RT>(p, L, stage, o, l, item_t(cur), item_hp(cur) * HPI + L.wh * RT);
         }
         TRACE_CLK(tc4);
         TRACE_ADD(10, tc4 - tc3);
@@ -749,23 +765,38 @@ int device_state(DeviceState** out, long n_items) {
     return SPINF_OK;
 }
 
-template <int D, int RT, bool WIN>
+template <int D, int RT, bool WIN, int NHW = 1>
 int launch(const AttnParams& p, int blocks, hipStream_t stream) {
     using G = Geo<D>;
-    static_assert(2 * G::BUFB + 2 * ENT_CAP * 8 + 4 * 32 * 144 + 64 <= 160 * 1024, "LDS budget");
-    hipLaunchKernelGGL((tree_attn_kernel<D, RT, WIN>), dim3(blocks), dim3(256), 0, stream, p);
+    static_assert(2 * G::BUFB + 2 * ENT_CAP * 8 + ((NHW == 2 && D == 256) ? 16 : 4 * NHW * 32 * 144) + 64 <= 160 * 1024, "LDS budget");
+    hipLaunchKernelGGL((tree_attn_kernel<D, RT, WIN, NHW>), dim3(blocks), dim3(256 * NHW), 0, stream, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: launch: %s", hipGetErrorString(e));
     // the exact pass over whatever the fast pass handed on (normally nothing: its workgroups read a zero count and leave)
-    hipLaunchKernelGGL((tree_attn_exact_kernel<D, RT, WIN>), dim3(blocks < 64 ? blocks : 64), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((tree_attn_exact_kernel<D, RT, WIN, RT * NHW>), dim3(blocks < 64 ? blocks : 64), dim3(256), 0, stream, p);
     e = hipGetLastError();
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: launch (exact pass): %s", hipGetErrorString(e));
     return SPINF_OK;
 }
 
+// heads per wave (rt) and head sets across waves (nhw) for a head geometry; an item holds rt * nhw heads of one GQA group.
+//   variant 0: eight waves (nhw = 2) wherever a group has an even number of heads, else one head per item
+//   variant 1: one head per item, four waves
+//   variant 2: four waves with two heads each where their registers fit (head dim <= 128), else as 1
+void pick_kernel(int hq, int hkv, int d, int variant, int* rt, int* nhw) {
+    const bool pairs = (hq / hkv) % 2 == 0;
+    *rt = 1;
+    *nhw = 1;
+    if (variant == 0 && pairs) *nhw = 2;
+    if (variant == 2 && pairs && d <= 128) *rt = 2;
+}
+
 template <int D>
-int launch_d(const AttnParams& p, int rt, bool win, int blocks, hipStream_t s) {
-    if (rt == 2) return win ? launch<D, 2, true>(p, blocks, s) : launch<D, 2, false>(p, blocks, s);
+int launch_d(const AttnParams& p, int rt, int nhw, bool win, int blocks, hipStream_t s) {
+    if (nhw == 2) return win ? launch<D, 1, true, 2>(p, blocks, s) : launch<D, 1, false, 2>(p, blocks, s);
+    if constexpr (D <= 128) {
+        if (rt == 2) return win ? launch<D, 2, true>(p, blocks, s) : launch<D, 2, false>(p, blocks, s);
+    }
     return win ? launch<D, 1, true>(p, blocks, s) : launch<D, 1, false>(p, blocks, s);
 }
 
@@ -788,12 +819,9 @@ extern "C" int spinf_attn_exact_items(int64_t* total) {
 
 extern "C" int spinf_attn_heads_per_item(int32_t hq, int32_t hkv, int32_t d, int32_t variant) {
     if (hq <= 0 || hkv <= 0 || hq % hkv) return 0;
-    const int group = hq / hkv;
-    // two heads of a GQA group per wave halve the LDS and L2 traffic per MFMA; at head dim 256 their accumulators and
-    // query fragments (384 registers, 512 with the next item's queries) do not fit, so that size runs one head per wave
-    int rt = (group % 2 == 0 && d <= 128) ? 2 : 1;
-    if (variant == 1) rt = 1;
-    return rt;
+    int rt, nhw;
+    pick_kernel(hq, hkv, d, variant, &rt, &nhw);
+    return rt * nhw;
 }
 
 extern "C" int spinf_tree_attn_fwd(const spinf_attn_args* a, void* stream) {
@@ -805,11 +833,13 @@ extern "C" int spinf_tree_attn_fwd(const spinf_attn_args* a, void* stream) {
     if (a->hq <= 0 || a->hkv <= 0 || a->hq % a->hkv) return spinf_fail(SPINF_E_ARG, "tree_attn: hq %d not a multiple of hkv %d", a->hq, a->hkv);
     if (a->n > INT32_MAX / 2) return spinf_fail(SPINF_E_ARG, "tree_attn: stream too long");
     if (!(a->scale > 0.f)) return spinf_fail(SPINF_E_ARG, "tree_attn: scale must be positive");
-    const int rt = spinf_attn_heads_per_item(a->hq, a->hkv, a->d, a->variant);
+    int rt, nhw;
+    pick_kernel(a->hq, a->hkv, a->d, a->variant, &rt, &nhw);
+    const int hpi = rt * nhw;
     const int64_t nqt = (a->n + SPINF_QTILE - 1) / SPINF_QTILE;
-    if (a->n_items != nqt * (a->hq / rt))
+    if (a->n_items != nqt * (a->hq / hpi))
         return spinf_fail(SPINF_E_ARG, "tree_attn: schedule has %lld items, %lld query tiles x %d head groups need %lld", (long long)a->n_items,
-                          (long long)nqt, a->hq / rt, (long long)(nqt * (a->hq / rt)));
+                          (long long)nqt, a->hq / hpi, (long long)(nqt * (a->hq / hpi)));
     const int64_t strides[8] = {a->q_tok, a->q_head, a->k_tok, a->k_head, a->v_tok, a->v_head, a->o_tok, a->o_head};
     for (int i = 0; i < 8; i++)
         if (strides[i] % 8) return spinf_fail(SPINF_E_ARG, "tree_attn: strides must be multiples of 8 elements");
@@ -834,8 +864,8 @@ extern "C" int spinf_tree_attn_fwd(const spinf_attn_args* a, void* stream) {
     const bool win = p.window > 0;
     hipStream_t s = (hipStream_t)stream;
     switch (a->d) {
-        case 64: return launch_d<64>(p, rt, win, blocks, s);
-        case 128: return launch_d<128>(p, rt, win, blocks, s);
-        default: return launch_d<256>(p, rt, win, blocks, s);
+        case 64: return launch_d<64>(p, rt, nhw, win, blocks, s);
+        case 128: return launch_d<128>(p, rt, nhw, win, blocks, s);
+        default: return launch_d<256>(p, rt, nhw, win, blocks, s);
     }
 }

@@ -11,13 +11,16 @@ The op is a thin wrapper over spinf_tree_attn_fwd of libspinf_tree.so; it runs o
 from __future__ import annotations
 
 import ctypes as C
+import os
 
 import torch
 
 from . import _lib
 from .masks import TreeMask
 
-VARIANT = 0  # kernel tuning variant handed to the library (0 = its default choice); results do not depend on it
+# kernel tuning variant handed to the library (0 = its default choice, 1 = one head per work item, 2 = eight waves per
+# workgroup where two heads share an item); results do not depend on it
+VARIANT = int(os.environ.get("SPINF_ATTN_VARIANT", "0"))
 
 
 @torch.library.custom_op("spinf::tree_attn", mutates_args=())

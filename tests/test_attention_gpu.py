@@ -92,7 +92,9 @@ def test_wide_score_range_takes_the_exact_pass(dev, d, hq, hkv):
     assert float(np.abs(out2.float().cpu().numpy() - _oracle(q, k2, v, b, cfg.scale)).max()) <= TOL
 
 
-def test_c4_shape_two_level_tree(dev):
+@pytest.mark.parametrize("variant", [0, 1, 2])
+def test_c4_shape_two_level_tree(dev, variant):
+    """variant 0: eight waves, heads of a pair on different waves; 1: one head per item; 2: four waves with two heads each"""
     rng = np.random.default_rng(5)
     lens, parents = [], []
     for _ in range(4):
@@ -103,16 +105,17 @@ def test_c4_shape_two_level_tree(dev):
     trees = [synth._tree(rng, 700, lens, parents), synth._tree(rng, 130, lens[:7], parents[:7])]
     cfg = synth.AttnConfig("C4-small", 32, 16, 128, 128 ** -0.5, 0.5, None, trees)
     cfg.batches = synth.pack(trees)
-    _check(cfg, cfg.batches[0], dev)
+    _check(cfg, cfg.batches[0], dev, variant=variant)
 
 
+@pytest.mark.parametrize("variant", [0, 1])
 @pytest.mark.parametrize("window", [64, 200, 1024])
-def test_sliding_window(dev, window):
+def test_sliding_window(dev, window, variant):
     rng = np.random.default_rng(11)
     trees = [synth._tree(rng, 1500, rng.integers(4, 25, 12)), synth._tree(rng, 90, [7, 9])]
     cfg = synth.AttnConfig("C3-small", 16, 8, 256, 1.0 / 16, 0.5, window, trees)
     cfg.batches = synth.pack(trees)
-    _check(cfg, cfg.batches[0], dev, window=window)
+    _check(cfg, cfg.batches[0], dev, window=window, variant=variant)
 
 
 def test_odd_group_and_mha(dev):
