@@ -212,6 +212,15 @@ __device__ __forceinline__ void apply_mask(f32x16 (&s_acc)[RT], const int* meta,
     }
 }
 
+// The lane index, recomputed on the spot (two instructions).  For the code between two items (output rows, the next item's
+// queries): a lane-dependent value kept in a register across the tile loop is spilled at head dim 256, and its reload is a
+// memory operation whose wait also waits for every output store issued before it, one store at a time.
+__device__ __forceinline__ int fresh_lane_id() {
+    int lane;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane));
+    return lane;
+}
+
 // normalise O^T and store it as rows: each wave stages 32 rows x 64 head dims at a time in its own LDS slice (144-byte
 // rows) and writes them out as 16-byte pieces, 8 lanes per 128-byte row segment
 template <int D, int RT>
@@ -220,6 +229,7 @@ __device__ __forceinline__ void store_rows(const AttnParams& p, const Lane<D>& L
     constexpr int NDT = D / 32;
     constexpr int SROW = 128 + 16;
     const int tok0 = t * SPINF_QTILE + 32 * L.wr;
+    const int lane = fresh_lane_id(), m = lane & 31, g = lane >> 5;
 #pragma unroll
     for (int rt = 0; rt < RT; rt++) {
         const float inv = 1.0f / lane32_sum(l[rt]);
@@ -233,11 +243,11 @@ __device__ __forceinline__ void store_rows(const AttnParams& p, const Lane<D>& L
                     bf16x4 r;
 #pragma unroll
                     for (int jj = 0; jj < 4; jj++) r[jj] = (__bf16)(o[rt][2 * qd + dd][4 * i4 + jj] * inv);
-                    *(bf16x4*)(stage + L.m * SROW + (32 * dd + 8 * i4 + 4 * L.g) * 2) = r;
+                    *(bf16x4*)(stage + m * SROW + (32 * dd + 8 * i4 + 4 * g) * 2) = r;
                 }
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                const int c = j * 64 + L.lane, row = c >> 3, col = c & 7;
+                const int c = j * 64 + lane, row = c >> 3, col = c & 7;
                 const bf16x8 val = *(const bf16x8*)(stage + row * SROW + col * 16);
                 if (tok0 + row < p.n) *(bf16x8*)(ob + (long)(tok0 + row) * p.o_tok + 64 * qd + col * 8) = val;
             }
@@ -409,7 +419,9 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
     constexpr int NS = D / 16;     // contraction steps of K Q^T
     constexpr int NDT = D / 32;    // 32-wide slices of the head dimension in O^T
     constexpr int NVF = 2 * NDT;   // V^T fragments of one 32-key block
-    constexpr int PFD = D >= 256 ? 4 : 8;   // fragment read-ahead depth: the vector register file (256) is the tight one at head dim 256
+    // fragment read-ahead depth: the register file is the tight one at head dim 256 (4 with one wave per SIMD, 3 with two:
+    // measured 0.374 / 0.351 / 0.343 / 0.368 ms on the 24-content pass for depths 4 / 2 / 3 / 1); no effect at 128
+    constexpr int PFD = D >= 256 ? (NHW == 2 ? 3 : 4) : 8;
     constexpr int PF = NS < PFD ? NS : PFD;     // K fragments read ahead of the MFMAs
     constexpr int VPF = NVF < PFD ? NVF : PFD;  // V^T fragments read ahead
     constexpr int EK = 16 / NS;    // softmax elements folded into one K Q^T step
@@ -467,12 +479,13 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
     auto item_hp = [](const int4& it) { return (int)((unsigned)it.z >> 20); };
 
     auto load_q = [&](const int4& it, bf16x8 (&dst)[RT][NS], int& a_q, int& p_q) __attribute__((always_inline)) {
-        const int tok = item_t(it) * SPINF_QTILE + 32 * L.wr + L.m;
+        const int lane = fresh_lane_id();
+        const int tok = item_t(it) * SPINF_QTILE + 32 * L.wr + (lane & 31);
         const int tok_c = tok < p.n ? tok : p.n - 1;
         const int h0 = item_hp(it) * HPI + L.wh * RT;
 #pragma unroll
         for (int rt = 0; rt < RT; rt++) {
-            const __bf16* qp = p.q + (long)tok_c * p.q_tok + (long)(h0 + rt) * p.q_head + 8 * L.g;
+            const __bf16* qp = p.q + (long)tok_c * p.q_tok + (long)(h0 + rt) * p.q_head + 8 * (lane >> 5);
 #pragma unroll
             for (int s = 0; s < NS; s++) dst[rt][s] = *(const bf16x8*)(qp + 16 * s);
         }
@@ -690,7 +703,10 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
         }
         // ---- item finished: output (or hand the item to the exact pass), switch to the next item
         TRACE_CLK(tc3);
-        if (__builtin_amdgcn_readfirstlane(__syncthreads_or(viol))) {
+        const int any_viol = __builtin_amdgcn_readfirstlane(__syncthreads_or(viol));
+        TRACE_CLK(tc3b);
+        TRACE_ADD(12, tc3b - tc3);
+        if (any_viol) {
             if (threadIdx.x == 0) p.redo[atomicAdd(&p.counters[NLIST + 1], 1)] = cur_idx;
         } else {
             // (the loop has already flipped par: the last tile came from buffer par ^ 1)
