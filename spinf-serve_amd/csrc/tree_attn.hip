@@ -3,9 +3,11 @@
 // Replaces the flex_attention call of spinf_serve/models/gemma4.py:107-118 and spinf_serve/models/qwen35/qwen.py:614,620;
 // the per-element visibility test is the predicate of spinf_serve/scorer.py:173-177.
 //
-// Work decomposition.  A work item = one 128-token query tile x RT query heads of one GQA group; 4 waves, wave w owns
-// tokens 32w..32w+31 of the tile for all RT heads, so a K or V fragment read from LDS feeds RT MFMAs and the mask of a
-// 32x32 block is evaluated once for all RT heads.  Scores are computed transposed, S^T = K Q^T, with
+// Work decomposition.  A work item = one 128-token query tile x the heads of one GQA group that share it: RT heads per
+// wave times NHW head sets across waves.  The default for an even group is RT = 1, NHW = 2: eight waves, wave w owns
+// tokens 32(w%4)..+31 of head w/4, two waves per SIMD on the same K / V tiles, so that one wave's softmax runs under
+// the other's MFMAs.  (NHW = 1 are the four-wave kernels: one head per wave for odd groups, or RT = 2 heads per wave at
+// head dim <= 128, where a K or V fragment read from LDS feeds two MFMAs.)  Scores are computed transposed, S^T = K Q^T, with
 // v_mfma_f32_32x32x16_bf16: a lane then owns ONE query row (column lane%32 of the 32x32 result) and 16 of the 32 keys,
 // so the softmax row reductions are in-lane plus one exchange with lane^32.  O^T = V^T P^T reuses the score registers
 // as the B operand without any shuffle; V^T fragments come from row-major V in LDS through ds_read_b64_tr_b16.
@@ -424,8 +426,6 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
     constexpr int PFD = D >= 256 ? (NHW == 2 ? 3 : 4) : 8;
     constexpr int PF = NS < PFD ? NS : PFD;     // K fragments read ahead of the MFMAs
     constexpr int VPF = NVF < PFD ? NVF : PFD;  // V^T fragments read ahead
-    constexpr int EK = 16 / NS;    // softmax elements folded into one K Q^T step
-    constexpr int EV = (16 + NVF - 1) / NVF;   // ... into one P V step
     __shared__ __attribute__((aligned(16))) char bufs[2 * G::BUFB];   // the two tile buffers
     __shared__ int2 ent_a[ENT_CAP];   // (key tile, bits) of the current item's plan entries base .. base + ENT_CAP - 1
     __shared__ int2 ent_b[ENT_CAP];   // first entries of the next item
@@ -527,8 +527,8 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
         sum += pr;
         pb[i2 >> 3][i2 & 7] = (__bf16)pr;
     };
-    // S^T = K Q^T for one 32-key block; `shadow(s)` is vector-ALU work of another block slotted in after step s
-    auto qk_phase = [&](const char* krow, f32x16 (&s_acc)[RT], auto shadow) __attribute__((always_inline)) {
+    // S^T = K Q^T for one 32-key block
+    auto qk_phase = [&](const char* krow, f32x16 (&s_acc)[RT]) __attribute__((always_inline)) {
 #pragma unroll
         for (int rt = 0; rt < RT; rt++)
 #pragma unroll
@@ -543,12 +543,11 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
             for (int rt = 0; rt < RT; rt++)
                 s_acc[rt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[s % PF], qf[rt][s], s_acc[rt], 0, 0, 0);
             if (s + PF < NS) kf[s % PF] = *(const bf16x8*)(krow + 32 * (s + PF));
-            shadow(s);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
     // O^T += V^T P^T for one 32-key block
-    auto pv_phase = [&](const char* vrow, const bf16x8 (&pb)[RT][2], auto shadow) __attribute__((always_inline)) {
+    auto pv_phase = [&](const char* vrow, const bf16x8 (&pb)[RT][2]) __attribute__((always_inline)) {
         s16x4 vlo[VPF], vhi[VPF];
         auto vload = [&](const int f, const int slot) __attribute__((always_inline)) {
             const char* vp = vrow + G::v_off(16 * (f / NDT)) + 64 * (f % NDT);
@@ -565,11 +564,9 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
             for (int rt = 0; rt < RT; rt++)
                 o[rt][f % NDT] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[rt][f / NDT], o[rt][f % NDT], 0, 0, 0);
             if (f + VPF < NVF) vload(f + VPF, f % VPF);
-            shadow(f);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
-    auto no_shadow = [](const int) __attribute__((always_inline)) {};
     auto compute_tile = [&](const char* buf, const int kt, const unsigned bits) __attribute__((always_inline)) {
         const bool a0 = bits & 1u, a1 = bits & 2u;
         if (!a0 && !a1) return;   // wave-uniform: no row of this wave sees a key of the tile
@@ -581,7 +578,7 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
         auto one_block = [&](const int sub) __attribute__((always_inline)) {
             f32x16 sa[RT];
             bf16x8 pa[RT][2];
-            qk_phase(kb + sub * G::SUBB, sa, no_shadow);
+            qk_phase(kb + sub * G::SUBB, sa);
             if ((bits >> (8 + sub)) & 1u) apply_mask<RT, WIN>(sa, meta, kt, sub, L.g, tok, art_q, pos_q, p.window);
 #pragma unroll
             for (int rt = 0; rt < RT; rt++) {
@@ -591,50 +588,12 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
                 for (int i2 = 0; i2 < 16; i2++) sm_elem(sa[rt], i2, ms, sum, pa[rt]);
                 l[rt] += sum;
             }
-            pv_phase(vb + sub * G::SUBB, pa, no_shadow);
+            pv_phase(vb + sub * G::SUBB, pa);
         };
-#ifndef SPINF_FUSE   // measured faster than the variant below, which hides each softmax behind the other block's MFMAs
+        // (hiding each block's softmax behind the other block's MFMAs inside one wave was measured slower than plain
+        // sequence: the second wave on the SIMD does that job)
         if (a0) one_block(0);
         if (a1) one_block(1);
-        return;
-#endif
-        if (a0 && a1) {
-            // both blocks: K Q^T(0) | K Q^T(1) with softmax(0) in its shadow | P V(0) with softmax(1) in its shadow | P V(1)
-            f32x16 sa[RT], sb[RT];
-            bf16x8 pa[RT][2], pb[RT][2];
-            float ms[RT], sum[RT];
-            qk_phase(kb, sa, no_shadow);
-            if ((bits >> 8) & 1u) apply_mask<RT, WIN>(sa, meta, kt, 0, L.g, tok, art_q, pos_q, p.window);
-            qk_phase(kb + G::SUBB, sb, [&](const int s) __attribute__((always_inline)) {
-                if (s == 0) {
-#pragma unroll
-                    for (int rt = 0; rt < RT; rt++) { ms[rt] = sm_head(rt, sa[rt]); sum[rt] = 0.f; }
-                }
-#pragma unroll
-                for (int rt = 0; rt < RT; rt++)
-#pragma unroll
-                    for (int e = 0; e < EK; e++) sm_elem(sa[rt], s * EK + e, ms[rt], sum[rt], pa[rt]);
-            });
-#pragma unroll
-            for (int rt = 0; rt < RT; rt++) l[rt] += sum[rt];
-            if ((bits >> 9) & 1u) apply_mask<RT, WIN>(sb, meta, kt, 1, L.g, tok, art_q, pos_q, p.window);
-            pv_phase(vb, pa, [&](const int f) __attribute__((always_inline)) {
-                if (f == 0) {
-#pragma unroll
-                    for (int rt = 0; rt < RT; rt++) { ms[rt] = sm_head(rt, sb[rt]); sum[rt] = 0.f; }
-                }
-#pragma unroll
-                for (int rt = 0; rt < RT; rt++)
-#pragma unroll
-                    for (int e = 0; e < EV; e++)
-                        if (f * EV + e < 16) sm_elem(sb[rt], f * EV + e, ms[rt], sum[rt], pb[rt]);
-            });
-#pragma unroll
-            for (int rt = 0; rt < RT; rt++) l[rt] += sum[rt];
-            pv_phase(vb + G::SUBB, pb, no_shadow);
-        } else {
-            one_block(a0 ? 0 : 1);
-        }
     };
 
     // ---- prologue: first item, its queries, entries and first tile; the second item is grabbed right away
