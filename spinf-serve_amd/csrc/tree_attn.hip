@@ -607,7 +607,7 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
     if (cur_ok) {
         load_q(cur, qf, art_q, pos_q);
         load_ent(cur, ent_cur, 0);
-        issue_tile<D, 4 * NHW>(p, lds_addr(bufs), cur.w, item_hp(cur) * HPI / p.group, L.w, L.lane, L.lane_k, L.lane_v);
+        if (L.wh == 0) issue_tile<D, 4>(p, lds_addr(bufs), cur.w, item_hp(cur) * HPI / p.group, L.w, L.lane, L.lane_k, L.lane_v);
     }
     grab(1);
     int gslot = 1;      // slot of s_next that holds the item after `cur`
@@ -615,6 +615,8 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
     int base = 0;       // first plan entry held in ent_cur
     int pstage = 0;     // next-item prefetch: 0 nothing, 1 descriptor known, 2 entries requested, 3 first tile requested
 
+    // The tile DMA is issued by waves 0..3 alone: with eight waves they are the older wave of each SIMD, win the issue
+    // arbitration and finish a tile step first, so the younger waves, which set the pace, are spared that work.
     // Item loop around a tile loop (two real loop levels on purpose: the accumulators are touched by the vector ALU only
     // outside the tile loop, so inside it they stay in the MFMA accumulator registers).
     // One tile step = one key tile of the current item from buffer `par`, the next tile (of this item or of the next one)
@@ -650,9 +652,9 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
                 __syncthreads();
             }
             if (i + 1 < ne) {
-                issue_tile<D, 4 * NHW>(p, oth, __builtin_amdgcn_readfirstlane(ent_cur[i + 1 - base].x), kvh, L.w, L.lane, L.lane_k, L.lane_v);
+                if (L.wh == 0) issue_tile<D, 4>(p, oth, __builtin_amdgcn_readfirstlane(ent_cur[i + 1 - base].x), kvh, L.w, L.lane, L.lane_k, L.lane_v);
             } else if (nxt_ok) {
-                issue_tile<D, 4 * NHW>(p, oth, nxt.w, item_hp(nxt) * HPI / p.group, L.w, L.lane, L.lane_k, L.lane_v);
+                if (L.wh == 0) issue_tile<D, 4>(p, oth, nxt.w, item_hp(nxt) * HPI / p.group, L.w, L.lane, L.lane_k, L.lane_v);
                 pstage = pstage == 2 ? 3 : -1;   // -1: tile requested before the entries (one-tile items)
             }
             const int2 en = ent_cur[i - base];
