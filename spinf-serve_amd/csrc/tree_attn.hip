@@ -5,7 +5,7 @@
 //
 // Work decomposition.  A work item = one 128-token query tile x the heads of one GQA group that share it: RT heads per
 // wave times NHW head sets across waves.  The default for an even group is RT = 1, NHW = 2: eight waves, wave w owns
-// tokens 32(w%4)..+31 of head w/4, two waves per SIMD on the same K / V tiles, so that one wave's softmax runs under
+// 32 tokens of head w/4 (row group w%4 for the first head, 3 - w%4 for the second), two waves per SIMD on the same K / V tiles, so that one wave's softmax runs under
 // the other's MFMAs.  (NHW = 1 are the four-wave kernels: one head per wave for odd groups, or RT = 2 heads per wave at
 // head dim <= 128, where a K or V fragment read from LDS feeds two MFMAs.)  Scores are computed transposed, S^T = K Q^T, with
 // v_mfma_f32_32x32x16_bf16: a lane then owns ONE query row (column lane%32 of the 32x32 result) and 16 of the 32 keys,
@@ -167,7 +167,7 @@ template <int D>
 struct Lane {
     using G = Geo<D>;
     int lane, m, g, w;
-    int wr, wh;                  // row group (tokens 32 wr ..) and head slot of this wave: w = 4 wh + wr
+    int wr, wh;                  // row group (tokens 32 wr ..) and head set of this wave
     int k_lane, v_lane;          // byte offsets of this lane's K fragment row / V^T fragment address inside a tile
     unsigned lane_k, lane_v;     // per-lane part of the DMA source addresses
     __device__ __forceinline__ Lane(const AttnParams& p) {
@@ -175,8 +175,10 @@ struct Lane {
         m = lane & 31;
         g = lane >> 5;
         w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-        wr = w & 3;
         wh = w >> 2;
+        // waves w and w + 4 share a SIMD: the second head set takes the row groups in reverse order, so that a SIMD's two waves
+        // together see about the same number of key blocks near the diagonal (row group k sees k + 1 of 4, or only its own branch)
+        wr = wh ? 3 - (w & 3) : (w & 3);
         // K fragment: row m of the 32-key block, 16-byte chunk g of each 32-byte step.  V^T fragment
         // (ds_read_b64_tr_b16): inside its 16-lane group a lane supplies the address of key row 4g + tr_j, head dims
         // 16 tr_mb + 4 tr_a .. +3 of the 32-wide slice, and receives head dim lane%32 of 4 consecutive keys.
