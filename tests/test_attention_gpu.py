@@ -119,10 +119,11 @@ def test_sliding_window(dev, window, variant):
 
 
 def test_odd_group_and_mha(dev):
+    """groups of 3 and 1 heads run one head per item; groups of 4 and 8 are split into pairs that share an item"""
     rng = np.random.default_rng(2)
     trees = [synth._tree(rng, 200, [9, 17, 4])]
-    for hq, hkv in ((6, 2), (4, 4), (3, 1)):
-        cfg = synth.AttnConfig("odd", hq, hkv, 128, 128 ** -0.5, 1.0, None, trees)
+    for hq, hkv, d in ((6, 2, 128), (4, 4, 128), (3, 1, 128), (8, 2, 128), (8, 1, 64), (4, 1, 256), (3, 3, 256)):
+        cfg = synth.AttnConfig("odd", hq, hkv, d, d ** -0.5, 1.0, None, trees)
         cfg.batches = synth.pack(trees)
         _check(cfg, cfg.batches[0], dev)
 
