@@ -51,6 +51,41 @@ def test_c_abi_rejects_bad_arguments(lib):
     lib.spinf_tileplan_free(out)
 
 
+def test_heads_per_item_follows_the_kernel_choice(lib):
+    """even GQA groups share an item between the heads of a pair (variant 0: across waves; variant 2: inside a wave, head
+    dim <= 128 only); odd groups, MHA and variant 1 run one head per item; the schedule must be built for this count"""
+    f = lib.spinf_attn_heads_per_item
+    for d in (64, 128, 256):
+        assert f(16, 8, d, 0) == 2 and f(8, 2, d, 0) == 2 and f(8, 1, d, 0) == 2
+        assert f(6, 2, d, 0) == 1 and f(4, 4, d, 0) == 1 and f(3, 1, d, 0) == 1
+        assert f(16, 8, d, 1) == 1
+        assert f(16, 8, d, 2) == (2 if d <= 128 else 1)
+    assert f(0, 1, 128, 0) == 0 and f(5, 2, 128, 0) == 0      # not a head geometry
+
+
+def test_gdn_argument_checks_come_before_any_launch(lib):
+    """spinf_gdn_fwd validates shapes, strides and alignment on the host and reports what it rejects"""
+    from spinf_serve_amd import _lib as L
+
+    def args(**kw):
+        a = L.GdnArgs()
+        for name in ("q", "k", "v", "g", "beta", "o", "cu"):
+            setattr(a, name, 0x1000)      # never dereferenced: every case below is rejected first
+        a.q_tok, a.v_tok, a.g_tok, a.o_tok = 2048, 4096, 32, 4096
+        a.h, a.hv, a.dk, a.dv, a.scale = 16, 32, 128, 128, 0.088
+        a.n_seg, a.max_len, a.mode = 1, 0, 0
+        for k_, v_ in kw.items():
+            setattr(a, k_, v_)
+        return a
+
+    for kw, word in ((dict(dk=64), b"key head dim"), (dict(dv=48), b"value head dim"), (dict(hv=30), b"multiple of h"),
+                     (dict(q_tok=2044), b"q/k row stride"), (dict(v_tok=4100), b"v/o row stride"), (dict(o_tok=1 << 31), b"below 2^31"),
+                     (dict(mode=7), b"unknown mode")):
+        assert lib.spinf_gdn_fwd(ctypes.byref(args(**kw)), None) == -1, kw
+        assert word in lib.spinf_last_error(), (kw, lib.spinf_last_error())
+    assert lib.spinf_gdn_fwd(ctypes.byref(args(n_seg=0)), None) == 0      # nothing to do is not an error
+
+
 def test_missing_library_fails_loudly(monkeypatch):
     from spinf_serve_amd import _lib
 
