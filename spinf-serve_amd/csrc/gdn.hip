@@ -219,7 +219,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void
     }
 }
 
-int gdn_wy_launch(const GdnParams& p, int tokens_per_chunk, hipStream_t stream);   // gdn_chunk.hip
+int gdn_wy_launch(GdnParams p, bool pairs, hipStream_t stream);   // gdn_chunk.hip
 
 extern "C" int spinf_gdn_fwd(const spinf_gdn_args* a, void* stream) {
     if (!a) return spinf_fail(SPINF_E_ARG, "gdn: null args");
@@ -243,10 +243,11 @@ extern "C" int spinf_gdn_fwd(const spinf_gdn_args* a, void* stream) {
     p.h = a->h; p.hv = a->hv; p.dk = a->dk; p.dv = a->dv; p.scale = a->scale;
     p.cu = (const long*)a->cu; p.idx = (const long*)a->idx; p.n_seg = a->n_seg;
     p.h0 = a->h0; p.h0_idx = (const long*)a->h0_idx; p.ht = a->ht; p.ht_idx = (const long*)a->ht_idx;
+    p.run = 1;
     hipStream_t s = (hipStream_t)stream;
-    if (a->mode == 1) return gdn_wy_launch(p, 32, s);
+    if (a->mode == 1) return gdn_wy_launch(p, false, s);
     if (a->mode != 0) return spinf_fail(SPINF_E_ARG, "gdn: unknown mode %d", a->mode);
-    if (a->dv == 128) return gdn_wy_launch(p, 16, s);   // the workgroup kernel shares the per-head work of the four 32-column waves
+    if (a->dv == 128) return gdn_wy_launch(p, true, s);   // the workgroup kernel shares the per-head work of the four 32-column waves
     const long blocks = a->n_seg * a->hv * (a->dv / 32);
     if (blocks > INT32_MAX) return spinf_fail(SPINF_E_ARG, "gdn: too many segments");
     hipLaunchKernelGGL(gdn_short_kernel, dim3((unsigned)blocks), dim3(64), 0, s, p);

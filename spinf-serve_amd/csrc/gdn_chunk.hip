@@ -31,7 +31,10 @@ using namespace gdn_tiles;
 __device__ long g_gdn_trace[16];
 extern "C" int spinf_debug_gdn_trace(long* out) { return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_gdn_trace), sizeof(long) * 16, 0, hipMemcpyDeviceToHost); }
 #define GT_CLK(v) const long v = clock64()
-#define GT_ADD(slot, val) do { if (NT == 2 && threadIdx.x == SPINF_TRACE_THREAD && blockIdx.x == 7) g_gdn_trace[slot] += (val); } while (0)
+#ifndef SPINF_TRACE_PAIRS
+#define SPINF_TRACE_PAIRS false
+#endif
+#define GT_ADD(slot, val) do { if (NT == 2 && PAIRS == SPINF_TRACE_PAIRS && threadIdx.x == SPINF_TRACE_THREAD && blockIdx.x == 7) g_gdn_trace[slot] += (val); } while (0)
 #else
 #define GT_CLK(v) do { } while (0)
 #define GT_ADD(slot, val) do { } while (0)
@@ -74,8 +77,9 @@ struct Tok<1> {
 
 }  // namespace
 
-template <int NT>
+template <int NT, bool PAIRS>
 __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
+    static_assert(!PAIRS || NT == 2, "a pair of segments takes the two token tiles of a 32-token chunk");
     constexpr int CH = 16 * NT;
     constexpr int LO = CH;                          // row stride (elements) of a wave's transposed output tile [32 values][CH tokens]
     constexpr int NTILES = NT * (NT + 1) / 2;       // 16 x 16 tiles of A / P on or below the diagonal
@@ -102,11 +106,62 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
     // same q and k rows: they get launch slots 8 apart, i.e. the same XCD at about the same time, so the second read hits L2.
     long slot = blockIdx.x;
     if (p.hv == 2 * p.h && gridDim.x % 16 == 0) slot = (slot / 16) * 16 + (slot % 8) * 2 + (slot % 16) / 8;
-    const long seg = slot / p.hv;
     const int hv = (int)(slot % p.hv);
     const int hk = hv / (p.hv / p.h);
-    const long bos = p.cu[seg], eos = p.cu[seg + 1];
-    const int T = (int)(eos - bos);
+    // Pairs (the recurrent entry point).  Consecutive segments that start from the same stored state, have at most 16 tokens
+    // and leave no state behind (the leaves that fork from one trunk) never change the state registers: they form a run that
+    // is taken TWO segments per chunk (one per 16-token tile: A, P and T are then block diagonal, the tiles do not see each
+    // other), with the state loaded once and the row prefetch running from one pair into the next.  The instructions of a
+    // chunk hardly depend on how many of its rows are in use, so this halves the work per leaf.  A workgroup owns a group of
+    // p.run consecutive segments (launching one workgroup per leaf would cost more in dispatch than the leaves in compute)
+    // and walks it run by run; any segment that is not such a leaf is a run of its own, walked chunk by chunk.
+    const long group = PAIRS ? p.run : 1;
+    const long s_begin = (slot / p.hv) * group, s_end = PAIRS ? min(p.n_seg, s_begin + group) : s_begin + 1;
+    // The group's segments are described once, by one thread each: first call row, length, and whether the segment continues
+    // the run of the one before it (both leaves of the same state); the bit mask of the latter gives the run lengths.
+    __shared__ long g_base[16];
+    __shared__ int g_len[16];
+    __shared__ unsigned g_follows;
+    if (PAIRS) {
+        if (tid < 16) {
+            const long s_ = s_begin + tid;
+            bool fol = false;
+            if (s_ < s_end) {
+                const long b0 = p.cu[s_], b1 = p.cu[s_ + 1];
+                g_base[tid] = b0;
+                g_len[tid] = (int)(b1 - b0);
+                if (tid > 0) {
+                    const bool keeps = p.ht != nullptr && p.ht_idx != nullptr && (p.ht_idx[s_] >= 0 || p.ht_idx[s_ - 1] >= 0);
+                    const bool same = (p.h0 != nullptr && p.h0_idx != nullptr) ? p.h0_idx[s_] == p.h0_idx[s_ - 1] : true;
+                    fol = b1 - b0 <= 16 && b0 - p.cu[s_ - 1] <= 16 && !keeps && same;
+                }
+            }
+            const unsigned long m = __builtin_amdgcn_ballot_w64(fol);     // lanes 0..15 of wave 0
+            if (tid == 0) g_follows = (unsigned)m;
+        }
+        lds_barrier();
+    }
+    const unsigned fol_mask = PAIRS ? (unsigned)__builtin_amdgcn_readfirstlane((int)g_follows) : 0u;
+  for (long seg = s_begin; seg < s_end; seg++) {
+    const int sl = (int)(seg - s_begin);
+    if (PAIRS && ((fol_mask >> sl) & 1u)) continue;     // taken by the run it belongs to
+    // the run: this segment and the followers right after it
+    const int run_len = PAIRS ? 1 + __builtin_ctz(~(fol_mask >> (sl + 1)) | (1u << 16)) : 1;
+    const bool run_mode = PAIRS && run_len > 1;
+    const long bos = PAIRS ? g_base[sl] : p.cu[seg];
+    const int T = PAIRS ? g_len[sl] : (int)(p.cu[seg + 1] - bos);
+    const int n_chunks = run_mode ? (run_len + 1) / 2 : (T + CH - 1) / CH;
+    // token tile cc of chunk j: its first call row and its number of rows (0: there is no such tile)
+    auto tile_of = [&](int j, int cc, long& base, int& len) __attribute__((always_inline)) {
+        if (run_mode) {
+            const bool there = 2 * j + cc < run_len;
+            base = there ? g_base[sl + 2 * j + cc] : 0;
+            len = there ? g_len[sl + 2 * j + cc] : 0;
+        } else {
+            base = bos + (long)j * CH + 16 * cc;
+            len = max(0, min(16, T - j * CH - 16 * cc));
+        }
+    };
     __bf16* Ow = Vs + w * 32 * LO;
 
     // ---- state: S[kt][vt][r] = S[16 kt + 4 q4 + r][32 w + 16 vt + c]
@@ -141,21 +196,26 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
     // Only the low half of an index is loaded: the register of an unused high half would be handed out again at once, and
     // whoever writes it first has to wait for the load (and with it for every load in flight).
     const int* idx_lo = (const int*)p.idx;
-    auto fetch_rows = [&](const int c0) __attribute__((always_inline)) {
-        const int L = min(CH, T - c0);      // <= 0: there is no such chunk
+    auto fetch_rows = [&](const int j) __attribute__((always_inline)) {
+        long base[NT];
+        int len[NT];
 #pragma unroll
         for (int cc = 0; cc < NT; cc++) {
-            const int row = (tid >> 4) + 16 * cc;
+            tile_of(j, cc, base[cc], len[cc]);
             ra[cc] = -1;
-            if (row < L) {
-                const long t = bos + c0 + row;
+            if ((tid >> 4) < len[cc]) {       // this thread's row of tile cc
+                const long t = base[cc] + (tid >> 4);
                 ra[cc] = p.idx ? idx_lo[2 * t] : (int)t;
             }
         }
         rb = -1;
-        if (tid < CH && tid < L) {
-            const long t = bos + c0 + tid;
-            rb = p.idx ? idx_lo[2 * t] : (int)t;
+        if (tid < CH) {                       // chunk row tid = row tid % 16 of tile tid / 16
+            const bool hi = NT == 2 && tid >= 16;
+            const int r = tid & 15;
+            if (r < (hi ? len[NT - 1] : len[0])) {
+                const long t = (hi ? base[NT - 1] : base[0]) + r;
+                rb = p.idx ? idx_lo[2 * t] : (int)t;
+            }
         }
     };
     auto fetch_data = [&]() __attribute__((always_inline)) {
@@ -180,16 +240,16 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
     };
     fetch_rows(0);
     fetch_data();
-    fetch_rows(CH);
+    fetch_rows(1);
 
-    for (int c0 = 0; c0 < T; c0 += CH) {
-        const int L = min(CH, T - c0);
+    for (int j = 0; j < n_chunks; j++) {
         GT_CLK(g0);
         lds_barrier();   // every wave is done with the previous chunk's tiles
         // ---- stage the chunk from the prefetch registers (rows >= L are zero): cumulative g, beta, stream rows, K / Q / V
         if (tid < CH) {
             float x = row_prefix_sum(pg);
-            if (NT == 2) x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x142, 0xa, 0xf, false));  // row_bcast:15 -> lanes 16..31
+            // row_bcast:15 -> lanes 16..31 (not for a pair: the second tile is another segment)
+            if (NT == 2 && !run_mode) x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x142, 0xa, 0xf, false));
             Gs[tid] = x;
             Bs[tid] = (float)pbeta;
             Rs[tid] = pr32;
@@ -223,6 +283,7 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
                 qk = mfma32(kj, qi, qk);
             }
             const int i = 16 * it + c;
+            const bool apart = run_mode && jt != it;     // a pair's tiles are different segments
             const float Gi = Gs[i], bi = Bs[i];
             const f32x4 Gj = *(const f32x4*)(Gs + 16 * jt + 4 * q4);
             f32x4 a4;
@@ -231,8 +292,8 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
             for (int r = 0; r < 4; r++) {
                 const int j = 16 * jt + 4 * q4 + r;
                 const float d = __expf(Gi - Gj[r]);
-                a4[r] = j < i ? -bi * kk[r] * d : 0.f;
-                p4[r] = (__bf16)(j <= i ? p.scale * qk[r] * d : 0.f);
+                a4[r] = (j < i && !apart) ? -bi * kk[r] * d : 0.f;
+                p4[r] = (__bf16)((j <= i && !apart) ? p.scale * qk[r] * d : 0.f);
             }
             *(f32x4*)(As + i * LA + 16 * jt + 4 * q4) = a4;
             *(bf16x4*)(Ps + i * LP + 16 * jt + 4 * q4) = p4;
@@ -353,8 +414,8 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
         }
         GT_CLK(g5);
         // the next chunk's rows are requested here, where few registers are live; they arrive during the state update
-        fetch_data();          // chunk c0 + CH, whose rows are known since the previous chunk
-        fetch_rows(c0 + 2 * CH);
+        fetch_data();          // chunk j + 1, whose rows are known since the previous chunk
+        fetch_rows(j + 2);
         GT_CLK(g5a);
         // ---- O[i][v] = s e^{G_i} (Q S)[i][v] + sum_j P[i][j] V'[j][v], rows i = 16 it + 4 q4 + r; through LDS for 16-byte stores
         f32x4 Gj[NT];
@@ -388,11 +449,12 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
             const __bf16* op = Ow + (8 * q4 + (c >> 2)) * LO + 16 * it + 4 * (c & 3);
             const bf16x4 lo = __builtin_bit_cast(bf16x4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)op));
             const bf16x4 hi = __builtin_bit_cast(bf16x4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(op + 4 * LO)));
-            if (row < L) *(bf16x8*)(p.o + row_offset(Rs[row], p.o_tok) + hv * VD + 32 * w + 8 * q4) = join(lo, hi);
+            const int orow = Rs[row];      // -1: no such row in this chunk
+            if (orow >= 0) *(bf16x8*)(p.o + row_offset(orow, p.o_tok) + hv * VD + 32 * w + 8 * q4) = join(lo, hi);
         }
         GT_CLK(g6);
         // ---- S[k][v] = e^{G_L} S[k][v] + sum_j K[j][k] (V' e^{G_L - G_j})[j][v]; skipped when nothing reads the state again
-        if (c0 + CH < T || keep) {
+        if (!run_mode && (j + 1 < n_chunks || keep)) {
             const float GL = Gs[CH - 1];
             const float eg = __expf(GL);
             tok_op vd[2];
@@ -429,20 +491,23 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
 #pragma unroll
                 for (int vt = 0; vt < 2; vt++) hp[(16 * kt + r) * VD + 16 * vt] = S[kt][vt][r];
     }
+  }
 }
 
-// 32-token chunks: 254 registers (the solve's preloaded triangle), two workgroups per compute unit.  16-token chunks: 168
-// registers, three workgroups per compute unit.
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gdn_wy32_kernel(const GdnParams p) { gdn_wy_body<2>(p); }
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void gdn_wy16_kernel(const GdnParams p) { gdn_wy_body<1>(p); }
+// 32-token chunks, 254 registers, two workgroups per compute unit; the recurrent entry point's kernel also pairs up leaves.
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gdn_wy32_kernel(const GdnParams p) { gdn_wy_body<2, false>(p); }
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gdn_wy_pairs_kernel(const GdnParams p) { gdn_wy_body<2, true>(p); }
 
-// tokens_per_chunk: 32 (long segments) or 16 (short segments)
-int gdn_wy_launch(const GdnParams& p, int tokens_per_chunk, hipStream_t stream) {
+// pairs: the recurrent entry point (short segments, leaves two to a chunk)
+int gdn_wy_launch(GdnParams p, bool pairs, hipStream_t stream) {
     if (p.dv != VD) return spinf_fail(SPINF_E_ARG, "gdn: value head dim %d, the chunked kernel is built for 128", p.dv);
-    const long blocks = p.n_seg * p.hv;
+    // segments per workgroup: as many as leave about eight workgroups per compute unit (of 256), 16 at most
+    p.run = 1;
+    while (pairs && p.run < 16 && (p.n_seg + 2 * p.run - 1) / (2 * p.run) * p.hv >= 2048) p.run *= 2;
+    const long blocks = (p.n_seg + p.run - 1) / p.run * p.hv;
     if (blocks > INT32_MAX) return spinf_fail(SPINF_E_ARG, "gdn: too many segments");
-    if (tokens_per_chunk == 32) hipLaunchKernelGGL(gdn_wy32_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, p);
-    else hipLaunchKernelGGL(gdn_wy16_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, p);
+    if (!pairs) hipLaunchKernelGGL(gdn_wy32_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL(gdn_wy_pairs_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "gdn: launch: %s", hipGetErrorString(e));
     return SPINF_OK;

@@ -21,6 +21,7 @@ struct GdnParams {
     int h, hv, dk, dv; float scale;
     const long* cu; const long* idx; long n_seg;
     const float* h0; const long* h0_idx; float* ht; const long* ht_idx;
+    int run;   // segments per workgroup of the recurrent entry point's kernel (set by its launcher)
 };
 
 namespace gdn_tiles {

@@ -83,7 +83,8 @@ def test_rows_by_index_and_skipped_states(dev):
             assert np.abs(_np(o[0, r]) - want).max() <= TOL, mode
 
 
-def test_segments_forked_from_one_state(dev):
+@pytest.mark.parametrize("mode", ["recurrent", "chunked"])
+def test_segments_forked_from_one_state(dev, mode):
     """many short segments that start from the same stored state (what a trunk's leaves look like), mixed with segments that
     are longer than a mini-chunk, keep their final state or start from another state: each must equal its own recurrence"""
     H, HV = 2, 4
@@ -99,7 +100,10 @@ def test_segments_forked_from_one_state(dev):
     ht = torch.full((n, HV, 128, 128), float("nan"), device=dev)
     ht_idx = torch.tensor([i if i in kept else -1 for i in range(n)], device=dev)
     args = [t[x][None] for x in ("q", "k", "v", "g", "beta")]
-    o = sa.recurrent(*args, 128 ** -0.5, cu, n, h0=h0, h0_idx=h0_idx, ht=ht, ht_idx=ht_idx)
+    if mode == "recurrent":
+        o = sa.recurrent(*args, 128 ** -0.5, cu, n, h0=h0, h0_idx=h0_idx, ht=ht, ht_idx=ht_idx)
+    else:
+        o = sa.chunked(*args, 128 ** -0.5, cu, cu_cpu, h0=h0, h0_idx=h0_idx, ht=ht, ht_idx=ht_idx)
     torch.cuda.synchronize()
     for s in range(n):
         a, b = int(cu_cpu[s]), int(cu_cpu[s + 1])
