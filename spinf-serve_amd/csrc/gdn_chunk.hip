@@ -329,12 +329,6 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
                 const float* T1s = Ts + 16 * LX;
                 const f32x4 G1 = *(const f32x4*)(Gs + 16 + 4 * q4), B1 = *(const f32x4*)(Bs + 16 + 4 * q4);
                 const f32x4 t11 = *(const f32x4*)(T1s + c * LX + 4 * q4);
-                f32x4 x = zero4();
-#pragma unroll
-                for (int s4 = 0; s4 < 4; s4++)        // X[j][i] = sum_m A_lo[m][j] T_11[i][m]
-                    x = mfma4(As[(16 + 4 * s4 + q4) * LA + c], T1s[c * LX + 4 * s4 + q4], x);
-#pragma unroll
-                for (int r = 0; r < 4; r++) Xs[(4 * q4 + r) * LX + c] = x[r];
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
                     u4[r] = (__bf16)(t11[r] * B1[r]);
@@ -342,11 +336,19 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
                 }
                 *(bf16x4*)(Tus + (16 + c) * LP + 16 + 4 * q4) = u4;
                 *(bf16x4*)(Tws + (16 + c) * LP + 16 + 4 * q4) = w4;
-                wave_lds_order();
                 f32x4 tlo = zero4();
+                if (!run_mode) {      // (a pair's tiles are different segments: A_lo = 0, so is T_lo)
+                    f32x4 x = zero4();
 #pragma unroll
-                for (int s4 = 0; s4 < 4; s4++)        // T_lo[16 + i][j'] = sum_j T_00[j][j'] X[j][i]
-                    tlo = mfma4(Ts[(4 * s4 + q4) * LX + c], Xs[(4 * s4 + q4) * LX + c], tlo);
+                    for (int s4 = 0; s4 < 4; s4++)        // X[j][i] = sum_m A_lo[m][j] T_11[i][m]
+                        x = mfma4(As[(16 + 4 * s4 + q4) * LA + c], T1s[c * LX + 4 * s4 + q4], x);
+#pragma unroll
+                    for (int r = 0; r < 4; r++) Xs[(4 * q4 + r) * LX + c] = x[r];
+                    wave_lds_order();
+#pragma unroll
+                    for (int s4 = 0; s4 < 4; s4++)        // T_lo[16 + i][j'] = sum_j T_00[j][j'] X[j][i]
+                        tlo = mfma4(Ts[(4 * s4 + q4) * LX + c], Xs[(4 * s4 + q4) * LX + c], tlo);
+                }
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
                     u4[r] = (__bf16)(tlo[r] * B0[r]);
