@@ -100,9 +100,10 @@ int spinf_attn_exact_items(int64_t* total);
  *
  *   q, k [rows, h, dk] (l2-normalised), v, o [rows, hv, dv] bf16; g [rows, hv] fp32 log decay; beta [rows, hv] bf16;
  *   strides in elements (q and k share q_tok, g and beta share g_tok; heads are dense inside a row); dk = dv = 128.
- *   cu, idx, h0_idx, ht_idx: int64 device arrays.  mode 0 = short segments (one wave per
- *   segment, head and 32 value columns, 16-token mini-chunks), 1 = long segments (one workgroup per segment and head,
- *   32-token chunks); both are the WY form of the same recurrence and either mode accepts any segment length.
+ *   cu, idx, h0_idx, ht_idx: int64 device arrays.  mode 0 = the recurrent entry point (short
+ *   segments; consecutive segments of at most 16 tokens that start from the same state and leave none behind are taken
+ *   two to a chunk), 1 = the chunked entry point (one workgroup per segment and head, 32-token chunks); both are the WY
+ *   form of the same recurrence and either mode accepts any segment length.
  *   v and o must be 16-byte aligned with row strides that are multiples of 8 elements.
  */
 typedef struct spinf_gdn_args {

@@ -15,8 +15,8 @@
 using namespace gdn_tiles;
 
 // ---------------------------------------------------------------------------------------------- short segments
-// The recurrent entry point for value head dims other than 128 (128 runs the workgroup kernel of gdn_chunk.hip on 16-token
-// chunks): meant for the short segments of a trie (a handful of tokens after a fork), thousands per call.
+// The recurrent entry point for value head dims other than 128 (128 runs the workgroup kernel of gdn_chunk.hip, leaves two
+// to a chunk): meant for the short segments of a trie (a handful of tokens after a fork), thousands per call.
 // One wave per (segment, value head, 32 value columns) and no workgroup barrier anywhere.  The wave walks its segment in
 // mini-chunks of 16 tokens with the same WY algebra as the workgroup kernel of gdn_chunk.hip (A = -strict_tril(beta_i K_i.K_j e^{G_i-G_j}),
 // T = (I - A)^-1, U = T diag(beta) V, -W = -T diag(beta e^G) K, V' = U - W S, O = s e^G Q S + P V', S <- e^{G_L} S +

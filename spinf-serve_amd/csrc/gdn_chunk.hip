@@ -1,10 +1,10 @@
 // Gated DeltaNet, chunked WY form, one fused kernel: stands in for gdn.chunked (spinf_serve/models/qwen35/gdn.py:109-133),
 // i.e. for fla's cumsum -> intra-chunk WY solve -> state recurrence (gdn.py:21-106) -> output pipeline, without writing
-// the per-chunk state snapshots or the w / u / v_new intermediates to memory; with 16-token chunks it also serves the
-// recurrent entry point (gdn.py:197-235) for value head dim 128.
+// the per-chunk state snapshots or the w / u / v_new intermediates to memory; it also serves the recurrent entry point
+// (gdn.py:197-235) for value head dim 128, where the leaves that fork from one state are taken two to a chunk.
 //
-// One workgroup (4 waves) owns one (segment, value head) and walks its chunks of 16 NT tokens in order (NT = 2 for long
-// segments, 1 for short ones); wave w owns value columns 32w .. 32w+31 of the state S [K=128, V=128], which never leaves its
+// One workgroup (4 waves) owns one (segment, value head) and walks its 32-token chunks (two 16-token tiles) in order;
+// wave w owns value columns 32w .. 32w+31 of the state S [K=128, V=128], which never leaves its
 // fp32 accumulator registers.  Per chunk, with G = cumsum(g), D_ij = e^{G_i - G_j}:
 //     A   = -strict_tril(beta_i (K K^T)_ij D_ij)         T = (I - A)^-1      (fp32: 16 x 16 blocks solved by substitution in
 //                                                                             registers, merged with fp32 MFMAs)
@@ -34,7 +34,7 @@ extern "C" int spinf_debug_gdn_trace(long* out) { return (int)hipMemcpyFromSymbo
 #ifndef SPINF_TRACE_PAIRS
 #define SPINF_TRACE_PAIRS false
 #endif
-#define GT_ADD(slot, val) do { if (NT == 2 && PAIRS == SPINF_TRACE_PAIRS && threadIdx.x == SPINF_TRACE_THREAD && blockIdx.x == 7) g_gdn_trace[slot] += (val); } while (0)
+#define GT_ADD(slot, val) do { if (PAIRS == SPINF_TRACE_PAIRS && threadIdx.x == SPINF_TRACE_THREAD && blockIdx.x == 7) g_gdn_trace[slot] += (val); } while (0)
 #else
 #define GT_CLK(v) do { } while (0)
 #define GT_ADD(slot, val) do { } while (0)
@@ -58,32 +58,15 @@ __device__ __forceinline__ bf16x4 zero_bf4() {
     for (int r = 0; r < 4; r++) z[r] = (__bf16)0.f;
     return z;
 }
-// products over a contraction index of 16 NT tokens: 16x16x32 for NT = 2 (operands of 8 slots), 16x16x16 for NT = 1
-__device__ __forceinline__ f32x4 mm(bf16x8 a, bf16x8 b, f32x4 c) { return mfma32(a, b, c); }
-__device__ __forceinline__ f32x4 mm(bf16x4 a, bf16x4 b, f32x4 c) { return mfma16(a, b, c); }
-
-template <int NT>
-struct Tok;
-template <>
-struct Tok<2> {
-    typedef bf16x8 op;
-    static __device__ __forceinline__ op make(bf16x4 lo, bf16x4 hi) { return join(lo, hi); }
-};
-template <>
-struct Tok<1> {
-    typedef bf16x4 op;
-    static __device__ __forceinline__ op make(bf16x4 lo, bf16x4) { return lo; }
-};
-
 }  // namespace
 
-template <int NT, bool PAIRS>
+template <bool PAIRS>
 __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
-    static_assert(!PAIRS || NT == 2, "a pair of segments takes the two token tiles of a 32-token chunk");
+    constexpr int NT = 2;                           // 16-token tiles per chunk
     constexpr int CH = 16 * NT;
     constexpr int LO = CH;                          // row stride (elements) of a wave's transposed output tile [32 values][CH tokens]
     constexpr int NTILES = NT * (NT + 1) / 2;       // 16 x 16 tiles of A / P on or below the diagonal
-    typedef typename Tok<NT>::op tok_op;            // operand of a product that contracts over the chunk's tokens
+    typedef bf16x8 tok_op;                          // operand of a product that contracts over the chunk's 32 tokens
     __shared__ __attribute__((aligned(16))) __bf16 Ks[CH * LD];
     __shared__ __attribute__((aligned(16))) __bf16 Qs[CH * LD];
     __shared__ __attribute__((aligned(16))) __bf16 Vs[CH * LD];      // V; later the waves' output tiles
@@ -210,7 +193,7 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
         }
         rb = -1;
         if (tid < CH) {                       // chunk row tid = row tid % 16 of tile tid / 16
-            const bool hi = NT == 2 && tid >= 16;
+            const bool hi = tid >= 16;
             const int r = tid & 15;
             if (r < (hi ? len[NT - 1] : len[0])) {
                 const long t = (hi ? base[NT - 1] : base[0]) + r;
@@ -249,7 +232,7 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
         if (tid < CH) {
             float x = row_prefix_sum(pg);
             // row_bcast:15 -> lanes 16..31 (not for a pair: the second tile is another segment)
-            if (NT == 2 && !run_mode) x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x142, 0xa, 0xf, false));
+            if (!run_mode) x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x142, 0xa, 0xf, false));
             Gs[tid] = x;
             Bs[tid] = (float)pbeta;
             Rs[tid] = pr32;
@@ -307,8 +290,8 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
         // Leaves T diag(beta) and -T diag(beta e^G) in LDS as bf16, tile by tile.
         if (w == 0) {
             float t[16];
-            const int blk = NT == 2 ? (q4 & 1) : 0;
-            unit_lower_inverse_row<NT == 2>(As + blk * (16 * LA + 16), LA, c, t);
+            const int blk = q4 & 1;
+            unit_lower_inverse_row<true>(As + blk * (16 * LA + 16), LA, c, t);
             // the rows pass through LDS to reach the lanes in operand order (row c, columns 4 q4 ..+3)
 #pragma unroll
             for (int j4 = 0; j4 < 4; j4++) *(f32x4*)(Ts + (16 * blk + c) * LX + 4 * j4) = f32x4{t[4 * j4], t[4 * j4 + 1], t[4 * j4 + 2], t[4 * j4 + 3]};
@@ -325,7 +308,7 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
             }
             *(bf16x4*)(Tus + c * LP + 4 * q4) = u4;
             *(bf16x4*)(Tws + c * LP + 4 * q4) = w4;
-            if (NT == 2) {
+            {
                 const float* T1s = Ts + 16 * LX;
                 const f32x4 G1 = *(const f32x4*)(Gs + 16 + 4 * q4), B1 = *(const f32x4*)(Bs + 16 + 4 * q4);
                 const f32x4 t11 = *(const f32x4*)(T1s + c * LX + 4 * q4);
@@ -370,24 +353,24 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
             for (int it = 0; it < NT; it++) {
                 const __bf16* up = Tus + (16 * it + c) * LP + 4 * q4;
                 const __bf16* wp = Tws + (16 * it + c) * LP + 4 * q4;
-                tu[it] = Tok<NT>::make(*(const bf16x4*)up, it ? *(const bf16x4*)(up + 16) : zero_bf4());
-                tw[it] = Tok<NT>::make(*(const bf16x4*)wp, it ? *(const bf16x4*)(wp + 16) : zero_bf4());
+                tu[it] = join(*(const bf16x4*)up, it ? *(const bf16x4*)(up + 16) : zero_bf4());
+                tw[it] = join(*(const bf16x4*)wp, it ? *(const bf16x4*)(wp + 16) : zero_bf4());
             }
 #pragma unroll
             for (int vt = 0; vt < 2; vt++) {
-                const tok_op vB = Tok<NT>::make(frag_tr4(Vs, LD, 0, 32 * w + 16 * vt, lane), NT == 2 ? frag_tr4(Vs, LD, 16, 32 * w + 16 * vt, lane) : zero_bf4());
+                const tok_op vB = join(frag_tr4(Vs, LD, 0, 32 * w + 16 * vt, lane), frag_tr4(Vs, LD, 16, 32 * w + 16 * vt, lane));
 #pragma unroll
                 for (int it = 0; it < NT; it++) {
-                    vp[it][vt] = mm(tu[it], vB, zero4());
+                    vp[it][vt] = mfma32(tu[it], vB, zero4());
                     qs[it][vt] = zero4();
                 }
             }
 #pragma unroll
             for (int h = 0; h < 2; h++) {
                 const int kt = 2 * w + h;
-                const tok_op kT = Tok<NT>::make(frag_tr4(Ks, LD, 0, 16 * kt, lane), NT == 2 ? frag_tr4(Ks, LD, 16, 16 * kt, lane) : zero_bf4());
+                const tok_op kT = join(frag_tr4(Ks, LD, 0, 16 * kt, lane), frag_tr4(Ks, LD, 16, 16 * kt, lane));
 #pragma unroll
-                for (int it = 0; it < NT; it++) *(bf16x4*)(Wn + (16 * it + c) * LW + 16 * kt + 4 * q4) = round4(mm(kT, tw[it], zero4()));
+                for (int it = 0; it < NT; it++) *(bf16x4*)(Wn + (16 * it + c) * LW + 16 * kt + 4 * q4) = round4(mfma32(kT, tw[it], zero4()));
             }
         }
         lds_barrier();   // -W visible; every wave has read its V columns
@@ -428,14 +411,14 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
 #pragma unroll
             for (int it = 0; it < NT; it++) {
                 const __bf16* pp = Ps + (16 * it + c) * LP + 4 * q4;
-                pA[it] = Tok<NT>::make(*(const bf16x4*)pp, it ? *(const bf16x4*)(pp + 16) : zero_bf4());
+                pA[it] = join(*(const bf16x4*)pp, it ? *(const bf16x4*)(pp + 16) : zero_bf4());
             }
 #pragma unroll
             for (int vt = 0; vt < 2; vt++) {
-                const tok_op vb = Tok<NT>::make(round4(vp[0][vt]), round4(vp[NT - 1][vt]));
+                const tok_op vb = join(round4(vp[0][vt]), round4(vp[NT - 1][vt]));
 #pragma unroll
                 for (int it = 0; it < NT; it++) {
-                    f32x4 o = mm(pA[it], vb, zero4());
+                    f32x4 o = mfma32(pA[it], vb, zero4());
 #pragma unroll
                     for (int r = 0; r < 4; r++) o[r] = __builtin_fmaf(p.scale * __expf(Gj[it][r]), qs[it][vt][r], o[r]);
                     *(bf16x4*)(Ow + (16 * vt + c) * LO + 16 * it + 4 * q4) = round4(o);      // O^T[v][i]
@@ -467,16 +450,16 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
                 for (int it = 0; it < NT; it++)
 #pragma unroll
                     for (int r = 0; r < 4; r++) d[it][r] = (__bf16)(vp[it][vt][r] * __expf(GL - Gj[it][r]));
-                vd[vt] = Tok<NT>::make(d[0], d[NT - 1]);
+                vd[vt] = join(d[0], d[NT - 1]);
             }
 #pragma unroll
             for (int kt = 0; kt < 8; kt++) {
-                const tok_op kT = Tok<NT>::make(frag_tr4(Ks, LD, 0, 16 * kt, lane), NT == 2 ? frag_tr4(Ks, LD, 16, 16 * kt, lane) : zero_bf4());
+                const tok_op kT = join(frag_tr4(Ks, LD, 0, 16 * kt, lane), frag_tr4(Ks, LD, 16, 16 * kt, lane));
 #pragma unroll
                 for (int vt = 0; vt < 2; vt++) {
 #pragma unroll
                     for (int r = 0; r < 4; r++) S[kt][vt][r] *= eg;
-                    S[kt][vt] = mm(kT, vd[vt], S[kt][vt]);
+                    S[kt][vt] = mfma32(kT, vd[vt], S[kt][vt]);
                 }
             }
         }
@@ -497,8 +480,8 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
 }
 
 // 32-token chunks, 254 registers, two workgroups per compute unit; the recurrent entry point's kernel also pairs up leaves.
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gdn_wy32_kernel(const GdnParams p) { gdn_wy_body<2, false>(p); }
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gdn_wy_pairs_kernel(const GdnParams p) { gdn_wy_body<2, true>(p); }
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gdn_wy32_kernel(const GdnParams p) { gdn_wy_body<false>(p); }
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gdn_wy_pairs_kernel(const GdnParams p) { gdn_wy_body<true>(p); }
 
 // pairs: the recurrent entry point (short segments, leaves two to a chunk)
 int gdn_wy_launch(GdnParams p, bool pairs, hipStream_t stream) {
