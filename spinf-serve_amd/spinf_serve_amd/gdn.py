@@ -1,8 +1,7 @@
 """Gated DeltaNet over trie segments with the reference's two entry points (spinf_serve/models/qwen35/gdn.py:109-133, 197-235).
 
-Both run in libspinf_tree.so as fused WY-form kernels: `recurrent` one wave per (segment, head, 32 values) on 16-token
-mini-chunks (short segments), `chunked` one workgroup per (segment, head) on 32-token chunks (long
-segments).  Unlike the reference's chunked(), the kernel reads and writes the stream rows through `idx` itself, so callers
+Both run in libspinf_tree.so as fused WY-form kernels, one workgroup per (segment, head) on 32-token chunks: `chunked` for
+long segments, `recurrent` for short ones (leaves that fork from one state are taken two to a chunk).  Unlike the reference's chunked(), the kernel reads and writes the stream rows through `idx` itself, so callers
 need no gather / scatter around it, and it writes no per-chunk state snapshots.
 
 q and k arrive l2-normalised; g is the log decay (fp32), beta the write strength, scale 1 / sqrt(K).
