@@ -409,9 +409,13 @@ __device__ long g_trace[16 * 4096];
 extern "C" int spinf_debug_trace(long* out, int n) { return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_trace), sizeof(long) * n, 0, hipMemcpyDeviceToHost); }
 #define TRACE_ADD(slot, val) do { if (threadIdx.x == 64 && blockIdx.x < 4096) g_trace[blockIdx.x * 16 + (slot)] += (val); } while (0)
 #define TRACE_CLK(var) const long var = clock64()
+#define TRACE_WALL(var) const long var = wall_clock64()
+#define TRACE_SET(slot, val) do { if (threadIdx.x == 64 && blockIdx.x < 4096) g_trace[blockIdx.x * 16 + (slot)] = (val); } while (0)
 #else
 #define TRACE_ADD(slot, val) do { } while (0)
 #define TRACE_CLK(var) do { } while (0)
+#define TRACE_WALL(var) do { } while (0)
+#define TRACE_SET(slot, val) do { } while (0)
 #endif
 
 // NHW = 1: four waves, each with RT heads of the item.  NHW = 2: eight waves, waves 4..7 take the item's second set of RT heads
@@ -439,6 +443,8 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
     __shared__ __attribute__((aligned(16))) char stage_all[STAGE_IN_TILE ? 16 : 4 * NHW * 32 * 144];
     __shared__ int s_next[2];         // item grabbed by thread 0 for the whole workgroup, double buffered
 
+    TRACE_CLK(tk0);
+    TRACE_WALL(tw0);
     const Lane<D> L(p);
     char* const stage_own = stage_all + (STAGE_IN_TILE ? 0 : L.w * 32 * 144);
 
@@ -611,8 +617,12 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
         load_ent(cur, ent_cur, 0);
         if (L.wh == 0) issue_tile<D, 4>(p, lds_addr(bufs), cur.w, item_hp(cur) * HPI / p.group, L.w, L.lane, L.lane_k, L.lane_v);
     }
-    grab(1);
+    // The item after the current one is fetched from the lists as late as the prefetch pipeline allows (three tile steps
+    // before the current item ends; at once for items shorter than that): an item fetched long before it starts keeps the
+    // workgroup busy long after the lists have run dry, and the pass ends with the last workgroup.
+    auto grab_step = [](const int ne) { return ne >= 4 ? ne - 3 : -1; };
     int gslot = 1;      // slot of s_next that holds the item after `cur`
+    if (cur_ok && grab_step(item_ne(cur)) < 0) grab(1);
     int i = 0;          // tile step inside the current item
     int base = 0;       // first plan entry held in ent_cur
     int pstage = 0;     // next-item prefetch: 0 nothing, 1 descriptor known, 2 entries requested, 3 first tile requested
@@ -627,9 +637,16 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
     while (cur_ok) {
         const int ne = item_ne(cur);
         const int kvh = item_hp(cur) * HPI / p.group;
+        const int grab_at = grab_step(ne);
         reset_acc();
         base = 0;
         pstage = 0;
+        nxt_ok = false;
+        TRACE_WALL(twi);
+        TRACE_SET(5, twi);
+        TRACE_SET(6, (long)ne);
+        TRACE_SET(4, (long)cur_idx);
+        TRACE_SET(3, (long)xcc);
         for (i = 0; i < ne; i++, par ^= 1) {
             const char* buf = bufs + par * G::BUFB;
             const unsigned oth = lds_addr(bufs + (par ^ 1) * G::BUFB);
@@ -639,7 +656,10 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
             TRACE_CLK(tc1);
             TRACE_ADD(8, tc1 - tc0);
             // next-item prefetch, one stage per step
-            if (pstage == 0) {
+            if (i < grab_at) {
+            } else if (i == grab_at) {
+                grab(gslot);
+            } else if (pstage == 0) {
                 nxt_idx = __builtin_amdgcn_readfirstlane(s_next[gslot]);
                 nxt_ok = nxt_idx >= 0;
                 if (nxt_ok) nxt = uniform4(p.items[nxt_idx]);
@@ -679,6 +699,10 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
         TRACE_CLK(tc4);
         TRACE_ADD(10, tc4 - tc3);
         TRACE_ADD(11, 1);
+        TRACE_WALL(twe);
+        TRACE_SET(13, tw0);
+        TRACE_SET(7, twe);
+        TRACE_SET(14, tc4 - tk0);
         cur_ok = nxt_ok;
         if (!cur_ok) break;
         // finish whatever of the next item's prefetch has not happened yet (one-tile items), then switch
@@ -688,7 +712,7 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
         load_q(cur, qf, art_q, pos_q);
         { int2* tmp = ent_cur; ent_cur = ent_nxt; ent_nxt = tmp; }
         gslot ^= 1;
-        grab(gslot);     // the item after the new current one; read at the next tile step's barrier
+        if (grab_step(item_ne(cur)) < 0) grab(gslot);   // short item: fetch its successor now; read at the next tile step's barrier
     }
     // ---- the last workgroup to finish resets the counters for the next launch
     __builtin_amdgcn_s_waitcnt(0x0f70);

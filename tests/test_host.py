@@ -289,14 +289,21 @@ def test_schedule_covers_every_tile_and_head_group_once():
             assert e0 == plan.qt_ptr[t] and ne == plan.qt_ptr[t + 1] - plan.qt_ptr[t] and ne >= 1
             assert kt0 == plan.kv_idx[e0]
         assert len(seen) == plan.n_qtiles * head_groups
-        # a list never splits the head groups of one query tile's job across lists more than necessary: within a list the
-        # items of one (job, head group) are contiguous
+        # a list is a body followed by a tail.  Body: the items of one (job, head group) are contiguous (they share keys).
+        # Tail: the list's lightest items, at most 128 of them, heaviest first, so that the workgroups finish close together.
         job_of_tile = {}
         for o in b.owners:
             for t in range(o.start // 128, -(-(o.start + o.n_tokens) // 128)):
                 job_of_tile[t] = o.job_id
         for l in range(8):
-            runs = [(job_of_tile.get(t, -1), ((z & 0xFFFFFFFF) >> 20)) for t, _, z, _ in items[list_ptr[l] : list_ptr[l + 1]].tolist()]
+            rows = items[list_ptr[l] : list_ptr[l + 1]].tolist()
+            # cost of an item: per key tile, the most 32-key blocks any of the four row groups sees (they move in step)
+            blocks = [sum(max(bin((int(x) >> (2 * w)) & 3).count("1") for w in range(4)) for x in plan.kv_bits[e0 : e0 + (z & 0xFFFFF)])
+                      for _, e0, z, _ in rows]
+            cut = len(rows)
+            while cut > 0 and len(rows) - cut < 128 and (cut == len(rows) or blocks[cut - 1] >= blocks[cut]):
+                cut -= 1
+            runs = [(job_of_tile.get(t, -1), ((z & 0xFFFFFFFF) >> 20)) for t, _, z, _ in rows[:cut]]
             compact = [r for i, r in enumerate(runs) if i == 0 or r != runs[i - 1]]
             assert len(compact) == len(set(compact))
 
