@@ -65,6 +65,10 @@ def main():
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--variant", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--rows", default="stream", choices=["stream", "compact", "scatter"],
+                    help="attention workloads: stream layout (default); compact = real rows only, read through the kernel's row map; "
+                         "scatter = real rows only, scattered into stream layout and gathered back around the call (the reference's way). "
+                         "The timed region then is the whole call, copies included; no CPU leg")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU's throughput; contents shard across GPUs with no exchange, run one process per GPU (--gpus 1)")
@@ -135,11 +139,32 @@ def main():
         sa.TilePlan.build(b.art, b.end, b.pos, None)
     plan_ms = 1e3 * (time.perf_counter() - tp0)
 
+    if args.rows != "stream":
+        args.no_cpu = True
+        # compact rows (the Qwen stack's call, spinf_serve/models/qwen35/qwen.py:613-622): q, k, v hold the real tokens only
+        compact = []
+        for b, ((q, k, v), masks) in zip(cfg.batches, work):
+            sidx = torch.from_numpy(np.flatnonzero(b.art >= 0)).to(dev)
+            compact.append((tuple(t[sidx].contiguous() for t in (q, k, v)), masks, sidx, b.length))
+        work = None
+
     def step():
         out = None
-        for (q, k, v), masks in work:
-            for w in layers:
-                out = sa.tree_attn(q, k, v, masks["sliding_attention" if w else "full_attention"], cfg.scale, variant=args.variant)
+        if args.rows == "stream":
+            for (q, k, v), masks in work:
+                for w in layers:
+                    out = sa.tree_attn(q, k, v, masks["sliding_attention" if w else "full_attention"], cfg.scale, variant=args.variant)
+        elif args.rows == "compact":   # the kernel goes through the row map
+            for (q, k, v), masks, sidx, _ in compact:
+                for w in layers:
+                    out = sa.tree_attn(q, k, v, masks["sliding_attention" if w else "full_attention"], cfg.scale, variant=args.variant, sidx=sidx)
+        else:                          # "scatter": the reference's three zero-filled scatters and the gather around the stream-layout call
+            for (q, k, v), masks, sidx, length in compact:
+                for w in layers:
+                    up = [t.new_zeros(length, t.shape[1], t.shape[2]).index_copy_(0, sidx, t) for t in (q, k, v)]
+                    o = sa.tree_attn(*up, masks["sliding_attention" if w else "full_attention"], cfg.scale, variant=args.variant)
+                    out = q.new_zeros(q.shape)
+                    out[: sidx.shape[0]] = o.index_select(0, sidx)
         return out
 
     wall, kern = timed(step, args.steps, args.warmup, torch)
@@ -150,9 +175,9 @@ def main():
     line.update(value=tokens * args.steps / wall, ms_per_step=1e3 * wall / args.steps, dtype="bf16",
                 config={"workload": WORKLOADS[args.workload], "contents": len(cfg.trees), "packed_tokens": cfg.n_real,
                         "stream_tokens": sum(b.length for b in cfg.batches), "passes": len(cfg.batches), "layers_per_step": len(layers),
-                        "visible_pairs": [cfg.pairs(w) for w in layers], "variant": args.variant},
+                        "visible_pairs": [cfg.pairs(w) for w in layers], "variant": args.variant, "rows": args.rows},
                 roofline={"bound": "mfma", "achieved": tfl, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": tfl / PEAK_BF16_TFLOPS,
-                          "traffic": TRAFFIC_BYTES.get(args.workload) if args.contents is None else None, "kernel_ms": ms,
+                          "traffic": TRAFFIC_BYTES.get(args.workload) if args.contents is None and args.rows == "stream" else None, "kernel_ms": ms,
                           "kernel_ms_min": float(np.min(kern)), "useful_flops": flops,
                           "algorithmic_bytes": cfg.bytes() * len(layers), "hbm_frac_at_algorithmic_bytes": cfg.bytes() * len(layers) / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS},
                 plan_build_ms_host=plan_ms, setup_s=setup_s)

@@ -44,8 +44,8 @@ int spinf_version(void);
  * spinf_tileplan_schedule turns the plan into the kernel's work lists for a given number of head groups (query heads /
  * heads per work item, see spinf_attn_heads_per_item): items[4*i..4*i+3] = {query tile, first entry, entries | head
  * group << 20, first key tile}; list_ptr[0..8] delimits eight lists of roughly equal weight (one per XCD), inside a list
- * the items of a job stay together, head group by head group, heaviest query tile first.  The order of the items never
- * changes a result.
+ * the items of a job stay together, head group by head group, heaviest query tile first; the lightest items of a list
+ * (8 % of its weight) sit at its end.  The order of the items never changes a result.
  */
 typedef struct spinf_tileplan spinf_tileplan;
 
@@ -57,6 +57,10 @@ int spinf_tileplan_counts(const spinf_tileplan* plan, int64_t counts[5]);
 int spinf_tileplan_export(const spinf_tileplan* plan, int32_t* qt_ptr, int32_t* kv_idx, uint32_t* kv_bits, int32_t* order);
 /* items [4 * n_qtiles * head_groups], list_ptr [9]: caller-allocated host arrays */
 int spinf_tileplan_schedule(const spinf_tileplan* plan, int32_t head_groups, int32_t* items, int32_t* list_ptr);
+/* Compact rows (tree_attention with sidx, spinf_serve/models/qwen35/qwen.py:613-622): row_of [n] = row of each stream
+ * position in tensors that hold the real tokens only, -1 for a pad position.  kv_row0 [entries] (caller-allocated) receives,
+ * per plan entry, the row of the entry's first key if its 64 keys are 64 consecutive rows, else -1.  Host arrays. */
+int spinf_tileplan_row0(const spinf_tileplan* plan, const int32_t* row_of, int32_t* kv_row0);
 void spinf_tileplan_free(spinf_tileplan* plan);
 
 /* ------------------------------------------------------------------------------------------------ attention
@@ -69,6 +73,9 @@ void spinf_tileplan_free(spinf_tileplan* plan);
  *   art, end, pos, kv_idx, kv_bits: device copies of the metadata and of the exported plan; items, list_ptr: device copy of
  *   the schedule for hq / spinf_attn_heads_per_item(hq, hkv, d, variant) head groups, n_items = query tiles x head groups
  *   window: the window the plan was built with (<= 0 global)
+ *   row_of, kv_row0 (both NULL, or both device arrays as spinf_tileplan_row0 describes them): compact rows.  q, k, v, out
+ *   then hold the real tokens only; the kernel reads and writes them through row_of instead of the three zero-filled
+ *   scatters and the gather of qwen.py:617-622.  Pad positions write nothing.  Results equal the scattered call's bit for bit.
  *
  * The kernel is persistent (one workgroup per CU pulling items from the lists) and keeps its list cursors in a small
  * per-device buffer of the library: launches that overlap on one device (different streams) are not supported.
@@ -81,7 +88,9 @@ typedef struct spinf_attn_args {
     const int32_t* kv_idx; const uint32_t* kv_bits; const int32_t* items; const int32_t* list_ptr;
     int64_t n_items;
     int32_t variant;   /* 0 = default kernel choice (eight waves, two heads of a GQA group per work item, where the group is even);
-                          1 = one head per work item, four waves; 2 = four waves with two heads each (head dim <= 128) */
+                          1 = one head per work item, four waves; 2 = four waves with two heads each (head dim <= 128,
+                          no compact rows) */
+    const int32_t* row_of; const int32_t* kv_row0;
 } spinf_attn_args;
 
 /* query heads one work item covers for this geometry (1 or 2); 0 for an invalid geometry */

@@ -255,4 +255,17 @@ extern "C" int spinf_tileplan_schedule(const spinf_tileplan* p, int32_t head_gro
     return SPINF_OK;
 }
 
+extern "C" int spinf_tileplan_row0(const spinf_tileplan* p, const int32_t* row_of, int32_t* kv_row0) {
+    if (!p || !row_of) return spinf_fail(SPINF_E_ARG, "tileplan_row0: null argument");
+    if (!kv_row0 && !p->kv_idx.empty()) return spinf_fail(SPINF_E_ARG, "tileplan_row0: null kv_row0");
+    for (size_t e = 0; e < p->kv_idx.size(); e++) {
+        const int64_t k0 = (int64_t)p->kv_idx[e] * SPINF_KTILE;
+        int32_t r0 = k0 + SPINF_KTILE <= p->n ? row_of[k0] : -1;
+        for (int64_t j = 1; r0 >= 0 && j < SPINF_KTILE; j++)
+            if (row_of[k0 + j] != r0 + j) r0 = -1;
+        kv_row0[e] = r0;
+    }
+    return SPINF_OK;
+}
+
 extern "C" void spinf_tileplan_free(spinf_tileplan* p) { delete p; }

@@ -57,6 +57,9 @@ struct AttnParams {
     int* counters;        // [0..NLIST) next item of each list, [NLIST] workgroups done, [NLIST+1] items awaiting the exact pass,
                           // [NLIST+2] exact-pass workgroups done; each kernel's last workgroup resets what it used
     int* redo;            // indices (into items) of the work items the fast pass handed to the exact pass
+    // compact rows (ROWS kernels): q, k, v, o hold the real tokens only; row_of[stream position] = row, -1 for a pad position;
+    // kv_row0[entry] = row of the entry's first key if its 64 keys are 64 consecutive rows, else -1
+    const int* row_of; const int* kv_row0;
 };
 
 // Softmax reference point.  The fast pass fixes each row's reference at the maximum of the first 32-key block in which
@@ -125,18 +128,19 @@ __device__ __forceinline__ unsigned lds_addr(const void* p) { return (unsigned)(
 // w*IPW .. w*IPW+IPW-1; lane -> (slot = which row of the region, 16-byte chunk of the row).  For a tile that lies fully inside
 // the stream every address is a wave-uniform base plus a per-lane constant (lane_k / lane_v, bytes), so the loop spends no
 // vector ALU on addressing; the last, partial tile clamps its rows per lane.
-template <int D, int NW = 4>
-__device__ __forceinline__ void issue_tile(const AttnParams& p, unsigned buf, int kt, int kvh, int w, int lane, unsigned lane_k, unsigned lane_v) {
+// ROWS (compact rows): row0 >= 0 says that the tile's keys are rows row0 .. row0 + 63; otherwise every lane looks its row up.
+template <int D, int NW = 4, bool ROWS = false>
+__device__ __forceinline__ void issue_tile(const AttnParams& p, unsigned buf, int kt, int row0, int kvh, int w, int lane, unsigned lane_k, unsigned lane_v) {
     using G = Geo<D>;
     constexpr int IPW = G::NREG / NW;   // DMA instructions per wave and tile
     static_assert(IPW >= 1 && IPW * NW == G::NREG, "the tile's regions must divide among the waves");
     const char* kbase = (const char*)(p.k + (long)kvh * p.k_head);
     const char* vbase = (const char*)(p.v + (long)kvh * p.v_head);
-    if (kt * 64 + 64 <= p.n) {
+    if (ROWS ? row0 >= 0 : kt * 64 + 64 <= p.n) {
 #pragma unroll
         for (int i = 0; i < IPW; i++) {
             const int reg = w * IPW + i;
-            const long row = (long)kt * 64 + reg;
+            const long row = (ROWS ? (long)row0 : (long)kt * 64) + reg;
             dma16_uniform(kbase + row * p.k_tok * 2, lane_k, buf + reg * G::KRS);
             dma16_uniform(vbase + row * p.v_tok * 2, lane_v, buf + G::KTILEB + reg * G::VRS);
         }
@@ -151,6 +155,10 @@ __device__ __forceinline__ void issue_tile(const AttnParams& p, unsigned buf, in
             const int reg = w * IPW + i;
             long grow = (long)kt * 64 + reg + G::NREG * slot;
             grow = grow < p.n ? grow : p.n - 1;
+            if (ROWS) {   // a pad position has no row: any row will do, its keys are visible to nobody but pad rows
+                const int r = p.row_of[grow];
+                grow = r < 0 ? 0 : r;
+            }
             dma16_lane(kbase + grow * p.k_tok * 2 + chunk * 16, buf + reg * G::KRS);
             dma16_lane(vbase + grow * p.v_tok * 2 + chunk * 16, buf + G::KTILEB + reg * G::VRS);
         }
@@ -227,13 +235,21 @@ __device__ __forceinline__ int fresh_lane_id() {
 
 // normalise O^T and store it as rows: each wave stages 32 rows x 64 head dims at a time in its own LDS slice (144-byte
 // rows) and writes them out as 16-byte pieces, 8 lanes per 128-byte row segment
-template <int D, int RT>
+template <int D, int RT, bool ROWS = false>
 __device__ __forceinline__ void store_rows(const AttnParams& p, const Lane<D>& L, char* stage, const f32x16 (&o)[RT][D / 32], const float (&l)[RT],
                                            int t, int h0) {
     constexpr int NDT = D / 32;
     constexpr int SROW = 128 + 16;
     const int tok0 = t * SPINF_QTILE + 32 * L.wr;
     const int lane = fresh_lane_id(), m = lane & 31, g = lane >> 5;
+    int orow[4] = {0, 0, 0, 0};   // compact rows: row of the four tokens this lane stores pieces of, -1 for a pad position
+    if (ROWS) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int tok = tok0 + ((j * 64 + lane) >> 3);
+            orow[j] = tok < p.n ? p.row_of[tok] : -1;
+        }
+    }
 #pragma unroll
     for (int rt = 0; rt < RT; rt++) {
         const float inv = 1.0f / lane32_sum(l[rt]);
@@ -253,7 +269,11 @@ __device__ __forceinline__ void store_rows(const AttnParams& p, const Lane<D>& L
             for (int j = 0; j < 4; j++) {
                 const int c = j * 64 + lane, row = c >> 3, col = c & 7;
                 const bf16x8 val = *(const bf16x8*)(stage + row * SROW + col * 16);
-                if (tok0 + row < p.n) *(bf16x8*)(ob + (long)(tok0 + row) * p.o_tok + 64 * qd + col * 8) = val;
+                if (ROWS) {
+                    if (orow[j] >= 0) *(bf16x8*)(ob + (long)orow[j] * p.o_tok + 64 * qd + col * 8) = val;
+                } else {
+                    if (tok0 + row < p.n) *(bf16x8*)(ob + (long)(tok0 + row) * p.o_tok + 64 * qd + col * 8) = val;
+                }
             }
         }
     }
@@ -263,8 +283,8 @@ __device__ __forceinline__ void store_rows(const AttnParams& p, const Lane<D>& L
 // Classic online softmax over one work item, one 32-key block at a time, nothing overlapped: the rare fallback, in a
 // kernel of its own because its accumulator rescaling (vector ALU on all of O) would cost the fast pass its register
 // allocation.
-template <int D, int RT, bool WIN>
-__device__ __forceinline__ void attn_item_exact(const AttnParams& p, const int4 item, const int h0, char* buf0, int2* ent, char* stage) {
+template <int D, int RT, bool WIN, bool ROWS>
+__device__ __forceinline__ void attn_item_exact(const AttnParams& p, const int4 item, const int h0, char* buf0, int2* ent, int* ent_row0, char* stage) {
     using G = Geo<D>;
     constexpr int NS = D / 16, NDT = D / 32;
     const Lane<D> L(p);
@@ -272,10 +292,15 @@ __device__ __forceinline__ void attn_item_exact(const AttnParams& p, const int4 
     const int kvh = h0 / p.group;
     const int tok = t * SPINF_QTILE + 32 * L.w + L.m;
     const int tok_c = tok < p.n ? tok : p.n - 1;
+    int q_row = tok_c;
+    if (ROWS) {   // a pad position has no row: it computes on some row's queries and stores nothing
+        q_row = p.row_of[tok_c];
+        q_row = q_row < 0 ? 0 : q_row;
+    }
     bf16x8 qf[RT][NS];
 #pragma unroll
     for (int rt = 0; rt < RT; rt++) {
-        const __bf16* qp = p.q + (long)tok_c * p.q_tok + (long)(h0 + rt) * p.q_head + 8 * L.g;
+        const __bf16* qp = p.q + (long)q_row * p.q_tok + (long)(h0 + rt) * p.q_head + 8 * L.g;
 #pragma unroll
         for (int s = 0; s < NS; s++) qf[rt][s] = *(const bf16x8*)(qp + 16 * s);
     }
@@ -294,20 +319,27 @@ __device__ __forceinline__ void attn_item_exact(const AttnParams& p, const int4 
     }
     int base = 0;
     __syncthreads();
-    if ((int)threadIdx.x < ne) ent[threadIdx.x] = make_int2(p.kv_idx[e0 + threadIdx.x], (int)p.kv_bits[e0 + threadIdx.x]);
+    if ((int)threadIdx.x < ne) {
+        ent[threadIdx.x] = make_int2(p.kv_idx[e0 + threadIdx.x], (int)p.kv_bits[e0 + threadIdx.x]);
+        if (ROWS) ent_row0[threadIdx.x] = p.kv_row0[e0 + threadIdx.x];
+    }
     __syncthreads();
     for (int i = 0; i < ne; i++) {
         if (i - base >= ENT_CAP) {
             __syncthreads();
             base = i;
-            if (i + (int)threadIdx.x < ne) ent[threadIdx.x] = make_int2(p.kv_idx[e0 + i + threadIdx.x], (int)p.kv_bits[e0 + i + threadIdx.x]);
+            if (i + (int)threadIdx.x < ne) {
+                ent[threadIdx.x] = make_int2(p.kv_idx[e0 + i + threadIdx.x], (int)p.kv_bits[e0 + i + threadIdx.x]);
+                if (ROWS) ent_row0[threadIdx.x] = p.kv_row0[e0 + i + threadIdx.x];
+            }
             __syncthreads();
         }
         const int2 en = ent[i - base];
         const int kt = __builtin_amdgcn_readfirstlane(en.x);
         const unsigned bits = (unsigned)__builtin_amdgcn_readfirstlane(en.y) >> (2 * L.w);
+        const int row0 = ROWS ? __builtin_amdgcn_readfirstlane(ent_row0[i - base]) : 0;
         __syncthreads();   // everyone is done with the buffer
-        issue_tile<D>(p, lds_addr(buf0), kt, kvh, L.w, L.lane, L.lane_k, L.lane_v);
+        issue_tile<D, 4, ROWS>(p, lds_addr(buf0), kt, row0, kvh, L.w, L.lane, L.lane_k, L.lane_v);
         __builtin_amdgcn_s_waitcnt(0x0f70);
         __syncthreads();
         const char* kb = buf0;
@@ -370,15 +402,16 @@ __device__ __forceinline__ void attn_item_exact(const AttnParams& p, const int4 
             }
         }
     }
-    store_rows<D, RT>(p, L, stage, o, l, t, h0);
+    store_rows<D, RT, ROWS>(p, L, stage, o, l, t, h0);
 }
 
 // An item of HPI heads is recomputed RT heads at a time.
-template <int D, int RT, bool WIN, int HPI>
+template <int D, int RT, bool WIN, int HPI, bool ROWS>
 __global__ __launch_bounds__(256) void tree_attn_exact_kernel(const AttnParams p) {
     using G = Geo<D>;
     __shared__ __attribute__((aligned(16))) char buf0[G::BUFB];
     __shared__ int2 ent[ENT_CAP];
+    __shared__ int ent_row0[ROWS ? ENT_CAP : 1];
     __shared__ __attribute__((aligned(16))) char stage_all[4 * 32 * 144];
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int n_redo = p.counters[NLIST + 1];
@@ -388,7 +421,7 @@ __global__ __launch_bounds__(256) void tree_attn_exact_kernel(const AttnParams p
         const int4 item = make_int4(__builtin_amdgcn_readfirstlane(it.x), __builtin_amdgcn_readfirstlane(it.y),
                                     __builtin_amdgcn_readfirstlane(it.z), __builtin_amdgcn_readfirstlane(it.w));
         const int hp = (int)((unsigned)item.z >> 20);
-        for (int sub = 0; sub < HPI; sub += RT) attn_item_exact<D, RT, WIN>(p, item, hp * HPI + sub, buf0, ent, stage_all + w * 32 * 144);
+        for (int sub = 0; sub < HPI; sub += RT) attn_item_exact<D, RT, WIN, ROWS>(p, item, hp * HPI + sub, buf0, ent, ent_row0, stage_all + w * 32 * 144);
     }
     __builtin_amdgcn_s_waitcnt(0x0f70);
     __syncthreads();
@@ -420,7 +453,8 @@ extern "C" int spinf_debug_trace(long* out, int n) { return (int)hipMemcpyFromSy
 
 // NHW = 1: four waves, each with RT heads of the item.  NHW = 2: eight waves, waves 4..7 take the item's second set of RT heads
 // on the same K / V tiles (two waves per SIMD: one wave's softmax runs under the other's MFMAs).
-template <int D, int RT, bool WIN, int NHW>
+// ROWS: q, k, v, o hold the real tokens only (compact rows); the stream positions of the plan are mapped through row_of.
+template <int D, int RT, bool WIN, int NHW, bool ROWS>
 __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p) {
     using G = Geo<D>;
     constexpr int HPI = RT * NHW;  // heads per work item
@@ -435,6 +469,8 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
     __shared__ __attribute__((aligned(16))) char bufs[2 * G::BUFB];   // the two tile buffers
     __shared__ int2 ent_a[ENT_CAP];   // (key tile, bits) of the current item's plan entries base .. base + ENT_CAP - 1
     __shared__ int2 ent_b[ENT_CAP];   // first entries of the next item
+    __shared__ int entr_a[ROWS ? ENT_CAP : 1];   // compact rows: first row of each entry's key tile, alongside ent_a / ent_b
+    __shared__ int entr_b[ROWS ? ENT_CAP : 1];
     // output staging, one slice per wave; with eight waves at head dim 256 there is no room left for it and the slices lie in
     // the tile buffer the item's last tile was computed from (free from the barrier after the tile loop until the next
     // item's first tile step requests a tile into it, which comes after that step's barrier)
@@ -477,6 +513,9 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
     bool viol = false;
     int2* ent_cur = ent_a;
     int2* ent_nxt = ent_b;
+    int* entr_cur = entr_a;
+    int* entr_nxt = entr_b;
+    int nxt_row0 = 0;   // compact rows: first row of the next item's first key tile
 
     auto uniform4 = [](const int4 v) __attribute__((always_inline)) {   // the same value in every lane: keep it in scalar registers
         return make_int4(__builtin_amdgcn_readfirstlane(v.x), __builtin_amdgcn_readfirstlane(v.y), __builtin_amdgcn_readfirstlane(v.z),
@@ -491,19 +530,26 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
         const int tok = item_t(it) * SPINF_QTILE + 32 * L.wr + (lane & 31);
         const int tok_c = tok < p.n ? tok : p.n - 1;
         const int h0 = item_hp(it) * HPI + L.wh * RT;
+        int q_row = tok_c;
+        if (ROWS) {   // a pad position has no row: it computes on some row's queries and stores nothing
+            q_row = p.row_of[tok_c];
+            q_row = q_row < 0 ? 0 : q_row;
+        }
 #pragma unroll
         for (int rt = 0; rt < RT; rt++) {
-            const __bf16* qp = p.q + (long)tok_c * p.q_tok + (long)(h0 + rt) * p.q_head + 8 * (lane >> 5);
+            const __bf16* qp = p.q + (long)q_row * p.q_tok + (long)(h0 + rt) * p.q_head + 8 * (lane >> 5);
 #pragma unroll
             for (int s = 0; s < NS; s++) dst[rt][s] = *(const bf16x8*)(qp + 16 * s);
         }
         a_q = tok < p.n ? p.art[tok_c] : -1;
         p_q = WIN ? p.pos[tok_c] : 0;
     };
-    auto load_ent = [&](const int4& it, int2* dst, const int from) __attribute__((always_inline)) {
+    auto load_ent = [&](const int4& it, int2* dst, int* dst_row0, const int from) __attribute__((always_inline)) {
         const int ne = item_ne(it);
-        if ((int)threadIdx.x < ENT_CAP && from + (int)threadIdx.x < ne)
+        if ((int)threadIdx.x < ENT_CAP && from + (int)threadIdx.x < ne) {
             dst[threadIdx.x] = make_int2(p.kv_idx[it.y + from + threadIdx.x], (int)p.kv_bits[it.y + from + threadIdx.x]);
+            if (ROWS) dst_row0[threadIdx.x] = p.kv_row0[it.y + from + threadIdx.x];
+        }
     };
     auto reset_acc = [&]() __attribute__((always_inline)) {
 #pragma unroll
@@ -614,8 +660,9 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
     }
     if (cur_ok) {
         load_q(cur, qf, art_q, pos_q);
-        load_ent(cur, ent_cur, 0);
-        if (L.wh == 0) issue_tile<D, 4>(p, lds_addr(bufs), cur.w, item_hp(cur) * HPI / p.group, L.w, L.lane, L.lane_k, L.lane_v);
+        load_ent(cur, ent_cur, entr_cur, 0);
+        const int row0 = ROWS ? __builtin_amdgcn_readfirstlane(p.kv_row0[cur.y]) : 0;
+        if (L.wh == 0) issue_tile<D, 4, ROWS>(p, lds_addr(bufs), cur.w, row0, item_hp(cur) * HPI / p.group, L.w, L.lane, L.lane_k, L.lane_v);
     }
     // The item after the current one is fetched from the lists as late as the prefetch pipeline allows (three tile steps
     // before the current item ends; at once for items shorter than that): an item fetched long before it starts keeps the
@@ -663,20 +710,23 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
                 nxt_idx = __builtin_amdgcn_readfirstlane(s_next[gslot]);
                 nxt_ok = nxt_idx >= 0;
                 if (nxt_ok) nxt = uniform4(p.items[nxt_idx]);
+                if (ROWS && nxt_ok) nxt_row0 = __builtin_amdgcn_readfirstlane(p.kv_row0[nxt.y]);
                 pstage = 1;
             } else if (pstage == 1) {
-                if (nxt_ok) load_ent(nxt, ent_nxt, 0);
+                if (nxt_ok) load_ent(nxt, ent_nxt, entr_nxt, 0);
                 pstage = 2;
             }
             if (i + 1 - base >= ENT_CAP) {       // slide the window of plan entries (uniform; long key lists only)
                 base = i;
-                load_ent(cur, ent_cur, i);
+                load_ent(cur, ent_cur, entr_cur, i);
                 __syncthreads();
             }
             if (i + 1 < ne) {
-                if (L.wh == 0) issue_tile<D, 4>(p, oth, __builtin_amdgcn_readfirstlane(ent_cur[i + 1 - base].x), kvh, L.w, L.lane, L.lane_k, L.lane_v);
+                const int row0 = ROWS ? __builtin_amdgcn_readfirstlane(entr_cur[i + 1 - base]) : 0;
+                if (L.wh == 0)
+                    issue_tile<D, 4, ROWS>(p, oth, __builtin_amdgcn_readfirstlane(ent_cur[i + 1 - base].x), row0, kvh, L.w, L.lane, L.lane_k, L.lane_v);
             } else if (nxt_ok) {
-                if (L.wh == 0) issue_tile<D, 4>(p, oth, nxt.w, item_hp(nxt) * HPI / p.group, L.w, L.lane, L.lane_k, L.lane_v);
+                if (L.wh == 0) issue_tile<D, 4, ROWS>(p, oth, nxt.w, nxt_row0, item_hp(nxt) * HPI / p.group, L.w, L.lane, L.lane_k, L.lane_v);
                 pstage = pstage == 2 ? 3 : -1;   // -1: tile requested before the entries (one-tile items)
             }
             const int2 en = ent_cur[i - base];
@@ -694,7 +744,7 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
         } else {
             // (the loop has already flipped par: the last tile came from buffer par ^ 1)
             char* const stage = STAGE_IN_TILE ? bufs + (par ^ 1) * G::BUFB + L.w * 32 * 144 : stage_own;
-            store_rows<D, RT>(p, L, stage, o, l, item_t(cur), item_hp(cur) * HPI + L.wh * RT);
+            store_rows<D, RT, ROWS>(p, L, stage, o, l, item_t(cur), item_hp(cur) * HPI + L.wh * RT);
         }
         TRACE_CLK(tc4);
         TRACE_ADD(10, tc4 - tc3);
@@ -706,11 +756,12 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
         cur_ok = nxt_ok;
         if (!cur_ok) break;
         // finish whatever of the next item's prefetch has not happened yet (one-tile items), then switch
-        if (pstage == -1) load_ent(nxt, ent_nxt, 0);
+        if (pstage == -1) load_ent(nxt, ent_nxt, entr_nxt, 0);
         cur = nxt;
         cur_idx = nxt_idx;
         load_q(cur, qf, art_q, pos_q);
         { int2* tmp = ent_cur; ent_cur = ent_nxt; ent_nxt = tmp; }
+        { int* tmp = entr_cur; entr_cur = entr_nxt; entr_nxt = tmp; }
         gslot ^= 1;
         if (grab_step(item_ne(cur)) < 0) grab(gslot);   // short item: fetch its successor now; read at the next tile step's barrier
     }
@@ -768,15 +819,15 @@ int device_state(DeviceState** out, long n_items) {
     return SPINF_OK;
 }
 
-template <int D, int RT, bool WIN, int NHW = 1>
+template <int D, int RT, bool WIN, int NHW, bool ROWS>
 int launch(const AttnParams& p, int blocks, hipStream_t stream) {
     using G = Geo<D>;
-    static_assert(2 * G::BUFB + 2 * ENT_CAP * 8 + ((NHW == 2 && D == 256) ? 16 : 4 * NHW * 32 * 144) + 64 <= 160 * 1024, "LDS budget");
-    hipLaunchKernelGGL((tree_attn_kernel<D, RT, WIN, NHW>), dim3(blocks), dim3(256 * NHW), 0, stream, p);
+    static_assert(2 * G::BUFB + 2 * ENT_CAP * 12 + ((NHW == 2 && D == 256) ? 16 : 4 * NHW * 32 * 144) + 64 <= 160 * 1024, "LDS budget");
+    hipLaunchKernelGGL((tree_attn_kernel<D, RT, WIN, NHW, ROWS>), dim3(blocks), dim3(256 * NHW), 0, stream, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: launch: %s", hipGetErrorString(e));
     // the exact pass over whatever the fast pass handed on (normally nothing: its workgroups read a zero count and leave)
-    hipLaunchKernelGGL((tree_attn_exact_kernel<D, RT, WIN, RT * NHW>), dim3(blocks < 64 ? blocks : 64), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((tree_attn_exact_kernel<D, RT, WIN, RT * NHW, ROWS>), dim3(blocks < 64 ? blocks : 64), dim3(256), 0, stream, p);
     e = hipGetLastError();
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: launch (exact pass): %s", hipGetErrorString(e));
     return SPINF_OK;
@@ -796,11 +847,15 @@ void pick_kernel(int hq, int hkv, int d, int variant, int* rt, int* nhw) {
 
 template <int D>
 int launch_d(const AttnParams& p, int rt, int nhw, bool win, int blocks, hipStream_t s) {
-    if (nhw == 2) return win ? launch<D, 1, true, 2>(p, blocks, s) : launch<D, 1, false, 2>(p, blocks, s);
-    if constexpr (D <= 128) {
-        if (rt == 2) return win ? launch<D, 2, true>(p, blocks, s) : launch<D, 2, false>(p, blocks, s);
+    if (p.row_of) {   // compact rows: the one-head-per-wave kernels only
+        if (nhw == 2) return win ? launch<D, 1, true, 2, true>(p, blocks, s) : launch<D, 1, false, 2, true>(p, blocks, s);
+        return win ? launch<D, 1, true, 1, true>(p, blocks, s) : launch<D, 1, false, 1, true>(p, blocks, s);
     }
-    return win ? launch<D, 1, true>(p, blocks, s) : launch<D, 1, false>(p, blocks, s);
+    if (nhw == 2) return win ? launch<D, 1, true, 2, false>(p, blocks, s) : launch<D, 1, false, 2, false>(p, blocks, s);
+    if constexpr (D <= 128) {
+        if (rt == 2) return win ? launch<D, 2, true, 1, false>(p, blocks, s) : launch<D, 2, false, 1, false>(p, blocks, s);
+    }
+    return win ? launch<D, 1, true, 1, false>(p, blocks, s) : launch<D, 1, false, 1, false>(p, blocks, s);
 }
 
 }  // namespace
@@ -838,6 +893,8 @@ extern "C" int spinf_tree_attn_fwd(const spinf_attn_args* a, void* stream) {
     if (!(a->scale > 0.f)) return spinf_fail(SPINF_E_ARG, "tree_attn: scale must be positive");
     int rt, nhw;
     pick_kernel(a->hq, a->hkv, a->d, a->variant, &rt, &nhw);
+    if ((a->row_of != nullptr) != (a->kv_row0 != nullptr)) return spinf_fail(SPINF_E_ARG, "tree_attn: row_of and kv_row0 come together");
+    if (a->row_of && rt != 1) return spinf_fail(SPINF_E_ARG, "tree_attn: variant %d does not take compact rows", a->variant);
     const int hpi = rt * nhw;
     const int64_t nqt = (a->n + SPINF_QTILE - 1) / SPINF_QTILE;
     if (a->n_items != nqt * (a->hq / hpi))
@@ -861,6 +918,7 @@ extern "C" int spinf_tree_attn_fwd(const spinf_attn_args* a, void* stream) {
     p.art = a->art; p.end = a->end; p.pos = a->pos;
     p.kv_idx = a->kv_idx; p.kv_bits = a->kv_bits;
     p.items = (const int4*)a->items; p.list_ptr = a->list_ptr;
+    p.row_of = a->row_of; p.kv_row0 = a->kv_row0;
     p.counters = st->counters;
     p.redo = st->counters + 64;
     const int blocks = (int)(a->n_items < st->cus ? a->n_items : st->cus);

@@ -23,6 +23,7 @@ class AttnArgs(C.Structure):
         ("art", C.c_void_p), ("end", C.c_void_p), ("pos", C.c_void_p),
         ("kv_idx", C.c_void_p), ("kv_bits", C.c_void_p), ("items", C.c_void_p), ("list_ptr", C.c_void_p),
         ("n_items", C.c_int64), ("variant", C.c_int32),
+        ("row_of", C.c_void_p), ("kv_row0", C.c_void_p),
     ]
 
 
@@ -58,12 +59,13 @@ def load_library():
     lib.spinf_tileplan_schedule.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p]
     lib.spinf_attn_heads_per_item.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_int32]
     lib.spinf_attn_heads_per_item.restype = C.c_int
+    lib.spinf_tileplan_row0.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
     lib.spinf_tileplan_free.argtypes = [C.c_void_p]
     lib.spinf_tileplan_free.restype = None
     lib.spinf_tree_attn_fwd.argtypes = [C.POINTER(AttnArgs), C.c_void_p]
     lib.spinf_attn_exact_items.argtypes = [C.POINTER(C.c_int64)]
     lib.spinf_gdn_fwd.argtypes = [C.POINTER(GdnArgs), C.c_void_p]
-    for name in ("spinf_tileplan_build", "spinf_tileplan_counts", "spinf_tileplan_export", "spinf_tileplan_schedule", "spinf_tree_attn_fwd", "spinf_attn_exact_items", "spinf_gdn_fwd"):
+    for name in ("spinf_tileplan_build", "spinf_tileplan_counts", "spinf_tileplan_export", "spinf_tileplan_schedule", "spinf_tileplan_row0", "spinf_tree_attn_fwd", "spinf_attn_exact_items", "spinf_gdn_fwd"):
         getattr(lib, name).restype = C.c_int
     _LIB = lib
     return lib

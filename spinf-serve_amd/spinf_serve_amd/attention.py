@@ -12,6 +12,7 @@ from __future__ import annotations
 
 import ctypes as C
 import os
+from typing import Optional
 
 import torch
 
@@ -26,21 +27,35 @@ VARIANT = int(os.environ.get("SPINF_ATTN_VARIANT", "0"))
 @torch.library.custom_op("spinf::tree_attn", mutates_args=())
 def _tree_attn_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, art: torch.Tensor, end: torch.Tensor, pos: torch.Tensor,
                   kv_idx: torch.Tensor, kv_bits: torch.Tensor, items: torch.Tensor, list_ptr: torch.Tensor, n_items: int,
-                  scale: float, window: int, variant: int) -> torch.Tensor:
-    """q [n, hq, d], k / v [n, hkv, d] (any token / head strides, d contiguous) -> out [n, hq, d] contiguous, bf16."""
+                  scale: float, window: int, variant: int, row_of: Optional[torch.Tensor], kv_row0: Optional[torch.Tensor],
+                  n_mapped: int) -> torch.Tensor:
+    """q [rows, hq, d], k / v [rows, hkv, d] (any token / head strides, d contiguous) -> out [rows, hq, d] contiguous, bf16.
+    rows = the stream length, or with row_of / kv_row0 (compact rows) any number of rows: the kernel maps stream positions to
+    rows through row_of; rows 0 .. n_mapped-1 are the rows row_of names (each written by the kernel), later rows come back zero."""
     if not q.is_cuda:
         raise RuntimeError("spinf::tree_attn runs on ROCm device tensors only (no CPU path)")
     if q.dtype != torch.bfloat16 or k.dtype != torch.bfloat16 or v.dtype != torch.bfloat16:
         raise ValueError("spinf::tree_attn takes bf16 q, k, v")
-    n, hq, d = q.shape
+    rows, hq, d = q.shape
     hkv = k.shape[1]
-    if k.shape != (n, hkv, d) or v.shape != (n, hkv, d):
+    if k.shape != (rows, hkv, d) or v.shape != (rows, hkv, d):
         raise ValueError(f"k / v shapes {tuple(k.shape)} {tuple(v.shape)} do not match q {tuple(q.shape)}")
     if q.stride(2) != 1 or k.stride(2) != 1 or v.stride(2) != 1:
         raise ValueError("the head dimension must be contiguous")
+    n = art.numel() if row_of is not None else rows
     if art.numel() < n:
         raise ValueError(f"mask built for {art.numel()} tokens, stream has {n}")
-    out = torch.empty((n, hq, d), dtype=torch.bfloat16, device=q.device)
+    if (row_of is None) != (kv_row0 is None):
+        raise ValueError("row_of and kv_row0 come together")
+    if row_of is not None:
+        if row_of.dtype != torch.int32 or kv_row0.dtype != torch.int32 or row_of.numel() != n or kv_row0.numel() != kv_idx.numel():
+            raise ValueError("row_of [n] and kv_row0 [entries] must be int32")
+        if not 0 <= n_mapped <= rows:
+            raise ValueError(f"{n_mapped} mapped rows, q has {rows}")
+        out = torch.empty((rows, hq, d), dtype=torch.bfloat16, device=q.device)
+        out[n_mapped:].zero_()
+    else:
+        out = torch.empty((rows, hq, d), dtype=torch.bfloat16, device=q.device)
     a = _lib.AttnArgs()
     a.q, a.k, a.v, a.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
     a.q_tok, a.q_head = q.stride(0), q.stride(1)
@@ -52,6 +67,8 @@ def _tree_attn_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, art: torch.
     a.kv_idx, a.kv_bits, a.items, a.list_ptr = kv_idx.data_ptr(), kv_bits.data_ptr(), items.data_ptr(), list_ptr.data_ptr()
     a.n_items = n_items
     a.variant = variant
+    if row_of is not None:
+        a.row_of, a.kv_row0 = row_of.data_ptr(), kv_row0.data_ptr()
     lib = _lib.load_library()
     with torch.cuda.device(q.device):
         stream = torch.cuda.current_stream(q.device).cuda_stream
@@ -60,25 +77,32 @@ def _tree_attn_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, art: torch.
 
 
 @_tree_attn_op.register_fake
-def _(q, k, v, art, end, pos, kv_idx, kv_bits, items, list_ptr, n_items, scale, window, variant):
+def _(q, k, v, art, end, pos, kv_idx, kv_bits, items, list_ptr, n_items, scale, window, variant, row_of, kv_row0, n_mapped):
     return torch.empty(q.shape, dtype=torch.bfloat16, device=q.device)
 
 
-def tree_attn(q, k, v, mask: TreeMask, scale=None, variant=None):
-    """q [n, hq, d], k / v [n, hkv, d] bf16 -> [n, hq, d]: softmax(scale q k^T under the tree mask) v."""
+def tree_attn(q, k, v, mask: TreeMask, scale=None, variant=None, sidx=None):
+    """q [n, hq, d], k / v [n, hkv, d] bf16 -> [n, hq, d]: softmax(scale q k^T under the tree mask) v.
+    sidx [R] (compact rows): q, k, v hold real tokens only, row r is stream position sidx[r]; the kernel reads and writes them
+    in place of the scatter into stream layout and the gather back (rows >= R come back zero)."""
     if not isinstance(mask, TreeMask):
         raise TypeError("attention_mask must be a TreeMask (masks.block_masks)")
-    if q.shape[0] != mask.n:
+    if sidx is None and q.shape[0] != mask.n:
         raise ValueError(f"mask describes {mask.n} tokens, q has {q.shape[0]}")
+    if sidx is not None and sidx.shape[0] > q.shape[0]:
+        raise ValueError(f"sidx names {sidx.shape[0]} rows, q has {q.shape[0]}")
     scale = float(q.shape[-1] ** -0.5 if scale is None else scale)
     variant = int(VARIANT if variant is None else variant)
+    if sidx is not None and variant == 2:
+        variant = 0   # the two-heads-per-wave kernels do not take compact rows
     hq, hkv, d = q.shape[1], k.shape[1], q.shape[2]
     per_item = _lib.load_library().spinf_attn_heads_per_item(hq, hkv, d, variant)
     if per_item <= 0:
         raise ValueError(f"{hq} query heads do not group over {hkv} key / value heads")
     items, list_ptr, n_items = mask.schedule(hq // per_item)
+    row_of, kv_row0 = mask.rows(sidx) if sidx is not None else (None, None)
     return _tree_attn_op(q, k, v, mask.art, mask.end, mask.pos, mask.kv_idx, mask.kv_bits, items, list_ptr, n_items,
-                         scale, int(mask.window), variant)
+                         scale, int(mask.window), variant, row_of, kv_row0, 0 if sidx is None else int(sidx.shape[0]))
 
 
 # K/V capture for extraction, as spinf_serve/models/gemma4.py:66-70: while CAPTURE[device] = {"window", "ranges": [(start, n, key)],
@@ -114,8 +138,9 @@ def register_tree_attention(name: str = "tree_flex") -> None:
 @torch.compiler.disable
 def tree_attention(q, k, v, mask, scale, sidx=None, plan=None, mod=None):
     """q [1, H, rows, d], k / v [1, Hkv, rows, d] -> [1, H, rows, d]   (spinf_serve/models/qwen35/qwen.py:604-623).
-    sidx (compact rows): stream position of each real row; rows are scattered into the stream layout the mask describes
-    (pads: zero rows attending to themselves) and the output gathered back."""
+    sidx (compact rows): stream position of each real row.  The reference scatters the rows into the stream layout the mask
+    describes (pads: zero rows attending to themselves) and gathers the output back; here the kernel goes through the row map
+    and the result for every real row is the same bit for bit."""
     cap = plan.cap if plan is not None else None
     if cap is not None:
         for r0, n, name in cap["ranges"]:
@@ -123,14 +148,6 @@ def tree_attention(q, k, v, mask, scale, sidx=None, plan=None, mod=None):
     if sidx is None:
         o = tree_attn(q[0].transpose(0, 1), k[0].transpose(0, 1), v[0].transpose(0, 1), mask, scale)
         return o.transpose(0, 1)[None]
-    T, R = mask.seq_lengths[0], sidx.shape[0]
-
-    def up(t):  # [1, h, rows, d] -> token-major stream layout [T, h, d]
-        s = t.new_zeros(T, t.shape[1], t.shape[3])
-        s.index_copy_(0, sidx, t[0, :, :R].transpose(0, 1))
-        return s
-
-    o = tree_attn(up(q), up(k), up(v), mask, scale)
-    out = q.new_zeros(q.shape)
-    out[0, :, :R] = o.index_select(0, sidx).transpose(0, 1)
-    return out
+    # compact rows: the kernel maps stream positions to rows itself (no scatter into stream layout, no gather back)
+    o = tree_attn(q[0].transpose(0, 1), k[0].transpose(0, 1), v[0].transpose(0, 1), mask, scale, sidx=sidx)
+    return o.transpose(0, 1)[None]

@@ -97,6 +97,26 @@ class TreeMask:
         self.kv_idx = _upload(plan.kv_idx if len(plan.kv_idx) else one, np.int32, device)
         self.kv_bits = _upload((plan.kv_bits if len(plan.kv_bits) else one.view(np.uint32)).view(np.int32), np.int32, device)
         self._sched = {}
+        self._rows = None
+
+    def rows(self, sidx):
+        """compact rows (spinf_serve/models/qwen35/qwen.py:613-622): sidx [R] = stream position of each real row (a device
+        tensor) -> (row_of [n], kv_row0 [entries]) int32 device tensors for the kernel: the row of each stream position (-1:
+        pad) and, per plan entry, the row of its first key where its 64 keys are consecutive rows (else -1).  Kept for the
+        sidx tensor it was built from (one forward: every layer passes the same tensor)."""
+        import torch
+
+        if self._rows is not None and self._rows[0] is sidx:
+            return self._rows[1], self._rows[2]
+        n = self.n
+        row_of = torch.full((n + 63,), -1, dtype=torch.int32, device=self.device)   # padded: every key tile is 64 long
+        row_of[sidx.to(self.device, torch.long)] = torch.arange(sidx.shape[0], dtype=torch.int32, device=self.device)
+        tiles = row_of[: (n + 63) // 64 * 64].view(-1, 64)
+        run = (tiles - tiles[:, :1]) == torch.arange(64, dtype=torch.int32, device=self.device)
+        tile_row0 = torch.where((tiles[:, 0] >= 0) & run.all(1), tiles[:, 0], torch.full_like(tiles[:, 0], -1))
+        kv_row0 = tile_row0[self.kv_idx.long()].contiguous()
+        self._rows = (sidx, row_of[:n].contiguous(), kv_row0)
+        return self._rows[1], self._rows[2]
 
     def schedule(self, head_groups: int):
         """device copy of the work lists for this many head groups (built on first use, then kept)"""

@@ -214,6 +214,82 @@ def test_reference_call_signatures(dev):
     assert (o3[0, :, len(real):] == 0).all()
 
 
+def _compact_case(name):
+    """-> (cfg, batch, window): streams with pads in different places"""
+    rng = np.random.default_rng(21)
+    if name == "c2":          # head dim 256, eight-wave kernel; alignment pads after every job
+        cfg = synth.attention_config("C2", contents=3)
+        return cfg, cfg.batches[0], None
+    if name == "gaps":        # pads INSIDE a job (aligned branch group), head dim 128
+        t = GroupedTree(rng.integers(5, 99, 300).tolist(), [rng.integers(5, 99, n).tolist() for n in (9, 12, 7, 30)], [], [], parents=[-1, -1, -1, -1], aligned=[2])
+        cfg = synth.AttnConfig("gaps", 8, 4, 128, 128 ** -0.5, 1.0, None, [t])
+        return cfg, synth.pack([t])[0], None
+    if name == "dense":       # no alignment: pads only at the end of the stream, head dim 64
+        trees = [synth._tree(rng, 100, [5, 6]), synth._tree(rng, 37, [3]), synth._tree(rng, 260, [11] * 6)]
+        cfg = synth.AttnConfig("dense", 4, 2, 64, 0.125, 1.0, None, trees)
+        return cfg, synth.pack(trees, align=False)[0], None
+    if name == "window":      # sliding layer
+        trees = [synth._tree(rng, 700, [9, 14, 30]), synth._tree(rng, 150, [8])]
+        cfg = synth.AttnConfig("window", 4, 2, 256, 1.0 / 16, 0.5, 200, trees)
+        return cfg, synth.pack(trees)[0], 200
+    trees = [synth._tree(rng, 200, [20, 9]), synth._tree(rng, 90, [7])]   # "mha": three heads, one head per work item
+    cfg = synth.AttnConfig("mha", 3, 3, 128, 128 ** -0.5, 1.0, None, trees)
+    return cfg, synth.pack(trees)[0], None
+
+
+@pytest.mark.parametrize("name", ["c2", "gaps", "dense", "window", "mha"])
+def test_compact_rows_equal_the_stream_layout_call(dev, name):
+    """tree_attention with sidx (spinf_serve/models/qwen35/qwen.py:613-622): q, k, v hold the real rows only.  The reference
+    scatters them into the stream layout (zero rows for pads) and gathers the output back; the kernel's row map must give the
+    same bits for every real row, zero for the rows after them, and must not touch memory of other rows."""
+    cfg, b, window = _compact_case(name)
+    q, k, v = synth.qkv(cfg, b, device=dev)
+    mask = sa.TreeMask.build(b.art, b.end, b.pos, window, device=dev)
+    real = np.flatnonzero(b.art >= 0)
+    sidx = torch.from_numpy(real).to(dev)
+    R = len(real)
+    rows = R + 37   # a few spare rows, as the reference's row buckets have
+    # the reference's way: zero rows at the pad positions of the stream layout
+    zq, zk, zv = (torch.zeros_like(t).index_copy_(0, sidx, t[sidx]) for t in (q, k, v))
+    want = sa.tree_attn(zq, zk, zv, mask, cfg.scale)[sidx]
+    ref = _oracle(zq, zk, zv, b, cfg.scale, window)
+    assert float(np.abs(want.float().cpu().numpy() - ref[real]).max()) <= TOL
+
+    def compact(t):
+        c = torch.full((rows, t.shape[1], t.shape[2]), 7.0, dtype=t.dtype, device=dev)   # spare rows hold junk on purpose
+        c[:R] = t[sidx]
+        return c
+
+    cq, ck, cv = compact(q), compact(k), compact(v)
+    got = sa.tree_attn(cq, ck, cv, mask, cfg.scale, sidx=sidx)
+    assert got.shape == (rows, cfg.hq, cfg.d)
+    assert torch.equal(got[:R], want)
+    assert (got[R:] == 0).all()
+    # through the Qwen stack's function, [1, heads, rows, d] views
+    o = sa.tree_attention(cq.transpose(0, 1)[None], ck.transpose(0, 1)[None], cv.transpose(0, 1)[None], mask, cfg.scale, sidx=sidx)
+    assert o.shape == (1, cfg.hq, rows, cfg.d) and torch.equal(o[0].transpose(0, 1), got)
+
+
+def test_compact_rows_through_the_exact_pass(dev):
+    """the rescaling pass reads and writes through the same row map"""
+    rng = np.random.default_rng(11)
+    trees = [synth._tree(rng, 300, [20, 9]), synth._tree(rng, 90, [7])]
+    cfg = synth.AttnConfig("wide", 4, 2, 128, 128 ** -0.5, 1.0, None, trees)
+    b = synth.pack(trees)[0]
+    q, k, v = synth.qkv(cfg, b, seed=3, device=dev)
+    k = k.clone()
+    k[96:] *= 60.0
+    mask = sa.TreeMask.build(b.art, b.end, b.pos, device=dev)
+    real = np.flatnonzero(b.art >= 0)
+    sidx = torch.from_numpy(real).to(dev)
+    want = sa.tree_attn(q, k, v, mask, cfg.scale)[sidx]
+    before = _exact_items()
+    got = sa.tree_attn(q[sidx].contiguous(), k[sidx].contiguous(), v[sidx].contiguous(), mask, cfg.scale, sidx=sidx)
+    torch.cuda.synchronize()
+    assert _exact_items() > before, "the exact pass did not run"
+    assert torch.equal(got, want)
+
+
 def test_argument_errors(dev):
     cfg = synth.attention_config("smoke")
     b = cfg.batches[0]

@@ -308,6 +308,35 @@ def test_schedule_covers_every_tile_and_head_group_once():
             assert len(compact) == len(set(compact))
 
 
+def test_row_map_of_a_plan_names_the_tiles_that_are_consecutive_rows():
+    """spinf_tileplan_row0: per plan entry, the compact row of the tile's first key where its 64 keys are 64 consecutive rows"""
+    import ctypes as C
+
+    rng = np.random.default_rng(5)
+    t = GroupedTree(rng.integers(5, 99, 300).tolist(), [rng.integers(5, 99, n).tolist() for n in (9, 12, 7, 30)], [], [], parents=[-1, -1, -1, -1], aligned=[2])
+    trees = [t, synth._tree(rng, 200, [20, 9]), synth._tree(rng, 64, [])]
+    b = synth.pack(trees)[0]
+    plan = sa.TilePlan.build(b.art, b.end, b.pos, None)
+    real = np.flatnonzero(b.art >= 0)
+    row_of = np.full(b.length, -1, np.int32)
+    row_of[real] = np.arange(len(real), dtype=np.int32)
+    got = np.full(len(plan.kv_idx), -7, np.int32)
+    lib = sa.load_library()
+    assert lib.spinf_tileplan_row0(plan._handle, row_of.ctypes.data_as(C.c_void_p), got.ctypes.data_as(C.c_void_p)) == 0
+    want = []
+    for kt in plan.kv_idx.tolist():
+        r = row_of[kt * 64 : kt * 64 + 64]
+        want.append(int(r[0]) if len(r) == 64 and r[0] >= 0 and (r == r[0] + np.arange(64)).all() else -1)
+    assert got.tolist() == want
+    assert -1 in want and max(want) > 0            # the case has both kinds of tile
+    # the mask's own (torch) construction of the two arrays agrees
+    import torch
+
+    mask = sa.TreeMask(plan, tuple(torch.from_numpy(np.ascontiguousarray(x)) for x in (b.art, b.end, b.pos)), torch.device("cpu"))
+    r_of, r0 = mask.rows(torch.from_numpy(real))
+    assert r_of.tolist() == row_of.tolist() and r0.tolist() == want
+
+
 def test_a_jobs_plan_does_not_depend_on_its_neighbours():
     """aligned jobs: a job's tile lists, relative to its first tile, are the same alone and packed (the host half of batch
     invariance, tests/test_packer.py:115-134)"""
