@@ -30,13 +30,15 @@ WORKLOADS = {
     "C4": "C4: contents x (8192-token trunk + 16 nodes x 32 + 192 leaves of U{6..10}), 32/16 heads, head_dim 128, one varlen pass",
     "copy": "plain device copy of 1 GiB (reads 1 GiB, writes 1 GiB per launch): the yardstick the FETCH_SIZE / WRITE_SIZE counters are scaled by",
     "C5": "C5: Gated DeltaNet, contents x (2048-token trunk + 32 branches x 12), 16 qk / 32 v heads, 128 x 128 fp32 state",
+    "C5_prologue": "C5's stream through the Gated DeltaNet layer's prologue: path convolution (4 taps) + silu + q/k l2 norm + beta + g from the input projection's rows",
+    "C5_gate": "C5's stream through the Gated DeltaNet layer's output gate: per-head rms norm x norm_w x silu(z)",
 }
 
 
 # HBM bytes per launch of the dominant kernel(s), from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE runs of this file (KiB per
 # dispatch), each scaled by what the same counter reads for `--workload copy` (whose traffic is known).  The figures and the
 # commands are in profiles/*_counters.md; a workload without a counter run has None.
-TRAFFIC_BYTES = {"C2": 800_516_096, "C5": 8_716_861_440}
+TRAFFIC_BYTES = {"C2": 800_516_096, "C5": 8_716_861_440, "C5_prologue": 10_777_077_760, "C5_gate": 7_650_867_200}
 
 
 def timed(fn, steps, warmup, torch):
@@ -98,6 +100,38 @@ def main():
                     config={"workload": WORKLOADS["copy"], "bytes_read": n, "bytes_written": n},
                     roofline={"bound": "hbm", "achieved": 2 * n / (ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                               "frac": 2 * n / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": 2 * n, "kernel_ms": ms})
+        print(json.dumps(line))
+        return
+
+    if args.workload in ("C5_prologue", "C5_gate"):
+        cfg = synth.gdn_config("C5", seed=args.seed, contents=args.contents)
+        plan = cfg.plan(dev)
+        T, h, hv, dk, dv = cfg.batch.length, 16, 32, 128, 128
+        kd, vd = h * dk, hv * dv
+        cd = 2 * kd + vd
+        gen = torch.Generator(device=dev).manual_seed(args.seed)
+        y = torch.randn((T, cd + vd + 2 * hv), generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+        if args.workload == "C5_prologue":
+            conv_w = torch.randn((cd, 4), generator=gen, device=dev) * 0.5
+            a_log = torch.rand(hv, generator=gen, device=dev)
+            dt_bias = torch.randn(hv, generator=gen, device=dev)
+            step = lambda: sa.gdn_prologue(y, plan.conv, conv_w, a_log, dt_bias, h, hv, dk, dv, True)  # noqa: E731
+            nbytes = T * ((cd + 2 * hv) * 2 + 32 + cd * 2 + hv * 6)     # q k v b a columns + taps in; q k v, g, beta out
+        else:
+            o = torch.randn((T, hv, dv), generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+            norm_w = torch.rand(dv, generator=gen, device=dev).to(torch.bfloat16) + 0.5
+            z = y[:, cd : cd + vd]
+            step = lambda: sa.gdn_gate(o, z, norm_w, 1e-6)  # noqa: E731
+            nbytes = T * 3 * vd * 2                                        # o, z in; out
+        wall, kern = timed(step, args.steps, args.warmup, torch)
+        ms = float(np.mean(kern))
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        line.update(metric="stream rows/s, Gated DeltaNet layer element-wise kernel", value=T * args.steps / wall, unit="rows/s",
+                    ms_per_step=1e3 * wall / args.steps, dtype="bf16 (fp32 arithmetic)",
+                    config={"workload": WORKLOADS[args.workload], "contents": len(cfg.trees), "rows": T},
+                    roofline={"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
+                              "traffic": TRAFFIC_BYTES[args.workload] if args.contents is None else None, "kernel_ms": ms,
+                              "algorithmic_bytes": nbytes})
         print(json.dumps(line))
         return
 

@@ -126,6 +126,32 @@ typedef struct spinf_gdn_args {
 
 int spinf_gdn_fwd(const spinf_gdn_args* args, void* stream);
 
+/* ------------------------------------------------------------------------------------------------ Gated DeltaNet layer, around the scan
+ * spinf_gdn_prologue replaces the element-wise work of GatedDeltaNet.forward before the scan
+ * (spinf_serve/models/qwen35/qwen.py:657-668): the 4-tap convolution along each token's path (conv [T, 4]: rows of the
+ * 3 path predecessors and of the token itself, a row index outside 0 .. T-1 = a zero row; weights conv_w [conv_dim, 4] fp32),
+ * silu, the split into q / k / v, with `normalize` the l2 norm x / sqrt(sum x^2 + 1e-6) of q and k per head, beta = sigmoid(b)
+ * and g = -exp(a_log) softplus(a + dt_bias).
+ *   y [T, y_tok] bf16: the input projection's rows, columns q (h dk) | k (h dk) | v (hv dv) | z (hv dv) | b (hv) | a (hv)
+ *   q, k [T, h, dk], v [T, hv, dv], beta [T, hv] bf16 and g [T, hv] fp32: dense outputs.  Values are rounded to bf16 where
+ *   the reference rounds them (after the silu, after the norm).
+ * spinf_gdn_gate replaces qwen.py:670-672 after the scan: out = bf16(norm_w * bf16(rms_norm(o))) * silu(z), rms_norm per
+ * head over dv with eps; o [T, hv, dv] (row stride o_tok), z = the z columns of y (row stride z_tok), out [T, hv dv] dense.
+ */
+typedef struct spinf_gdn_pre_args {
+    const void* y; int64_t y_tok;
+    const int64_t* conv; const float* conv_w; const float* a_log; const float* dt_bias;
+    void* q; void* k; void* v; float* g; void* beta;
+    int64_t T; int32_t h, hv, dk, dv; int32_t normalize;
+} spinf_gdn_pre_args;
+int spinf_gdn_prologue(const spinf_gdn_pre_args* args, void* stream);
+
+typedef struct spinf_gdn_gate_args {
+    const void* o; int64_t o_tok; const void* z; int64_t z_tok; const void* norm_w; float eps;
+    void* out; int64_t T; int32_t hv, dv;
+} spinf_gdn_gate_args;
+int spinf_gdn_gate(const spinf_gdn_gate_args* args, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

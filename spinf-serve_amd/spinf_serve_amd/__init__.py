@@ -16,4 +16,5 @@ from .packer import BLOCK, Batch, GroupedTree, Owner, Packer, ReadPlan, Tree, bu
 from .masks import TreeMask, TilePlan, block_masks  # noqa: F401
 from .attention import CAPTURE, register_tree_attention, tree_attention, tree_attn, tree_flex_forward  # noqa: F401
 from .gdn import chunked, recurrent  # noqa: F401
+from .gdn_layer import gdn_gate, gdn_prologue  # noqa: F401
 from .qwen_plan import Call, TreePlan, gdn_tree, tree_plan  # noqa: F401

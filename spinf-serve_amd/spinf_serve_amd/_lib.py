@@ -27,6 +27,22 @@ class AttnArgs(C.Structure):
     ]
 
 
+class GdnPreArgs(C.Structure):
+    _fields_ = [
+        ("y", C.c_void_p), ("y_tok", C.c_int64),
+        ("conv", C.c_void_p), ("conv_w", C.c_void_p), ("a_log", C.c_void_p), ("dt_bias", C.c_void_p),
+        ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("g", C.c_void_p), ("beta", C.c_void_p),
+        ("T", C.c_int64), ("h", C.c_int32), ("hv", C.c_int32), ("dk", C.c_int32), ("dv", C.c_int32), ("normalize", C.c_int32),
+    ]
+
+
+class GdnGateArgs(C.Structure):
+    _fields_ = [
+        ("o", C.c_void_p), ("o_tok", C.c_int64), ("z", C.c_void_p), ("z_tok", C.c_int64), ("norm_w", C.c_void_p), ("eps", C.c_float),
+        ("out", C.c_void_p), ("T", C.c_int64), ("hv", C.c_int32), ("dv", C.c_int32),
+    ]
+
+
 class GdnArgs(C.Structure):
     _fields_ = [
         ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("g", C.c_void_p), ("beta", C.c_void_p), ("o", C.c_void_p),
@@ -65,7 +81,9 @@ def load_library():
     lib.spinf_tree_attn_fwd.argtypes = [C.POINTER(AttnArgs), C.c_void_p]
     lib.spinf_attn_exact_items.argtypes = [C.POINTER(C.c_int64)]
     lib.spinf_gdn_fwd.argtypes = [C.POINTER(GdnArgs), C.c_void_p]
-    for name in ("spinf_tileplan_build", "spinf_tileplan_counts", "spinf_tileplan_export", "spinf_tileplan_schedule", "spinf_tileplan_row0", "spinf_tree_attn_fwd", "spinf_attn_exact_items", "spinf_gdn_fwd"):
+    lib.spinf_gdn_prologue.argtypes = [C.POINTER(GdnPreArgs), C.c_void_p]
+    lib.spinf_gdn_gate.argtypes = [C.POINTER(GdnGateArgs), C.c_void_p]
+    for name in ("spinf_tileplan_build", "spinf_tileplan_counts", "spinf_tileplan_export", "spinf_tileplan_schedule", "spinf_tileplan_row0", "spinf_tree_attn_fwd", "spinf_attn_exact_items", "spinf_gdn_fwd", "spinf_gdn_prologue", "spinf_gdn_gate"):
         getattr(lib, name).restype = C.c_int
     _LIB = lib
     return lib
