@@ -51,6 +51,11 @@ typedef struct spinf_tileplan spinf_tileplan;
 
 int spinf_tileplan_build(const int32_t* art, const int32_t* end, const int32_t* pos, int64_t n, int32_t window,
                          spinf_tileplan** out);
+/* The same with image groups (spinf_serve/scorer.py:184-198, spinf_serve/packer.py:456-468,485): grp [n], -1 = no group; tokens
+ * of one group also see each other both ways.  grp_mode 1: also past the window (the "unified" checkpoint: every layer);
+ * 2: only within the window (sliding layers of the other checkpoint; its global layers take no groups). */
+int spinf_tileplan_build_groups(const int32_t* art, const int32_t* end, const int32_t* pos, const int32_t* grp, int32_t grp_mode,
+                                int64_t n, int32_t window, spinf_tileplan** out);
 /* counts[0] query tiles, [1] entries, [2] active 32x32 blocks, [3] masked 32x32 blocks, [4] n */
 int spinf_tileplan_counts(const spinf_tileplan* plan, int64_t counts[5]);
 /* qt_ptr [n_qtiles+1], kv_idx [entries], kv_bits [entries], order [n_qtiles]: caller-allocated host arrays */
@@ -76,6 +81,7 @@ void spinf_tileplan_free(spinf_tileplan* plan);
  *   row_of, kv_row0 (both NULL, or both device arrays as spinf_tileplan_row0 describes them): compact rows.  q, k, v, out
  *   then hold the real tokens only; the kernel reads and writes them through row_of instead of the three zero-filled
  *   scatters and the gather of qwen.py:617-622.  Pad positions write nothing.  Results equal the scattered call's bit for bit.
+ *   grp, grp_mode: the image groups the plan was built with (spinf_tileplan_build_groups); stream layout, variant 0 / 1.
  *
  * The kernel is persistent (one workgroup per CU pulling items from the lists) and keeps its list cursors in a small
  * per-device buffer of the library: launches that overlap on one device (different streams) are not supported.
@@ -91,6 +97,7 @@ typedef struct spinf_attn_args {
                           1 = one head per work item, four waves; 2 = four waves with two heads each (head dim <= 128,
                           no compact rows) */
     const int32_t* row_of; const int32_t* kv_row0;
+    const int32_t* grp; int32_t grp_mode;   /* image groups, as given to spinf_tileplan_build_groups (device copy of grp), or NULL */
 } spinf_attn_args;
 
 /* query heads one work item covers for this geometry (1 or 2); 0 for an invalid geometry */

@@ -13,8 +13,10 @@ import numpy as np
 from .layout import BLOCK
 
 
-def dense_tree_mask(art, end, pos=None, window=None):
-    """visible[q, k]: token q attends to token k (scorer.py:173-177).  window: sliding layers add pos[q]-pos[k] < W."""
+def dense_tree_mask(art, end, pos=None, window=None, grp=None, grp_windowed=False):
+    """visible[q, k]: token q attends to token k (scorer.py:173-177).  window: sliding layers add pos[q]-pos[k] < W.
+    grp (scorer.py:184-198): the tokens of an image group also attend to each other both ways; past the window (full_img /
+    sliding_img of a model with _vision_bidir_all), or with grp_windowed only within it (the other sliding_img)."""
     art = np.asarray(art)
     end = np.asarray(end)
     n = len(art)
@@ -22,9 +24,17 @@ def dense_tree_mask(art, end, pos=None, window=None):
     k = np.arange(n)[None, :]
     m = (k <= q) & (art[q] >= 0) & (art[k] == art[q]) & (q < end[k])
     m = m | (q == k)
+    inw = None
     if window is not None:
         pos = np.asarray(pos).astype(np.int64)
-        m = m & (pos[:, None] - pos[None, :] < window)
+        inw = pos[:, None] - pos[None, :] < window
+        m = m & inw
+    if grp is not None:
+        grp = np.asarray(grp)
+        same = (grp[:, None] == grp[None, :]) & (grp[:, None] >= 0)
+        if grp_windowed and inw is not None:
+            same = same & inw
+        m = m | same
     return m
 
 

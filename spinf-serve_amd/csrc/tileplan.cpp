@@ -1,6 +1,7 @@
 // Tile-plan compiler: stream metadata -> per-query-tile list of visible key tiles with 32x32 activity / mask bits.
 // Stands in for block_tables (spinf_serve/packer.py:426-491); the visibility predicate is the one of
-// spinf_serve/scorer.py:173-177.  Host code, no global state.
+// spinf_serve/scorer.py:173-177, with the image groups of scorer.py:184-198 (the tokens of a group also see each other both
+// ways).  Host code, no global state.
 #include "spinf_tree.h"
 #include "common.h"
 
@@ -31,20 +32,39 @@ struct Blk {            // aggregates of one 32-token block
     bool any_real;
 };
 
-inline bool visible(const int32_t* art, const int32_t* end, const int32_t* pos, int32_t window, int64_t q, int64_t k) {
+// grp_mode 1: the group term holds past the window; 2: it is windowed like the rest (scorer.py:186-198)
+inline bool visible(const int32_t* art, const int32_t* end, const int32_t* pos, const int32_t* grp, int32_t grp_mode, int32_t window,
+                    int64_t q, int64_t k) {
     if (q == k) return true;
-    bool v = k <= q && art[q] >= 0 && art[k] == art[q] && q < (int64_t)end[k];
-    if (v && window > 0) v = ((int64_t)pos[q] - (int64_t)pos[k]) < (int64_t)window;
-    return v;
+    const bool in_window = window <= 0 || ((int64_t)pos[q] - (int64_t)pos[k]) < (int64_t)window;
+    const bool v = k <= q && art[q] >= 0 && art[k] == art[q] && q < (int64_t)end[k] && in_window;
+    if (v || !grp) return v;
+    return grp[q] >= 0 && grp[q] == grp[k] && (grp_mode == 1 || in_window);
+}
+
+// do two sorted lists share a value?
+inline bool share(const std::vector<int32_t>& a, const std::vector<int32_t>& b) {
+    size_t i = 0, j = 0;
+    while (i < a.size() && j < b.size()) {
+        if (a[i] == b[j]) return true;
+        if (a[i] < b[j]) i++; else j++;
+    }
+    return false;
 }
 
 }  // namespace
 
 extern "C" int spinf_tileplan_build(const int32_t* art, const int32_t* end, const int32_t* pos, int64_t n, int32_t window,
                                     spinf_tileplan** out) {
+    return spinf_tileplan_build_groups(art, end, pos, nullptr, 0, n, window, out);
+}
+
+extern "C" int spinf_tileplan_build_groups(const int32_t* art, const int32_t* end, const int32_t* pos, const int32_t* grp, int32_t grp_mode,
+                                           int64_t n, int32_t window, spinf_tileplan** out) {
     if (!out) return spinf_fail(SPINF_E_ARG, "tileplan_build: out is null");
     *out = nullptr;
     if (n < 0 || (n > 0 && (!art || !end || !pos))) return spinf_fail(SPINF_E_ARG, "tileplan_build: null metadata");
+    if (grp && grp_mode != 1 && grp_mode != 2) return spinf_fail(SPINF_E_ARG, "tileplan_build: group mode %d not in {1, 2}", grp_mode);
     if (n > (int64_t)1 << 30) return spinf_fail(SPINF_E_ARG, "tileplan_build: stream too long");
     spinf_tileplan* p = new (std::nothrow) spinf_tileplan;
     if (!p) return spinf_fail(SPINF_E_NOMEM, "tileplan_build: out of memory");
@@ -77,6 +97,18 @@ extern "C" int spinf_tileplan_build(const int32_t* art, const int32_t* end, cons
             }
             if (B.job == -3) B.job = -2;
         }
+        // image groups: the distinct groups of every block (sorted), the last position of every group
+        std::vector<std::vector<int32_t>> bgrp(grp ? nb : 0);
+        std::unordered_map<int32_t, int64_t> glast;
+        if (grp) {
+            for (int64_t i = 0; i < n; i++) {
+                if (grp[i] < 0) continue;
+                std::vector<int32_t>& g = bgrp[i / SPINF_SUB];
+                if (std::find(g.begin(), g.end(), grp[i]) == g.end()) g.push_back(grp[i]);
+                glast[grp[i]] = i;
+            }
+            for (auto& g : bgrp) std::sort(g.begin(), g.end());
+        }
         // first stream position of every job: the lowest key any of its rows may see
         std::unordered_map<int32_t, int64_t> first;
         std::vector<int64_t> jfirst(n);
@@ -93,12 +125,13 @@ extern "C" int spinf_tileplan_build(const int32_t* art, const int32_t* end, cons
         group.assign(nqt, -1);
         for (int64_t t = 0; t < nqt; t++) {
             const int64_t q0 = t * SPINF_QTILE, q1 = std::min<int64_t>(n, q0 + SPINF_QTILE);
-            int64_t lo_key = q0;
+            int64_t lo_key = q0, hi_key = q1;   // keys [lo_key, hi_key) can matter: the rows' jobs so far, and their groups to the end
             for (int64_t q = q0; q < q1; q++) {
                 lo_key = std::min(lo_key, jfirst[q]);
                 if (group[t] < 0 && art[q] >= 0) group[t] = art[q];
+                if (grp && grp[q] >= 0) hi_key = std::max(hi_key, glast[grp[q]] + 1);
             }
-            for (int64_t j = lo_key / SPINF_KTILE; j * SPINF_KTILE < q1; j++) {
+            for (int64_t j = lo_key / SPINF_KTILE; j * SPINF_KTILE < hi_key; j++) {
                 uint32_t bits = 0;
                 for (int w = 0; w < SPINF_QTILE / SPINF_SUB; w++) {
                     const int64_t rb = q0 / SPINF_SUB + w;
@@ -108,10 +141,18 @@ extern "C" int spinf_tileplan_build(const int32_t* art, const int32_t* end, cons
                         const int64_t kb = j * (SPINF_KTILE / SPINF_SUB) + s;
                         if (kb >= nb) break;
                         const Blk& K = blk[kb];
-                        if (K.lo > R.hi - 1) continue;                       // every key after every row
+                        const bool grouped = grp && share(bgrp[rb], bgrp[kb]);   // some row and some key are of one image
+                        if (K.lo > R.hi - 1 && !grouped) continue;           // every key after every row
                         const bool below = K.hi - 1 < R.lo;                  // every key strictly before every row
                         bool any, all;
-                        if (below && K.max_end <= R.lo) { any = false; all = false; }
+                        if (grouped) {
+                            any = false; all = (R.hi - R.lo) == SPINF_SUB && (K.hi - K.lo) == SPINF_SUB;
+                            for (int64_t q = R.lo; q < R.hi; q++)
+                                for (int64_t k = K.lo; k < K.hi; k++) {
+                                    const bool v = visible(art, end, pos, grp, grp_mode, W, q, k);
+                                    any |= v; all &= v;
+                                }
+                        } else if (below && K.max_end <= R.lo) { any = false; all = false; }
                         else if (below && W > 0 && R.any_real && K.any_real && R.min_pos - K.max_pos >= W) { any = false; all = false; }
                         else if (K.hi - 1 <= R.lo && R.all_real && K.all_real && R.job >= 0 && R.job == K.job && K.min_end >= R.hi &&
                                  (W == 0 || R.max_pos - K.min_pos < W) && (R.hi - R.lo) == SPINF_SUB && (K.hi - K.lo) == SPINF_SUB) {
@@ -120,7 +161,7 @@ extern "C" int spinf_tileplan_build(const int32_t* art, const int32_t* end, cons
                             any = false; all = (R.hi - R.lo) == SPINF_SUB && (K.hi - K.lo) == SPINF_SUB;
                             for (int64_t q = R.lo; q < R.hi; q++)
                                 for (int64_t k = K.lo; k < K.hi; k++) {
-                                    const bool v = visible(art, end, pos, W, q, k);
+                                    const bool v = visible(art, end, pos, nullptr, 0, W, q, k);
                                     any |= v; all &= v;
                                 }
                         }

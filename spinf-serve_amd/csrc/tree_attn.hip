@@ -60,6 +60,7 @@ struct AttnParams {
     // compact rows (ROWS kernels): q, k, v, o hold the real tokens only; row_of[stream position] = row, -1 for a pad position;
     // kv_row0[entry] = row of the entry's first key if its 64 keys are 64 consecutive rows, else -1
     const int* row_of; const int* kv_row0;
+    const int* grp;       // image groups (GRP kernels): -1 none; the tokens of a group see each other both ways
 };
 
 // Softmax reference point.  The fast pass fixes each row's reference at the maximum of the first 32-key block in which
@@ -93,8 +94,8 @@ struct Geo {
     static constexpr int NREG = 64 / RPI;              // regions per tile
     static constexpr int KRS = 1024 + 16, VRS = 1024 + 64;
     static constexpr int KTILEB = NREG * KRS, VTILEB = NREG * VRS;
-    static constexpr int METAB = 3 * 64 * 4;
-    static constexpr int BUFB = KTILEB + VTILEB + METAB;   // K tile | V tile | art,end,pos of the keys
+    static constexpr int METAB = 4 * 64 * 4;
+    static constexpr int BUFB = KTILEB + VTILEB + METAB;   // K tile | V tile | art, end, pos, grp of the keys
     static constexpr int SUBB = (32 / NREG) * ROWB;        // byte offset of rows 32.. relative to rows 0.. (same regions)
     __host__ __device__ static constexpr int k_off(int row) { return (row % NREG) * KRS + (row / NREG) * ROWB; }
     __host__ __device__ static constexpr int v_off(int row) { return (row % NREG) * VRS + (row / NREG) * ROWB; }
@@ -129,7 +130,7 @@ __device__ __forceinline__ unsigned lds_addr(const void* p) { return (unsigned)(
 // the stream every address is a wave-uniform base plus a per-lane constant (lane_k / lane_v, bytes), so the loop spends no
 // vector ALU on addressing; the last, partial tile clamps its rows per lane.
 // ROWS (compact rows): row0 >= 0 says that the tile's keys are rows row0 .. row0 + 63; otherwise every lane looks its row up.
-template <int D, int NW = 4, bool ROWS = false>
+template <int D, int NW = 4, bool ROWS = false, int GRP = 0>
 __device__ __forceinline__ void issue_tile(const AttnParams& p, unsigned buf, int kt, int row0, int kvh, int w, int lane, unsigned lane_k, unsigned lane_v) {
     using G = Geo<D>;
     constexpr int IPW = G::NREG / NW;   // DMA instructions per wave and tile
@@ -144,8 +145,8 @@ __device__ __forceinline__ void issue_tile(const AttnParams& p, unsigned buf, in
             dma16_uniform(kbase + row * p.k_tok * 2, lane_k, buf + reg * G::KRS);
             dma16_uniform(vbase + row * p.v_tok * 2, lane_v, buf + G::KTILEB + reg * G::VRS);
         }
-        if (w < 3) {   // wave 0: art, wave 1: end, wave 2: pos of the 64 keys
-            const int* src = (w == 0 ? p.art : w == 1 ? p.end : p.pos) + (long)kt * 64;
+        if (w < (GRP ? 4 : 3)) {   // wave 0: art, wave 1: end, wave 2: pos, wave 3: grp of the 64 keys
+            const int* src = (w == 0 ? p.art : w == 1 ? p.end : w == 2 ? p.pos : p.grp) + (long)kt * 64;
             dma4_lane(src + lane, buf + G::KTILEB + G::VTILEB + w * 256);
         }
     } else {
@@ -162,10 +163,10 @@ __device__ __forceinline__ void issue_tile(const AttnParams& p, unsigned buf, in
             dma16_lane(kbase + grow * p.k_tok * 2 + chunk * 16, buf + reg * G::KRS);
             dma16_lane(vbase + grow * p.v_tok * 2 + chunk * 16, buf + G::KTILEB + reg * G::VRS);
         }
-        if (w < 3) {
+        if (w < (GRP ? 4 : 3)) {
             long gk = (long)kt * 64 + lane;
             gk = gk < p.n ? gk : p.n - 1;
-            dma4_lane((w == 0 ? p.art : w == 1 ? p.end : p.pos) + gk, buf + G::KTILEB + G::VTILEB + w * 256);
+            dma4_lane((w == 0 ? p.art : w == 1 ? p.end : w == 2 ? p.pos : p.grp) + gk, buf + G::KTILEB + G::VTILEB + w * 256);
         }
     }
 }
@@ -199,25 +200,31 @@ struct Lane {
 };
 
 // mask of one 32-key block: register i of the S^T tile holds key 8*(i/4) + 4g + i%4 of the block
-template <int RT, bool WIN>
-__device__ __forceinline__ void apply_mask(f32x16 (&s_acc)[RT], const int* meta, int kt, int sub, int g, int tok, int art_q, int pos_q, int window) {
+// GRP 1: a key of the row's image group is visible whatever the rest says; GRP 2: if it also lies within the window
+template <int RT, bool WIN, int GRP = 0>
+__device__ __forceinline__ void apply_mask(f32x16 (&s_acc)[RT], const int* meta, int kt, int sub, int g, int tok, int art_q, int pos_q, int window,
+                                           int grp_q = -1) {
 #pragma unroll
     for (int i4 = 0; i4 < 4; i4++) {
         const int ko = 32 * sub + 8 * i4 + 4 * g;
         const int4 ka = *(const int4*)(meta + ko);
         const int4 ke = *(const int4*)(meta + 64 + ko);
-        int4 kp = make_int4(0, 0, 0, 0);
+        int4 kp = make_int4(0, 0, 0, 0), kgr = make_int4(-1, -1, -1, -1);
         if (WIN) kp = *(const int4*)(meta + 128 + ko);
+        if (GRP) kgr = *(const int4*)(meta + 192 + ko);
         const int kg = kt * 64 + ko;
         const int kav[4] = {ka.x, ka.y, ka.z, ka.w};
         const int kev[4] = {ke.x, ke.y, ke.z, ke.w};
         const int kpv[4] = {kp.x, kp.y, kp.z, kp.w};
+        const int kgv[4] = {kgr.x, kgr.y, kgr.z, kgr.w};
 #pragma unroll
         for (int jj = 0; jj < 4; jj++) {
             const int kk = kg + jj;
             bool vis = (kk <= tok) & (art_q >= 0) & (kav[jj] == art_q) & (tok < kev[jj]);
+            if (GRP == 1 && WIN) vis = vis & ((pos_q - kpv[jj]) < window);   // the group term below is not windowed
+            if (GRP) vis = vis | ((grp_q >= 0) & (kgv[jj] == grp_q));
             vis = vis | (kk == tok);
-            if (WIN) vis = vis & ((pos_q - kpv[jj]) < window);
+            if (WIN && GRP != 1) vis = vis & ((pos_q - kpv[jj]) < window);
 #pragma unroll
             for (int rt = 0; rt < RT; rt++) s_acc[rt][4 * i4 + jj] = vis ? s_acc[rt][4 * i4 + jj] : -INFINITY;
         }
@@ -283,7 +290,7 @@ __device__ __forceinline__ void store_rows(const AttnParams& p, const Lane<D>& L
 // Classic online softmax over one work item, one 32-key block at a time, nothing overlapped: the rare fallback, in a
 // kernel of its own because its accumulator rescaling (vector ALU on all of O) would cost the fast pass its register
 // allocation.
-template <int D, int RT, bool WIN, bool ROWS>
+template <int D, int RT, bool WIN, bool ROWS, int GRP>
 __device__ __forceinline__ void attn_item_exact(const AttnParams& p, const int4 item, const int h0, char* buf0, int2* ent, int* ent_row0, char* stage) {
     using G = Geo<D>;
     constexpr int NS = D / 16, NDT = D / 32;
@@ -306,6 +313,7 @@ __device__ __forceinline__ void attn_item_exact(const AttnParams& p, const int4 
     }
     const int art_q = tok < p.n ? p.art[tok_c] : -1;
     const int pos_q = WIN ? p.pos[tok_c] : 0;
+    const int grp_q = GRP && tok < p.n ? p.grp[tok_c] : -1;
     f32x16 o[RT][NDT];
     float M[RT], l[RT];
 #pragma unroll
@@ -339,7 +347,7 @@ __device__ __forceinline__ void attn_item_exact(const AttnParams& p, const int4 
         const unsigned bits = (unsigned)__builtin_amdgcn_readfirstlane(en.y) >> (2 * L.w);
         const int row0 = ROWS ? __builtin_amdgcn_readfirstlane(ent_row0[i - base]) : 0;
         __syncthreads();   // everyone is done with the buffer
-        issue_tile<D, 4, ROWS>(p, lds_addr(buf0), kt, row0, kvh, L.w, L.lane, L.lane_k, L.lane_v);
+        issue_tile<D, 4, ROWS, GRP>(p, lds_addr(buf0), kt, row0, kvh, L.w, L.lane, L.lane_k, L.lane_v);
         __builtin_amdgcn_s_waitcnt(0x0f70);
         __syncthreads();
         const char* kb = buf0;
@@ -361,7 +369,7 @@ __device__ __forceinline__ void attn_item_exact(const AttnParams& p, const int4 
 #pragma unroll
                 for (int rt = 0; rt < RT; rt++) s_acc[rt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[rt][s], s_acc[rt], 0, 0, 0);
             }
-            if ((bits >> (8 + sub)) & 1u) apply_mask<RT, WIN>(s_acc, meta, kt, sub, L.g, tok, art_q, pos_q, p.window);
+            if ((bits >> (8 + sub)) & 1u) apply_mask<RT, WIN, GRP>(s_acc, meta, kt, sub, L.g, tok, art_q, pos_q, p.window, grp_q);
             bf16x8 pb[RT][2];
 #pragma unroll
             for (int rt = 0; rt < RT; rt++) {
@@ -406,7 +414,7 @@ __device__ __forceinline__ void attn_item_exact(const AttnParams& p, const int4 
 }
 
 // An item of HPI heads is recomputed RT heads at a time.
-template <int D, int RT, bool WIN, int HPI, bool ROWS>
+template <int D, int RT, bool WIN, int HPI, bool ROWS, int GRP>
 __global__ __launch_bounds__(256) void tree_attn_exact_kernel(const AttnParams p) {
     using G = Geo<D>;
     __shared__ __attribute__((aligned(16))) char buf0[G::BUFB];
@@ -421,7 +429,7 @@ __global__ __launch_bounds__(256) void tree_attn_exact_kernel(const AttnParams p
         const int4 item = make_int4(__builtin_amdgcn_readfirstlane(it.x), __builtin_amdgcn_readfirstlane(it.y),
                                     __builtin_amdgcn_readfirstlane(it.z), __builtin_amdgcn_readfirstlane(it.w));
         const int hp = (int)((unsigned)item.z >> 20);
-        for (int sub = 0; sub < HPI; sub += RT) attn_item_exact<D, RT, WIN, ROWS>(p, item, hp * HPI + sub, buf0, ent, ent_row0, stage_all + w * 32 * 144);
+        for (int sub = 0; sub < HPI; sub += RT) attn_item_exact<D, RT, WIN, ROWS, GRP>(p, item, hp * HPI + sub, buf0, ent, ent_row0, stage_all + w * 32 * 144);
     }
     __builtin_amdgcn_s_waitcnt(0x0f70);
     __syncthreads();
@@ -454,7 +462,8 @@ extern "C" int spinf_debug_trace(long* out, int n) { return (int)hipMemcpyFromSy
 // NHW = 1: four waves, each with RT heads of the item.  NHW = 2: eight waves, waves 4..7 take the item's second set of RT heads
 // on the same K / V tiles (two waves per SIMD: one wave's softmax runs under the other's MFMAs).
 // ROWS: q, k, v, o hold the real tokens only (compact rows); the stream positions of the plan are mapped through row_of.
-template <int D, int RT, bool WIN, int NHW, bool ROWS>
+// GRP: image groups (1: their tokens see each other whatever the window, 2: within the window).
+template <int D, int RT, bool WIN, int NHW, bool ROWS, int GRP>
 __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p) {
     using G = Geo<D>;
     constexpr int HPI = RT * NHW;  // heads per work item
@@ -507,7 +516,7 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
     int cur_idx = -1, nxt_idx = -1;
     bool cur_ok = false, nxt_ok = false;
     bf16x8 qf[RT][NS];
-    int art_q = -1, pos_q = 0;
+    int art_q = -1, pos_q = 0, grp_q = -1;
     f32x16 o[RT][NDT];
     float M[RT], l[RT];
     bool viol = false;
@@ -525,7 +534,7 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
     auto item_ne = [](const int4& it) { return it.z & 0xfffff; };
     auto item_hp = [](const int4& it) { return (int)((unsigned)it.z >> 20); };
 
-    auto load_q = [&](const int4& it, bf16x8 (&dst)[RT][NS], int& a_q, int& p_q) __attribute__((always_inline)) {
+    auto load_q = [&](const int4& it, bf16x8 (&dst)[RT][NS], int& a_q, int& p_q, int& g_q) __attribute__((always_inline)) {
         const int lane = fresh_lane_id();
         const int tok = item_t(it) * SPINF_QTILE + 32 * L.wr + (lane & 31);
         const int tok_c = tok < p.n ? tok : p.n - 1;
@@ -543,6 +552,7 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
         }
         a_q = tok < p.n ? p.art[tok_c] : -1;
         p_q = WIN ? p.pos[tok_c] : 0;
+        g_q = GRP && tok < p.n ? p.grp[tok_c] : -1;
     };
     auto load_ent = [&](const int4& it, int2* dst, int* dst_row0, const int from) __attribute__((always_inline)) {
         const int ne = item_ne(it);
@@ -633,7 +643,7 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
             f32x16 sa[RT];
             bf16x8 pa[RT][2];
             qk_phase(kb + sub * G::SUBB, sa);
-            if ((bits >> (8 + sub)) & 1u) apply_mask<RT, WIN>(sa, meta, kt, sub, L.g, tok, art_q, pos_q, p.window);
+            if ((bits >> (8 + sub)) & 1u) apply_mask<RT, WIN, GRP>(sa, meta, kt, sub, L.g, tok, art_q, pos_q, p.window, grp_q);
 #pragma unroll
             for (int rt = 0; rt < RT; rt++) {
                 const float ms = sm_head(rt, sa[rt]);
@@ -659,10 +669,10 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
         if (cur_ok) cur = uniform4(p.items[cur_idx]);
     }
     if (cur_ok) {
-        load_q(cur, qf, art_q, pos_q);
+        load_q(cur, qf, art_q, pos_q, grp_q);
         load_ent(cur, ent_cur, entr_cur, 0);
         const int row0 = ROWS ? __builtin_amdgcn_readfirstlane(p.kv_row0[cur.y]) : 0;
-        if (L.wh == 0) issue_tile<D, 4, ROWS>(p, lds_addr(bufs), cur.w, row0, item_hp(cur) * HPI / p.group, L.w, L.lane, L.lane_k, L.lane_v);
+        if (L.wh == 0) issue_tile<D, 4, ROWS, GRP>(p, lds_addr(bufs), cur.w, row0, item_hp(cur) * HPI / p.group, L.w, L.lane, L.lane_k, L.lane_v);
     }
     // The item after the current one is fetched from the lists as late as the prefetch pipeline allows (three tile steps
     // before the current item ends; at once for items shorter than that): an item fetched long before it starts keeps the
@@ -724,9 +734,9 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
             if (i + 1 < ne) {
                 const int row0 = ROWS ? __builtin_amdgcn_readfirstlane(entr_cur[i + 1 - base]) : 0;
                 if (L.wh == 0)
-                    issue_tile<D, 4, ROWS>(p, oth, __builtin_amdgcn_readfirstlane(ent_cur[i + 1 - base].x), row0, kvh, L.w, L.lane, L.lane_k, L.lane_v);
+                    issue_tile<D, 4, ROWS, GRP>(p, oth, __builtin_amdgcn_readfirstlane(ent_cur[i + 1 - base].x), row0, kvh, L.w, L.lane, L.lane_k, L.lane_v);
             } else if (nxt_ok) {
-                if (L.wh == 0) issue_tile<D, 4, ROWS>(p, oth, nxt.w, nxt_row0, item_hp(nxt) * HPI / p.group, L.w, L.lane, L.lane_k, L.lane_v);
+                if (L.wh == 0) issue_tile<D, 4, ROWS, GRP>(p, oth, nxt.w, nxt_row0, item_hp(nxt) * HPI / p.group, L.w, L.lane, L.lane_k, L.lane_v);
                 pstage = pstage == 2 ? 3 : -1;   // -1: tile requested before the entries (one-tile items)
             }
             const int2 en = ent_cur[i - base];
@@ -759,7 +769,7 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
         if (pstage == -1) load_ent(nxt, ent_nxt, entr_nxt, 0);
         cur = nxt;
         cur_idx = nxt_idx;
-        load_q(cur, qf, art_q, pos_q);
+        load_q(cur, qf, art_q, pos_q, grp_q);
         { int2* tmp = ent_cur; ent_cur = ent_nxt; ent_nxt = tmp; }
         { int* tmp = entr_cur; entr_cur = entr_nxt; entr_nxt = tmp; }
         gslot ^= 1;
@@ -819,15 +829,15 @@ int device_state(DeviceState** out, long n_items) {
     return SPINF_OK;
 }
 
-template <int D, int RT, bool WIN, int NHW, bool ROWS>
+template <int D, int RT, bool WIN, int NHW, bool ROWS, int GRP = 0>
 int launch(const AttnParams& p, int blocks, hipStream_t stream) {
     using G = Geo<D>;
     static_assert(2 * G::BUFB + 2 * ENT_CAP * 12 + ((NHW == 2 && D == 256) ? 16 : 4 * NHW * 32 * 144) + 64 <= 160 * 1024, "LDS budget");
-    hipLaunchKernelGGL((tree_attn_kernel<D, RT, WIN, NHW, ROWS>), dim3(blocks), dim3(256 * NHW), 0, stream, p);
+    hipLaunchKernelGGL((tree_attn_kernel<D, RT, WIN, NHW, ROWS, GRP>), dim3(blocks), dim3(256 * NHW), 0, stream, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: launch: %s", hipGetErrorString(e));
     // the exact pass over whatever the fast pass handed on (normally nothing: its workgroups read a zero count and leave)
-    hipLaunchKernelGGL((tree_attn_exact_kernel<D, RT, WIN, RT * NHW, ROWS>), dim3(blocks < 64 ? blocks : 64), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((tree_attn_exact_kernel<D, RT, WIN, RT * NHW, ROWS, GRP>), dim3(blocks < 64 ? blocks : 64), dim3(256), 0, stream, p);
     e = hipGetLastError();
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: launch (exact pass): %s", hipGetErrorString(e));
     return SPINF_OK;
@@ -846,7 +856,15 @@ void pick_kernel(int hq, int hkv, int d, int variant, int* rt, int* nhw) {
 }
 
 template <int D>
-int launch_d(const AttnParams& p, int rt, int nhw, bool win, int blocks, hipStream_t s) {
+int launch_d(const AttnParams& p, int rt, int nhw, bool win, int grp_mode, int blocks, hipStream_t s) {
+    if (p.grp) {   // image groups: the one-head-per-wave kernels, stream layout
+        if (nhw == 2) {
+            if (!win) return launch<D, 1, false, 2, false, 1>(p, blocks, s);
+            return grp_mode == 1 ? launch<D, 1, true, 2, false, 1>(p, blocks, s) : launch<D, 1, true, 2, false, 2>(p, blocks, s);
+        }
+        if (!win) return launch<D, 1, false, 1, false, 1>(p, blocks, s);
+        return grp_mode == 1 ? launch<D, 1, true, 1, false, 1>(p, blocks, s) : launch<D, 1, true, 1, false, 2>(p, blocks, s);
+    }
     if (p.row_of) {   // compact rows: the one-head-per-wave kernels only
         if (nhw == 2) return win ? launch<D, 1, true, 2, true>(p, blocks, s) : launch<D, 1, false, 2, true>(p, blocks, s);
         return win ? launch<D, 1, true, 1, true>(p, blocks, s) : launch<D, 1, false, 1, true>(p, blocks, s);
@@ -895,6 +913,8 @@ extern "C" int spinf_tree_attn_fwd(const spinf_attn_args* a, void* stream) {
     pick_kernel(a->hq, a->hkv, a->d, a->variant, &rt, &nhw);
     if ((a->row_of != nullptr) != (a->kv_row0 != nullptr)) return spinf_fail(SPINF_E_ARG, "tree_attn: row_of and kv_row0 come together");
     if (a->row_of && rt != 1) return spinf_fail(SPINF_E_ARG, "tree_attn: variant %d does not take compact rows", a->variant);
+    if (a->grp && (a->grp_mode != 1 && a->grp_mode != 2)) return spinf_fail(SPINF_E_ARG, "tree_attn: group mode %d not in {1, 2}", a->grp_mode);
+    if (a->grp && (rt != 1 || a->row_of)) return spinf_fail(SPINF_E_ARG, "tree_attn: image groups go with variant 0 / 1 and the stream layout only");
     const int hpi = rt * nhw;
     const int64_t nqt = (a->n + SPINF_QTILE - 1) / SPINF_QTILE;
     if (a->n_items != nqt * (a->hq / hpi))
@@ -919,14 +939,15 @@ extern "C" int spinf_tree_attn_fwd(const spinf_attn_args* a, void* stream) {
     p.kv_idx = a->kv_idx; p.kv_bits = a->kv_bits;
     p.items = (const int4*)a->items; p.list_ptr = a->list_ptr;
     p.row_of = a->row_of; p.kv_row0 = a->kv_row0;
+    p.grp = a->grp;
     p.counters = st->counters;
     p.redo = st->counters + 64;
     const int blocks = (int)(a->n_items < st->cus ? a->n_items : st->cus);
     const bool win = p.window > 0;
     hipStream_t s = (hipStream_t)stream;
     switch (a->d) {
-        case 64: return launch_d<64>(p, rt, nhw, win, blocks, s);
-        case 128: return launch_d<128>(p, rt, nhw, win, blocks, s);
-        default: return launch_d<256>(p, rt, nhw, win, blocks, s);
+        case 64: return launch_d<64>(p, rt, nhw, win, a->grp_mode, blocks, s);
+        case 128: return launch_d<128>(p, rt, nhw, win, a->grp_mode, blocks, s);
+        default: return launch_d<256>(p, rt, nhw, win, a->grp_mode, blocks, s);
     }
 }

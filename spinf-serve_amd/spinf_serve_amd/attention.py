@@ -28,7 +28,7 @@ VARIANT = int(os.environ.get("SPINF_ATTN_VARIANT", "0"))
 def _tree_attn_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, art: torch.Tensor, end: torch.Tensor, pos: torch.Tensor,
                   kv_idx: torch.Tensor, kv_bits: torch.Tensor, items: torch.Tensor, list_ptr: torch.Tensor, n_items: int,
                   scale: float, window: int, variant: int, row_of: Optional[torch.Tensor], kv_row0: Optional[torch.Tensor],
-                  n_mapped: int) -> torch.Tensor:
+                  n_mapped: int, grp: Optional[torch.Tensor], grp_mode: int) -> torch.Tensor:
     """q [rows, hq, d], k / v [rows, hkv, d] (any token / head strides, d contiguous) -> out [rows, hq, d] contiguous, bf16.
     rows = the stream length, or with row_of / kv_row0 (compact rows) any number of rows: the kernel maps stream positions to
     rows through row_of; rows 0 .. n_mapped-1 are the rows row_of names (each written by the kernel), later rows come back zero."""
@@ -69,6 +69,10 @@ def _tree_attn_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, art: torch.
     a.variant = variant
     if row_of is not None:
         a.row_of, a.kv_row0 = row_of.data_ptr(), kv_row0.data_ptr()
+    if grp is not None:
+        if grp.dtype != torch.int32 or grp.numel() < n:
+            raise ValueError("grp must be int32 [n]")
+        a.grp, a.grp_mode = grp.data_ptr(), grp_mode
     lib = _lib.load_library()
     with torch.cuda.device(q.device):
         stream = torch.cuda.current_stream(q.device).cuda_stream
@@ -77,7 +81,7 @@ def _tree_attn_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, art: torch.
 
 
 @_tree_attn_op.register_fake
-def _(q, k, v, art, end, pos, kv_idx, kv_bits, items, list_ptr, n_items, scale, window, variant, row_of, kv_row0, n_mapped):
+def _(q, k, v, art, end, pos, kv_idx, kv_bits, items, list_ptr, n_items, scale, window, variant, row_of, kv_row0, n_mapped, grp, grp_mode):
     return torch.empty(q.shape, dtype=torch.bfloat16, device=q.device)
 
 
@@ -93,8 +97,10 @@ def tree_attn(q, k, v, mask: TreeMask, scale=None, variant=None, sidx=None):
         raise ValueError(f"sidx names {sidx.shape[0]} rows, q has {q.shape[0]}")
     scale = float(q.shape[-1] ** -0.5 if scale is None else scale)
     variant = int(VARIANT if variant is None else variant)
-    if sidx is not None and variant == 2:
-        variant = 0   # the two-heads-per-wave kernels do not take compact rows
+    if (sidx is not None or mask.grp is not None) and variant == 2:
+        variant = 0   # the two-heads-per-wave kernels take neither compact rows nor image groups
+    if sidx is not None and mask.grp is not None:
+        raise ValueError("image groups go with the stream layout (no sidx)")
     hq, hkv, d = q.shape[1], k.shape[1], q.shape[2]
     per_item = _lib.load_library().spinf_attn_heads_per_item(hq, hkv, d, variant)
     if per_item <= 0:
@@ -102,7 +108,8 @@ def tree_attn(q, k, v, mask: TreeMask, scale=None, variant=None, sidx=None):
     items, list_ptr, n_items = mask.schedule(hq // per_item)
     row_of, kv_row0 = mask.rows(sidx) if sidx is not None else (None, None)
     return _tree_attn_op(q, k, v, mask.art, mask.end, mask.pos, mask.kv_idx, mask.kv_bits, items, list_ptr, n_items,
-                         scale, int(mask.window), variant, row_of, kv_row0, 0 if sidx is None else int(sidx.shape[0]))
+                         scale, int(mask.window), variant, row_of, kv_row0, 0 if sidx is None else int(sidx.shape[0]),
+                         mask.grp, int(mask.grp_mode))
 
 
 # K/V capture for extraction, as spinf_serve/models/gemma4.py:66-70: while CAPTURE[device] = {"window", "ranges": [(start, n, key)],

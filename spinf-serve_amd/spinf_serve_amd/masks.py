@@ -17,10 +17,10 @@ from . import _lib
 class TilePlan:
     """host arrays of a compiled plan (see include/spinf_tree.h) and the native handle that makes its work lists"""
 
-    def __init__(self, handle, qt_ptr, kv_idx, kv_bits, order, n, window, active_blocks, masked_blocks):
+    def __init__(self, handle, qt_ptr, kv_idx, kv_bits, order, n, window, active_blocks, masked_blocks, grp_mode=0):
         self._handle = handle
         self.qt_ptr, self.kv_idx, self.kv_bits, self.order = qt_ptr, kv_idx, kv_bits, order
-        self.n, self.window = n, window
+        self.n, self.window, self.grp_mode = n, window, grp_mode
         self.active_blocks, self.masked_blocks = active_blocks, masked_blocks
         self._schedules = {}
 
@@ -33,7 +33,9 @@ class TilePlan:
                 pass
 
     @classmethod
-    def build(cls, art, end, pos, window=None) -> "TilePlan":
+    def build(cls, art, end, pos, window=None, grp=None, grp_windowed=False) -> "TilePlan":
+        """grp (image groups, spinf_serve/scorer.py:184-198): [n] int32, -1 none; the tokens of a group also see each other both
+        ways, past the window unless grp_windowed"""
         lib = _lib.load_library()
         art = np.ascontiguousarray(art, np.int32)
         end = np.ascontiguousarray(end, np.int32)
@@ -43,7 +45,16 @@ class TilePlan:
             raise ValueError("art, end and pos differ in length")
         w = int(window) if window else 0
         h = C.c_void_p()
-        _lib.check(lib.spinf_tileplan_build(art.ctypes.data, end.ctypes.data, pos.ctypes.data, n, w, C.byref(h)), "tileplan_build")
+        mode = 0
+        if grp is None:
+            _lib.check(lib.spinf_tileplan_build(art.ctypes.data, end.ctypes.data, pos.ctypes.data, n, w, C.byref(h)), "tileplan_build")
+        else:
+            grp = np.ascontiguousarray(grp, np.int32)
+            if len(grp) != n:
+                raise ValueError("grp differs in length from art")
+            mode = 2 if grp_windowed else 1
+            _lib.check(lib.spinf_tileplan_build_groups(art.ctypes.data, end.ctypes.data, pos.ctypes.data, grp.ctypes.data, mode, n, w, C.byref(h)),
+                       "tileplan_build_groups")
         try:
             counts = (C.c_int64 * 5)()
             _lib.check(lib.spinf_tileplan_counts(h, counts), "tileplan_counts")
@@ -56,7 +67,7 @@ class TilePlan:
         except Exception:
             lib.spinf_tileplan_free(h)
             raise
-        return cls(h, qt_ptr, kv_idx[:nent], kv_bits[:nent], order[:nqt], n, w, int(counts[2]), int(counts[3]))
+        return cls(h, qt_ptr, kv_idx[:nent], kv_bits[:nent], order[:nqt], n, w, int(counts[2]), int(counts[3]), mode)
 
     @property
     def n_qtiles(self) -> int:
@@ -86,8 +97,10 @@ class TreeMask:
     """Device-side handle: the stream's metadata + one compiled plan.  ``seq_lengths`` mirrors BlockMask.seq_lengths
     (spinf_serve/models/qwen35/qwen.py:615 reads it)."""
 
-    def __init__(self, plan: TilePlan, meta, device):
+    def __init__(self, plan: TilePlan, meta, device, grp=None):
         self.plan = plan
+        self.grp = grp                      # device copy of the image groups the plan was built with, or None
+        self.grp_mode = plan.grp_mode if grp is not None else 0
         self.n = plan.n
         self.window = plan.window
         self.seq_lengths = (plan.n, plan.n)
@@ -129,22 +142,30 @@ class TreeMask:
         return got
 
     @classmethod
-    def build(cls, art, end, pos, window=None, device="cuda", meta=None):
-        """compile the plan on the host and upload it; ``meta``: device art / end / pos tensors to share with another mask"""
+    def build(cls, art, end, pos, window=None, device="cuda", meta=None, grp=None, grp_windowed=False, grp_dev=None):
+        """compile the plan on the host and upload it; ``meta``: device art / end / pos tensors to share with another mask;
+        grp: image groups (see TilePlan.build), grp_dev: their device copy to share"""
         import torch
 
         device = torch.device(device)
         if meta is None:
             meta = tuple(_upload(a, np.int32, device) for a in (art, end, pos))
-        return cls(TilePlan.build(art, end, pos, window), meta, device)
+        if grp is not None and grp_dev is None:
+            grp_dev = _upload(grp, np.int32, device)
+        return cls(TilePlan.build(art, end, pos, window, grp, grp_windowed), meta, device, grp_dev if grp is not None else None)
 
 
-def block_masks(batch, sliding_window=None, device="cuda"):
+def block_masks(batch, sliding_window=None, device="cuda", grp=None, bidir_all=True):
     """-> {"full_attention": TreeMask, "sliding_attention": TreeMask}: the dict Scorer._block_masks returns
     (spinf_serve/scorer.py:207-238).  With a window the sliding plan is always built (the reference's always_window,
-    spinf_serve/packer.py:448-450); without one both keys name the global mask."""
-    full = TreeMask.build(batch.art, batch.end, batch.pos, None, device)
+    spinf_serve/packer.py:448-450); without one both keys name the global mask.
+    grp: image groups of the stream's tokens (-1 none).  bidir_all (the model's _vision_bidir_all, scorer.py:186-198): the
+    tokens of an image see each other both ways on every layer and past the window; otherwise on the sliding layers only,
+    within the window, and the global layers stay causal."""
+    full = TreeMask.build(batch.art, batch.end, batch.pos, None, device, grp=grp if bidir_all else None)
     if not sliding_window:
         return {"full_attention": full, "sliding_attention": full}
-    slid = TreeMask.build(batch.art, batch.end, batch.pos, sliding_window, device, meta=(full.art, full.end, full.pos))
+    grp_dev = full.grp if grp is not None else None
+    slid = TreeMask.build(batch.art, batch.end, batch.pos, sliding_window, device, meta=(full.art, full.end, full.pos), grp=grp,
+                          grp_windowed=not bidir_all, grp_dev=grp_dev)
     return {"full_attention": full, "sliding_attention": slid}

@@ -9,6 +9,7 @@ import torch
 
 import spinf_serve_amd as sa
 from oracle import attention as oattn
+from oracle import mask as omask
 from spinf_serve_amd import synth
 from spinf_serve_amd.packer import GroupedTree
 
@@ -288,6 +289,72 @@ def test_compact_rows_through_the_exact_pass(dev):
     torch.cuda.synchronize()
     assert _exact_items() > before, "the exact pass did not run"
     assert torch.equal(got, want)
+
+
+def _image_stream(seed=8):
+    """two jobs with image placeholders: groups that straddle tile borders, two in one block, one inside a branch"""
+    rng = np.random.default_rng(seed)
+    t1 = GroupedTree(rng.integers(5, 99, 700).tolist(), [rng.integers(5, 99, n).tolist() for n in (40, 9, 70)], [], [], parents=[-1, -1, -1])
+    t2 = synth._tree(rng, 150, [20])
+    trees = [t1, t2]
+    b = synth.pack(trees)[0]
+    grp = np.full(b.length, -1, np.int32)
+    for gid, (a, e) in enumerate([(10, 22), (24, 30), (100, 356), (500, 530), (705, 735), (768 + 128 + 5, 768 + 128 + 40)]):
+        grp[a:e] = gid
+    grp[b.art < 0] = -1
+    return trees, b, grp
+
+
+@pytest.mark.parametrize("hq,hkv,d", [(4, 2, 256), (3, 3, 128), (4, 1, 64)])
+@pytest.mark.parametrize("window,windowed", [(None, False), (64, False), (64, True)])
+def test_image_groups_see_each_other_both_ways(dev, hq, hkv, d, window, windowed):
+    """spinf_serve/scorer.py:184-198: the placeholders of an image attend to each other both ways (later keys too), on the
+    global layers, on the sliding layers past the window, or on the sliding layers within it"""
+    trees, b, grp = _image_stream()
+    cfg = synth.AttnConfig("img", hq, hkv, d, d ** -0.5, 1.0, window, trees)
+    q, k, v = synth.qkv(cfg, b, device=dev)
+    mask = sa.TreeMask.build(b.art, b.end, b.pos, window, device=dev, grp=grp, grp_windowed=windowed)
+    out = sa.tree_attn(q, k, v, mask, cfg.scale)
+    dense = omask.dense_tree_mask(b.art, b.end, b.pos, window, grp, windowed)
+    ref = oattn.masked_attention(q.float().cpu().numpy(), k.float().cpu().numpy(), v.float().cpu().numpy(), dense, cfg.scale)
+    got = out.float().cpu().numpy()
+    assert float(np.abs(got - ref).max()) <= TOL
+    # the groups matter: without them the same rows come out differently
+    plain = sa.tree_attn(q, k, v, sa.TreeMask.build(b.art, b.end, b.pos, window, device=dev), cfg.scale).float().cpu().numpy()
+    assert np.abs(plain[grp >= 0] - ref[grp >= 0]).max() > 10 * TOL
+    assert np.array_equal(plain[(grp < 0) & (b.art < 0)], got[(grp < 0) & (b.art < 0)])      # pads: their own V row either way
+
+
+def test_block_masks_with_images(dev):
+    """bidir_all (the unified checkpoint): groups on both masks; otherwise the global mask stays causal and the sliding one
+    takes the groups within the window (scorer.py:186-198)"""
+    trees, b, grp = _image_stream()
+    cfg = synth.AttnConfig("img", 4, 2, 128, 128 ** -0.5, 1.0, 64, trees)
+    q, k, v = synth.qkv(cfg, b, device=dev)
+    qn, kn, vn = (t.float().cpu().numpy() for t in (q, k, v))
+    for bidir_all in (True, False):
+        masks = sa.block_masks(b, sliding_window=64, device=dev, grp=grp, bidir_all=bidir_all)
+        want_full = omask.dense_tree_mask(b.art, b.end, b.pos, None, grp if bidir_all else None)
+        want_slid = omask.dense_tree_mask(b.art, b.end, b.pos, 64, grp, not bidir_all)
+        for name, dense in (("full_attention", want_full), ("sliding_attention", want_slid)):
+            got = sa.tree_attn(q, k, v, masks[name], cfg.scale).float().cpu().numpy()
+            assert float(np.abs(got - oattn.masked_attention(qn, kn, vn, dense, cfg.scale)).max()) <= TOL, (bidir_all, name)
+
+
+def test_image_groups_through_the_exact_pass(dev):
+    trees, b, grp = _image_stream()
+    cfg = synth.AttnConfig("img", 4, 2, 128, 128 ** -0.5, 1.0, None, trees)
+    q, k, v = synth.qkv(cfg, b, seed=3, device=dev)
+    k = k.clone()
+    k[96:] *= 60.0
+    mask = sa.TreeMask.build(b.art, b.end, b.pos, None, device=dev, grp=grp)
+    before = _exact_items()
+    out = sa.tree_attn(q, k, v, mask, cfg.scale)
+    torch.cuda.synchronize()
+    assert _exact_items() > before, "the exact pass did not run"
+    dense = omask.dense_tree_mask(b.art, b.end, b.pos, None, grp)
+    ref = oattn.masked_attention(q.float().cpu().numpy(), k.float().cpu().numpy(), v.float().cpu().numpy(), dense, cfg.scale)
+    assert float(np.abs(out.float().cpu().numpy() - ref).max()) <= TOL
 
 
 def test_argument_errors(dev):

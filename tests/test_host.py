@@ -211,12 +211,12 @@ def test_reads_see_exactly_their_prompt():
 
 
 # ------------------------------------------------------------------------------------------------ tile plan
-def _check_plan(art, end, pos, window):
+def _check_plan(art, end, pos, window, grp=None, grp_windowed=False):
     """exactness of the compiled plan against the dense mask at 32 x 32 granularity: a set bit <=> some pair visible,
     a clear mask bit <=> every pair visible, unlisted tiles <=> nothing visible; key tiles ascending"""
-    plan = sa.TilePlan.build(art, end, pos, window)
+    plan = sa.TilePlan.build(art, end, pos, window, grp, grp_windowed)
     n = len(art)
-    m = omask.dense_tree_mask(art, end, pos, window)
+    m = omask.dense_tree_mask(art, end, pos, window, grp, grp_windowed)
     nqt = -(-n // 128)
     assert plan.n_qtiles == nqt and sorted(plan.order.tolist()) == list(range(nqt))
     active = masked = 0
@@ -241,6 +241,51 @@ def _check_plan(art, end, pos, window):
                         assert not (bits >> (8 + 2 * w + s) & 1)
     assert (active, masked) == (plan.active_blocks, plan.masked_blocks)
     return plan
+
+
+def _image_stream(seed=8):
+    """two jobs with image placeholders: groups that straddle tile borders, two in one block, one in a branch"""
+    rng = np.random.default_rng(seed)
+    t1 = GroupedTree(rng.integers(5, 99, 700).tolist(), [rng.integers(5, 99, n).tolist() for n in (40, 9, 70)], [], [], parents=[-1, -1, -1])
+    t2 = synth._tree(rng, 150, [20])
+    b = synth.pack([t1, t2])[0]
+    grp = np.full(b.length, -1, np.int32)
+    for gid, (a, e) in enumerate([(10, 22), (24, 30), (100, 356), (500, 530), (705, 735), (768 + 128 + 5, 768 + 128 + 40)]):
+        grp[a:e] = gid
+    grp[b.art < 0] = -1
+    return b, grp
+
+
+def test_image_group_mask_literal():
+    """scorer.py:184-198 on six tokens of one job, tokens 2..4 one image: they see each other both ways, the rest stays causal"""
+    art, end = np.zeros(6, np.int32), np.full(6, 6, np.int32)
+    grp = np.array([-1, -1, 0, 0, 0, -1], np.int32)
+    want = np.array([[1, 0, 0, 0, 0, 0],
+                     [1, 1, 0, 0, 0, 0],
+                     [1, 1, 1, 1, 1, 0],
+                     [1, 1, 1, 1, 1, 0],
+                     [1, 1, 1, 1, 1, 0],
+                     [1, 1, 1, 1, 1, 1]], bool)
+    assert np.array_equal(omask.dense_tree_mask(art, end, grp=grp), want)
+    pos = np.arange(6)
+    # window 2, group term not windowed: the image still sees itself whole; windowed: only neighbours at distance < 2
+    w_all = omask.dense_tree_mask(art, end, pos, 2, grp)
+    assert w_all[2].tolist() == [0, 1, 1, 1, 1, 0] and w_all[4].tolist() == [0, 0, 1, 1, 1, 0] and w_all[5].tolist() == [0, 0, 0, 0, 1, 1]
+    w_win = omask.dense_tree_mask(art, end, pos, 2, grp, grp_windowed=True)
+    assert w_win[2].tolist() == [0, 1, 1, 1, 1, 0] and w_win[4].tolist() == [0, 0, 0, 1, 1, 0]   # later keys: pos[q] - pos[k] < 0 < W
+
+
+def test_tileplan_with_image_groups_is_exact():
+    b, grp = _image_stream()
+    for window, windowed in ((None, False), (64, False), (64, True), (300, True)):
+        plan = _check_plan(b.art, b.end, b.pos, window, grp, windowed)
+    # a query tile lists the LATER key tiles of its images (packer.py:456-468)
+    plan = sa.TilePlan.build(b.art, b.end, b.pos, None, grp)
+    kts = plan.kv_idx[plan.qt_ptr[0] : plan.qt_ptr[1]].tolist()      # tile 0 holds the start of the image at 100 .. 355
+    assert kts == [0, 1, 2, 3, 4, 5]
+    # without groups the same stream lists nothing after the diagonal
+    plain = sa.TilePlan.build(b.art, b.end, b.pos, None)
+    assert plain.kv_idx[plain.qt_ptr[0] : plain.qt_ptr[1]].tolist() == [0, 1]
 
 
 def test_tileplan_is_exact_on_golden_streams(golden):
