@@ -32,6 +32,7 @@ WORKLOADS = {
     "C5": "C5: Gated DeltaNet, contents x (2048-token trunk + 32 branches x 12), 16 qk / 32 v heads, 128 x 128 fp32 state",
     "C5_prologue": "C5's stream through the Gated DeltaNet layer's prologue: path convolution (4 taps) + silu + q/k l2 norm + beta + g from the input projection's rows",
     "C5_gate": "C5's stream through the Gated DeltaNet layer's output gate: per-head rms norm x norm_w x silu(z)",
+    "LM": "lm head read-out of one chunk of 1,024 read rows: soft-capping (30) + log-softmax over 262,144 fp32 logits + 8 option columns",
 }
 
 
@@ -100,6 +101,26 @@ def main():
                     config={"workload": WORKLOADS["copy"], "bytes_read": n, "bytes_written": n},
                     roofline={"bound": "hbm", "achieved": 2 * n / (ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                               "frac": 2 * n / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": 2 * n, "kernel_ms": ms})
+        print(json.dumps(line))
+        return
+
+    if args.workload == "LM":
+        rows, vocab, cap = 1024, 262144, 30.0
+        gen = torch.Generator(device=dev).manual_seed(args.seed)
+        logits = torch.randn((rows, vocab), generator=gen, device=dev) * 12
+        cols = torch.randint(0, vocab, (8,), generator=gen, device=dev)
+        if args.rows == "scatter":   # the reference's own lines (scorer.py:351-353, :254), for comparison
+            step = lambda: torch.log_softmax((torch.tanh(logits / cap) * cap).float(), dim=-1)[:, cols]  # noqa: E731
+        else:
+            step = lambda: sa.lm_logprobs(logits, cols, cap)  # noqa: E731
+        wall, kern = timed(step, args.steps, args.warmup, torch)
+        ms = float(np.mean(kern))
+        nbytes = rows * vocab * 4 + rows * 8 * 4
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        line.update(metric="read rows/s, lm head read-out", value=rows * args.steps / wall, unit="rows/s", ms_per_step=1e3 * wall / args.steps,
+                    dtype="f32", config={"workload": WORKLOADS["LM"], "rows": rows, "vocab": vocab, "way": "torch ops" if args.rows == "scatter" else "kernel"},
+                    roofline={"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS, "traffic": None,
+                              "kernel_ms": ms, "algorithmic_bytes": nbytes})
         print(json.dumps(line))
         return
 

@@ -159,6 +159,21 @@ typedef struct spinf_gdn_gate_args {
 } spinf_gdn_gate_args;
 int spinf_gdn_gate(const spinf_gdn_gate_args* args, void* stream);
 
+/* ------------------------------------------------------------------------------------------------ lm head read-out
+ * Replaces the lines after the logits GEMM in Scorer._logprobs and the column selection of Scorer._forward
+ * (spinf_serve/scorer.py:351-353 and :254): out[r, c] = log_softmax(softcap * tanh(logits[r] / softcap))[cols[c]], or the whole
+ * row with cols == NULL (the extraction rows, scorer.py:260).  softcap 0 = none.
+ *   logits [rows, ld >= vocab]: fp32 (dtype 0) or bf16 (dtype 1) device matrix, rows 16-byte aligned; cols [n_cols] int64
+ *   device array of column indices in 0 .. vocab-1; out [rows, out_ld] fp32.
+ */
+typedef struct spinf_lm_args {
+    const void* logits; int64_t ld; int32_t dtype;
+    int64_t rows, vocab; float softcap;
+    const int64_t* cols; int64_t n_cols;
+    float* out; int64_t out_ld;
+} spinf_lm_args;
+int spinf_lm_logprobs(const spinf_lm_args* args, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -17,4 +17,5 @@ from .masks import TreeMask, TilePlan, block_masks  # noqa: F401
 from .attention import CAPTURE, register_tree_attention, tree_attention, tree_attn, tree_flex_forward  # noqa: F401
 from .gdn import chunked, recurrent  # noqa: F401
 from .gdn_layer import gdn_gate, gdn_prologue  # noqa: F401
+from .lm_head import lm_logprobs  # noqa: F401
 from .qwen_plan import Call, TreePlan, gdn_tree, tree_plan  # noqa: F401

@@ -44,6 +44,15 @@ class GdnGateArgs(C.Structure):
     ]
 
 
+class LmArgs(C.Structure):
+    _fields_ = [
+        ("logits", C.c_void_p), ("ld", C.c_int64), ("dtype", C.c_int32),
+        ("rows", C.c_int64), ("vocab", C.c_int64), ("softcap", C.c_float),
+        ("cols", C.c_void_p), ("n_cols", C.c_int64),
+        ("out", C.c_void_p), ("out_ld", C.c_int64),
+    ]
+
+
 class GdnArgs(C.Structure):
     _fields_ = [
         ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("g", C.c_void_p), ("beta", C.c_void_p), ("o", C.c_void_p),
@@ -85,7 +94,8 @@ def load_library():
     lib.spinf_gdn_fwd.argtypes = [C.POINTER(GdnArgs), C.c_void_p]
     lib.spinf_gdn_prologue.argtypes = [C.POINTER(GdnPreArgs), C.c_void_p]
     lib.spinf_gdn_gate.argtypes = [C.POINTER(GdnGateArgs), C.c_void_p]
-    for name in ("spinf_tileplan_build", "spinf_tileplan_build_groups", "spinf_tileplan_counts", "spinf_tileplan_export", "spinf_tileplan_schedule", "spinf_tileplan_row0", "spinf_tree_attn_fwd", "spinf_attn_exact_items", "spinf_gdn_fwd", "spinf_gdn_prologue", "spinf_gdn_gate"):
+    lib.spinf_lm_logprobs.argtypes = [C.POINTER(LmArgs), C.c_void_p]
+    for name in ("spinf_tileplan_build", "spinf_tileplan_build_groups", "spinf_tileplan_counts", "spinf_tileplan_export", "spinf_tileplan_schedule", "spinf_tileplan_row0", "spinf_tree_attn_fwd", "spinf_attn_exact_items", "spinf_gdn_fwd", "spinf_gdn_prologue", "spinf_gdn_gate", "spinf_lm_logprobs"):
         getattr(lib, name).restype = C.c_int
     _LIB = lib
     return lib
