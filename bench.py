@@ -26,6 +26,7 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E (published)
 
 WORKLOADS = {
     "C2": "C2: 24 contents x (470-token trunk + 56 branches of U{8..16} tokens) in one varlen pass, 16 query / 8 KV heads, head_dim 256, scale 1/16, Q/K/V ~ 0.5 N(0,1), global layer",
+    "C2_512": "C2's stream at the head geometry of the Gemma-4 full-attention layers: 16 query heads / 1 KV head, head_dim 512, global layer",
     "C3": "C3: 512 contents, trunk lognormal(median 800, sigma 0.6) clipped 64..4096, U{8..64} branches of U{4..24}, passes <= 65,536 tokens, 16/8 heads, head_dim 256, one sliding (W=1024) + one global layer per pass",
     "C4": "C4: contents x (8192-token trunk + 16 nodes x 32 + 192 leaves of U{6..10}), 32/16 heads, head_dim 128, one varlen pass",
     "copy": "plain device copy of 1 GiB (reads 1 GiB, writes 1 GiB per launch): the yardstick the FETCH_SIZE / WRITE_SIZE counters are scaled by",

@@ -74,7 +74,7 @@ void spinf_tileplan_free(spinf_tileplan* plan);
  * GQA (query head h reads key/value head h / (hq / hkv)).  bf16 in, fp32 softmax and accumulation, bf16 out.
  *
  *   q [n, hq, d], k / v [n, hkv, d], out [n, hq, d]: bf16 device tensors, d contiguous; *_tok / *_head are the token
- *   and head strides in elements (multiples of 8).  d is 64, 128 or 256.
+ *   and head strides in elements (multiples of 8).  d is 64, 128, 256 or 512 (512: a single-pass kernel, one head per item).
  *   art, end, pos, kv_idx, kv_bits: device copies of the metadata and of the exported plan; items, list_ptr: device copy of
  *   the schedule for hq / spinf_attn_heads_per_item(hq, hkv, d, variant) head groups, n_items = query tiles x head groups
  *   window: the window the plan was built with (<= 0 global)

@@ -61,6 +61,7 @@ struct AttnParams {
     // kv_row0[entry] = row of the entry's first key if its 64 keys are 64 consecutive rows, else -1
     const int* row_of; const int* kv_row0;
     const int* grp;       // image groups (GRP kernels): -1 none; the tokens of a group see each other both ways
+    int all_items;        // > 0: the exact kernel is the only pass and takes items 0 .. all_items-1 (head dim 512)
 };
 
 // Softmax reference point.  The fast pass fixes each row's reference at the maximum of the first 32-key block in which
@@ -96,9 +97,9 @@ struct Geo {
     static constexpr int KTILEB = NREG * KRS, VTILEB = NREG * VRS;
     static constexpr int METAB = 4 * 64 * 4;
     static constexpr int BUFB = KTILEB + VTILEB + METAB;   // K tile | V tile | art, end, pos, grp of the keys
-    static constexpr int SUBB = (32 / NREG) * ROWB;        // byte offset of rows 32.. relative to rows 0.. (same regions)
     __host__ __device__ static constexpr int k_off(int row) { return (row % NREG) * KRS + (row / NREG) * ROWB; }
     __host__ __device__ static constexpr int v_off(int row) { return (row % NREG) * VRS + (row / NREG) * ROWB; }
+    static constexpr int KSUB = k_off(32), VSUB = v_off(32);   // byte offsets of rows 32.. relative to rows 0..
 };
 
 // One wave-wide DMA instruction: 64 lanes x `16` (or 4) bytes from global memory straight into 1 KiB (256 B) of contiguous
@@ -356,8 +357,8 @@ __device__ __forceinline__ void attn_item_exact(const AttnParams& p, const int4 
 #pragma unroll 1
         for (int sub = 0; sub < 2; sub++) {
             if (!((bits >> sub) & 1u)) continue;
-            const char* krow = kb + L.k_lane + sub * G::SUBB;
-            const char* vrow = vb + L.v_lane + sub * G::SUBB;
+            const char* krow = kb + L.k_lane + sub * G::KSUB;
+            const char* vrow = vb + L.v_lane + sub * G::VSUB;
             f32x16 s_acc[RT];
 #pragma unroll
             for (int rt = 0; rt < RT; rt++)
@@ -368,6 +369,8 @@ __device__ __forceinline__ void attn_item_exact(const AttnParams& p, const int4 
                 const bf16x8 kf = *(const bf16x8*)(krow + 32 * s);
 #pragma unroll
                 for (int rt = 0; rt < RT; rt++) s_acc[rt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[rt][s], s_acc[rt], 0, 0, 0);
+                // at head dim 512 the registers are full (O 256, Q 128): keep the scheduler from hoisting every fragment read
+                if (D > 256 && s % 4 == 3) __builtin_amdgcn_sched_barrier(0);
             }
             if ((bits >> (8 + sub)) & 1u) apply_mask<RT, WIN, GRP>(s_acc, meta, kt, sub, L.g, tok, art_q, pos_q, p.window, grp_q);
             bf16x8 pb[RT][2];
@@ -383,9 +386,11 @@ __device__ __forceinline__ void attn_item_exact(const AttnParams& p, const int4 
                 const float alpha = up ? __builtin_amdgcn_exp2f(M[rt] - mn) : 1.0f;
                 if (__builtin_amdgcn_ballot_w64(up && M[rt] != -INFINITY) != 0) {   // rows without a key so far hold zeros
 #pragma unroll
-                    for (int dt = 0; dt < NDT; dt++)
+                    for (int dt = 0; dt < NDT; dt++) {
 #pragma unroll
                         for (int i2 = 0; i2 < 16; i2++) o[rt][dt][i2] *= alpha;
+                        if (D > 256) __builtin_amdgcn_sched_barrier(0);   // one slice at a time through the vector registers
+                    }
                 }
                 l[rt] *= alpha;
                 M[rt] = mn;
@@ -407,6 +412,7 @@ __device__ __forceinline__ void attn_item_exact(const AttnParams& p, const int4 
                 const bf16x8 a = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
 #pragma unroll
                 for (int rt = 0; rt < RT; rt++) o[rt][f % NDT] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[rt][f / NDT], o[rt][f % NDT], 0, 0, 0);
+                if (D > 256 && f % 4 == 3) __builtin_amdgcn_sched_barrier(0);
             }
         }
     }
@@ -422,15 +428,16 @@ __global__ __launch_bounds__(256) void tree_attn_exact_kernel(const AttnParams p
     __shared__ int ent_row0[ROWS ? ENT_CAP : 1];
     __shared__ __attribute__((aligned(16))) char stage_all[4 * 32 * 144];
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int n_redo = p.counters[NLIST + 1];
+    const int n_redo = p.all_items > 0 ? p.all_items : p.counters[NLIST + 1];
     if (n_redo == 0) return;   // the normal case: the fast pass handed nothing on (every workgroup reads the same count)
     for (int j = blockIdx.x; j < n_redo; j += gridDim.x) {
-        const int4 it = p.items[p.redo[j]];
+        const int4 it = p.items[p.all_items > 0 ? j : p.redo[j]];
         const int4 item = make_int4(__builtin_amdgcn_readfirstlane(it.x), __builtin_amdgcn_readfirstlane(it.y),
                                     __builtin_amdgcn_readfirstlane(it.z), __builtin_amdgcn_readfirstlane(it.w));
         const int hp = (int)((unsigned)item.z >> 20);
         for (int sub = 0; sub < HPI; sub += RT) attn_item_exact<D, RT, WIN, ROWS, GRP>(p, item, hp * HPI + sub, buf0, ent, ent_row0, stage_all + w * 32 * 144);
     }
+    if (p.all_items > 0) return;   // no hand-over to account for
     __builtin_amdgcn_s_waitcnt(0x0f70);
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -642,7 +649,7 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
         auto one_block = [&](const int sub) __attribute__((always_inline)) {
             f32x16 sa[RT];
             bf16x8 pa[RT][2];
-            qk_phase(kb + sub * G::SUBB, sa);
+            qk_phase(kb + sub * G::KSUB, sa);
             if ((bits >> (8 + sub)) & 1u) apply_mask<RT, WIN, GRP>(sa, meta, kt, sub, L.g, tok, art_q, pos_q, p.window, grp_q);
 #pragma unroll
             for (int rt = 0; rt < RT; rt++) {
@@ -652,7 +659,7 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
                 for (int i2 = 0; i2 < 16; i2++) sm_elem(sa[rt], i2, ms, sum, pa[rt]);
                 l[rt] += sum;
             }
-            pv_phase(vb + sub * G::SUBB, pa);
+            pv_phase(vb + sub * G::VSUB, pa);
         };
         // (hiding each block's softmax behind the other block's MFMAs inside one wave was measured slower than plain
         // sequence: the second wave on the SIMD does that job)
@@ -851,6 +858,7 @@ void pick_kernel(int hq, int hkv, int d, int variant, int* rt, int* nhw) {
     const bool pairs = (hq / hkv) % 2 == 0;
     *rt = 1;
     *nhw = 1;
+    if (d > 256) return;   // head dim 512: one head per item, the single-pass kernel
     if (variant == 0 && pairs) *nhw = 2;
     if (variant == 2 && pairs && d <= 128) *rt = 2;
 }
@@ -874,6 +882,28 @@ int launch_d(const AttnParams& p, int rt, int nhw, bool win, int grp_mode, int b
         if (rt == 2) return win ? launch<D, 2, true, 1, false>(p, blocks, s) : launch<D, 2, false, 1, false>(p, blocks, s);
     }
     return win ? launch<D, 1, true, 1, false>(p, blocks, s) : launch<D, 1, false, 1, false>(p, blocks, s);
+}
+
+// Head dim 512 (the full-attention layers of the Gemma-4 checkpoints, one key / value head): a 64-key K / V tile fills most of the
+// LDS, so there is one tile buffer and no fast pass; every item goes through the online-softmax kernel.
+template <bool WIN, bool ROWS, int GRP>
+int launch_512(AttnParams p, long n_items, int blocks, hipStream_t stream) {
+    using G = Geo<512>;
+    static_assert(G::BUFB + ENT_CAP * 12 + 4 * 32 * 144 + 64 <= 160 * 1024, "LDS budget");
+    p.all_items = (int)n_items;
+    hipLaunchKernelGGL((tree_attn_exact_kernel<512, 1, WIN, 1, ROWS, GRP>), dim3(blocks), dim3(256), 0, stream, p);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: launch (head dim 512): %s", hipGetErrorString(e));
+    return SPINF_OK;
+}
+
+int launch_d512(const AttnParams& p, bool win, int grp_mode, long n_items, int blocks, hipStream_t s) {
+    if (p.grp) {
+        if (!win) return launch_512<false, false, 1>(p, n_items, blocks, s);
+        return grp_mode == 1 ? launch_512<true, false, 1>(p, n_items, blocks, s) : launch_512<true, false, 2>(p, n_items, blocks, s);
+    }
+    if (p.row_of) return win ? launch_512<true, true, 0>(p, n_items, blocks, s) : launch_512<false, true, 0>(p, n_items, blocks, s);
+    return win ? launch_512<true, false, 0>(p, n_items, blocks, s) : launch_512<false, false, 0>(p, n_items, blocks, s);
 }
 
 }  // namespace
@@ -905,7 +935,7 @@ extern "C" int spinf_tree_attn_fwd(const spinf_attn_args* a, void* stream) {
     if (a->n <= 0 || a->n_items <= 0) return SPINF_OK;
     if (!a->q || !a->k || !a->v || !a->out || !a->art || !a->end || !a->pos || !a->kv_idx || !a->kv_bits || !a->items || !a->list_ptr)
         return spinf_fail(SPINF_E_ARG, "tree_attn: null pointer");
-    if (a->d != 64 && a->d != 128 && a->d != 256) return spinf_fail(SPINF_E_ARG, "tree_attn: head dim %d not in {64,128,256}", a->d);
+    if (a->d != 64 && a->d != 128 && a->d != 256 && a->d != 512) return spinf_fail(SPINF_E_ARG, "tree_attn: head dim %d not in {64,128,256,512}", a->d);
     if (a->hq <= 0 || a->hkv <= 0 || a->hq % a->hkv) return spinf_fail(SPINF_E_ARG, "tree_attn: hq %d not a multiple of hkv %d", a->hq, a->hkv);
     if (a->n > INT32_MAX / 2) return spinf_fail(SPINF_E_ARG, "tree_attn: stream too long");
     if (!(a->scale > 0.f)) return spinf_fail(SPINF_E_ARG, "tree_attn: scale must be positive");
@@ -940,6 +970,7 @@ extern "C" int spinf_tree_attn_fwd(const spinf_attn_args* a, void* stream) {
     p.items = (const int4*)a->items; p.list_ptr = a->list_ptr;
     p.row_of = a->row_of; p.kv_row0 = a->kv_row0;
     p.grp = a->grp;
+    p.all_items = 0;
     p.counters = st->counters;
     p.redo = st->counters + 64;
     const int blocks = (int)(a->n_items < st->cus ? a->n_items : st->cus);
@@ -948,6 +979,7 @@ extern "C" int spinf_tree_attn_fwd(const spinf_attn_args* a, void* stream) {
     switch (a->d) {
         case 64: return launch_d<64>(p, rt, nhw, win, a->grp_mode, blocks, s);
         case 128: return launch_d<128>(p, rt, nhw, win, a->grp_mode, blocks, s);
-        default: return launch_d<256>(p, rt, nhw, win, a->grp_mode, blocks, s);
+        case 256: return launch_d<256>(p, rt, nhw, win, a->grp_mode, blocks, s);
+        default: return launch_d512(p, win, a->grp_mode, (long)a->n_items, blocks, s);
     }
 }

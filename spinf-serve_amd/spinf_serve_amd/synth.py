@@ -89,6 +89,11 @@ def attention_config(name: str, seed: int = 0, contents: int | None = None) -> A
         trees = [_tree(rng, 470, rng.integers(8, 17, 56)) for _ in range(n)]
         cfg = AttnConfig(name, 16, 8, 256, 1.0 / 16, 0.5, None, trees)
         cfg.batches = pack(trees)
+    elif name == "C2_512":   # C2's stream at the head geometry of the Gemma-4 full-attention layers
+        n = contents or 24
+        trees = [_tree(rng, 470, rng.integers(8, 17, 56)) for _ in range(n)]
+        cfg = AttnConfig(name, 16, 1, 512, 512 ** -0.5, 0.5, None, trees)
+        cfg.batches = pack(trees)
     elif name == "C3":
         n = contents or 512
         trees = []

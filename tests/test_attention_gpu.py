@@ -357,6 +357,34 @@ def test_image_groups_through_the_exact_pass(dev):
     assert float(np.abs(out.float().cpu().numpy() - ref).max()) <= TOL
 
 
+@pytest.mark.parametrize("hq,hkv", [(8, 1), (4, 2)])
+def test_head_dim_512(dev, hq, hkv):
+    """the full-attention layers of the Gemma-4 checkpoints: head dim 512, one key / value head (spinf_serve/models/gemma4.py:39-41)"""
+    rng = np.random.default_rng(12)
+    trees = [synth._tree(rng, 300, [20, 9, 14]), synth._tree(rng, 90, [7]), synth._tree(rng, 33, [])]
+    cfg = synth.AttnConfig("d512", hq, hkv, 512, 512 ** -0.5, 0.5, None, trees)
+    b = synth.pack(trees)[0]
+    _check(cfg, b, dev)
+    _check(cfg, b, dev, window=100)
+    # bit-identical per job alone and packed
+    q, k, v = synth.qkv(cfg, b, device=dev)
+    mask = sa.TreeMask.build(b.art, b.end, b.pos, device=dev)
+    packed = sa.tree_attn(q, k, v, mask, cfg.scale)
+    o = b.owners[1]
+    b1 = synth.pack([trees[1]])[0]
+    m1 = sa.TreeMask.build(b1.art, b1.end, b1.pos, device=dev)
+    sl = slice(o.start, o.start + o.n_tokens)
+    pad = b1.length - o.n_tokens
+    ext = lambda t: torch.cat([t[sl], t.new_zeros(pad, *t.shape[1:])])  # noqa: E731
+    alone = sa.tree_attn(ext(q), ext(k), ext(v), m1, cfg.scale)
+    assert torch.equal(alone[: o.n_tokens], packed[sl])
+    # compact rows
+    real = np.flatnonzero(b.art >= 0)
+    sidx = torch.from_numpy(real).to(dev)
+    got = sa.tree_attn(q[sidx].contiguous(), k[sidx].contiguous(), v[sidx].contiguous(), mask, cfg.scale, sidx=sidx)
+    assert torch.equal(got, packed[sidx])
+
+
 def test_argument_errors(dev):
     cfg = synth.attention_config("smoke")
     b = cfg.batches[0]
