@@ -56,6 +56,10 @@ int spinf_tileplan_build(const int32_t* art, const int32_t* end, const int32_t* 
  * 2: only within the window (sliding layers of the other checkpoint; its global layers take no groups). */
 int spinf_tileplan_build_groups(const int32_t* art, const int32_t* end, const int32_t* pos, const int32_t* grp, int32_t grp_mode,
                                 int64_t n, int32_t window, spinf_tileplan** out);
+/* The same with the keys per entry chosen: 64 (SPINF_KTILE, what the two calls above build) or 32, where an entry is a single
+ * 32-key sub-tile (bits 2w and 8+2w only).  The attention kernel takes 32-key plans for head dim 512, 64-key plans otherwise. */
+int spinf_tileplan_build_ktile(const int32_t* art, const int32_t* end, const int32_t* pos, const int32_t* grp, int32_t grp_mode,
+                               int64_t n, int32_t window, int32_t ktile, spinf_tileplan** out);
 /* counts[0] query tiles, [1] entries, [2] active 32x32 blocks, [3] masked 32x32 blocks, [4] n */
 int spinf_tileplan_counts(const spinf_tileplan* plan, int64_t counts[5]);
 /* qt_ptr [n_qtiles+1], kv_idx [entries], kv_bits [entries], order [n_qtiles]: caller-allocated host arrays */
@@ -74,7 +78,7 @@ void spinf_tileplan_free(spinf_tileplan* plan);
  * GQA (query head h reads key/value head h / (hq / hkv)).  bf16 in, fp32 softmax and accumulation, bf16 out.
  *
  *   q [n, hq, d], k / v [n, hkv, d], out [n, hq, d]: bf16 device tensors, d contiguous; *_tok / *_head are the token
- *   and head strides in elements (multiples of 8).  d is 64, 128, 256 or 512 (512: a single-pass kernel, one head per item).
+ *   and head strides in elements (multiples of 8).  d is 64, 128, 256 or 512 (512: one head per item, and a plan of 32-key entries).
  *   art, end, pos, kv_idx, kv_bits: device copies of the metadata and of the exported plan; items, list_ptr: device copy of
  *   the schedule for hq / spinf_attn_heads_per_item(hq, hkv, d, variant) head groups, n_items = query tiles x head groups
  *   window: the window the plan was built with (<= 0 global)
@@ -98,6 +102,7 @@ typedef struct spinf_attn_args {
                           no compact rows) */
     const int32_t* row_of; const int32_t* kv_row0;
     const int32_t* grp; int32_t grp_mode;   /* image groups, as given to spinf_tileplan_build_groups (device copy of grp), or NULL */
+    int32_t ktile;                          /* keys per plan entry: 0 or 64; 32 with d = 512 (and only then) */
 } spinf_attn_args;
 
 /* query heads one work item covers for this geometry (1 or 2); 0 for an invalid geometry */

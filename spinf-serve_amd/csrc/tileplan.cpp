@@ -14,6 +14,7 @@
 struct spinf_tileplan {
     int64_t n = 0;
     int32_t window = 0;
+    int32_t ktile = SPINF_KTILE;     // keys per entry: 64, or 32 for the head dim 512 kernel (one sub-tile per entry)
     std::vector<int32_t> qt_ptr, kv_idx, order;
     std::vector<uint32_t> kv_bits;
     std::vector<int64_t> weight;     // cost of a query tile in 32 x 32 blocks: per key tile, 4 x the most blocks any row group sees
@@ -56,13 +57,19 @@ inline bool share(const std::vector<int32_t>& a, const std::vector<int32_t>& b) 
 
 extern "C" int spinf_tileplan_build(const int32_t* art, const int32_t* end, const int32_t* pos, int64_t n, int32_t window,
                                     spinf_tileplan** out) {
-    return spinf_tileplan_build_groups(art, end, pos, nullptr, 0, n, window, out);
+    return spinf_tileplan_build_ktile(art, end, pos, nullptr, 0, n, window, SPINF_KTILE, out);
 }
 
 extern "C" int spinf_tileplan_build_groups(const int32_t* art, const int32_t* end, const int32_t* pos, const int32_t* grp, int32_t grp_mode,
                                            int64_t n, int32_t window, spinf_tileplan** out) {
+    return spinf_tileplan_build_ktile(art, end, pos, grp, grp_mode, n, window, SPINF_KTILE, out);
+}
+
+extern "C" int spinf_tileplan_build_ktile(const int32_t* art, const int32_t* end, const int32_t* pos, const int32_t* grp, int32_t grp_mode,
+                                          int64_t n, int32_t window, int32_t ktile, spinf_tileplan** out) {
     if (!out) return spinf_fail(SPINF_E_ARG, "tileplan_build: out is null");
     *out = nullptr;
+    if (ktile != SPINF_KTILE && ktile != SPINF_SUB) return spinf_fail(SPINF_E_ARG, "tileplan_build: key tile %d not in {64, 32}", ktile);
     if (n < 0 || (n > 0 && (!art || !end || !pos))) return spinf_fail(SPINF_E_ARG, "tileplan_build: null metadata");
     if (grp && grp_mode != 1 && grp_mode != 2) return spinf_fail(SPINF_E_ARG, "tileplan_build: group mode %d not in {1, 2}", grp_mode);
     if (n > (int64_t)1 << 30) return spinf_fail(SPINF_E_ARG, "tileplan_build: stream too long");
@@ -70,6 +77,7 @@ extern "C" int spinf_tileplan_build_groups(const int32_t* art, const int32_t* en
     if (!p) return spinf_fail(SPINF_E_NOMEM, "tileplan_build: out of memory");
     try {
         p->n = n;
+        p->ktile = ktile;
         p->window = window > 0 ? window : 0;
         const int32_t W = p->window;
         const int64_t nqt = (n + SPINF_QTILE - 1) / SPINF_QTILE;
@@ -131,14 +139,14 @@ extern "C" int spinf_tileplan_build_groups(const int32_t* art, const int32_t* en
                 if (group[t] < 0 && art[q] >= 0) group[t] = art[q];
                 if (grp && grp[q] >= 0) hi_key = std::max(hi_key, glast[grp[q]] + 1);
             }
-            for (int64_t j = lo_key / SPINF_KTILE; j * SPINF_KTILE < hi_key; j++) {
+            for (int64_t j = lo_key / ktile; j * ktile < hi_key; j++) {
                 uint32_t bits = 0;
                 for (int w = 0; w < SPINF_QTILE / SPINF_SUB; w++) {
                     const int64_t rb = q0 / SPINF_SUB + w;
                     if (rb >= nb) break;
                     const Blk& R = blk[rb];
-                    for (int s = 0; s < SPINF_KTILE / SPINF_SUB; s++) {
-                        const int64_t kb = j * (SPINF_KTILE / SPINF_SUB) + s;
+                    for (int s = 0; s < ktile / SPINF_SUB; s++) {
+                        const int64_t kb = j * (ktile / SPINF_SUB) + s;
                         if (kb >= nb) break;
                         const Blk& K = blk[kb];
                         const bool grouped = grp && share(bgrp[rb], bgrp[kb]);   // some row and some key are of one image
@@ -300,9 +308,9 @@ extern "C" int spinf_tileplan_row0(const spinf_tileplan* p, const int32_t* row_o
     if (!p || !row_of) return spinf_fail(SPINF_E_ARG, "tileplan_row0: null argument");
     if (!kv_row0 && !p->kv_idx.empty()) return spinf_fail(SPINF_E_ARG, "tileplan_row0: null kv_row0");
     for (size_t e = 0; e < p->kv_idx.size(); e++) {
-        const int64_t k0 = (int64_t)p->kv_idx[e] * SPINF_KTILE;
-        int32_t r0 = k0 + SPINF_KTILE <= p->n ? row_of[k0] : -1;
-        for (int64_t j = 1; r0 >= 0 && j < SPINF_KTILE; j++)
+        const int64_t k0 = (int64_t)p->kv_idx[e] * p->ktile;
+        int32_t r0 = k0 + p->ktile <= p->n ? row_of[k0] : -1;
+        for (int64_t j = 1; r0 >= 0 && j < p->ktile; j++)
             if (row_of[k0 + j] != r0 + j) r0 = -1;
         kv_row0[e] = r0;
     }

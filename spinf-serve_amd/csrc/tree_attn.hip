@@ -61,7 +61,6 @@ struct AttnParams {
     // kv_row0[entry] = row of the entry's first key if its 64 keys are 64 consecutive rows, else -1
     const int* row_of; const int* kv_row0;
     const int* grp;       // image groups (GRP kernels): -1 none; the tokens of a group see each other both ways
-    int all_items;        // > 0: the exact kernel is the only pass and takes items 0 .. all_items-1 (head dim 512)
 };
 
 // Softmax reference point.  The fast pass fixes each row's reference at the maximum of the first 32-key block in which
@@ -82,9 +81,9 @@ __device__ __forceinline__ float lane32_sum(float x) {
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
-template <int D>
+template <int D, int TK = 64>
 struct Geo {
-    // LDS image of one 64-row K or V tile.  One wave-wide 16-byte DMA instruction fills 1 KiB of contiguous LDS (a
+    // LDS image of one K or V tile of TK rows (64; 32 at head dim 512, where two 64-row tile buffers would not fit).  One wave-wide 16-byte DMA instruction fills 1 KiB of contiguous LDS (a
     // "region"); a region holds rows r, r + NREG, r + 2 NREG ... so that consecutive rows lie in consecutive regions, and
     // regions are padded apart: by 16 bytes for K (the b128 fragment reads of 16 consecutive rows then cover all 64
     // banks) and by 64 bytes for V (the transposing reads touch 64 bytes of each of 4 consecutive rows).  Every address
@@ -92,7 +91,8 @@ struct Geo {
     static constexpr int ROWB = D * 2;                 // bytes of one K / V row
     static constexpr int CPR = ROWB / 16;              // 16-byte chunks per row
     static constexpr int RPI = 1024 / ROWB;            // rows per region
-    static constexpr int NREG = 64 / RPI;              // regions per tile
+    static constexpr int NREG = TK / RPI;              // regions per tile
+    static_assert(RPI >= 1 && NREG >= 4 && NREG <= 64, "tile geometry");
     static constexpr int KRS = 1024 + 16, VRS = 1024 + 64;
     static constexpr int KTILEB = NREG * KRS, VTILEB = NREG * VRS;
     static constexpr int METAB = 4 * 64 * 4;
@@ -131,31 +131,31 @@ __device__ __forceinline__ unsigned lds_addr(const void* p) { return (unsigned)(
 // the stream every address is a wave-uniform base plus a per-lane constant (lane_k / lane_v, bytes), so the loop spends no
 // vector ALU on addressing; the last, partial tile clamps its rows per lane.
 // ROWS (compact rows): row0 >= 0 says that the tile's keys are rows row0 .. row0 + 63; otherwise every lane looks its row up.
-template <int D, int NW = 4, bool ROWS = false, int GRP = 0>
+template <int D, int NW = 4, bool ROWS = false, int GRP = 0, int TK = 64>
 __device__ __forceinline__ void issue_tile(const AttnParams& p, unsigned buf, int kt, int row0, int kvh, int w, int lane, unsigned lane_k, unsigned lane_v) {
-    using G = Geo<D>;
+    using G = Geo<D, TK>;
     constexpr int IPW = G::NREG / NW;   // DMA instructions per wave and tile
     static_assert(IPW >= 1 && IPW * NW == G::NREG, "the tile's regions must divide among the waves");
     const char* kbase = (const char*)(p.k + (long)kvh * p.k_head);
     const char* vbase = (const char*)(p.v + (long)kvh * p.v_head);
-    if (ROWS ? row0 >= 0 : kt * 64 + 64 <= p.n) {
+    if (ROWS ? row0 >= 0 : kt * TK + TK <= p.n) {
 #pragma unroll
         for (int i = 0; i < IPW; i++) {
             const int reg = w * IPW + i;
-            const long row = (ROWS ? (long)row0 : (long)kt * 64) + reg;
+            const long row = (ROWS ? (long)row0 : (long)kt * TK) + reg;
             dma16_uniform(kbase + row * p.k_tok * 2, lane_k, buf + reg * G::KRS);
             dma16_uniform(vbase + row * p.v_tok * 2, lane_v, buf + G::KTILEB + reg * G::VRS);
         }
         if (w < (GRP ? 4 : 3)) {   // wave 0: art, wave 1: end, wave 2: pos, wave 3: grp of the 64 keys
-            const int* src = (w == 0 ? p.art : w == 1 ? p.end : w == 2 ? p.pos : p.grp) + (long)kt * 64;
-            dma4_lane(src + lane, buf + G::KTILEB + G::VTILEB + w * 256);
+            const int* src = (w == 0 ? p.art : w == 1 ? p.end : w == 2 ? p.pos : p.grp) + (long)kt * TK;
+            dma4_lane(src + (TK < 64 ? lane % TK : lane), buf + G::KTILEB + G::VTILEB + w * 256);   // (64 lanes: a 32-key tile's twice)
         }
     } else {
         const int slot = lane / G::CPR, chunk = lane % G::CPR;
 #pragma unroll
         for (int i = 0; i < IPW; i++) {
             const int reg = w * IPW + i;
-            long grow = (long)kt * 64 + reg + G::NREG * slot;
+            long grow = (long)kt * TK + reg + G::NREG * slot;
             grow = grow < p.n ? grow : p.n - 1;
             if (ROWS) {   // a pad position has no row: any row will do, its keys are visible to nobody but pad rows
                 const int r = p.row_of[grow];
@@ -165,7 +165,7 @@ __device__ __forceinline__ void issue_tile(const AttnParams& p, unsigned buf, in
             dma16_lane(vbase + grow * p.v_tok * 2 + chunk * 16, buf + G::KTILEB + reg * G::VRS);
         }
         if (w < (GRP ? 4 : 3)) {
-            long gk = (long)kt * 64 + lane;
+            long gk = (long)kt * TK + (TK < 64 ? lane % TK : lane);
             gk = gk < p.n ? gk : p.n - 1;
             dma4_lane((w == 0 ? p.art : w == 1 ? p.end : w == 2 ? p.pos : p.grp) + gk, buf + G::KTILEB + G::VTILEB + w * 256);
         }
@@ -173,9 +173,9 @@ __device__ __forceinline__ void issue_tile(const AttnParams& p, unsigned buf, in
 }
 
 // Everything a wave needs to know about its place in the workgroup and its LDS fragment addresses.
-template <int D>
+template <int D, int TK = 64>
 struct Lane {
-    using G = Geo<D>;
+    using G = Geo<D, TK>;
     int lane, m, g, w;
     int wr, wh;                  // row group (tokens 32 wr ..) and head set of this wave
     int k_lane, v_lane;          // byte offsets of this lane's K fragment row / V^T fragment address inside a tile
@@ -202,7 +202,7 @@ struct Lane {
 
 // mask of one 32-key block: register i of the S^T tile holds key 8*(i/4) + 4g + i%4 of the block
 // GRP 1: a key of the row's image group is visible whatever the rest says; GRP 2: if it also lies within the window
-template <int RT, bool WIN, int GRP = 0>
+template <int RT, bool WIN, int GRP = 0, int TK = 64>
 __device__ __forceinline__ void apply_mask(f32x16 (&s_acc)[RT], const int* meta, int kt, int sub, int g, int tok, int art_q, int pos_q, int window,
                                            int grp_q = -1) {
 #pragma unroll
@@ -213,7 +213,7 @@ __device__ __forceinline__ void apply_mask(f32x16 (&s_acc)[RT], const int* meta,
         int4 kp = make_int4(0, 0, 0, 0), kgr = make_int4(-1, -1, -1, -1);
         if (WIN) kp = *(const int4*)(meta + 128 + ko);
         if (GRP) kgr = *(const int4*)(meta + 192 + ko);
-        const int kg = kt * 64 + ko;
+        const int kg = kt * TK + ko;
         const int kav[4] = {ka.x, ka.y, ka.z, ka.w};
         const int kev[4] = {ke.x, ke.y, ke.z, ke.w};
         const int kpv[4] = {kp.x, kp.y, kp.z, kp.w};
@@ -241,10 +241,21 @@ __device__ __forceinline__ int fresh_lane_id() {
     return lane;
 }
 
+// An accumulator element read into a vector register by an explicit move.  At head dim 512 the 256 accumulators of O must stay
+// in the accumulator registers; a plain vector ALU use of them makes the register allocator keep ALL of O in vector
+// registers for the whole kernel (the query fragments then live in scratch memory).
+template <bool VIA_ACC>
+__device__ __forceinline__ float acc_value(float a) {
+    if (!VIA_ACC) return a;
+    float v;
+    asm("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(a));
+    return v;
+}
+
 // normalise O^T and store it as rows: each wave stages 32 rows x 64 head dims at a time in its own LDS slice (144-byte
 // rows) and writes them out as 16-byte pieces, 8 lanes per 128-byte row segment
-template <int D, int RT, bool ROWS = false>
-__device__ __forceinline__ void store_rows(const AttnParams& p, const Lane<D>& L, char* stage, const f32x16 (&o)[RT][D / 32], const float (&l)[RT],
+template <int D, int RT, bool ROWS = false, class LaneT>
+__device__ __forceinline__ void store_rows(const AttnParams& p, const LaneT& L, char* stage, const f32x16 (&o)[RT][D / 32], const float (&l)[RT],
                                            int t, int h0) {
     constexpr int NDT = D / 32;
     constexpr int SROW = 128 + 16;
@@ -270,7 +281,7 @@ __device__ __forceinline__ void store_rows(const AttnParams& p, const Lane<D>& L
                 for (int i4 = 0; i4 < 4; i4++) {
                     bf16x4 r;
 #pragma unroll
-                    for (int jj = 0; jj < 4; jj++) r[jj] = (__bf16)(o[rt][2 * qd + dd][4 * i4 + jj] * inv);
+                    for (int jj = 0; jj < 4; jj++) r[jj] = (__bf16)(acc_value<(D > 256)>(o[rt][2 * qd + dd][4 * i4 + jj]) * inv);
                     *(bf16x4*)(stage + m * SROW + (32 * dd + 8 * i4 + 4 * g) * 2) = r;
                 }
 #pragma unroll
@@ -291,11 +302,11 @@ __device__ __forceinline__ void store_rows(const AttnParams& p, const Lane<D>& L
 // Classic online softmax over one work item, one 32-key block at a time, nothing overlapped: the rare fallback, in a
 // kernel of its own because its accumulator rescaling (vector ALU on all of O) would cost the fast pass its register
 // allocation.
-template <int D, int RT, bool WIN, bool ROWS, int GRP>
+template <int D, int RT, bool WIN, bool ROWS, int GRP, int TK>
 __device__ __forceinline__ void attn_item_exact(const AttnParams& p, const int4 item, const int h0, char* buf0, int2* ent, int* ent_row0, char* stage) {
-    using G = Geo<D>;
+    using G = Geo<D, TK>;
     constexpr int NS = D / 16, NDT = D / 32;
-    const Lane<D> L(p);
+    const Lane<D, TK> L(p);
     const int t = item.x, e0 = item.y, ne = item.z & 0xfffff;   // heads h0 .. h0 + RT - 1 of the item
     const int kvh = h0 / p.group;
     const int tok = t * SPINF_QTILE + 32 * L.w + L.m;
@@ -348,14 +359,14 @@ __device__ __forceinline__ void attn_item_exact(const AttnParams& p, const int4 
         const unsigned bits = (unsigned)__builtin_amdgcn_readfirstlane(en.y) >> (2 * L.w);
         const int row0 = ROWS ? __builtin_amdgcn_readfirstlane(ent_row0[i - base]) : 0;
         __syncthreads();   // everyone is done with the buffer
-        issue_tile<D, 4, ROWS, GRP>(p, lds_addr(buf0), kt, row0, kvh, L.w, L.lane, L.lane_k, L.lane_v);
+        issue_tile<D, 4, ROWS, GRP, TK>(p, lds_addr(buf0), kt, row0, kvh, L.w, L.lane, L.lane_k, L.lane_v);
         __builtin_amdgcn_s_waitcnt(0x0f70);
         __syncthreads();
         const char* kb = buf0;
         const char* vb = buf0 + G::KTILEB;
         const int* meta = (const int*)(buf0 + G::KTILEB + G::VTILEB);
 #pragma unroll 1
-        for (int sub = 0; sub < 2; sub++) {
+        for (int sub = 0; sub < TK / 32; sub++) {
             if (!((bits >> sub) & 1u)) continue;
             const char* krow = kb + L.k_lane + sub * G::KSUB;
             const char* vrow = vb + L.v_lane + sub * G::VSUB;
@@ -372,7 +383,7 @@ __device__ __forceinline__ void attn_item_exact(const AttnParams& p, const int4 
                 // at head dim 512 the registers are full (O 256, Q 128): keep the scheduler from hoisting every fragment read
                 if (D > 256 && s % 4 == 3) __builtin_amdgcn_sched_barrier(0);
             }
-            if ((bits >> (8 + sub)) & 1u) apply_mask<RT, WIN, GRP>(s_acc, meta, kt, sub, L.g, tok, art_q, pos_q, p.window, grp_q);
+            if ((bits >> (8 + sub)) & 1u) apply_mask<RT, WIN, GRP, TK>(s_acc, meta, kt, sub, L.g, tok, art_q, pos_q, p.window, grp_q);
             bf16x8 pb[RT][2];
 #pragma unroll
             for (int rt = 0; rt < RT; rt++) {
@@ -420,24 +431,23 @@ __device__ __forceinline__ void attn_item_exact(const AttnParams& p, const int4 
 }
 
 // An item of HPI heads is recomputed RT heads at a time.
-template <int D, int RT, bool WIN, int HPI, bool ROWS, int GRP>
+template <int D, int RT, bool WIN, int HPI, bool ROWS, int GRP, int TK = 64>
 __global__ __launch_bounds__(256) void tree_attn_exact_kernel(const AttnParams p) {
-    using G = Geo<D>;
+    using G = Geo<D, TK>;
     __shared__ __attribute__((aligned(16))) char buf0[G::BUFB];
     __shared__ int2 ent[ENT_CAP];
     __shared__ int ent_row0[ROWS ? ENT_CAP : 1];
     __shared__ __attribute__((aligned(16))) char stage_all[4 * 32 * 144];
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int n_redo = p.all_items > 0 ? p.all_items : p.counters[NLIST + 1];
+    const int n_redo = p.counters[NLIST + 1];
     if (n_redo == 0) return;   // the normal case: the fast pass handed nothing on (every workgroup reads the same count)
     for (int j = blockIdx.x; j < n_redo; j += gridDim.x) {
-        const int4 it = p.items[p.all_items > 0 ? j : p.redo[j]];
+        const int4 it = p.items[p.redo[j]];
         const int4 item = make_int4(__builtin_amdgcn_readfirstlane(it.x), __builtin_amdgcn_readfirstlane(it.y),
                                     __builtin_amdgcn_readfirstlane(it.z), __builtin_amdgcn_readfirstlane(it.w));
         const int hp = (int)((unsigned)item.z >> 20);
-        for (int sub = 0; sub < HPI; sub += RT) attn_item_exact<D, RT, WIN, ROWS, GRP>(p, item, hp * HPI + sub, buf0, ent, ent_row0, stage_all + w * 32 * 144);
+        for (int sub = 0; sub < HPI; sub += RT) attn_item_exact<D, RT, WIN, ROWS, GRP, TK>(p, item, hp * HPI + sub, buf0, ent, ent_row0, stage_all + w * 32 * 144);
     }
-    if (p.all_items > 0) return;   // no hand-over to account for
     __builtin_amdgcn_s_waitcnt(0x0f70);
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -470,16 +480,16 @@ extern "C" int spinf_debug_trace(long* out, int n) { return (int)hipMemcpyFromSy
 // on the same K / V tiles (two waves per SIMD: one wave's softmax runs under the other's MFMAs).
 // ROWS: q, k, v, o hold the real tokens only (compact rows); the stream positions of the plan are mapped through row_of.
 // GRP: image groups (1: their tokens see each other whatever the window, 2: within the window).
-template <int D, int RT, bool WIN, int NHW, bool ROWS, int GRP>
+template <int D, int RT, bool WIN, int NHW, bool ROWS, int GRP, int TK = 64>
 __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p) {
-    using G = Geo<D>;
+    using G = Geo<D, TK>;
     constexpr int HPI = RT * NHW;  // heads per work item
     constexpr int NS = D / 16;     // contraction steps of K Q^T
     constexpr int NDT = D / 32;    // 32-wide slices of the head dimension in O^T
     constexpr int NVF = 2 * NDT;   // V^T fragments of one 32-key block
     // fragment read-ahead depth: the register file is the tight one at head dim 256 (4 with one wave per SIMD, 3 with two:
     // measured 0.374 / 0.351 / 0.343 / 0.368 ms on the 24-content pass for depths 4 / 2 / 3 / 1); no effect at 128
-    constexpr int PFD = D >= 256 ? (NHW == 2 ? 3 : 4) : 8;
+    constexpr int PFD = D > 256 ? 2 : D == 256 ? (NHW == 2 ? 3 : 4) : 8;
     constexpr int PF = NS < PFD ? NS : PFD;     // K fragments read ahead of the MFMAs
     constexpr int VPF = NVF < PFD ? NVF : PFD;  // V^T fragments read ahead
     __shared__ __attribute__((aligned(16))) char bufs[2 * G::BUFB];   // the two tile buffers
@@ -490,14 +500,14 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
     // output staging, one slice per wave; with eight waves at head dim 256 there is no room left for it and the slices lie in
     // the tile buffer the item's last tile was computed from (free from the barrier after the tile loop until the next
     // item's first tile step requests a tile into it, which comes after that step's barrier)
-    constexpr bool STAGE_IN_TILE = NHW == 2 && D == 256;
-    static_assert(!STAGE_IN_TILE || 8 * 32 * 144 <= G::BUFB, "the staging slices must fit a tile buffer");
+    constexpr bool STAGE_IN_TILE = (NHW == 2 && D == 256) || D == 512;
+    static_assert(!STAGE_IN_TILE || 4 * NHW * 32 * 144 <= G::BUFB, "the staging slices must fit a tile buffer");
     __shared__ __attribute__((aligned(16))) char stage_all[STAGE_IN_TILE ? 16 : 4 * NHW * 32 * 144];
     __shared__ int s_next[2];         // item grabbed by thread 0 for the whole workgroup, double buffered
 
     TRACE_CLK(tk0);
     TRACE_WALL(tw0);
-    const Lane<D> L(p);
+    const Lane<D, TK> L(p);
     char* const stage_own = stage_all + (STAGE_IN_TILE ? 0 : L.w * 32 * 144);
 
     // ---- work lists: start with the list of this workgroup's XCD, continue with the following ones
@@ -650,7 +660,7 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
             f32x16 sa[RT];
             bf16x8 pa[RT][2];
             qk_phase(kb + sub * G::KSUB, sa);
-            if ((bits >> (8 + sub)) & 1u) apply_mask<RT, WIN, GRP>(sa, meta, kt, sub, L.g, tok, art_q, pos_q, p.window, grp_q);
+            if ((bits >> (8 + sub)) & 1u) apply_mask<RT, WIN, GRP, TK>(sa, meta, kt, sub, L.g, tok, art_q, pos_q, p.window, grp_q);
 #pragma unroll
             for (int rt = 0; rt < RT; rt++) {
                 const float ms = sm_head(rt, sa[rt]);
@@ -664,7 +674,7 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
         // (hiding each block's softmax behind the other block's MFMAs inside one wave was measured slower than plain
         // sequence: the second wave on the SIMD does that job)
         if (a0) one_block(0);
-        if (a1) one_block(1);
+        if (TK > 32 && a1) one_block(1);
     };
 
     // ---- prologue: first item, its queries, entries and first tile; the second item is grabbed right away
@@ -679,7 +689,7 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
         load_q(cur, qf, art_q, pos_q, grp_q);
         load_ent(cur, ent_cur, entr_cur, 0);
         const int row0 = ROWS ? __builtin_amdgcn_readfirstlane(p.kv_row0[cur.y]) : 0;
-        if (L.wh == 0) issue_tile<D, 4, ROWS, GRP>(p, lds_addr(bufs), cur.w, row0, item_hp(cur) * HPI / p.group, L.w, L.lane, L.lane_k, L.lane_v);
+        if (L.wh == 0) issue_tile<D, 4, ROWS, GRP, TK>(p, lds_addr(bufs), cur.w, row0, item_hp(cur) * HPI / p.group, L.w, L.lane, L.lane_k, L.lane_v);
     }
     // The item after the current one is fetched from the lists as late as the prefetch pipeline allows (three tile steps
     // before the current item ends; at once for items shorter than that): an item fetched long before it starts keeps the
@@ -741,9 +751,9 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
             if (i + 1 < ne) {
                 const int row0 = ROWS ? __builtin_amdgcn_readfirstlane(entr_cur[i + 1 - base]) : 0;
                 if (L.wh == 0)
-                    issue_tile<D, 4, ROWS, GRP>(p, oth, __builtin_amdgcn_readfirstlane(ent_cur[i + 1 - base].x), row0, kvh, L.w, L.lane, L.lane_k, L.lane_v);
+                    issue_tile<D, 4, ROWS, GRP, TK>(p, oth, __builtin_amdgcn_readfirstlane(ent_cur[i + 1 - base].x), row0, kvh, L.w, L.lane, L.lane_k, L.lane_v);
             } else if (nxt_ok) {
-                if (L.wh == 0) issue_tile<D, 4, ROWS, GRP>(p, oth, nxt.w, nxt_row0, item_hp(nxt) * HPI / p.group, L.w, L.lane, L.lane_k, L.lane_v);
+                if (L.wh == 0) issue_tile<D, 4, ROWS, GRP, TK>(p, oth, nxt.w, nxt_row0, item_hp(nxt) * HPI / p.group, L.w, L.lane, L.lane_k, L.lane_v);
                 pstage = pstage == 2 ? 3 : -1;   // -1: tile requested before the entries (one-tile items)
             }
             const int2 en = ent_cur[i - base];
@@ -836,15 +846,15 @@ int device_state(DeviceState** out, long n_items) {
     return SPINF_OK;
 }
 
-template <int D, int RT, bool WIN, int NHW, bool ROWS, int GRP = 0>
+template <int D, int RT, bool WIN, int NHW, bool ROWS, int GRP = 0, int TK = 64>
 int launch(const AttnParams& p, int blocks, hipStream_t stream) {
-    using G = Geo<D>;
-    static_assert(2 * G::BUFB + 2 * ENT_CAP * 12 + ((NHW == 2 && D == 256) ? 16 : 4 * NHW * 32 * 144) + 64 <= 160 * 1024, "LDS budget");
-    hipLaunchKernelGGL((tree_attn_kernel<D, RT, WIN, NHW, ROWS, GRP>), dim3(blocks), dim3(256 * NHW), 0, stream, p);
+    using G = Geo<D, TK>;
+    static_assert(2 * G::BUFB + 2 * ENT_CAP * 12 + (((NHW == 2 && D == 256) || D == 512) ? 16 : 4 * NHW * 32 * 144) + 64 <= 160 * 1024, "LDS budget");
+    hipLaunchKernelGGL((tree_attn_kernel<D, RT, WIN, NHW, ROWS, GRP, TK>), dim3(blocks), dim3(256 * NHW), 0, stream, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: launch: %s", hipGetErrorString(e));
     // the exact pass over whatever the fast pass handed on (normally nothing: its workgroups read a zero count and leave)
-    hipLaunchKernelGGL((tree_attn_exact_kernel<D, RT, WIN, RT * NHW, ROWS, GRP>), dim3(blocks < 64 ? blocks : 64), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((tree_attn_exact_kernel<D, RT, WIN, RT * NHW, ROWS, GRP, TK>), dim3(blocks < 64 ? blocks : 64), dim3(256), 0, stream, p);
     e = hipGetLastError();
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: launch (exact pass): %s", hipGetErrorString(e));
     return SPINF_OK;
@@ -884,26 +894,15 @@ int launch_d(const AttnParams& p, int rt, int nhw, bool win, int grp_mode, int b
     return win ? launch<D, 1, true, 1, false>(p, blocks, s) : launch<D, 1, false, 1, false>(p, blocks, s);
 }
 
-// Head dim 512 (the full-attention layers of the Gemma-4 checkpoints, one key / value head): a 64-key K / V tile fills most of the
-// LDS, so there is one tile buffer and no fast pass; every item goes through the online-softmax kernel.
-template <bool WIN, bool ROWS, int GRP>
-int launch_512(AttnParams p, long n_items, int blocks, hipStream_t stream) {
-    using G = Geo<512>;
-    static_assert(G::BUFB + ENT_CAP * 12 + 4 * 32 * 144 + 64 <= 160 * 1024, "LDS budget");
-    p.all_items = (int)n_items;
-    hipLaunchKernelGGL((tree_attn_exact_kernel<512, 1, WIN, 1, ROWS, GRP>), dim3(blocks), dim3(256), 0, stream, p);
-    const hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: launch (head dim 512): %s", hipGetErrorString(e));
-    return SPINF_OK;
-}
-
-int launch_d512(const AttnParams& p, bool win, int grp_mode, long n_items, int blocks, hipStream_t s) {
+// Head dim 512 (the full-attention layers of the Gemma-4 checkpoints, one key / value head): two 64-key K / V tile buffers would
+// not fit the LDS, so the tiles are 32 keys (the plan is built with 32-key entries); four waves, one head per item.
+int launch_d512(const AttnParams& p, bool win, int grp_mode, int blocks, hipStream_t s) {
     if (p.grp) {
-        if (!win) return launch_512<false, false, 1>(p, n_items, blocks, s);
-        return grp_mode == 1 ? launch_512<true, false, 1>(p, n_items, blocks, s) : launch_512<true, false, 2>(p, n_items, blocks, s);
+        if (!win) return launch<512, 1, false, 1, false, 1, 32>(p, blocks, s);
+        return grp_mode == 1 ? launch<512, 1, true, 1, false, 1, 32>(p, blocks, s) : launch<512, 1, true, 1, false, 2, 32>(p, blocks, s);
     }
-    if (p.row_of) return win ? launch_512<true, true, 0>(p, n_items, blocks, s) : launch_512<false, true, 0>(p, n_items, blocks, s);
-    return win ? launch_512<true, false, 0>(p, n_items, blocks, s) : launch_512<false, false, 0>(p, n_items, blocks, s);
+    if (p.row_of) return win ? launch<512, 1, true, 1, true, 0, 32>(p, blocks, s) : launch<512, 1, false, 1, true, 0, 32>(p, blocks, s);
+    return win ? launch<512, 1, true, 1, false, 0, 32>(p, blocks, s) : launch<512, 1, false, 1, false, 0, 32>(p, blocks, s);
 }
 
 }  // namespace
@@ -943,6 +942,8 @@ extern "C" int spinf_tree_attn_fwd(const spinf_attn_args* a, void* stream) {
     pick_kernel(a->hq, a->hkv, a->d, a->variant, &rt, &nhw);
     if ((a->row_of != nullptr) != (a->kv_row0 != nullptr)) return spinf_fail(SPINF_E_ARG, "tree_attn: row_of and kv_row0 come together");
     if (a->row_of && rt != 1) return spinf_fail(SPINF_E_ARG, "tree_attn: variant %d does not take compact rows", a->variant);
+    if ((a->d == 512) != (a->ktile == 32) || (a->ktile != 0 && a->ktile != 32 && a->ktile != 64))
+        return spinf_fail(SPINF_E_ARG, "tree_attn: plan entries of %d keys with head dim %d (32 goes with 512, 64 with the others)", a->ktile ? a->ktile : 64, a->d);
     if (a->grp && (a->grp_mode != 1 && a->grp_mode != 2)) return spinf_fail(SPINF_E_ARG, "tree_attn: group mode %d not in {1, 2}", a->grp_mode);
     if (a->grp && (rt != 1 || a->row_of)) return spinf_fail(SPINF_E_ARG, "tree_attn: image groups go with variant 0 / 1 and the stream layout only");
     const int hpi = rt * nhw;
@@ -970,7 +971,6 @@ extern "C" int spinf_tree_attn_fwd(const spinf_attn_args* a, void* stream) {
     p.items = (const int4*)a->items; p.list_ptr = a->list_ptr;
     p.row_of = a->row_of; p.kv_row0 = a->kv_row0;
     p.grp = a->grp;
-    p.all_items = 0;
     p.counters = st->counters;
     p.redo = st->counters + 64;
     const int blocks = (int)(a->n_items < st->cus ? a->n_items : st->cus);
@@ -980,6 +980,6 @@ extern "C" int spinf_tree_attn_fwd(const spinf_attn_args* a, void* stream) {
         case 64: return launch_d<64>(p, rt, nhw, win, a->grp_mode, blocks, s);
         case 128: return launch_d<128>(p, rt, nhw, win, a->grp_mode, blocks, s);
         case 256: return launch_d<256>(p, rt, nhw, win, a->grp_mode, blocks, s);
-        default: return launch_d512(p, win, a->grp_mode, (long)a->n_items, blocks, s);
+        default: return launch_d512(p, win, a->grp_mode, blocks, s);
     }
 }

@@ -24,7 +24,7 @@ class AttnArgs(C.Structure):
         ("kv_idx", C.c_void_p), ("kv_bits", C.c_void_p), ("items", C.c_void_p), ("list_ptr", C.c_void_p),
         ("n_items", C.c_int64), ("variant", C.c_int32),
         ("row_of", C.c_void_p), ("kv_row0", C.c_void_p),
-        ("grp", C.c_void_p), ("grp_mode", C.c_int32),
+        ("grp", C.c_void_p), ("grp_mode", C.c_int32), ("ktile", C.c_int32),
     ]
 
 
@@ -81,6 +81,7 @@ def load_library():
     lib.spinf_version.restype = C.c_int
     lib.spinf_tileplan_build.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.POINTER(C.c_void_p)]
     lib.spinf_tileplan_build_groups.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_int32, C.POINTER(C.c_void_p)]
+    lib.spinf_tileplan_build_ktile.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_int32, C.c_int32, C.POINTER(C.c_void_p)]
     lib.spinf_tileplan_counts.argtypes = [C.c_void_p, C.POINTER(C.c_int64)]
     lib.spinf_tileplan_export.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
     lib.spinf_tileplan_schedule.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p]
@@ -95,7 +96,7 @@ def load_library():
     lib.spinf_gdn_prologue.argtypes = [C.POINTER(GdnPreArgs), C.c_void_p]
     lib.spinf_gdn_gate.argtypes = [C.POINTER(GdnGateArgs), C.c_void_p]
     lib.spinf_lm_logprobs.argtypes = [C.POINTER(LmArgs), C.c_void_p]
-    for name in ("spinf_tileplan_build", "spinf_tileplan_build_groups", "spinf_tileplan_counts", "spinf_tileplan_export", "spinf_tileplan_schedule", "spinf_tileplan_row0", "spinf_tree_attn_fwd", "spinf_attn_exact_items", "spinf_gdn_fwd", "spinf_gdn_prologue", "spinf_gdn_gate", "spinf_lm_logprobs"):
+    for name in ("spinf_tileplan_build", "spinf_tileplan_build_groups", "spinf_tileplan_build_ktile", "spinf_tileplan_counts", "spinf_tileplan_export", "spinf_tileplan_schedule", "spinf_tileplan_row0", "spinf_tree_attn_fwd", "spinf_attn_exact_items", "spinf_gdn_fwd", "spinf_gdn_prologue", "spinf_gdn_gate", "spinf_lm_logprobs"):
         getattr(lib, name).restype = C.c_int
     _LIB = lib
     return lib

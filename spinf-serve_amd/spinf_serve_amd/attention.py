@@ -28,7 +28,7 @@ VARIANT = int(os.environ.get("SPINF_ATTN_VARIANT", "0"))
 def _tree_attn_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, art: torch.Tensor, end: torch.Tensor, pos: torch.Tensor,
                   kv_idx: torch.Tensor, kv_bits: torch.Tensor, items: torch.Tensor, list_ptr: torch.Tensor, n_items: int,
                   scale: float, window: int, variant: int, row_of: Optional[torch.Tensor], kv_row0: Optional[torch.Tensor],
-                  n_mapped: int, grp: Optional[torch.Tensor], grp_mode: int) -> torch.Tensor:
+                  n_mapped: int, grp: Optional[torch.Tensor], grp_mode: int, ktile: int) -> torch.Tensor:
     """q [rows, hq, d], k / v [rows, hkv, d] (any token / head strides, d contiguous) -> out [rows, hq, d] contiguous, bf16.
     rows = the stream length, or with row_of / kv_row0 (compact rows) any number of rows: the kernel maps stream positions to
     rows through row_of; rows 0 .. n_mapped-1 are the rows row_of names (each written by the kernel), later rows come back zero."""
@@ -67,6 +67,7 @@ def _tree_attn_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, art: torch.
     a.kv_idx, a.kv_bits, a.items, a.list_ptr = kv_idx.data_ptr(), kv_bits.data_ptr(), items.data_ptr(), list_ptr.data_ptr()
     a.n_items = n_items
     a.variant = variant
+    a.ktile = ktile
     if row_of is not None:
         a.row_of, a.kv_row0 = row_of.data_ptr(), kv_row0.data_ptr()
     if grp is not None:
@@ -81,7 +82,7 @@ def _tree_attn_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, art: torch.
 
 
 @_tree_attn_op.register_fake
-def _(q, k, v, art, end, pos, kv_idx, kv_bits, items, list_ptr, n_items, scale, window, variant, row_of, kv_row0, n_mapped, grp, grp_mode):
+def _(q, k, v, art, end, pos, kv_idx, kv_bits, items, list_ptr, n_items, scale, window, variant, row_of, kv_row0, n_mapped, grp, grp_mode, ktile):
     return torch.empty(q.shape, dtype=torch.bfloat16, device=q.device)
 
 
@@ -102,6 +103,7 @@ def tree_attn(q, k, v, mask: TreeMask, scale=None, variant=None, sidx=None):
     if sidx is not None and mask.grp is not None:
         raise ValueError("image groups go with the stream layout (no sidx)")
     hq, hkv, d = q.shape[1], k.shape[1], q.shape[2]
+    mask = mask.for_head_dim(d)
     per_item = _lib.load_library().spinf_attn_heads_per_item(hq, hkv, d, variant)
     if per_item <= 0:
         raise ValueError(f"{hq} query heads do not group over {hkv} key / value heads")
@@ -109,7 +111,7 @@ def tree_attn(q, k, v, mask: TreeMask, scale=None, variant=None, sidx=None):
     row_of, kv_row0 = mask.rows(sidx) if sidx is not None else (None, None)
     return _tree_attn_op(q, k, v, mask.art, mask.end, mask.pos, mask.kv_idx, mask.kv_bits, items, list_ptr, n_items,
                          scale, int(mask.window), variant, row_of, kv_row0, 0 if sidx is None else int(sidx.shape[0]),
-                         mask.grp, int(mask.grp_mode))
+                         mask.grp, int(mask.grp_mode), int(mask.plan.ktile))
 
 
 # K/V capture for extraction, as spinf_serve/models/gemma4.py:66-70: while CAPTURE[device] = {"window", "ranges": [(start, n, key)],

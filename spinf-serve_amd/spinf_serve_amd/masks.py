@@ -17,8 +17,9 @@ from . import _lib
 class TilePlan:
     """host arrays of a compiled plan (see include/spinf_tree.h) and the native handle that makes its work lists"""
 
-    def __init__(self, handle, qt_ptr, kv_idx, kv_bits, order, n, window, active_blocks, masked_blocks, grp_mode=0):
+    def __init__(self, handle, qt_ptr, kv_idx, kv_bits, order, n, window, active_blocks, masked_blocks, grp_mode=0, ktile=64):
         self._handle = handle
+        self.ktile = ktile
         self.qt_ptr, self.kv_idx, self.kv_bits, self.order = qt_ptr, kv_idx, kv_bits, order
         self.n, self.window, self.grp_mode = n, window, grp_mode
         self.active_blocks, self.masked_blocks = active_blocks, masked_blocks
@@ -33,9 +34,9 @@ class TilePlan:
                 pass
 
     @classmethod
-    def build(cls, art, end, pos, window=None, grp=None, grp_windowed=False) -> "TilePlan":
+    def build(cls, art, end, pos, window=None, grp=None, grp_windowed=False, ktile=64) -> "TilePlan":
         """grp (image groups, spinf_serve/scorer.py:184-198): [n] int32, -1 none; the tokens of a group also see each other both
-        ways, past the window unless grp_windowed"""
+        ways, past the window unless grp_windowed.  ktile: keys per entry, 64, or 32 for the head dim 512 kernel."""
         lib = _lib.load_library()
         art = np.ascontiguousarray(art, np.int32)
         end = np.ascontiguousarray(end, np.int32)
@@ -46,15 +47,15 @@ class TilePlan:
         w = int(window) if window else 0
         h = C.c_void_p()
         mode = 0
-        if grp is None:
-            _lib.check(lib.spinf_tileplan_build(art.ctypes.data, end.ctypes.data, pos.ctypes.data, n, w, C.byref(h)), "tileplan_build")
-        else:
+        gptr = None
+        if grp is not None:
             grp = np.ascontiguousarray(grp, np.int32)
             if len(grp) != n:
                 raise ValueError("grp differs in length from art")
             mode = 2 if grp_windowed else 1
-            _lib.check(lib.spinf_tileplan_build_groups(art.ctypes.data, end.ctypes.data, pos.ctypes.data, grp.ctypes.data, mode, n, w, C.byref(h)),
-                       "tileplan_build_groups")
+            gptr = grp.ctypes.data
+        _lib.check(lib.spinf_tileplan_build_ktile(art.ctypes.data, end.ctypes.data, pos.ctypes.data, gptr, mode, n, w, int(ktile), C.byref(h)),
+                   "tileplan_build")
         try:
             counts = (C.c_int64 * 5)()
             _lib.check(lib.spinf_tileplan_counts(h, counts), "tileplan_counts")
@@ -67,7 +68,7 @@ class TilePlan:
         except Exception:
             lib.spinf_tileplan_free(h)
             raise
-        return cls(h, qt_ptr, kv_idx[:nent], kv_bits[:nent], order[:nqt], n, w, int(counts[2]), int(counts[3]), mode)
+        return cls(h, qt_ptr, kv_idx[:nent], kv_bits[:nent], order[:nqt], n, w, int(counts[2]), int(counts[3]), mode, int(ktile))
 
     @property
     def n_qtiles(self) -> int:
@@ -97,8 +98,10 @@ class TreeMask:
     """Device-side handle: the stream's metadata + one compiled plan.  ``seq_lengths`` mirrors BlockMask.seq_lengths
     (spinf_serve/models/qwen35/qwen.py:615 reads it)."""
 
-    def __init__(self, plan: TilePlan, meta, device, grp=None):
+    def __init__(self, plan: TilePlan, meta, device, grp=None, host=None):
         self.plan = plan
+        self._host = host                   # (art, end, pos, grp, grp_windowed) on the host, for a plan of another key-tile size
+        self._other = None
         self.grp = grp                      # device copy of the image groups the plan was built with, or None
         self.grp_mode = plan.grp_mode if grp is not None else 0
         self.n = plan.n
@@ -112,6 +115,21 @@ class TreeMask:
         self._sched = {}
         self._rows = None
 
+    def for_head_dim(self, d: int) -> "TreeMask":
+        """the mask with the plan granularity the kernel of this head dim takes: 32-key entries at 512, 64-key ones otherwise
+        (the second plan is compiled on first use and shares the device metadata)"""
+        ktile = 32 if d == 512 else 64
+        if ktile == self.plan.ktile:
+            return self
+        if self._other is None:
+            if self._host is None:
+                raise ValueError(f"this mask was built for key tiles of {self.plan.ktile}; head dim {d} takes {ktile}")
+            art, end, pos, grp, grp_windowed = self._host
+            plan = TilePlan.build(art, end, pos, self.window, grp, grp_windowed, ktile)
+            self._other = TreeMask(plan, (self.art, self.end, self.pos), self.device, self.grp)
+            self._other._other = self
+        return self._other
+
     def rows(self, sidx):
         """compact rows (spinf_serve/models/qwen35/qwen.py:613-622): sidx [R] = stream position of each real row (a device
         tensor) -> (row_of [n], kv_row0 [entries]) int32 device tensors for the kernel: the row of each stream position (-1:
@@ -124,8 +142,9 @@ class TreeMask:
         n = self.n
         row_of = torch.full((n + 63,), -1, dtype=torch.int32, device=self.device)   # padded: every key tile is 64 long
         row_of[sidx.to(self.device, torch.long)] = torch.arange(sidx.shape[0], dtype=torch.int32, device=self.device)
-        tiles = row_of[: (n + 63) // 64 * 64].view(-1, 64)
-        run = (tiles - tiles[:, :1]) == torch.arange(64, dtype=torch.int32, device=self.device)
+        kt = self.plan.ktile
+        tiles = row_of[: (n + kt - 1) // kt * kt].view(-1, kt)
+        run = (tiles - tiles[:, :1]) == torch.arange(kt, dtype=torch.int32, device=self.device)
         tile_row0 = torch.where((tiles[:, 0] >= 0) & run.all(1), tiles[:, 0], torch.full_like(tiles[:, 0], -1))
         kv_row0 = tile_row0[self.kv_idx.long()].contiguous()
         self._rows = (sidx, row_of[:n].contiguous(), kv_row0)
@@ -152,7 +171,8 @@ class TreeMask:
             meta = tuple(_upload(a, np.int32, device) for a in (art, end, pos))
         if grp is not None and grp_dev is None:
             grp_dev = _upload(grp, np.int32, device)
-        return cls(TilePlan.build(art, end, pos, window, grp, grp_windowed), meta, device, grp_dev if grp is not None else None)
+        return cls(TilePlan.build(art, end, pos, window, grp, grp_windowed), meta, device, grp_dev if grp is not None else None,
+                   host=(art, end, pos, grp, grp_windowed))
 
 
 def block_masks(batch, sliding_window=None, device="cuda", grp=None, bidir_all=True):
