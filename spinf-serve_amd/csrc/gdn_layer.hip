@@ -58,7 +58,7 @@ __device__ __forceinline__ bf16x8 load_row(const __bf16* y, long y_tok, long row
     return v;
 }
 
-constexpr int MAX_TOK = 64;   // tokens a workgroup walks over at most
+constexpr int MAX_TOK = 128;  // tokens a workgroup walks over at most
 
 __global__ __launch_bounds__(256) void gdn_prologue_kernel(const PreParams p) {
     const int c0 = (blockIdx.y * 256 + threadIdx.x) * LANE_CH;
@@ -145,9 +145,12 @@ __global__ __launch_bounds__(256) void gdn_prologue_kernel(const PreParams p) {
                 acc += (float)x2[i] * w[i][2];
                 acc += (float)x3[i] * w[i][3];
                 s[i] = (__bf16)silu(acc);
-                ss += (float)s[i] * (float)s[i];
             }
-            ss = head_sum(ss, p.head_lanes);   // l2 norm over the head; every lane takes part in the exchange
+            if (__builtin_amdgcn_ballot_w64(norm) != 0) {   // (a wave of v channels skips the norm's sums altogether)
+#pragma unroll
+                for (int i = 0; i < LANE_CH; i++) ss += (float)s[i] * (float)s[i];
+                ss = head_sum(ss, p.head_lanes);   // l2 norm over the head; every lane of the wave takes part in the exchange
+            }
             if (norm) {
                 const float r = rsqrtf(ss + 1e-6f);
 #pragma unroll
