@@ -178,3 +178,35 @@ def test_deep_trie(dev):
     o = sa.gdn_tree(t["q"], t["k"], t["v"], t["g"], t["beta"], cfg.plan(dev))
     want = ogdn.tree_scan(*(_np(t[x]) for x in ("q", "k", "v", "g", "beta")), cfg.batch.prev, cfg.batch.art >= 0)
     assert float(np.abs(_np(o) - want).max()) <= TOL
+
+
+def test_decoder_steps_rerun_the_recurrence_from_the_prefix_state(dev):
+    """the extraction decoder's call (spinf_serve/models/qwen35/qwen_decode.py:305-318): every step each slot re-runs the recurrence
+    from its group's prefix state over its template rows plus the tokens generated so far, read out of row caches through idx,
+    outputs written into a buffer at the same rows; no per-slot state is kept.  Two groups, slots of different template lengths."""
+    H, HV, R = 2, 4, 512
+    rng = np.random.default_rng(2)
+    t = _inputs(R, H, HV, dev, seed=9)                       # the row caches: any row may belong to any slot
+    caches = [t[x][None] for x in ("q", "k", "v", "g", "beta")]
+    states = (torch.randn((2, HV, 128, 128), device=dev) * 0.1).contiguous()   # the two groups' prefix states
+    slot_group = [0, 0, 0, 1, 1]
+    templates = [5, 17, 30, 9, 40]
+    free = list(rng.permutation(R))
+    rows = [[int(free.pop()) for _ in range(n)] for n in templates]            # each slot's template rows, scattered
+    o_buf = torch.full((1, R, HV, 128), float("nan"), device=dev, dtype=torch.bfloat16)
+    h0_idx = torch.tensor(slot_group, device=dev)
+    for step in range(4):
+        for r in rows:
+            r.append(int(free.pop()))                                            # the step's new token of every slot
+        lens = [len(r) for r in rows]
+        cu = torch.tensor(np.concatenate([[0], np.cumsum(lens)]), dtype=torch.int64, device=dev)
+        idx = torch.tensor([x for r in rows for x in r], dtype=torch.int64, device=dev)
+        sa.recurrent(*caches, 128 ** -0.5, cu, len(rows), h0=states, h0_idx=h0_idx, idx=idx, o=o_buf)
+        torch.cuda.synchronize()
+        for s, r in enumerate(rows):
+            want, _ = ogdn.recurrent(*(_np(t[x][r]) for x in ("q", "k", "v", "g", "beta")), h0=_np(states[slot_group[s]]))
+            assert float(np.abs(_np(o_buf[0, r[-1]]) - want[-1]).max()) <= TOL, (step, s)   # the decoder reads the new token's row
+            assert float(np.abs(_np(o_buf[0, r]) - want).max()) <= TOL
+    used = sorted(x for r in rows for x in r)
+    untouched = np.setdiff1d(np.arange(R), used)
+    assert torch.isnan(o_buf[0, untouched].float()).all()                         # rows of no slot are never written
