@@ -102,6 +102,17 @@ struct Geo {
     static constexpr int KSUB = k_off(32), VSUB = v_off(32);   // byte offsets of rows 32.. relative to rows 0..
 };
 
+// A tile buffer: the K tile at the key head dim D, the V tile at DV head dims (DV = D, except at head dim 512, where O^T is
+// computed 256 dims at a time: see launch_d512), then art, end, pos, grp of the keys.
+template <int D, int TK, int DV>
+struct TileGeo {
+    using K = Geo<D, TK>;
+    using V = Geo<DV, TK>;
+    static constexpr int KTILEB = K::KTILEB, VTILEB = V::VTILEB;
+    static constexpr int BUFB = KTILEB + VTILEB + K::METAB;
+    static constexpr int KSUB = K::KSUB, VSUB = V::VSUB;
+};
+
 // One wave-wide DMA instruction: 64 lanes x `16` (or 4) bytes from global memory straight into 1 KiB (256 B) of contiguous
 // LDS at byte address `lds`.  Written as inline assembly on purpose: the compiler then does not track these LDS writes, so
 // it never makes the fragment reads of the OTHER tile buffer wait for them (it cannot tell the two buffers apart once the
@@ -131,38 +142,50 @@ __device__ __forceinline__ unsigned lds_addr(const void* p) { return (unsigned)(
 // the stream every address is a wave-uniform base plus a per-lane constant (lane_k / lane_v, bytes), so the loop spends no
 // vector ALU on addressing; the last, partial tile clamps its rows per lane.
 // ROWS (compact rows): row0 >= 0 says that the tile's keys are rows row0 .. row0 + 63; otherwise every lane looks its row up.
-template <int D, int NW = 4, bool ROWS = false, int GRP = 0, int TK = 64>
+template <int D, int NW = 4, bool ROWS = false, int GRP = 0, int TK = 64, int DV = D>
 __device__ __forceinline__ void issue_tile(const AttnParams& p, unsigned buf, int kt, int row0, int kvh, int w, int lane, unsigned lane_k, unsigned lane_v) {
-    using G = Geo<D, TK>;
-    constexpr int IPW = G::NREG / NW;   // DMA instructions per wave and tile
-    static_assert(IPW >= 1 && IPW * NW == G::NREG, "the tile's regions must divide among the waves");
+    using G = TileGeo<D, TK, DV>;
+    using GK = typename G::K;
+    using GV = typename G::V;
+    constexpr int IPWK = GK::NREG / NW, IPWV = GV::NREG / NW;   // DMA instructions per wave and tile
+    static_assert(IPWK >= 1 && IPWK * NW == GK::NREG && IPWV >= 1 && IPWV * NW == GV::NREG, "the tile's regions must divide among the waves");
     const char* kbase = (const char*)(p.k + (long)kvh * p.k_head);
     const char* vbase = (const char*)(p.v + (long)kvh * p.v_head);
     if (ROWS ? row0 >= 0 : kt * TK + TK <= p.n) {
+        const long first = ROWS ? (long)row0 : (long)kt * TK;
 #pragma unroll
-        for (int i = 0; i < IPW; i++) {
-            const int reg = w * IPW + i;
-            const long row = (ROWS ? (long)row0 : (long)kt * TK) + reg;
-            dma16_uniform(kbase + row * p.k_tok * 2, lane_k, buf + reg * G::KRS);
-            dma16_uniform(vbase + row * p.v_tok * 2, lane_v, buf + G::KTILEB + reg * G::VRS);
+        for (int i = 0; i < IPWK; i++) {
+            const int reg = w * IPWK + i;
+            dma16_uniform(kbase + (first + reg) * p.k_tok * 2, lane_k, buf + reg * GK::KRS);
+        }
+#pragma unroll
+        for (int i = 0; i < IPWV; i++) {
+            const int reg = w * IPWV + i;
+            dma16_uniform(vbase + (first + reg) * p.v_tok * 2, lane_v, buf + G::KTILEB + reg * GV::VRS);
         }
         if (w < (GRP ? 4 : 3)) {   // wave 0: art, wave 1: end, wave 2: pos, wave 3: grp of the 64 keys
             const int* src = (w == 0 ? p.art : w == 1 ? p.end : w == 2 ? p.pos : p.grp) + (long)kt * TK;
             dma4_lane(src + (TK < 64 ? lane % TK : lane), buf + G::KTILEB + G::VTILEB + w * 256);   // (64 lanes: a 32-key tile's twice)
         }
     } else {
-        const int slot = lane / G::CPR, chunk = lane % G::CPR;
-#pragma unroll
-        for (int i = 0; i < IPW; i++) {
-            const int reg = w * IPW + i;
-            long grow = (long)kt * TK + reg + G::NREG * slot;
+        auto row_at = [&](const int reg, const int nreg, const int slot) {
+            long grow = (long)kt * TK + reg + nreg * slot;
             grow = grow < p.n ? grow : p.n - 1;
             if (ROWS) {   // a pad position has no row: any row will do, its keys are visible to nobody but pad rows
                 const int r = p.row_of[grow];
                 grow = r < 0 ? 0 : r;
             }
-            dma16_lane(kbase + grow * p.k_tok * 2 + chunk * 16, buf + reg * G::KRS);
-            dma16_lane(vbase + grow * p.v_tok * 2 + chunk * 16, buf + G::KTILEB + reg * G::VRS);
+            return grow;
+        };
+#pragma unroll
+        for (int i = 0; i < IPWK; i++) {
+            const int reg = w * IPWK + i;
+            dma16_lane(kbase + row_at(reg, GK::NREG, lane / GK::CPR) * p.k_tok * 2 + (lane % GK::CPR) * 16, buf + reg * GK::KRS);
+        }
+#pragma unroll
+        for (int i = 0; i < IPWV; i++) {
+            const int reg = w * IPWV + i;
+            dma16_lane(vbase + row_at(reg, GV::NREG, lane / GV::CPR) * p.v_tok * 2 + (lane % GV::CPR) * 16, buf + G::KTILEB + reg * GV::VRS);
         }
         if (w < (GRP ? 4 : 3)) {
             long gk = (long)kt * TK + (TK < 64 ? lane % TK : lane);
@@ -173,9 +196,10 @@ __device__ __forceinline__ void issue_tile(const AttnParams& p, unsigned buf, in
 }
 
 // Everything a wave needs to know about its place in the workgroup and its LDS fragment addresses.
-template <int D, int TK = 64>
+template <int D, int TK = 64, int DV = D>
 struct Lane {
-    using G = Geo<D, TK>;
+    using GK = Geo<D, TK>;
+    using GV = Geo<DV, TK>;
     int lane, m, g, w;
     int wr, wh;                  // row group (tokens 32 wr ..) and head set of this wave
     int k_lane, v_lane;          // byte offsets of this lane's K fragment row / V^T fragment address inside a tile
@@ -193,10 +217,10 @@ struct Lane {
         // (ds_read_b64_tr_b16): inside its 16-lane group a lane supplies the address of key row 4g + tr_j, head dims
         // 16 tr_mb + 4 tr_a .. +3 of the 32-wide slice, and receives head dim lane%32 of 4 consecutive keys.
         const int tr_a = lane & 3, tr_j = (lane >> 2) & 3, tr_mb = (lane >> 4) & 1;
-        k_lane = G::k_off(m) + 16 * g;
-        v_lane = G::v_off(4 * g + tr_j) + 32 * tr_mb + 8 * tr_a;
-        lane_k = (unsigned)((lane / G::CPR) * G::NREG * p.k_tok * 2 + (lane % G::CPR) * 16);
-        lane_v = (unsigned)((lane / G::CPR) * G::NREG * p.v_tok * 2 + (lane % G::CPR) * 16);
+        k_lane = GK::k_off(m) + 16 * g;
+        v_lane = GV::v_off(4 * g + tr_j) + 32 * tr_mb + 8 * tr_a;
+        lane_k = (unsigned)((lane / GK::CPR) * GK::NREG * p.k_tok * 2 + (lane % GK::CPR) * 16);
+        lane_v = (unsigned)((lane / GV::CPR) * GV::NREG * p.v_tok * 2 + (lane % GV::CPR) * 16);
     }
 };
 
@@ -302,11 +326,11 @@ __device__ __forceinline__ void store_rows(const AttnParams& p, const LaneT& L, 
 // Classic online softmax over one work item, one 32-key block at a time, nothing overlapped: the rare fallback, in a
 // kernel of its own because its accumulator rescaling (vector ALU on all of O) would cost the fast pass its register
 // allocation.
-template <int D, int RT, bool WIN, bool ROWS, int GRP, int TK>
+template <int D, int RT, bool WIN, bool ROWS, int GRP, int TK, int DV>
 __device__ __forceinline__ void attn_item_exact(const AttnParams& p, const int4 item, const int h0, char* buf0, int2* ent, int* ent_row0, char* stage) {
-    using G = Geo<D, TK>;
-    constexpr int NS = D / 16, NDT = D / 32;
-    const Lane<D, TK> L(p);
+    using G = TileGeo<D, TK, DV>;
+    constexpr int NS = D / 16, NDT = DV / 32;
+    const Lane<D, TK, DV> L(p);
     const int t = item.x, e0 = item.y, ne = item.z & 0xfffff;   // heads h0 .. h0 + RT - 1 of the item
     const int kvh = h0 / p.group;
     const int tok = t * SPINF_QTILE + 32 * L.w + L.m;
@@ -359,7 +383,7 @@ __device__ __forceinline__ void attn_item_exact(const AttnParams& p, const int4 
         const unsigned bits = (unsigned)__builtin_amdgcn_readfirstlane(en.y) >> (2 * L.w);
         const int row0 = ROWS ? __builtin_amdgcn_readfirstlane(ent_row0[i - base]) : 0;
         __syncthreads();   // everyone is done with the buffer
-        issue_tile<D, 4, ROWS, GRP, TK>(p, lds_addr(buf0), kt, row0, kvh, L.w, L.lane, L.lane_k, L.lane_v);
+        issue_tile<D, 4, ROWS, GRP, TK, DV>(p, lds_addr(buf0), kt, row0, kvh, L.w, L.lane, L.lane_k, L.lane_v);
         __builtin_amdgcn_s_waitcnt(0x0f70);
         __syncthreads();
         const char* kb = buf0;
@@ -417,9 +441,9 @@ __device__ __forceinline__ void attn_item_exact(const AttnParams& p, const int4 
             }
 #pragma unroll
             for (int f = 0; f < 2 * NDT; f++) {
-                const char* vp = vrow + G::v_off(16 * (f / NDT)) + 64 * (f % NDT);
+                const char* vp = vrow + G::V::v_off(16 * (f / NDT)) + 64 * (f % NDT);
                 const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)vp);
-                const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vp + G::v_off(8)));
+                const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vp + G::V::v_off(8)));
                 const bf16x8 a = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
 #pragma unroll
                 for (int rt = 0; rt < RT; rt++) o[rt][f % NDT] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[rt][f / NDT], o[rt][f % NDT], 0, 0, 0);
@@ -427,13 +451,13 @@ __device__ __forceinline__ void attn_item_exact(const AttnParams& p, const int4 
             }
         }
     }
-    store_rows<D, RT, ROWS>(p, L, stage, o, l, t, h0);
+    store_rows<DV, RT, ROWS>(p, L, stage, o, l, t, h0);
 }
 
 // An item of HPI heads is recomputed RT heads at a time.
-template <int D, int RT, bool WIN, int HPI, bool ROWS, int GRP, int TK = 64>
+template <int D, int RT, bool WIN, int HPI, bool ROWS, int GRP, int TK = 64, int DV = D>
 __global__ __launch_bounds__(256) void tree_attn_exact_kernel(const AttnParams p) {
-    using G = Geo<D, TK>;
+    using G = TileGeo<D, TK, DV>;
     __shared__ __attribute__((aligned(16))) char buf0[G::BUFB];
     __shared__ int2 ent[ENT_CAP];
     __shared__ int ent_row0[ROWS ? ENT_CAP : 1];
@@ -446,7 +470,7 @@ __global__ __launch_bounds__(256) void tree_attn_exact_kernel(const AttnParams p
         const int4 item = make_int4(__builtin_amdgcn_readfirstlane(it.x), __builtin_amdgcn_readfirstlane(it.y),
                                     __builtin_amdgcn_readfirstlane(it.z), __builtin_amdgcn_readfirstlane(it.w));
         const int hp = (int)((unsigned)item.z >> 20);
-        for (int sub = 0; sub < HPI; sub += RT) attn_item_exact<D, RT, WIN, ROWS, GRP, TK>(p, item, hp * HPI + sub, buf0, ent, ent_row0, stage_all + w * 32 * 144);
+        for (int sub = 0; sub < HPI; sub += RT) attn_item_exact<D, RT, WIN, ROWS, GRP, TK, DV>(p, item, hp * HPI + sub, buf0, ent, ent_row0, stage_all + w * 32 * 144);
     }
     __builtin_amdgcn_s_waitcnt(0x0f70);
     __syncthreads();
@@ -480,16 +504,16 @@ extern "C" int spinf_debug_trace(long* out, int n) { return (int)hipMemcpyFromSy
 // on the same K / V tiles (two waves per SIMD: one wave's softmax runs under the other's MFMAs).
 // ROWS: q, k, v, o hold the real tokens only (compact rows); the stream positions of the plan are mapped through row_of.
 // GRP: image groups (1: their tokens see each other whatever the window, 2: within the window).
-template <int D, int RT, bool WIN, int NHW, bool ROWS, int GRP, int TK = 64>
+template <int D, int RT, bool WIN, int NHW, bool ROWS, int GRP, int TK = 64, int DV = D>
 __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p) {
-    using G = Geo<D, TK>;
+    using G = TileGeo<D, TK, DV>;
     constexpr int HPI = RT * NHW;  // heads per work item
     constexpr int NS = D / 16;     // contraction steps of K Q^T
-    constexpr int NDT = D / 32;    // 32-wide slices of the head dimension in O^T
+    constexpr int NDT = DV / 32;   // 32-wide slices of the (value) head dimension in O^T
     constexpr int NVF = 2 * NDT;   // V^T fragments of one 32-key block
     // fragment read-ahead depth: the register file is the tight one at head dim 256 (4 with one wave per SIMD, 3 with two:
     // measured 0.374 / 0.351 / 0.343 / 0.368 ms on the 24-content pass for depths 4 / 2 / 3 / 1); no effect at 128
-    constexpr int PFD = D > 256 ? 2 : D == 256 ? (NHW == 2 ? 3 : 4) : 8;
+    constexpr int PFD = D >= 256 ? (NHW == 2 ? 3 : 4) : 8;
     constexpr int PF = NS < PFD ? NS : PFD;     // K fragments read ahead of the MFMAs
     constexpr int VPF = NVF < PFD ? NVF : PFD;  // V^T fragments read ahead
     __shared__ __attribute__((aligned(16))) char bufs[2 * G::BUFB];   // the two tile buffers
@@ -500,14 +524,14 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
     // output staging, one slice per wave; with eight waves at head dim 256 there is no room left for it and the slices lie in
     // the tile buffer the item's last tile was computed from (free from the barrier after the tile loop until the next
     // item's first tile step requests a tile into it, which comes after that step's barrier)
-    constexpr bool STAGE_IN_TILE = (NHW == 2 && D == 256) || D == 512;
+    constexpr bool STAGE_IN_TILE = NHW == 2 && D == 256;
     static_assert(!STAGE_IN_TILE || 4 * NHW * 32 * 144 <= G::BUFB, "the staging slices must fit a tile buffer");
     __shared__ __attribute__((aligned(16))) char stage_all[STAGE_IN_TILE ? 16 : 4 * NHW * 32 * 144];
     __shared__ int s_next[2];         // item grabbed by thread 0 for the whole workgroup, double buffered
 
     TRACE_CLK(tk0);
     TRACE_WALL(tw0);
-    const Lane<D, TK> L(p);
+    const Lane<D, TK, DV> L(p);
     char* const stage_own = stage_all + (STAGE_IN_TILE ? 0 : L.w * 32 * 144);
 
     // ---- work lists: start with the list of this workgroup's XCD, continue with the following ones
@@ -631,9 +655,9 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
     auto pv_phase = [&](const char* vrow, const bf16x8 (&pb)[RT][2]) __attribute__((always_inline)) {
         s16x4 vlo[VPF], vhi[VPF];
         auto vload = [&](const int f, const int slot) __attribute__((always_inline)) {
-            const char* vp = vrow + G::v_off(16 * (f / NDT)) + 64 * (f % NDT);
+            const char* vp = vrow + G::V::v_off(16 * (f / NDT)) + 64 * (f % NDT);
             vlo[slot] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)vp);
-            vhi[slot] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vp + G::v_off(8)));
+            vhi[slot] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vp + G::V::v_off(8)));
         };
 #pragma unroll
         for (int f = 0; f < VPF; f++) vload(f, f);
@@ -689,7 +713,7 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
         load_q(cur, qf, art_q, pos_q, grp_q);
         load_ent(cur, ent_cur, entr_cur, 0);
         const int row0 = ROWS ? __builtin_amdgcn_readfirstlane(p.kv_row0[cur.y]) : 0;
-        if (L.wh == 0) issue_tile<D, 4, ROWS, GRP, TK>(p, lds_addr(bufs), cur.w, row0, item_hp(cur) * HPI / p.group, L.w, L.lane, L.lane_k, L.lane_v);
+        if (L.wh == 0) issue_tile<D, 4, ROWS, GRP, TK, DV>(p, lds_addr(bufs), cur.w, row0, item_hp(cur) * HPI / p.group, L.w, L.lane, L.lane_k, L.lane_v);
     }
     // The item after the current one is fetched from the lists as late as the prefetch pipeline allows (three tile steps
     // before the current item ends; at once for items shorter than that): an item fetched long before it starts keeps the
@@ -751,9 +775,9 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
             if (i + 1 < ne) {
                 const int row0 = ROWS ? __builtin_amdgcn_readfirstlane(entr_cur[i + 1 - base]) : 0;
                 if (L.wh == 0)
-                    issue_tile<D, 4, ROWS, GRP, TK>(p, oth, __builtin_amdgcn_readfirstlane(ent_cur[i + 1 - base].x), row0, kvh, L.w, L.lane, L.lane_k, L.lane_v);
+                    issue_tile<D, 4, ROWS, GRP, TK, DV>(p, oth, __builtin_amdgcn_readfirstlane(ent_cur[i + 1 - base].x), row0, kvh, L.w, L.lane, L.lane_k, L.lane_v);
             } else if (nxt_ok) {
-                if (L.wh == 0) issue_tile<D, 4, ROWS, GRP, TK>(p, oth, nxt.w, nxt_row0, item_hp(nxt) * HPI / p.group, L.w, L.lane, L.lane_k, L.lane_v);
+                if (L.wh == 0) issue_tile<D, 4, ROWS, GRP, TK, DV>(p, oth, nxt.w, nxt_row0, item_hp(nxt) * HPI / p.group, L.w, L.lane, L.lane_k, L.lane_v);
                 pstage = pstage == 2 ? 3 : -1;   // -1: tile requested before the entries (one-tile items)
             }
             const int2 en = ent_cur[i - base];
@@ -771,7 +795,7 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
         } else {
             // (the loop has already flipped par: the last tile came from buffer par ^ 1)
             char* const stage = STAGE_IN_TILE ? bufs + (par ^ 1) * G::BUFB + L.w * 32 * 144 : stage_own;
-            store_rows<D, RT, ROWS>(p, L, stage, o, l, item_t(cur), item_hp(cur) * HPI + L.wh * RT);
+            store_rows<DV, RT, ROWS>(p, L, stage, o, l, item_t(cur), item_hp(cur) * HPI + L.wh * RT);
         }
         TRACE_CLK(tc4);
         TRACE_ADD(10, tc4 - tc3);
@@ -846,15 +870,15 @@ int device_state(DeviceState** out, long n_items) {
     return SPINF_OK;
 }
 
-template <int D, int RT, bool WIN, int NHW, bool ROWS, int GRP = 0, int TK = 64>
+template <int D, int RT, bool WIN, int NHW, bool ROWS, int GRP = 0, int TK = 64, int DV = D>
 int launch(const AttnParams& p, int blocks, hipStream_t stream) {
-    using G = Geo<D, TK>;
-    static_assert(2 * G::BUFB + 2 * ENT_CAP * 12 + (((NHW == 2 && D == 256) || D == 512) ? 16 : 4 * NHW * 32 * 144) + 64 <= 160 * 1024, "LDS budget");
-    hipLaunchKernelGGL((tree_attn_kernel<D, RT, WIN, NHW, ROWS, GRP, TK>), dim3(blocks), dim3(256 * NHW), 0, stream, p);
+    using G = TileGeo<D, TK, DV>;
+    static_assert(2 * G::BUFB + 2 * ENT_CAP * 12 + ((NHW == 2 && D == 256) ? 16 : 4 * NHW * 32 * 144) + 64 <= 160 * 1024, "LDS budget");
+    hipLaunchKernelGGL((tree_attn_kernel<D, RT, WIN, NHW, ROWS, GRP, TK, DV>), dim3(blocks), dim3(256 * NHW), 0, stream, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: launch: %s", hipGetErrorString(e));
     // the exact pass over whatever the fast pass handed on (normally nothing: its workgroups read a zero count and leave)
-    hipLaunchKernelGGL((tree_attn_exact_kernel<D, RT, WIN, RT * NHW, ROWS, GRP, TK>), dim3(blocks < 64 ? blocks : 64), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((tree_attn_exact_kernel<D, RT, WIN, RT * NHW, ROWS, GRP, TK, DV>), dim3(blocks < 64 ? blocks : 64), dim3(256), 0, stream, p);
     e = hipGetLastError();
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: launch (exact pass): %s", hipGetErrorString(e));
     return SPINF_OK;
@@ -894,15 +918,29 @@ int launch_d(const AttnParams& p, int rt, int nhw, bool win, int grp_mode, int b
     return win ? launch<D, 1, true, 1, false>(p, blocks, s) : launch<D, 1, false, 1, false>(p, blocks, s);
 }
 
-// Head dim 512 (the full-attention layers of the Gemma-4 checkpoints, one key / value head): two 64-key K / V tile buffers would
-// not fit the LDS, so the tiles are 32 keys (the plan is built with 32-key entries); four waves, one head per item.
+// Head dim 512 (the full-attention layers of the Gemma-4 checkpoints, one key / value head).  O^T for 32 rows x 512 dims is 256
+// accumulator registers per lane, which with the score tile and the 128 query registers leaves the register allocator no way
+// out but scratch memory.  So the output is computed 256 dims at a time, in two launches over the same plan: each computes the
+// scores over all 512 dims (that part is done twice) and P V for one half of V's columns.  Tiles are 32 keys (the plan is
+// built with 32-key entries): a K tile of 32 KB and a half-width V tile of 16 KB, twice, fit the LDS with room to spare.
+template <bool WIN, bool ROWS, int GRP>
+int launch_512(const AttnParams& p, int blocks, hipStream_t s) {
+    for (int half = 0; half < 2; half++) {
+        AttnParams ph = p;
+        ph.v = p.v + 256 * half;
+        ph.o = p.o + 256 * half;
+        if (int rc = launch<512, 1, WIN, 1, ROWS, GRP, 32, 256>(ph, blocks, s)) return rc;
+    }
+    return SPINF_OK;
+}
+
 int launch_d512(const AttnParams& p, bool win, int grp_mode, int blocks, hipStream_t s) {
     if (p.grp) {
-        if (!win) return launch<512, 1, false, 1, false, 1, 32>(p, blocks, s);
-        return grp_mode == 1 ? launch<512, 1, true, 1, false, 1, 32>(p, blocks, s) : launch<512, 1, true, 1, false, 2, 32>(p, blocks, s);
+        if (!win) return launch_512<false, false, 1>(p, blocks, s);
+        return grp_mode == 1 ? launch_512<true, false, 1>(p, blocks, s) : launch_512<true, false, 2>(p, blocks, s);
     }
-    if (p.row_of) return win ? launch<512, 1, true, 1, true, 0, 32>(p, blocks, s) : launch<512, 1, false, 1, true, 0, 32>(p, blocks, s);
-    return win ? launch<512, 1, true, 1, false, 0, 32>(p, blocks, s) : launch<512, 1, false, 1, false, 0, 32>(p, blocks, s);
+    if (p.row_of) return win ? launch_512<true, true, 0>(p, blocks, s) : launch_512<false, true, 0>(p, blocks, s);
+    return win ? launch_512<true, false, 0>(p, blocks, s) : launch_512<false, false, 0>(p, blocks, s);
 }
 
 }  // namespace
