@@ -265,17 +265,6 @@ __device__ __forceinline__ int fresh_lane_id() {
     return lane;
 }
 
-// An accumulator element read into a vector register by an explicit move.  At head dim 512 the 256 accumulators of O must stay
-// in the accumulator registers; a plain vector ALU use of them makes the register allocator keep ALL of O in vector
-// registers for the whole kernel (the query fragments then live in scratch memory).
-template <bool VIA_ACC>
-__device__ __forceinline__ float acc_value(float a) {
-    if (!VIA_ACC) return a;
-    float v;
-    asm("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(a));
-    return v;
-}
-
 // normalise O^T and store it as rows: each wave stages 32 rows x 64 head dims at a time in its own LDS slice (144-byte
 // rows) and writes them out as 16-byte pieces, 8 lanes per 128-byte row segment
 template <int D, int RT, bool ROWS = false, class LaneT>
@@ -305,7 +294,7 @@ __device__ __forceinline__ void store_rows(const AttnParams& p, const LaneT& L, 
                 for (int i4 = 0; i4 < 4; i4++) {
                     bf16x4 r;
 #pragma unroll
-                    for (int jj = 0; jj < 4; jj++) r[jj] = (__bf16)(acc_value<(D > 256)>(o[rt][2 * qd + dd][4 * i4 + jj]) * inv);
+                    for (int jj = 0; jj < 4; jj++) r[jj] = (__bf16)(o[rt][2 * qd + dd][4 * i4 + jj] * inv);
                     *(bf16x4*)(stage + m * SROW + (32 * dd + 8 * i4 + 4 * g) * 2) = r;
                 }
 #pragma unroll
@@ -404,8 +393,6 @@ __device__ __forceinline__ void attn_item_exact(const AttnParams& p, const int4 
                 const bf16x8 kf = *(const bf16x8*)(krow + 32 * s);
 #pragma unroll
                 for (int rt = 0; rt < RT; rt++) s_acc[rt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[rt][s], s_acc[rt], 0, 0, 0);
-                // at head dim 512 the registers are full (O 256, Q 128): keep the scheduler from hoisting every fragment read
-                if (D > 256 && s % 4 == 3) __builtin_amdgcn_sched_barrier(0);
             }
             if ((bits >> (8 + sub)) & 1u) apply_mask<RT, WIN, GRP, TK>(s_acc, meta, kt, sub, L.g, tok, art_q, pos_q, p.window, grp_q);
             bf16x8 pb[RT][2];
@@ -421,11 +408,9 @@ __device__ __forceinline__ void attn_item_exact(const AttnParams& p, const int4 
                 const float alpha = up ? __builtin_amdgcn_exp2f(M[rt] - mn) : 1.0f;
                 if (__builtin_amdgcn_ballot_w64(up && M[rt] != -INFINITY) != 0) {   // rows without a key so far hold zeros
 #pragma unroll
-                    for (int dt = 0; dt < NDT; dt++) {
+                    for (int dt = 0; dt < NDT; dt++)
 #pragma unroll
                         for (int i2 = 0; i2 < 16; i2++) o[rt][dt][i2] *= alpha;
-                        if (D > 256) __builtin_amdgcn_sched_barrier(0);   // one slice at a time through the vector registers
-                    }
                 }
                 l[rt] *= alpha;
                 M[rt] = mn;
@@ -447,7 +432,6 @@ __device__ __forceinline__ void attn_item_exact(const AttnParams& p, const int4 
                 const bf16x8 a = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
 #pragma unroll
                 for (int rt = 0; rt < RT; rt++) o[rt][f % NDT] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[rt][f / NDT], o[rt][f % NDT], 0, 0, 0);
-                if (D > 256 && f % 4 == 3) __builtin_amdgcn_sched_barrier(0);
             }
         }
     }
