@@ -466,3 +466,51 @@ def test_tree_plan_compact_rows_keep_and_levels():
     # the oracle's restatement agrees
     levels, n_keep, _ = oplan.tree_plan(s.prev, real, short=4)
     assert n_keep == ip.n_keep and [[c["kind"] for c in lv] for lv in levels] == [[c.kind for c in lv] for lv in ip.levels]
+
+
+def test_tileplan_is_exact_on_random_forests():
+    """random forests (two-level trees, aligned branch groups, dense or aligned packing, with and without a window, image groups
+    and 32-key entries): the compiled plan equals the dense mask block by block"""
+    from hypothesis import given, settings
+    from hypothesis import strategies as st
+
+    @settings(max_examples=30, deadline=None, derandomize=True)
+    @given(st.integers(0, 2 ** 31 - 1))
+    def run(seed):
+        rng = np.random.default_rng(seed)
+        trees = []
+        for _ in range(int(rng.integers(1, 4))):
+            nb = int(rng.integers(0, 6))
+            lens = [int(x) for x in rng.integers(1, 40, nb)]
+            parents = [-1 if i == 0 or rng.random() < 0.5 else int(rng.integers(0, i)) for i in range(nb)]
+            parents = [p if p < 0 or parents[p] < 0 else -1 for p in parents]          # at most two levels, parents first
+            aligned = [i for i in range(nb) if parents[i] < 0 and rng.random() < 0.2]
+            trunk = int(rng.integers(0 if nb else 1, 300))
+            trees.append(GroupedTree(rng.integers(5, 99, trunk).tolist(), [rng.integers(5, 99, n).tolist() for n in lens], [], [],
+                                     parents=parents, aligned=aligned))
+        b = synth.pack(trees, align=bool(rng.integers(0, 2)))[0]
+        window = [None, 17, 100][int(rng.integers(0, 3))]
+        grp = None
+        if rng.random() < 0.5:
+            grp = np.full(b.length, -1, np.int32)
+            for gid in range(int(rng.integers(1, 4))):
+                a = int(rng.integers(0, b.length))
+                grp[a : a + int(rng.integers(1, 90))] = gid
+            grp[b.art < 0] = -1
+        windowed = bool(rng.integers(0, 2)) and window is not None
+        _check_plan(b.art, b.end, b.pos, window, grp, windowed)
+        # 32-key entries: the same blocks, one sub-tile per entry
+        p64 = sa.TilePlan.build(b.art, b.end, b.pos, window, grp, windowed)
+        p32 = sa.TilePlan.build(b.art, b.end, b.pos, window, grp, windowed, ktile=32)
+        assert (p32.active_blocks, p32.masked_blocks) == (p64.active_blocks, p64.masked_blocks)
+        assert not (p32.kv_bits & np.uint32(0xAAAA)).any()                              # only sub-tile 0 of an entry
+        for t in range(p64.n_qtiles):
+            want = set()
+            for e in range(p64.qt_ptr[t], p64.qt_ptr[t + 1]):
+                for s_ in range(2):
+                    if int(p64.kv_bits[e]) & (0x55 << s_):
+                        want.add((2 * int(p64.kv_idx[e]) + s_, (int(p64.kv_bits[e]) >> s_) & 0x5555))
+            got = {(int(p32.kv_idx[e]), int(p32.kv_bits[e])) for e in range(p32.qt_ptr[t], p32.qt_ptr[t + 1])}
+            assert got == want, t
+
+    run()
