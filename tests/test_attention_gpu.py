@@ -385,6 +385,48 @@ def test_head_dim_512(dev, hq, hkv):
     assert torch.equal(got, packed[sidx])
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_random_forests_against_the_oracle(dev, seed):
+    """seeded random cases over everything at once: forest shape, packing, head geometry, window, image groups or compact rows"""
+    rng = np.random.default_rng(1000 + seed)
+    trees = []
+    for _ in range(int(rng.integers(1, 4))):
+        nb = int(rng.integers(0, 6))
+        lens = [int(x) for x in rng.integers(1, 40, nb)]
+        parents = [-1 if i == 0 or rng.random() < 0.5 else int(rng.integers(0, i)) for i in range(nb)]
+        parents = [p_ if p_ < 0 or parents[p_] < 0 else -1 for p_ in parents]
+        aligned = [i for i in range(nb) if parents[i] < 0 and rng.random() < 0.2]
+        trunk = int(rng.integers(0 if nb else 1, 400))
+        trees.append(GroupedTree(rng.integers(5, 99, trunk).tolist(), [rng.integers(5, 99, n).tolist() for n in lens], [], [],
+                                 parents=parents, aligned=aligned))
+    b = synth.pack(trees, align=bool(rng.integers(0, 2)))[0]
+    hq, hkv, d = [(4, 2, 64), (8, 2, 128), (3, 3, 128), (4, 2, 256), (2, 1, 256), (4, 1, 512)][int(rng.integers(0, 6))]
+    window = [None, 23, 150][int(rng.integers(0, 3))]
+    mode = int(rng.integers(0, 3))          # 0 plain, 1 image groups, 2 compact rows
+    grp, windowed = None, False
+    if mode == 1:
+        grp = np.full(b.length, -1, np.int32)
+        for gid in range(int(rng.integers(1, 4))):
+            a = int(rng.integers(0, b.length))
+            grp[a : a + int(rng.integers(1, 90))] = gid
+        grp[b.art < 0] = -1
+        windowed = bool(rng.integers(0, 2)) and window is not None
+    cfg = synth.AttnConfig("rand", hq, hkv, d, d ** -0.5, 1.0, window, trees)
+    q, k, v = synth.qkv(cfg, b, seed=seed, device=dev)
+    print(f"case seed={seed} n={b.length} heads={hq}/{hkv} d={d} window={window} mode={mode}", flush=True)
+    mask = sa.TreeMask.build(b.art, b.end, b.pos, window, device=dev, grp=grp, grp_windowed=windowed)
+    dense = omask.dense_tree_mask(b.art, b.end, b.pos, window, grp, windowed)
+    ref = oattn.masked_attention(q.float().cpu().numpy(), k.float().cpu().numpy(), v.float().cpu().numpy(), dense, cfg.scale)
+    if mode == 2:
+        real = np.flatnonzero(b.art >= 0)
+        sidx = torch.from_numpy(real).to(dev)
+        got = sa.tree_attn(q[sidx].contiguous(), k[sidx].contiguous(), v[sidx].contiguous(), mask, cfg.scale, sidx=sidx).float().cpu().numpy()
+        assert float(np.abs(got - ref[real]).max()) <= TOL
+    else:
+        got = sa.tree_attn(q, k, v, mask, cfg.scale).float().cpu().numpy()
+        assert float(np.abs(got - ref).max()) <= TOL
+
+
 def test_argument_errors(dev):
     cfg = synth.attention_config("smoke")
     b = cfg.batches[0]
