@@ -179,6 +179,36 @@ typedef struct spinf_lm_args {
 } spinf_lm_args;
 int spinf_lm_logprobs(const spinf_lm_args* args, void* stream);
 
+/* ------------------------------------------------------------------------------------------------ extraction-decode attention
+ * Replaces _x_attention of spinf_serve/decode.py:71-104 (the attention interface "x_decode"): one decoding step for the
+ * Q = slots x beams queries of each of G groups.  A query attends to its group's prefix, to its own slot's template and to the
+ * tokens its own beam generated; the three key ranges stay in the decoder's three caches (decode.py:129-155):
+ *   q [G, H, Q, d] bf16 with element strides q_g, q_h, q_q (head dim contiguous); out [G, Q, H, d] bf16 contiguous;
+ *   kp, vp [G, h, Lp, d], pos_p [G, Lp] (position, -1 = padding: decode.py:136,146,152);
+ *   kt, vt [G, h, Tt, d], pos_t [G, Tt], own_t [G, Tt] (slot that owns the template token, -1 = padding; the reference's mask_t
+ *   is own_t == q / beam, decode.py:161-162);
+ *   gk, gv [G, h, Q, S, d]: entry s of query q is visible to q alone, for s <= *step (device scalar, decode.py:92; step >= 0);
+ *   qpos [G, Q] int64 device (decode.py:170), read on sliding layers only: window > 0 hides prefix / template keys with
+ *   qpos - pos >= window (decode.py:88-89); window 0 = global layer.  softcap 0 = none (decode.py:86-87).
+ * All caches contiguous, 16-byte aligned, d in {64, 128, 256}, H a multiple of h.  The key stream of a (group, kv head) can be
+ * split over nsplit workgroups; nsplit > 1 needs a workspace of the size spinf_xdecode_plan reports (partial results, fp32),
+ * which the caller owns.  Calls are stream-ordered; nothing is allocated.
+ */
+typedef struct spinf_xdec_args {
+    const void* q; int64_t q_g, q_h, q_q;
+    const void* kp; const void* vp; const int32_t* pos_p;
+    const void* kt; const void* vt; const int32_t* pos_t; const int32_t* own_t;
+    const void* gk; const void* gv;
+    const int64_t* qpos; const int64_t* step;
+    void* out;
+    void* workspace; int64_t workspace_bytes; int32_t nsplit;
+    int32_t G, H, h, Q, S, Lp, Tt, d, beam, window;
+    float scale, softcap;
+} spinf_xdec_args;
+/* suggested nsplit for these sizes (enough workgroups to fill the GPU) and the workspace it needs (0 for nsplit 1) */
+int spinf_xdecode_plan(const spinf_xdec_args* args, int32_t* nsplit, int64_t* workspace_bytes);
+int spinf_xdecode_attn_fwd(const spinf_xdec_args* args, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

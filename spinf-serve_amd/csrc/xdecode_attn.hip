@@ -1,0 +1,403 @@
+// Extraction-decode attention ("x_decode") for gfx950 (MI355X): one decoding step of every slot x beam of every group.
+//
+// Replaces _x_attention of spinf_serve/decode.py:71-104.  A query (group g, slot x beam q, head) attends to three key
+// ranges that live in three caches and are never copied per slot or per beam:
+//   the group's prefix        kp, vp [G, h, Lp, D]   visible to every query of the group where pos_p >= 0,
+//   the slots' templates      kt, vt [G, h, Tt, D]   key j visible to the queries of slot own_t[j] (q / beam == own_t[j]),
+//   the beams' own tokens     gk, gv [G, h, Q, S, D] key (q', s) visible to query q' alone and only for s <= step,
+// on sliding layers the first two also only where qpos[g, q] - pos < window.  The softmax runs over the three ranges
+// together (decode.py:96).
+//
+// Layout of the work.  The three ranges are taken as ONE stream of keys per (group, kv head), cut into tiles of 32 keys:
+// prefix | templates | generated (row-major over (q, s), which is how gk / gv lie in memory).  The rows of a (group, kv
+// head) are its Q queries x r = H / h heads, row = q * r + head % r, so that the rows of one 32-row block are neighbouring
+// queries and their generated keys one contiguous piece of the stream.  A workgroup of four waves owns up to 128 rows (wave w the
+// rows 32 w ..) and a contiguous share of the key tiles (blockIdx: split); it visits the prefix / template tiles of its share and those generated
+// tiles that hold keys of its own queries.  K / V tiles go global -> LDS by DMA, double buffered, one barrier per tile, and are
+// shared by the four waves, so every key is read from memory once per 128 rows.  Scores are S^T = K Q^T with
+// v_mfma_f32_32x32x16_bf16 (a lane owns one query row), classic online softmax with a lazily raised reference, O^T = V^T P^T
+// with V^T fragments read through ds_read_b64_tr_b16.  With more than one split every workgroup leaves (O, reference, sum)
+// per row in a workspace and xdec_combine_kernel merges them; with one split the workgroup writes the output itself.
+//
+// A row's result depends on its own keys only (fixed tile order, masked entries are exact zeros), so a group's outputs do
+// not depend on which other groups share the call.
+#include <hip/hip_runtime.h>
+
+#include "spinf_tree.h"
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+#include "attn_tiles.h"
+
+namespace {
+
+constexpr int XTK = 32;            // keys per tile
+constexpr int XROWS = 128;         // rows per workgroup
+constexpr float XTAU = 8.f;        // the reference point is raised when a tile's maximum exceeds it by more than this (log2 units)
+constexpr int RANGE_EMPTY = 1;     // lo = 1 > hi = 0: a key nobody sees
+constexpr int POS_ALWAYS = 0x3fffffff;   // position of a key the window never hides
+
+struct XdecParams {
+    const __bf16* q; long q_g, q_h, q_q;
+    const __bf16 *kp, *vp, *kt, *vt, *gk, *gv;
+    const int *pos_p, *pos_t, *own_t;
+    const long long* qpos;
+    const long long* step;
+    __bf16* out;
+    float* part_o; float* part_ml;
+    int G, H, h, r, Q, Lp, Tt, S, beam, window;
+    int R, nchunk, nsplit;
+    float c, cap_in, cap_out;
+};
+
+// key tiles of a workgroup that owns the queries qlo .. qhi: the tiles with prefix / template keys, then the tiles that hold
+// the generated keys of its queries (a tile holding both kinds counts as the first kind)
+struct TileList {
+    int nshared, gt0, nt;
+    __host__ __device__ TileList(int Lp, int Tt, int S, int qlo, int qhi) {
+        const long lk = (long)Lp + Tt;
+        nshared = (int)((lk + XTK - 1) / XTK);
+        const long a = (lk + (long)qlo * S) / XTK, b = (lk + (long)(qhi + 1) * S + XTK - 1) / XTK;
+        gt0 = (int)(a > nshared ? a : nshared);
+        const int ngen = (int)(b > gt0 ? b - gt0 : 0);
+        nt = nshared + ngen;
+    }
+    __host__ __device__ int tile(int i) const { return i < nshared ? i : gt0 + i - nshared; }
+};
+
+template <int D, bool WIN, bool CAP>
+__global__ __launch_bounds__(256) void xdec_kernel(const XdecParams p) {
+    using GK = Geo<D, XTK>;
+    constexpr int KTILEB = GK::KTILEB, VTILEB = GK::VTILEB, METAB = 2 * XTK * 4;
+    constexpr int BUFB = KTILEB + VTILEB + METAB;
+    constexpr int NS = D / 16, NDT = D / 32;
+    constexpr int IPW = GK::NREG / 4;
+    static_assert(IPW >= 1 && IPW * 4 == GK::NREG, "the tile's regions must divide among the four waves");
+    __shared__ __attribute__((aligned(16))) char bufs[2 * BUFB];
+
+    const int lane = threadIdx.x & 63, m = lane & 31, g2 = lane >> 5;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    // blockIdx.x = chunk * (G h nsplit) + (g h + hh) * nsplit + split: the row chunks of one (group, kv head) are a multiple of
+    // 8 workgroups apart when G h nsplit is, i.e. they share an XCD's L2
+    const int per_chunk = p.G * p.h * p.nsplit;
+    const int chunk = blockIdx.x / per_chunk;
+    const int rest = blockIdx.x - chunk * per_chunk;
+    const int split = rest % p.nsplit, gh = rest / p.nsplit;
+    const int g = gh / p.h, hh = gh - g * p.h;
+
+    const int row0 = chunk * XROWS + 32 * w;
+    const int row = row0 + m;
+    const bool valid = row < p.R;
+    const int rowc = valid ? row : p.R - 1;
+    const int qi = rowc / p.r, head = hh * p.r + (rowc - qi * p.r);
+    const bool wave_on = row0 < p.R;
+    const int qlo_w = row0 / p.r, qhi_w = ((row0 + 31 < p.R ? row0 + 31 : p.R - 1)) / p.r;
+    const int last_row = chunk * XROWS + XROWS - 1 < p.R ? chunk * XROWS + XROWS - 1 : p.R - 1;
+    const TileList tl(p.Lp, p.Tt, p.S, (chunk * XROWS) / p.r, last_row / p.r);
+    const int per = (tl.nt + p.nsplit - 1) / p.nsplit;
+    const int i0 = split * per, i1 = i0 + per < tl.nt ? i0 + per : tl.nt;
+
+    const long ltot = (long)p.Lp + p.Tt + (long)p.Q * p.S;
+    const int step = (int)*p.step;
+    const int qpos_q = WIN ? (int)p.qpos[(long)g * p.Q + qi] : 0;
+
+    bf16x8 qf[NS];
+    {
+        const __bf16* qp = p.q + (long)g * p.q_g + (long)head * p.q_h + (long)qi * p.q_q + 8 * g2;
+#pragma unroll
+        for (int s = 0; s < NS; s++) qf[s] = *(const bf16x8*)(qp + 16 * s);
+    }
+    f32x16 o[NDT];
+#pragma unroll
+    for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) o[dt][i] = 0.f;
+    float M = -INFINITY, l = 0.f;
+
+    // fragment addresses inside a tile (see Geo): K row m, 16-byte chunk g2 of each 32-byte step; V^T through the transposing read
+    const int tr_a = lane & 3, tr_j = (lane >> 2) & 3, tr_mb = (lane >> 4) & 1;
+    const int k_lane = GK::k_off(m) + 16 * g2;
+    const int v_lane = GK::v_off(4 * g2 + tr_j) + 32 * tr_mb + 8 * tr_a;
+
+    // element offset of key `key` of the stream inside its cache, and which cache (0 prefix, 1 templates, 2 generated)
+    auto locate = [&](long key, int& which) -> long {
+        key = key < ltot ? key : ltot - 1;
+        if (key < p.Lp) { which = 0; return ((long)gh * p.Lp + key) * D; }
+        if (key < (long)p.Lp + p.Tt) { which = 1; return ((long)gh * p.Tt + (key - p.Lp)) * D; }
+        which = 2;
+        return ((long)gh * p.Q * p.S + (key - p.Lp - p.Tt)) * D;
+    };
+    auto issue = [&](const unsigned buf, const int tile) {
+#pragma unroll
+        for (int i = 0; i < IPW; i++) {
+            const int reg = w * IPW + i;
+            int which;
+            const long off = locate((long)tile * XTK + reg + GK::NREG * (lane / GK::CPR), which) + (lane % GK::CPR) * 8;
+            const __bf16* kb = which == 0 ? p.kp : which == 1 ? p.kt : p.gk;
+            const __bf16* vb = which == 0 ? p.vp : which == 1 ? p.vt : p.gv;
+            dma16_lane((const char*)(kb + off), buf + reg * GK::KRS);
+            dma16_lane((const char*)(vb + off), buf + KTILEB + reg * GK::VRS);
+        }
+        if (w == 0 && lane < XTK) {   // who may see the key (queries lo .. hi) and the key's position
+            const long key = (long)tile * XTK + lane;
+            int range = RANGE_EMPTY, kpos = POS_ALWAYS;
+            if (key < p.Lp) {
+                kpos = p.pos_p[(long)g * p.Lp + key];
+                if (kpos >= 0) range = (p.Q - 1) << 16;
+            } else if (key < (long)p.Lp + p.Tt) {
+                const long j = (long)g * p.Tt + (key - p.Lp);
+                const int own = p.own_t[j];
+                kpos = p.pos_t[j];
+                if (own >= 0 && own * p.beam < p.Q) {
+                    const int hi = own * p.beam + p.beam - 1;
+                    range = (own * p.beam) | ((hi < p.Q ? hi : p.Q - 1) << 16);
+                }
+            } else if (key < ltot) {
+                const int idx = (int)(key - p.Lp - p.Tt), qq = idx / p.S;
+                if (idx - qq * p.S <= step) range = qq | (qq << 16);
+            }
+            int* meta = (int*)(bufs + (buf - lds_addr(bufs)) + KTILEB + VTILEB);
+            meta[lane] = range;
+            meta[XTK + lane] = kpos;
+        }
+    };
+
+    const unsigned buf_base = lds_addr(bufs);
+    if (i0 < i1) issue(buf_base, tl.tile(i0));
+    for (int i = i0; i < i1; i++) {
+        __builtin_amdgcn_s_waitcnt(0x0f70);   // this wave's share of tile i has landed
+        __syncthreads();                      // ... and everybody's; all waves are done with tile i - 1
+        const int b = (i - i0) & 1;
+        if (i + 1 < i1) issue(buf_base + (b ^ 1) * BUFB, tl.tile(i + 1));
+        const char* kb = bufs + b * BUFB;
+        const char* vb = kb + KTILEB;
+        const int* meta = (const int*)(kb + KTILEB + VTILEB);
+        {   // does any key of the tile belong to a query of this wave?
+            const unsigned rg = (unsigned)meta[m];
+            const int lo = rg & 0xffff, hi = rg >> 16;
+            const bool need = wave_on && lo <= hi && lo <= qhi_w && hi >= qlo_w;
+            if (__builtin_amdgcn_ballot_w64(need) == 0) continue;
+        }
+        const char* krow = kb + k_lane;
+        const char* vrow = vb + v_lane;
+        f32x16 s_acc;
+#pragma unroll
+        for (int i2 = 0; i2 < 16; i2++) s_acc[i2] = 0.f;
+#pragma unroll
+        for (int s = 0; s < NS; s++) {
+            const bf16x8 kf = *(const bf16x8*)(krow + 32 * s);
+            s_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[s], s_acc, 0, 0, 0);
+        }
+        // register i of the S^T tile holds key 8 (i / 4) + 4 g2 + i % 4 of the tile
+        float mx = -INFINITY;
+#pragma unroll
+        for (int i4 = 0; i4 < 4; i4++) {
+            const int ko = 8 * i4 + 4 * g2;
+            const int4 rg4 = *(const int4*)(meta + ko);
+            const int4 kp4 = *(const int4*)(meta + XTK + ko);
+            const int rgv[4] = {rg4.x, rg4.y, rg4.z, rg4.w};
+            const int kpv[4] = {kp4.x, kp4.y, kp4.z, kp4.w};
+#pragma unroll
+            for (int jj = 0; jj < 4; jj++) {
+                const int lo = rgv[jj] & 0xffff, hi = (unsigned)rgv[jj] >> 16;
+                bool vis = (lo <= qi) & (qi <= hi);
+                if (WIN) vis = vis & ((qpos_q - kpv[jj]) < p.window);
+                float t = s_acc[4 * i4 + jj];
+                if (CAP) {   // softcap * tanh(score * scale / softcap), in log2 units
+                    const float e = __builtin_amdgcn_exp2f(t * p.cap_in);   // exp(2 y), y = score * scale / softcap
+                    t = p.cap_out * (1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f));
+                } else {
+                    t *= p.c;
+                }
+                t = vis ? t : -INFINITY;
+                s_acc[4 * i4 + jj] = t;
+                mx = fmaxf(mx, t);
+            }
+        }
+        mx = lane32_max(mx);
+        const bool up = mx > M + XTAU;
+        const float mn = up ? mx : M;
+        const float alpha = up ? __builtin_amdgcn_exp2f(M - mn) : 1.0f;
+        if (__builtin_amdgcn_ballot_w64(up && M != -INFINITY) != 0) {   // rows without a key so far hold zeros
+#pragma unroll
+            for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+                for (int i2 = 0; i2 < 16; i2++) o[dt][i2] *= alpha;
+        }
+        l *= alpha;
+        M = mn;
+        const float ms = mn == -INFINITY ? 0.f : mn;
+        bf16x8 pb[2];
+        float sum = 0.f;
+#pragma unroll
+        for (int i2 = 0; i2 < 16; i2++) {
+            const float pr = __builtin_amdgcn_exp2f(s_acc[i2] - ms);
+            sum += pr;
+            pb[i2 >> 3][i2 & 7] = (__bf16)pr;
+        }
+        l += sum;
+#pragma unroll
+        for (int f = 0; f < 2 * NDT; f++) {
+            const char* vp = vrow + GK::v_off(16 * (f / NDT)) + 64 * (f % NDT);
+            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)vp);
+            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vp + GK::v_off(8)));
+            const bf16x8 a = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+            o[f % NDT] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[f / NDT], o[f % NDT], 0, 0, 0);
+        }
+    }
+
+    // register i of O^T tile dt holds head dim 32 dt + 8 (i / 4) + 4 g2 + i % 4 of this lane's row
+    const float lsum = lane32_sum(l);
+    if (!valid) return;
+    if (p.nsplit == 1) {
+        const float inv = 1.0f / lsum;
+        __bf16* ob = p.out + (((long)g * p.Q + qi) * p.H + head) * D;
+#pragma unroll
+        for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+            for (int i4 = 0; i4 < 4; i4++) {
+                bf16x4 r;
+#pragma unroll
+                for (int jj = 0; jj < 4; jj++) r[jj] = (__bf16)(o[dt][4 * i4 + jj] * inv);
+                *(bf16x4*)(ob + 32 * dt + 8 * i4 + 4 * g2) = r;
+            }
+    } else {
+        const long prow = (((long)g * p.H + head) * p.Q + qi) * p.nsplit + split;
+        float* po = p.part_o + prow * D;
+#pragma unroll
+        for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+            for (int i4 = 0; i4 < 4; i4++)
+                *(float4*)(po + 32 * dt + 8 * i4 + 4 * g2) = make_float4(o[dt][4 * i4], o[dt][4 * i4 + 1], o[dt][4 * i4 + 2], o[dt][4 * i4 + 3]);
+        if (g2 == 0) *(float2*)(p.part_ml + prow * 2) = make_float2(M, lsum);
+    }
+}
+
+// out = sum_s 2^(M_s - M*) O_s / sum_s 2^(M_s - M*) l_s over the splits of a row, splits in ascending order; one thread per 4 head dims
+template <int D>
+__global__ __launch_bounds__(256) void xdec_combine_kernel(const XdecParams p, const long n_rows) {
+    const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+    const long rowid = idx / (D / 4);
+    const int d4 = (int)(idx - rowid * (D / 4));
+    if (rowid >= n_rows) return;
+    const float* ml = p.part_ml + rowid * p.nsplit * 2;
+    float mstar = -INFINITY;
+    for (int s = 0; s < p.nsplit; s++) mstar = fmaxf(mstar, ml[2 * s]);
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    float lsum = 0.f;
+    for (int s = 0; s < p.nsplit; s++) {
+        const float ms = ml[2 * s];
+        if (ms == -INFINITY) continue;
+        const float wgt = __builtin_amdgcn_exp2f(ms - mstar);
+        const float4 x = *(const float4*)(p.part_o + (rowid * p.nsplit + s) * D + 4 * d4);
+        acc.x += wgt * x.x; acc.y += wgt * x.y; acc.z += wgt * x.z; acc.w += wgt * x.w;
+        lsum += wgt * ml[2 * s + 1];
+    }
+    const float inv = 1.0f / lsum;
+    const long gg = rowid / ((long)p.H * p.Q);
+    const int head = (int)((rowid / p.Q) % p.H), qi = (int)(rowid % p.Q);
+    bf16x4 r;
+    r[0] = (__bf16)(acc.x * inv); r[1] = (__bf16)(acc.y * inv); r[2] = (__bf16)(acc.z * inv); r[3] = (__bf16)(acc.w * inv);
+    *(bf16x4*)(p.out + ((gg * p.Q + qi) * p.H + head) * D + 4 * d4) = r;
+}
+
+int check_args(const spinf_xdec_args* a) {
+    if (!a) return spinf_fail(SPINF_E_ARG, "xdecode_attn: null args");
+    if (a->G < 0 || a->H <= 0 || a->h <= 0 || a->H % a->h || a->Q < 0 || a->S <= 0 || a->Lp < 0 || a->Tt < 0 || a->beam <= 0)
+        return spinf_fail(SPINF_E_ARG, "xdecode_attn: bad sizes (G %d H %d h %d Q %d S %d Lp %d Tt %d beam %d)", a->G, a->H, a->h, a->Q, a->S, a->Lp, a->Tt, a->beam);
+    if (a->d != 64 && a->d != 128 && a->d != 256) return spinf_fail(SPINF_E_ARG, "xdecode_attn: head dim %d not supported (64, 128, 256)", a->d);
+    if (a->Q > 32767 || (int64_t)a->Q * (a->H / a->h) > (1 << 20)) return spinf_fail(SPINF_E_ARG, "xdecode_attn: %d queries per group out of range", a->Q);
+    if ((int64_t)a->Lp + a->Tt + (int64_t)a->Q * a->S > (1 << 30)) return spinf_fail(SPINF_E_ARG, "xdecode_attn: key stream too long");
+    if ((int64_t)a->G * a->h > (1 << 24)) return spinf_fail(SPINF_E_ARG, "xdecode_attn: too many (group, kv head) pairs");
+    if (a->window < 0) return spinf_fail(SPINF_E_ARG, "xdecode_attn: window %d", a->window);
+    if (a->softcap < 0.f) return spinf_fail(SPINF_E_ARG, "xdecode_attn: softcap %g", (double)a->softcap);
+    return SPINF_OK;
+}
+
+int n_chunks(const spinf_xdec_args* a) { return (int)(((int64_t)a->Q * (a->H / a->h) + XROWS - 1) / XROWS); }
+
+template <int D>
+int launch_d(const XdecParams& p, bool cap, int blocks, hipStream_t s) {
+    const bool win = p.window > 0;
+    if (win && cap) hipLaunchKernelGGL((xdec_kernel<D, true, true>), dim3(blocks), dim3(256), 0, s, p);
+    else if (win) hipLaunchKernelGGL((xdec_kernel<D, true, false>), dim3(blocks), dim3(256), 0, s, p);
+    else if (cap) hipLaunchKernelGGL((xdec_kernel<D, false, true>), dim3(blocks), dim3(256), 0, s, p);
+    else hipLaunchKernelGGL((xdec_kernel<D, false, false>), dim3(blocks), dim3(256), 0, s, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "xdecode_attn: launch: %s", hipGetErrorString(e));
+    if (p.nsplit > 1) {
+        const long n_rows = (long)p.G * p.H * p.Q;
+        const long threads = n_rows * (D / 4);
+        hipLaunchKernelGGL((xdec_combine_kernel<D>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, p, n_rows);
+        e = hipGetLastError();
+        if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "xdecode_attn: launch (combine): %s", hipGetErrorString(e));
+    }
+    return SPINF_OK;
+}
+
+}  // namespace
+
+extern "C" int spinf_xdecode_plan(const spinf_xdec_args* a, int32_t* nsplit, int64_t* workspace_bytes) {
+    const int rc = check_args(a);
+    if (rc) return rc;
+    if (!nsplit || !workspace_bytes) return spinf_fail(SPINF_E_ARG, "xdecode_plan: null output");
+    *nsplit = 1;
+    *workspace_bytes = 0;
+    if (a->G == 0 || a->Q == 0) return SPINF_OK;
+    const int r = a->H / a->h;
+    const long base = (long)a->G * a->h * n_chunks(a);
+    // two workgroups per CU of 256; a split should still have 8 tiles of the first row chunk's list
+    const int first_hi = (int)(((int64_t)a->Q * r < XROWS ? (int64_t)a->Q * r : XROWS) - 1) / r;
+    const TileList tl(a->Lp, a->Tt, a->S, 0, first_hi);
+    long want = (512 + base - 1) / base;
+    const long most = tl.nt / 8 > 1 ? tl.nt / 8 : 1;
+    want = want < most ? want : most;
+    want = want < 16 ? want : 16;
+    *nsplit = (int32_t)(want < 1 ? 1 : want);
+    if (*nsplit > 1) *workspace_bytes = (int64_t)a->G * a->H * a->Q * *nsplit * (a->d + 2) * 4;
+    return SPINF_OK;
+}
+
+extern "C" int spinf_xdecode_attn_fwd(const spinf_xdec_args* a, void* stream) {
+    const int rc = check_args(a);
+    if (rc) return rc;
+    if (a->G == 0 || a->Q == 0) return SPINF_OK;
+    if (!a->q || !a->out || !a->gk || !a->gv || !a->step) return spinf_fail(SPINF_E_ARG, "xdecode_attn: null pointer (q, out, gk, gv, step)");
+    if (a->Lp > 0 && (!a->kp || !a->vp || !a->pos_p)) return spinf_fail(SPINF_E_ARG, "xdecode_attn: prefix of %d keys without kp / vp / pos_p", a->Lp);
+    if (a->Tt > 0 && (!a->kt || !a->vt || !a->pos_t || !a->own_t)) return spinf_fail(SPINF_E_ARG, "xdecode_attn: %d template keys without kt / vt / pos_t / own_t", a->Tt);
+    if (a->window > 0 && !a->qpos) return spinf_fail(SPINF_E_ARG, "xdecode_attn: a sliding layer needs qpos");
+    if (a->q_q % 8 || a->q_h % 8 || a->q_g % 8) return spinf_fail(SPINF_E_ARG, "xdecode_attn: query strides must be multiples of 8 elements");
+    for (const void* ptr : {a->q, (const void*)a->out, a->kp, a->vp, a->kt, a->vt, a->gk, a->gv})
+        if ((uintptr_t)ptr % 16) return spinf_fail(SPINF_E_ARG, "xdecode_attn: q, out and the caches must be 16-byte aligned");
+    if (a->nsplit < 1 || a->nsplit > 64) return spinf_fail(SPINF_E_ARG, "xdecode_attn: nsplit %d (1 .. 64)", a->nsplit);
+    const int64_t need = a->nsplit > 1 ? (int64_t)a->G * a->H * a->Q * a->nsplit * (a->d + 2) * 4 : 0;
+    if (need > 0 && (!a->workspace || a->workspace_bytes < need || (uintptr_t)a->workspace % 16))
+        return spinf_fail(SPINF_E_ARG, "xdecode_attn: %d splits need a 16-byte aligned workspace of %lld bytes", a->nsplit, (long long)need);
+    XdecParams p;
+    p.q = (const __bf16*)a->q; p.q_g = a->q_g; p.q_h = a->q_h; p.q_q = a->q_q;
+    p.kp = (const __bf16*)a->kp; p.vp = (const __bf16*)a->vp; p.kt = (const __bf16*)a->kt; p.vt = (const __bf16*)a->vt;
+    p.gk = (const __bf16*)a->gk; p.gv = (const __bf16*)a->gv;
+    p.pos_p = a->pos_p; p.pos_t = a->pos_t; p.own_t = a->own_t;
+    p.qpos = (const long long*)a->qpos; p.step = (const long long*)a->step;
+    p.out = (__bf16*)a->out;
+    p.part_o = (float*)a->workspace;
+    p.part_ml = p.part_o ? p.part_o + (int64_t)a->G * a->H * a->Q * a->nsplit * a->d : nullptr;
+    p.G = a->G; p.H = a->H; p.h = a->h; p.r = a->H / a->h; p.Q = a->Q; p.Lp = a->Lp; p.Tt = a->Tt; p.S = a->S; p.beam = a->beam;
+    p.window = a->window;
+    p.R = p.Q * p.r; p.nchunk = n_chunks(a); p.nsplit = a->nsplit;
+    const float log2e = 1.4426950408889634f;
+    p.c = a->scale * log2e;
+    p.cap_in = a->softcap > 0.f ? 2.0f * log2e * a->scale / a->softcap : 0.f;
+    p.cap_out = a->softcap * log2e;
+    const long blocks = (long)p.G * p.h * p.nsplit * p.nchunk;
+    if (blocks > 0x7fffffffL) return spinf_fail(SPINF_E_ARG, "xdecode_attn: too many workgroups");
+    const bool cap = a->softcap > 0.f;
+    hipStream_t s = (hipStream_t)stream;
+    switch (a->d) {
+        case 64: return launch_d<64>(p, cap, (int)blocks, s);
+        case 128: return launch_d<128>(p, cap, (int)blocks, s);
+        default: return launch_d<256>(p, cap, (int)blocks, s);
+    }
+}

@@ -5,6 +5,7 @@
   attention   tree_attn custom op, tree_flex_forward, tree_attention (gemma4.py:98-119, qwen.py:604-623)
   gdn         recurrent, chunked (spinf_serve/models/qwen35/gdn.py)
   qwen_plan   tree_plan, gdn_tree (spinf_serve/models/qwen35/qwen.py:158-276, 514-590)
+  decode      XCaches, GroupKV, x_attention: the extraction decoder's attention step (spinf_serve/decode.py:35-104)
   synth       seeded synthetic workloads of the benchmark configurations
 
 All device work goes through libspinf_tree.so (HIP, gfx950); there is no CPU or PyTorch fallback: importing the
@@ -18,4 +19,5 @@ from .attention import CAPTURE, register_tree_attention, tree_attention, tree_at
 from .gdn import chunked, recurrent  # noqa: F401
 from .gdn_layer import gdn_gate, gdn_prologue  # noqa: F401
 from .lm_head import lm_logprobs  # noqa: F401
+from .decode import GroupKV, XCaches, x_attention, xdecode_attn  # noqa: F401
 from .qwen_plan import Call, TreePlan, gdn_tree, tree_plan  # noqa: F401

@@ -53,6 +53,21 @@ class LmArgs(C.Structure):
     ]
 
 
+class XdecArgs(C.Structure):
+    _fields_ = [
+        ("q", C.c_void_p), ("q_g", C.c_int64), ("q_h", C.c_int64), ("q_q", C.c_int64),
+        ("kp", C.c_void_p), ("vp", C.c_void_p), ("pos_p", C.c_void_p),
+        ("kt", C.c_void_p), ("vt", C.c_void_p), ("pos_t", C.c_void_p), ("own_t", C.c_void_p),
+        ("gk", C.c_void_p), ("gv", C.c_void_p),
+        ("qpos", C.c_void_p), ("step", C.c_void_p),
+        ("out", C.c_void_p),
+        ("workspace", C.c_void_p), ("workspace_bytes", C.c_int64), ("nsplit", C.c_int32),
+        ("G", C.c_int32), ("H", C.c_int32), ("h", C.c_int32), ("Q", C.c_int32), ("S", C.c_int32), ("Lp", C.c_int32), ("Tt", C.c_int32),
+        ("d", C.c_int32), ("beam", C.c_int32), ("window", C.c_int32),
+        ("scale", C.c_float), ("softcap", C.c_float),
+    ]
+
+
 class GdnArgs(C.Structure):
     _fields_ = [
         ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("g", C.c_void_p), ("beta", C.c_void_p), ("o", C.c_void_p),
@@ -96,7 +111,9 @@ def load_library():
     lib.spinf_gdn_prologue.argtypes = [C.POINTER(GdnPreArgs), C.c_void_p]
     lib.spinf_gdn_gate.argtypes = [C.POINTER(GdnGateArgs), C.c_void_p]
     lib.spinf_lm_logprobs.argtypes = [C.POINTER(LmArgs), C.c_void_p]
-    for name in ("spinf_tileplan_build", "spinf_tileplan_build_groups", "spinf_tileplan_build_ktile", "spinf_tileplan_counts", "spinf_tileplan_export", "spinf_tileplan_schedule", "spinf_tileplan_row0", "spinf_tree_attn_fwd", "spinf_attn_exact_items", "spinf_gdn_fwd", "spinf_gdn_prologue", "spinf_gdn_gate", "spinf_lm_logprobs"):
+    lib.spinf_xdecode_plan.argtypes = [C.POINTER(XdecArgs), C.POINTER(C.c_int32), C.POINTER(C.c_int64)]
+    lib.spinf_xdecode_attn_fwd.argtypes = [C.POINTER(XdecArgs), C.c_void_p]
+    for name in ("spinf_tileplan_build", "spinf_tileplan_build_groups", "spinf_tileplan_build_ktile", "spinf_tileplan_counts", "spinf_tileplan_export", "spinf_tileplan_schedule", "spinf_tileplan_row0", "spinf_tree_attn_fwd", "spinf_attn_exact_items", "spinf_gdn_fwd", "spinf_gdn_prologue", "spinf_gdn_gate", "spinf_lm_logprobs", "spinf_xdecode_plan", "spinf_xdecode_attn_fwd"):
         getattr(lib, name).restype = C.c_int
     _LIB = lib
     return lib

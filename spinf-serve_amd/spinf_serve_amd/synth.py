@@ -215,3 +215,62 @@ def gdn_inputs(cfg: GdnConfig, seed: int = 0, device="cuda"):
         "beta": chunks((cfg.hv,), lambda x: torch.sigmoid(x).to(torch.bfloat16)),
         "g": chunks((cfg.hv,), lambda x: -F.softplus(x)),
     }
+
+
+# ------------------------------------------------------------------------------------------------ extraction decode step
+def xdecode_case(G=4, H=16, h=8, d=256, slots=4, beam=6, S=17, prefix=(300, 470), template=(6, 14), window=None, step=None, seed=0,
+                 device="cuda", layer=0):
+    """A synthetic decoding step of the extraction decoder (spinf_serve/decode.py:106-171): G groups with `slots` slots each
+    (Q = slots * beam queries), prefix lengths uniform in `prefix`, template lengths uniform in `template` per slot, S generated
+    entries per query of which 0 .. step are written.  A sliding layer (window) stores the last window - 1 prefix tokens
+    (spinf_serve/models/gemma4.py:100-106).  K, V ~ 0.5 N(0, 1) bf16, queries N(0, 1) bf16.
+    -> (query [G, H, Q, d] as the transposed view of [G, Q, H, d], XCaches)"""
+    import torch
+
+    from .decode import XCaches
+
+    rng = np.random.default_rng(seed)
+    Q = slots * beam
+    P = rng.integers(prefix[0], prefix[1] + 1, G)
+    T = rng.integers(template[0], template[1] + 1, (G, slots))
+    stored = np.minimum(P, window - 1) if window else P
+    Lp, Tt = int(stored.max()), int(T.sum(1).max())
+    pos_p = np.full((G, Lp), -1, np.int32)
+    pos_t = np.full((G, Tt), -1, np.int32)
+    own_t = np.full((G, Tt), -1, np.int32)
+    qpos = np.zeros((G, Q), np.int64)
+    step = S - 1 if step is None else step
+    for g in range(G):
+        pos_p[g, : stored[g]] = np.arange(P[g] - stored[g], P[g])
+        o = 0
+        for j in range(slots):
+            pos_t[g, o : o + T[g, j]] = np.arange(P[g], P[g] + T[g, j])
+            own_t[g, o : o + T[g, j]] = j
+            o += T[g, j]
+            qpos[g, j * beam : (j + 1) * beam] = P[g] + T[g, j] + step
+    gen = torch.Generator().manual_seed(seed)
+
+    def rnd(*shape, s=0.5):
+        return (torch.randn(*shape, generator=gen) * s).to(torch.bfloat16).to(device)
+
+    c = XCaches(beam=beam)
+    c.kp[layer], c.vp[layer] = rnd(G, h, Lp, d), rnd(G, h, Lp, d)
+    c.kt[layer], c.vt[layer] = rnd(G, h, Tt, d), rnd(G, h, Tt, d)
+    c.gk[layer], c.gv[layer] = rnd(G, h, Q, S, d), rnd(G, h, Q, S, d)
+    c.pos_p[layer] = torch.from_numpy(pos_p).to(device)
+    c.pos_t, c.own_t = torch.from_numpy(pos_t).to(device), torch.from_numpy(own_t).to(device)
+    c.qpos = torch.from_numpy(qpos).to(device)
+    c.step_t = torch.full((1,), step, dtype=torch.int64, device=device)
+    query = rnd(G, Q, H, d, s=1.0).transpose(1, 2)
+    return query, c
+
+
+def xdecode_bytes(c, layer=0, H=None) -> int:
+    """algorithmic bytes of one step: every stored prefix / template key and value row once, the written generated entries once
+    (entries 0 .. step), the queries and the outputs once"""
+    kp, kt, gk = c.kp[layer], c.kt[layer], c.gk[layer]
+    G, h, Lp, d = kp.shape
+    Q, S = gk.shape[2], gk.shape[3]
+    step = int(c.step_t.item())
+    rows = int((c.pos_p[layer] >= 0).sum().item()) * h + int((c.own_t >= 0).sum().item()) * h + G * h * Q * (step + 1)
+    return rows * d * 2 * 2 + 2 * G * Q * (H or h) * d * 2
