@@ -1,6 +1,6 @@
 """Benchmark of the tree-mask packed-prefill attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C2|C3|C4|C5|copy] [--seed S] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C2|C3|C4|C5|XDEC|LM|copy ...] [--seed S] [--no-cpu]
 
 A step is one pass of the attention op (one layer's call through the C ABI) over one packed synthetic stream already
 resident in HBM; the tile plan is compiled once per stream, outside the timed region, as the reference builds its block
@@ -33,6 +33,8 @@ WORKLOADS = {
     "C5": "C5: Gated DeltaNet, contents x (2048-token trunk + 32 branches x 12), 16 qk / 32 v heads, 128 x 128 fp32 state",
     "C5_prologue": "C5's stream through the Gated DeltaNet layer's prologue: path convolution (4 taps) + silu + q/k l2 norm + beta + g from the input projection's rows",
     "C5_gate": "C5's stream through the Gated DeltaNet layer's output gate: per-head rms norm x norm_w x silu(z)",
+    "XDEC": "extraction-decode attention step: 24 groups x (470-token prefix + 8 slots with templates of U{8..16} tokens) x 6 beams = 48 queries per group, 33 generated entries per query all written (step 32), 16 query / 8 KV heads, head_dim 256, scale 1/16, global layer",
+    "XDEC_long": "extraction-decode attention step: 64 groups x (U{1024..4096}-token prefix + 8 slots with templates of U{8..16} tokens) x 6 beams, 33 generated entries (step 32), 16 / 8 heads, head_dim 256, global layer",
     "LM": "lm head read-out of one chunk of 1,024 read rows: soft-capping (30) + log-softmax over 262,144 fp32 logits + 8 option columns",
 }
 
@@ -122,6 +124,57 @@ def main():
                     dtype="f32", config={"workload": WORKLOADS["LM"], "rows": rows, "vocab": vocab, "way": "torch ops" if args.rows == "scatter" else "kernel"},
                     roofline={"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS, "traffic": None,
                               "kernel_ms": ms, "algorithmic_bytes": nbytes})
+        print(json.dumps(line))
+        return
+
+    if args.workload in ("XDEC", "XDEC_long"):
+        from oracle import xdecode as ox
+
+        long = args.workload == "XDEC_long"
+        G = args.contents or (64 if long else 24)
+        q, c = synth.xdecode_case(G=G, H=16, h=8, d=256, slots=8, beam=6, S=33, prefix=(1024, 4096) if long else (470, 470), template=(8, 16),
+                                  step=32, seed=args.seed, device=dev)
+        Q, scale = q.shape[2], 1 / 16
+        if args.rows == "scatter":   # the reference's own way (decode.py:81-103: three einsums, masks, one softmax, three einsums), for comparison
+            kp, vp, kt, vt, gk, gv = (t[0] for t in (c.kp, c.vp, c.kt, c.vt, c.gk, c.gv))
+            mp = (c.pos_p[0] >= 0)[:, None, None, None, :]
+            mt = (c.own_t[:, None, :] == (torch.arange(Q, device=dev) // c.beam)[None, :, None])[:, None, None]
+            mg = (torch.arange(33, device=dev) > c.step_t)
+            ninf = torch.finfo(torch.float32).min
+
+            def step():
+                qq = q.reshape(G, 8, 2, Q, 256)
+                sp = (torch.einsum("ghrqd,ghkd->ghrqk", qq, kp).float() * scale).masked_fill(~mp, ninf)
+                st = (torch.einsum("ghrqd,ghkd->ghrqk", qq, kt).float() * scale).masked_fill(~mt, ninf)
+                sg = (torch.einsum("ghrqd,ghqsd->ghrqs", qq, gk).float() * scale).masked_fill(mg, ninf)
+                a = torch.softmax(torch.cat([sp, st, sg], -1), -1).to(vp.dtype)
+                Lp, Lt = sp.shape[-1], st.shape[-1]
+                out = torch.einsum("ghrqk,ghkd->ghrqd", a[..., :Lp], vp).float()
+                out += torch.einsum("ghrqk,ghkd->ghrqd", a[..., Lp : Lp + Lt], vt).float()
+                out += torch.einsum("ghrqs,ghqsd->ghrqd", a[..., Lp + Lt :], gv).float()
+                return out.reshape(G, 16, Q, 256).transpose(1, 2).contiguous().to(q.dtype)
+        else:
+            step = lambda: sa.xdecode_attn(q, c, 0, scale)  # noqa: E731
+        wall, kern = timed(step, args.steps, args.warmup, torch)
+        ms = float(np.mean(kern))
+        nbytes = synth.xdecode_bytes(c, 0, H=16)
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        cpu = None
+        if not args.no_cpu and args.rows != "scatter":   # the float64 oracle on the first groups, one core
+            ng = min(G, 2)
+            sub = [t[0][:ng].float().cpu().numpy() for t in (c.kp, c.vp, c.kt, c.vt, c.gk, c.gv)]
+            t0 = time.perf_counter()
+            ox.x_attention(q[:ng].float().cpu().numpy(), sub[0], sub[1], c.pos_p[0][:ng].cpu().numpy(), sub[2], sub[3], c.pos_t[:ng].cpu().numpy(),
+                           c.own_t[:ng].cpu().numpy(), sub[4], sub[5], c.qpos[:ng].cpu().numpy(), 32, c.beam, scale)
+            dt = time.perf_counter() - t0
+            cpu = {"value": ng * Q / dt, "unit": "queries/s", "cores": 1, "kind": "port", "sample": f"{ng} of {G} groups through the numpy float64 oracle"}
+        line.update(metric="decoded queries/s, extraction-decode attention step (one layer)", value=G * Q * args.steps / wall, unit="queries/s",
+                    ms_per_step=1e3 * wall / args.steps, dtype="bf16",
+                    config={"workload": WORKLOADS[args.workload], "groups": G, "queries": G * Q, "nsplit": sa.decode.plan_splits(G, 16, 8, Q, 33, c.kp[0].shape[2], c.kt[0].shape[2], 256, 6)[0],
+                            "way": "torch ops" if args.rows == "scatter" else "kernel"},
+                    roofline={"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS, "traffic": None,
+                              "kernel_ms": ms, "algorithmic_bytes": nbytes},
+                    cpu_baseline=cpu)
         print(json.dumps(line))
         return
 

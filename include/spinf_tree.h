@@ -190,6 +190,8 @@ int spinf_lm_logprobs(const spinf_lm_args* args, void* stream);
  *   gk, gv [G, h, Q, S, d]: entry s of query q is visible to q alone, for s <= *step (device scalar, decode.py:92; step >= 0);
  *   qpos [G, Q] int64 device (decode.py:170), read on sliding layers only: window > 0 hides prefix / template keys with
  *   qpos - pos >= window (decode.py:88-89); window 0 = global layer.  softcap 0 = none (decode.py:86-87).
+ *   len_p, len_t [G] int32 device, each may be NULL: a group's prefix holds keys (pos_p >= 0) only in its first len_p[g] entries,
+ *   its template range (own_t >= 0) only in its first len_t[g]; the entries behind are padding and are not read.  NULL = Lp / Tt.
  * All caches contiguous, 16-byte aligned, d in {64, 128, 256}, H a multiple of h.  The key stream of a (group, kv head) can be
  * split over nsplit workgroups; nsplit > 1 needs a workspace of the size spinf_xdecode_plan reports (partial results, fp32),
  * which the caller owns.  Calls are stream-ordered; nothing is allocated.
@@ -198,6 +200,7 @@ typedef struct spinf_xdec_args {
     const void* q; int64_t q_g, q_h, q_q;
     const void* kp; const void* vp; const int32_t* pos_p;
     const void* kt; const void* vt; const int32_t* pos_t; const int32_t* own_t;
+    const int32_t* len_p; const int32_t* len_t;
     const void* gk; const void* gv;
     const int64_t* qpos; const int64_t* step;
     void* out;

@@ -42,35 +42,48 @@ constexpr int POS_ALWAYS = 0x3fffffff;   // position of a key the window never h
 struct XdecParams {
     const __bf16* q; long q_g, q_h, q_q;
     const __bf16 *kp, *vp, *kt, *vt, *gk, *gv;
-    const int *pos_p, *pos_t, *own_t;
+    const int *pos_p, *pos_t, *own_t, *len_p, *len_t;
     const long long* qpos;
     const long long* step;
     __bf16* out;
     float* part_o; float* part_ml;
     int G, H, h, r, Q, Lp, Tt, S, beam, window;
-    int R, nchunk, nsplit;
+    int R, nchunk, nsplit, per;
     float c, cap_in, cap_out;
 };
 
-// key tiles of a workgroup that owns the queries qlo .. qhi: the tiles with prefix / template keys, then the tiles that hold
-// the generated keys of its queries (a tile holding both kinds counts as the first kind)
+// Key tiles (32 keys of the stream prefix | templates | generated) of a workgroup that owns the queries qlo .. qhi of a group
+// whose prefix holds keys in its first len_p entries only and whose template range in its first len_t: the tiles of those
+// prefix entries, of those template entries, and of the generated entries of its queries; a tile is listed once.
 struct TileList {
-    int nshared, gt0, nt;
-    __host__ __device__ TileList(int Lp, int Tt, int S, int qlo, int qhi) {
+    int e0, s1, e1, s2, nt;
+    __host__ __device__ TileList(int Lp, int Tt, int S, int len_p, int len_t, int qlo, int qhi) {
         const long lk = (long)Lp + Tt;
-        nshared = (int)((lk + XTK - 1) / XTK);
-        const long a = (lk + (long)qlo * S) / XTK, b = (lk + (long)(qhi + 1) * S + XTK - 1) / XTK;
-        gt0 = (int)(a > nshared ? a : nshared);
-        const int ngen = (int)(b > gt0 ? b - gt0 : 0);
-        nt = nshared + ngen;
+        e0 = (len_p + XTK - 1) / XTK;
+        s1 = len_t > 0 ? Lp / XTK : e0;
+        s1 = s1 > e0 ? s1 : e0;
+        e1 = len_t > 0 ? (int)(((long)Lp + len_t + XTK - 1) / XTK) : s1;
+        e1 = e1 > s1 ? e1 : s1;
+        s2 = (int)((lk + (long)qlo * S) / XTK);
+        s2 = s2 > e1 ? s2 : e1;
+        int e2 = (int)((lk + (long)(qhi + 1) * S + XTK - 1) / XTK);
+        e2 = e2 > s2 ? e2 : s2;
+        nt = e0 + (e1 - s1) + (e2 - s2);
     }
-    __host__ __device__ int tile(int i) const { return i < nshared ? i : gt0 + i - nshared; }
+    __host__ __device__ int tile(int i) const { return i < e0 ? i : i < e0 + (e1 - s1) ? s1 + (i - e0) : s2 + (i - e0 - (e1 - s1)); }
 };
+
+// entries of a group's prefix / template range that can hold keys (the whole range when the caller gave no lengths)
+__device__ __forceinline__ int group_len(const int* len, long g, int full) {
+    if (!len) return full;
+    const int n = len[g];
+    return n < 0 ? 0 : n < full ? n : full;
+}
 
 template <int D, bool WIN, bool CAP>
 __global__ __launch_bounds__(256) void xdec_kernel(const XdecParams p) {
     using GK = Geo<D, XTK>;
-    constexpr int KTILEB = GK::KTILEB, VTILEB = GK::VTILEB, METAB = 2 * XTK * 4;
+    constexpr int KTILEB = GK::KTILEB, VTILEB = GK::VTILEB, METAB = 2 * XTK * 4 + 16;   // (range, position) of the tile's keys, the tile's no-mask flag
     constexpr int BUFB = KTILEB + VTILEB + METAB;
     constexpr int NS = D / 16, NDT = D / 32;
     constexpr int IPW = GK::NREG / 4;
@@ -95,9 +108,10 @@ __global__ __launch_bounds__(256) void xdec_kernel(const XdecParams p) {
     const bool wave_on = row0 < p.R;
     const int qlo_w = row0 / p.r, qhi_w = ((row0 + 31 < p.R ? row0 + 31 : p.R - 1)) / p.r;
     const int last_row = chunk * XROWS + XROWS - 1 < p.R ? chunk * XROWS + XROWS - 1 : p.R - 1;
-    const TileList tl(p.Lp, p.Tt, p.S, (chunk * XROWS) / p.r, last_row / p.r);
-    const int per = (tl.nt + p.nsplit - 1) / p.nsplit;
-    const int i0 = split * per, i1 = i0 + per < tl.nt ? i0 + per : tl.nt;
+    const TileList tl(p.Lp, p.Tt, p.S, group_len(p.len_p, g, p.Lp), group_len(p.len_t, g, p.Tt), (chunk * XROWS) / p.r, last_row / p.r);
+    // a split is p.per tiles of the list: a group with a short prefix has fewer splits than p.nsplit, the rest leave at once
+    const int i0 = split * p.per, i1 = i0 + p.per < tl.nt ? i0 + p.per : tl.nt;
+    if (i0 >= i1) return;
 
     const long ltot = (long)p.Lp + p.Tt + (long)p.Q * p.S;
     const int step = (int)*p.step;
@@ -129,48 +143,88 @@ __global__ __launch_bounds__(256) void xdec_kernel(const XdecParams p) {
         which = 2;
         return ((long)gh * p.Q * p.S + (key - p.Lp - p.Tt)) * D;
     };
+    // the cache pointers as opaque scalar values: picking one per lane is then a register select (left as fields of the
+    // argument block, the compiler picks the FIELD per lane and loads the pointer from memory in front of every DMA, with a
+    // wait that also waits for the DMA before it)
+    const char* const kp_s = uniform_ptr((const char*)p.kp); const char* const vp_s = uniform_ptr((const char*)p.vp);
+    const char* const kt_s = uniform_ptr((const char*)p.kt); const char* const vt_s = uniform_ptr((const char*)p.vt);
+    const char* const gk_s = uniform_ptr((const char*)p.gk); const char* const gv_s = uniform_ptr((const char*)p.gv);
     auto issue = [&](const unsigned buf, const int tile) {
+#ifdef XDEC_NO_DMA
+        return;
+#endif
 #pragma unroll
         for (int i = 0; i < IPW; i++) {
             const int reg = w * IPW + i;
             int which;
             const long off = locate((long)tile * XTK + reg + GK::NREG * (lane / GK::CPR), which) + (lane % GK::CPR) * 8;
-            const __bf16* kb = which == 0 ? p.kp : which == 1 ? p.kt : p.gk;
-            const __bf16* vb = which == 0 ? p.vp : which == 1 ? p.vt : p.gv;
-            dma16_lane((const char*)(kb + off), buf + reg * GK::KRS);
-            dma16_lane((const char*)(vb + off), buf + KTILEB + reg * GK::VRS);
-        }
-        if (w == 0 && lane < XTK) {   // who may see the key (queries lo .. hi) and the key's position
-            const long key = (long)tile * XTK + lane;
-            int range = RANGE_EMPTY, kpos = POS_ALWAYS;
-            if (key < p.Lp) {
-                kpos = p.pos_p[(long)g * p.Lp + key];
-                if (kpos >= 0) range = (p.Q - 1) << 16;
-            } else if (key < (long)p.Lp + p.Tt) {
-                const long j = (long)g * p.Tt + (key - p.Lp);
-                const int own = p.own_t[j];
-                kpos = p.pos_t[j];
-                if (own >= 0 && own * p.beam < p.Q) {
-                    const int hi = own * p.beam + p.beam - 1;
-                    range = (own * p.beam) | ((hi < p.Q ? hi : p.Q - 1) << 16);
-                }
-            } else if (key < ltot) {
-                const int idx = (int)(key - p.Lp - p.Tt), qq = idx / p.S;
-                if (idx - qq * p.S <= step) range = qq | (qq << 16);
-            }
-            int* meta = (int*)(bufs + (buf - lds_addr(bufs)) + KTILEB + VTILEB);
-            meta[lane] = range;
-            meta[XTK + lane] = kpos;
+            const char* kb = which == 0 ? kp_s : which == 1 ? kt_s : gk_s;
+            const char* vb = which == 0 ? vp_s : which == 1 ? vt_s : gv_s;
+            dma16_lane(kb + off * 2, buf + reg * GK::KRS);
+            dma16_lane(vb + off * 2, buf + KTILEB + reg * GK::VRS);
         }
     };
+    // Key `lane` of a tile (lanes 0 .. 31 of wave 0): who may see it (queries lo .. hi, packed lo | hi << 16) and its position.
+    // The two values it needs from memory are loaded BEFORE the DMA of the tile ahead of it and turned into the LDS words one
+    // iteration later, after the loop's own wait: a wait for them between a DMA's issue and the end of the tile's
+    // arithmetic would wait for the DMA as well (one counter for all memory operations, in order).
+    auto load_raw = [&](const int tile, int& r0, int& r1) {
+        const long key = (long)tile * XTK + lane;
+        const bool pre = key < p.Lp, tem = !pre && key < (long)p.Lp + p.Tt;
+        const int* a0 = pre ? p.pos_p + (long)g * p.Lp + key : p.own_t + (long)g * p.Tt + (key - p.Lp);
+        const int* a1 = p.pos_t + (long)g * p.Tt + (key - p.Lp);
+        r0 = 0; r1 = 0;
+        if (pre || tem) r0 = *a0;
+        if (tem) r1 = *a1;
+    };
+    auto put_meta = [&](int* meta, const int tile, const int r0, const int r1) {
+        const long key = (long)tile * XTK + lane;
+        int range = RANGE_EMPTY, kpos = POS_ALWAYS;
+        if (key < p.Lp) {
+            kpos = r0;
+            if (kpos >= 0) range = (p.Q - 1) << 16;
+        } else if (key < (long)p.Lp + p.Tt) {
+            kpos = r1;
+            if (r0 >= 0 && r0 * p.beam < p.Q) {
+                const int hi = r0 * p.beam + p.beam - 1;
+                range = (r0 * p.beam) | ((hi < p.Q ? hi : p.Q - 1) << 16);
+            }
+        } else if (key < ltot) {
+            const int idx = (int)(key - p.Lp - p.Tt), qq = idx / p.S;
+            if (idx - qq * p.S <= step) range = qq | (qq << 16);
+        }
+        meta[lane] = range;
+        meta[XTK + lane] = kpos;
+        // a tile whose 32 keys every query sees needs no mask (sliding layers: not decided here)
+        const bool all = __builtin_amdgcn_ballot_w64(range != ((p.Q - 1) << 16)) == 0;
+        if (lane == 0) meta[2 * XTK] = !WIN && all;
+    };
+    const bool meta_lane = w == 0 && lane < XTK;
+    int m_r0 = 0, m_r1 = 0;
 
     const unsigned buf_base = lds_addr(bufs);
-    if (i0 < i1) issue(buf_base, tl.tile(i0));
+    if (i0 < i1) {
+        if (meta_lane) {
+            load_raw(tl.tile(i0), m_r0, m_r1);
+            put_meta((int*)(bufs + KTILEB + VTILEB), tl.tile(i0), m_r0, m_r1);
+            if (i0 + 1 < i1) load_raw(tl.tile(i0 + 1), m_r0, m_r1);
+        }
+        issue(buf_base, tl.tile(i0));
+    }
     for (int i = i0; i < i1; i++) {
         __builtin_amdgcn_s_waitcnt(0x0f70);   // this wave's share of tile i has landed
         __syncthreads();                      // ... and everybody's; all waves are done with tile i - 1
         const int b = (i - i0) & 1;
-        if (i + 1 < i1) issue(buf_base + (b ^ 1) * BUFB, tl.tile(i + 1));
+        if (i + 1 < i1) {
+            if (meta_lane) {
+                put_meta((int*)(bufs + (b ^ 1) * BUFB + KTILEB + VTILEB), tl.tile(i + 1), m_r0, m_r1);
+                if (i + 2 < i1) load_raw(tl.tile(i + 2), m_r0, m_r1);
+            }
+            issue(buf_base + (b ^ 1) * BUFB, tl.tile(i + 1));
+        }
+#ifdef XDEC_NO_COMPUTE
+        continue;
+#endif
         const char* kb = bufs + b * BUFB;
         const char* vb = kb + KTILEB;
         const int* meta = (const int*)(kb + KTILEB + VTILEB);
@@ -192,28 +246,36 @@ __global__ __launch_bounds__(256) void xdec_kernel(const XdecParams p) {
         }
         // register i of the S^T tile holds key 8 (i / 4) + 4 g2 + i % 4 of the tile
         float mx = -INFINITY;
+        auto to_log2 = [&](float t) {
+            if (CAP) {   // softcap * tanh(score * scale / softcap), in log2 units
+                const float e = __builtin_amdgcn_exp2f(t * p.cap_in);   // exp(2 y), y = score * scale / softcap
+                return p.cap_out * (1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f));
+            }
+            return t * p.c;
+        };
+        if (__builtin_amdgcn_readfirstlane(meta[2 * XTK])) {   // every row sees every key of the tile
 #pragma unroll
-        for (int i4 = 0; i4 < 4; i4++) {
-            const int ko = 8 * i4 + 4 * g2;
-            const int4 rg4 = *(const int4*)(meta + ko);
-            const int4 kp4 = *(const int4*)(meta + XTK + ko);
-            const int rgv[4] = {rg4.x, rg4.y, rg4.z, rg4.w};
-            const int kpv[4] = {kp4.x, kp4.y, kp4.z, kp4.w};
+            for (int i2 = 0; i2 < 16; i2++) {
+                s_acc[i2] = to_log2(s_acc[i2]);
+                mx = fmaxf(mx, s_acc[i2]);
+            }
+        } else {
 #pragma unroll
-            for (int jj = 0; jj < 4; jj++) {
-                const int lo = rgv[jj] & 0xffff, hi = (unsigned)rgv[jj] >> 16;
-                bool vis = (lo <= qi) & (qi <= hi);
-                if (WIN) vis = vis & ((qpos_q - kpv[jj]) < p.window);
-                float t = s_acc[4 * i4 + jj];
-                if (CAP) {   // softcap * tanh(score * scale / softcap), in log2 units
-                    const float e = __builtin_amdgcn_exp2f(t * p.cap_in);   // exp(2 y), y = score * scale / softcap
-                    t = p.cap_out * (1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f));
-                } else {
-                    t *= p.c;
+            for (int i4 = 0; i4 < 4; i4++) {
+                const int ko = 8 * i4 + 4 * g2;
+                const int4 rg4 = *(const int4*)(meta + ko);
+                const int4 kp4 = *(const int4*)(meta + XTK + ko);
+                const int rgv[4] = {rg4.x, rg4.y, rg4.z, rg4.w};
+                const int kpv[4] = {kp4.x, kp4.y, kp4.z, kp4.w};
+#pragma unroll
+                for (int jj = 0; jj < 4; jj++) {
+                    const int lo = rgv[jj] & 0xffff, hi = (unsigned)rgv[jj] >> 16;
+                    bool vis = (lo <= qi) & (qi <= hi);
+                    if (WIN) vis = vis & ((qpos_q - kpv[jj]) < p.window);
+                    const float t = vis ? to_log2(s_acc[4 * i4 + jj]) : -INFINITY;
+                    s_acc[4 * i4 + jj] = t;
+                    mx = fmaxf(mx, t);
                 }
-                t = vis ? t : -INFINITY;
-                s_acc[4 * i4 + jj] = t;
-                mx = fmaxf(mx, t);
             }
         }
         mx = lane32_max(mx);
@@ -282,12 +344,19 @@ __global__ __launch_bounds__(256) void xdec_combine_kernel(const XdecParams p, c
     const long rowid = idx / (D / 4);
     const int d4 = (int)(idx - rowid * (D / 4));
     if (rowid >= n_rows) return;
+    const long gg = rowid / ((long)p.H * p.Q);
+    const int head = (int)((rowid / p.Q) % p.H), qi = (int)(rowid % p.Q);
+    // the splits that exist for this row: those of its row chunk's tile list
+    const int chunk = (qi * p.r + head % p.r) / XROWS;
+    const int last_row = chunk * XROWS + XROWS - 1 < p.R ? chunk * XROWS + XROWS - 1 : p.R - 1;
+    const TileList tl(p.Lp, p.Tt, p.S, group_len(p.len_p, gg, p.Lp), group_len(p.len_t, gg, p.Tt), (chunk * XROWS) / p.r, last_row / p.r);
+    const int ns = (tl.nt + p.per - 1) / p.per;
     const float* ml = p.part_ml + rowid * p.nsplit * 2;
     float mstar = -INFINITY;
-    for (int s = 0; s < p.nsplit; s++) mstar = fmaxf(mstar, ml[2 * s]);
+    for (int s = 0; s < ns; s++) mstar = fmaxf(mstar, ml[2 * s]);
     float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
     float lsum = 0.f;
-    for (int s = 0; s < p.nsplit; s++) {
+    for (int s = 0; s < ns; s++) {
         const float ms = ml[2 * s];
         if (ms == -INFINITY) continue;
         const float wgt = __builtin_amdgcn_exp2f(ms - mstar);
@@ -296,8 +365,6 @@ __global__ __launch_bounds__(256) void xdec_combine_kernel(const XdecParams p, c
         lsum += wgt * ml[2 * s + 1];
     }
     const float inv = 1.0f / lsum;
-    const long gg = rowid / ((long)p.H * p.Q);
-    const int head = (int)((rowid / p.Q) % p.H), qi = (int)(rowid % p.Q);
     bf16x4 r;
     r[0] = (__bf16)(acc.x * inv); r[1] = (__bf16)(acc.y * inv); r[2] = (__bf16)(acc.z * inv); r[3] = (__bf16)(acc.w * inv);
     *(bf16x4*)(p.out + ((gg * p.Q + qi) * p.H + head) * D + 4 * d4) = r;
@@ -337,6 +404,14 @@ int launch_d(const XdecParams& p, bool cap, int blocks, hipStream_t s) {
     return SPINF_OK;
 }
 
+
+// tiles of the longest list of the call: the first row chunk of a group whose prefix and template ranges are full
+int max_tiles(const spinf_xdec_args* a) {
+    const int r = a->H / a->h;
+    const int first_hi = (int)(((int64_t)a->Q * r < XROWS ? (int64_t)a->Q * r : XROWS) - 1) / r;
+    return TileList(a->Lp, a->Tt, a->S, a->Lp, a->Tt, 0, first_hi).nt;
+}
+
 }  // namespace
 
 extern "C" int spinf_xdecode_plan(const spinf_xdec_args* a, int32_t* nsplit, int64_t* workspace_bytes) {
@@ -346,16 +421,22 @@ extern "C" int spinf_xdecode_plan(const spinf_xdec_args* a, int32_t* nsplit, int
     *nsplit = 1;
     *workspace_bytes = 0;
     if (a->G == 0 || a->Q == 0) return SPINF_OK;
-    const int r = a->H / a->h;
+    // 512 workgroups run at a time (two per CU of 256).  Take the split count with the fewest tile steps one after the other:
+    // rounds of workgroups x (tiles per split + 2 for a workgroup's start and end + what a split's partial results cost in
+    // memory traffic, written and read back, in tiles), a split keeping at least 8 tiles.
     const long base = (long)a->G * a->h * n_chunks(a);
-    // two workgroups per CU of 256; a split should still have 8 tiles of the first row chunk's list
-    const int first_hi = (int)(((int64_t)a->Q * r < XROWS ? (int64_t)a->Q * r : XROWS) - 1) / r;
-    const TileList tl(a->Lp, a->Tt, a->S, 0, first_hi);
-    long want = (512 + base - 1) / base;
-    const long most = tl.nt / 8 > 1 ? tl.nt / 8 : 1;
-    want = want < most ? want : most;
-    want = want < 16 ? want : 16;
-    *nsplit = (int32_t)(want < 1 ? 1 : want);
+    const int nt = max_tiles(a);
+    long best = -1;
+    for (int ns = 1; ns <= 16; ns++) {
+        const int per = (nt + ns - 1) / ns;
+        if (ns > 1 && per < 8) break;
+        const long rounds = (base * ns + 511) / 512;
+        const int r = a->H / a->h;
+        const long rows = (int64_t)a->Q * r < XROWS ? (int64_t)a->Q * r : XROWS;
+        const long partial_tiles = ns > 1 ? (rows * (a->d + 2) * 8 + XTK * a->d * 4 - 1) / (XTK * a->d * 4) : 0;
+        const long cost = rounds * (per + 2 + partial_tiles);
+        if (best < 0 || cost < best) { best = cost; *nsplit = ns; }
+    }
     if (*nsplit > 1) *workspace_bytes = (int64_t)a->G * a->H * a->Q * *nsplit * (a->d + 2) * 4;
     return SPINF_OK;
 }
@@ -379,7 +460,7 @@ extern "C" int spinf_xdecode_attn_fwd(const spinf_xdec_args* a, void* stream) {
     p.q = (const __bf16*)a->q; p.q_g = a->q_g; p.q_h = a->q_h; p.q_q = a->q_q;
     p.kp = (const __bf16*)a->kp; p.vp = (const __bf16*)a->vp; p.kt = (const __bf16*)a->kt; p.vt = (const __bf16*)a->vt;
     p.gk = (const __bf16*)a->gk; p.gv = (const __bf16*)a->gv;
-    p.pos_p = a->pos_p; p.pos_t = a->pos_t; p.own_t = a->own_t;
+    p.pos_p = a->pos_p; p.pos_t = a->pos_t; p.own_t = a->own_t; p.len_p = a->len_p; p.len_t = a->len_t;
     p.qpos = (const long long*)a->qpos; p.step = (const long long*)a->step;
     p.out = (__bf16*)a->out;
     p.part_o = (float*)a->workspace;
@@ -387,6 +468,7 @@ extern "C" int spinf_xdecode_attn_fwd(const spinf_xdec_args* a, void* stream) {
     p.G = a->G; p.H = a->H; p.h = a->h; p.r = a->H / a->h; p.Q = a->Q; p.Lp = a->Lp; p.Tt = a->Tt; p.S = a->S; p.beam = a->beam;
     p.window = a->window;
     p.R = p.Q * p.r; p.nchunk = n_chunks(a); p.nsplit = a->nsplit;
+    p.per = (max_tiles(a) + p.nsplit - 1) / p.nsplit;
     const float log2e = 1.4426950408889634f;
     p.c = a->scale * log2e;
     p.cap_in = a->softcap > 0.f ? 2.0f * log2e * a->scale / a->softcap : 0.f;

@@ -58,6 +58,7 @@ class XdecArgs(C.Structure):
         ("q", C.c_void_p), ("q_g", C.c_int64), ("q_h", C.c_int64), ("q_q", C.c_int64),
         ("kp", C.c_void_p), ("vp", C.c_void_p), ("pos_p", C.c_void_p),
         ("kt", C.c_void_p), ("vt", C.c_void_p), ("pos_t", C.c_void_p), ("own_t", C.c_void_p),
+        ("len_p", C.c_void_p), ("len_t", C.c_void_p),
         ("gk", C.c_void_p), ("gv", C.c_void_p),
         ("qpos", C.c_void_p), ("step", C.c_void_p),
         ("out", C.c_void_p),

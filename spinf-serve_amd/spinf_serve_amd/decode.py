@@ -41,7 +41,22 @@ class XCaches:
     qpos: Optional[torch.Tensor] = None
     step_t: Optional[torch.Tensor] = None
     beam: int = 6
+    len_p: dict = field(default_factory=dict)   # by layer: [G] int32, entries of each group's prefix that can hold keys (set_lengths)
+    len_t: Optional[torch.Tensor] = None        # [G] int32, the same for the template range
     _work: dict = field(default_factory=dict)   # workspace of the split launches, by (device, bytes needed)
+
+    def set_lengths(self) -> None:
+        """once per decoder, after the caches are filled: how far each group's prefix (pos_p >= 0) and template range
+        (own_t >= 0) reach; the kernel then neither reads nor schedules the padding behind (decode.py:136-150 pads every group
+        to the longest)"""
+        def reach(valid):   # [G, L] bool -> index of the last True + 1
+            L = valid.shape[1]
+            idx = torch.arange(1, L + 1, device=valid.device, dtype=torch.int32)
+            return (valid * idx).amax(1).to(torch.int32).contiguous() if L else torch.zeros(valid.shape[0], dtype=torch.int32, device=valid.device)
+
+        for li, pos in self.pos_p.items():
+            self.len_p[li] = reach(pos >= 0)
+        self.len_t = reach(self.own_t >= 0)
 
     def workspace(self, device, nbytes: int) -> torch.Tensor:
         w = self._work.get(device)
@@ -79,7 +94,7 @@ def _i32(t: Optional[torch.Tensor], what: str) -> Optional[torch.Tensor]:
 @torch.library.custom_op("spinf::xdecode_attn", mutates_args=())
 def _xdecode_op(query: torch.Tensor, kp: torch.Tensor, vp: torch.Tensor, pos_p: torch.Tensor, kt: torch.Tensor, vt: torch.Tensor,
                 pos_t: torch.Tensor, own_t: torch.Tensor, gk: torch.Tensor, gv: torch.Tensor, qpos: torch.Tensor, step_t: torch.Tensor,
-                workspace: Optional[torch.Tensor], nsplit: int, beam: int, scale: float, window: int, softcap: float) -> torch.Tensor:
+                len_p: Optional[torch.Tensor], len_t: Optional[torch.Tensor], workspace: Optional[torch.Tensor], nsplit: int, beam: int, scale: float, window: int, softcap: float) -> torch.Tensor:
     if not query.is_cuda:
         raise RuntimeError("spinf::xdecode_attn runs on ROCm device tensors only (no CPU path)")
     G, H, Q, d = query.shape
@@ -103,6 +118,11 @@ def _xdecode_op(query: torch.Tensor, kp: torch.Tensor, vp: torch.Tensor, pos_p: 
     a.kp, a.vp, a.pos_p = kp.data_ptr(), vp.data_ptr(), _i32(pos_p, "pos_p").data_ptr()
     a.kt, a.vt, a.pos_t, a.own_t = kt.data_ptr(), vt.data_ptr(), _i32(pos_t, "pos_t").data_ptr(), _i32(own_t, "own_t").data_ptr()
     a.gk, a.gv, a.qpos, a.step = gk.data_ptr(), gv.data_ptr(), qpos.data_ptr(), step_t.data_ptr()
+    for name, t in (("len_p", len_p), ("len_t", len_t)):
+        if t is not None:
+            if tuple(t.shape) != (G,):
+                raise ValueError(f"{name} must hold one length per group")
+            setattr(a, name, _i32(t, name).data_ptr())
     a.out = out.data_ptr()
     a.nsplit = nsplit
     if workspace is not None:
@@ -116,7 +136,7 @@ def _xdecode_op(query: torch.Tensor, kp: torch.Tensor, vp: torch.Tensor, pos_p: 
 
 
 @_xdecode_op.register_fake
-def _(query, kp, vp, pos_p, kt, vt, pos_t, own_t, gk, gv, qpos, step_t, workspace, nsplit, beam, scale, window, softcap):
+def _(query, kp, vp, pos_p, kt, vt, pos_t, own_t, gk, gv, qpos, step_t, len_p, len_t, workspace, nsplit, beam, scale, window, softcap):
     G, H, Q, d = query.shape
     return torch.empty((G, Q, H, d), dtype=torch.bfloat16, device=query.device)
 
@@ -142,7 +162,7 @@ def xdecode_attn(query, caches: XCaches, layer_idx: int, scale=None, window=None
         nbytes = G * H * Q * nsplit * (d + 2) * 4 if nsplit > 1 else 0
     work = c.workspace(query.device, nbytes) if nbytes else None
     return _xdecode_op(query, kp, c.vp[layer_idx], c.pos_p[layer_idx], c.kt[layer_idx], c.vt[layer_idx], c.pos_t, c.own_t, gk, c.gv[layer_idx],
-                       c.qpos, c.step_t, work, int(nsplit), int(c.beam), float(scale if scale is not None else d**-0.5), int(window or 0),
+                       c.qpos, c.step_t, c.len_p.get(layer_idx), c.len_t, work, int(nsplit), int(c.beam), float(scale if scale is not None else d**-0.5), int(window or 0),
                        float(softcap or 0.0))
 
 

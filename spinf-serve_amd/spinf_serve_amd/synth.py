@@ -261,6 +261,7 @@ def xdecode_case(G=4, H=16, h=8, d=256, slots=4, beam=6, S=17, prefix=(300, 470)
     c.pos_t, c.own_t = torch.from_numpy(pos_t).to(device), torch.from_numpy(own_t).to(device)
     c.qpos = torch.from_numpy(qpos).to(device)
     c.step_t = torch.full((1,), step, dtype=torch.int64, device=device)
+    c.set_lengths()
     query = rnd(G, Q, H, d, s=1.0).transpose(1, 2)
     return query, c
 

@@ -164,6 +164,7 @@ def test_a_group_alone_or_among_others_bit_for_bit(dev, nsplit):
         one = decode.XCaches(beam=c.beam, pos_t=c.pos_t[g : g + 1].contiguous(), own_t=c.own_t[g : g + 1].contiguous(), qpos=c.qpos[g : g + 1].contiguous(), step_t=c.step_t)
         for name in ("kp", "vp", "kt", "vt", "gk", "gv", "pos_p"):
             getattr(one, name)[0] = getattr(c, name)[0][g : g + 1].contiguous()
+        one.set_lengths()
         alone = sa.xdecode_attn(q[g : g + 1], one, 0, 1 / 16, nsplit=nsplit)
         assert torch.equal(alone[0], full[g])
 
