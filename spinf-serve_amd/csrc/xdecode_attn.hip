@@ -13,8 +13,11 @@
 // head) are its Q queries x r = H / h heads, row = q * r + head % r, so that the rows of one 32-row block are neighbouring
 // queries and their generated keys one contiguous piece of the stream.  A workgroup of four waves owns up to 128 rows (wave w the
 // rows 32 w ..) and a contiguous share of the key tiles (blockIdx: split); it visits the prefix / template tiles of its share and those generated
-// tiles that hold keys of its own queries.  K / V tiles go global -> LDS by DMA, double buffered, one barrier per tile, and are
-// shared by the four waves, so every key is read from memory once per 128 rows.  Scores are S^T = K Q^T with
+// tiles that hold keys of its own queries.  K / V tiles go global -> LDS by DMA (global_load_lds) into a ring of four buffers, three
+// tiles ahead of the arithmetic, one barrier per tile, and are shared by the four waves, so every key is read from memory once
+// per 128 rows; padding behind a group's own prefix / template length is neither read nor scheduled.  The loop issues no memory
+// operation but these DMAs (the words that say who sees a key ride along), so its wait can count them: all but the two
+// youngest tiles' worth.  Scores are S^T = K Q^T with
 // v_mfma_f32_32x32x16_bf16 (a lane owns one query row), classic online softmax with a lazily raised reference, O^T = V^T P^T
 // with V^T fragments read through ds_read_b64_tr_b16.  With more than one split every workgroup leaves (O, reference, sum)
 // per row in a workspace and xdec_combine_kernel merges them; with one split the workgroup writes the output itself.
@@ -36,6 +39,7 @@ namespace {
 constexpr int XTK = 32;            // keys per tile
 constexpr int XROWS = 128;         // rows per workgroup
 constexpr float XTAU = 8.f;        // the reference point is raised when a tile's maximum exceeds it by more than this (log2 units)
+constexpr int NBUF = 4;            // tile buffers in LDS: the DMA runs NBUF - 1 tiles ahead of the arithmetic
 constexpr int RANGE_EMPTY = 1;     // lo = 1 > hi = 0: a key nobody sees
 constexpr int POS_ALWAYS = 0x3fffffff;   // position of a key the window never hides
 
@@ -80,15 +84,19 @@ __device__ __forceinline__ int group_len(const int* len, long g, int full) {
     return n < 0 ? 0 : n < full ? n : full;
 }
 
+// s_waitcnt immediate that waits for all but the n youngest vector memory operations (gfx9 encoding: vmcnt in bits 3:0 and 15:14)
+constexpr int vmcnt_imm(int n) { return 0x0f70 | (n & 15) | ((n >> 4) << 14); }
+
 template <int D, bool WIN, bool CAP>
 __global__ __launch_bounds__(256) void xdec_kernel(const XdecParams p) {
     using GK = Geo<D, XTK>;
-    constexpr int KTILEB = GK::KTILEB, VTILEB = GK::VTILEB, METAB = 2 * XTK * 4 + 16;   // (range, position) of the tile's keys, the tile's no-mask flag
+    constexpr int KTILEB = GK::KTILEB, VTILEB = GK::VTILEB, METAB = 2 * 256 + 2 * XTK * 4;   // two words per key as they lie in memory (by DMA), then (range, position) per key
     constexpr int BUFB = KTILEB + VTILEB + METAB;
     constexpr int NS = D / 16, NDT = D / 32;
     constexpr int IPW = GK::NREG / 4;
     static_assert(IPW >= 1 && IPW * 4 == GK::NREG, "the tile's regions must divide among the four waves");
-    __shared__ __attribute__((aligned(16))) char bufs[2 * BUFB];
+    static_assert(NBUF * BUFB <= 160 * 1024, "LDS budget");
+    __shared__ __attribute__((aligned(16))) char bufs[NBUF * BUFB];
 
     const int lane = threadIdx.x & 63, m = lane & 31, g2 = lane >> 5;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -143,43 +151,57 @@ __global__ __launch_bounds__(256) void xdec_kernel(const XdecParams p) {
         which = 2;
         return ((long)gh * p.Q * p.S + (key - p.Lp - p.Tt)) * D;
     };
-    // the cache pointers as opaque scalar values: picking one per lane is then a register select (left as fields of the
-    // argument block, the compiler picks the FIELD per lane and loads the pointer from memory in front of every DMA, with a
-    // wait that also waits for the DMA before it)
-    const char* const kp_s = uniform_ptr((const char*)p.kp); const char* const vp_s = uniform_ptr((const char*)p.vp);
-    const char* const kt_s = uniform_ptr((const char*)p.kt); const char* const vt_s = uniform_ptr((const char*)p.vt);
-    const char* const gk_s = uniform_ptr((const char*)p.gk); const char* const gv_s = uniform_ptr((const char*)p.gv);
+    // per-lane part of a DMA's source address when the tile's 32 keys are 32 consecutive rows of one cache
+    const unsigned lane_src = (unsigned)((lane / GK::CPR) * GK::NREG * D * 2 + (lane % GK::CPR) * 16);
+    constexpr int DMAS = 2 * IPW + 2;   // DMA instructions per wave and tile: its share of K and of V, two words per key
+    // Starts the DMA of a tile: K and V rows, and for every key the two words that say who sees it (prefix: position; template:
+    // owning slot, position), which every wave copies to the same place (so that all waves have the same number of DMAs in
+    // flight and the loop's wait can count them).  No other memory operation is issued inside the loop.
     auto issue = [&](const unsigned buf, const int tile) {
-#ifdef XDEC_NO_DMA
-        return;
-#endif
+        const long k0 = (long)tile * XTK, lk = (long)p.Lp + p.Tt;
+        const int which = k0 + XTK <= p.Lp ? 0 : (k0 >= p.Lp && k0 + XTK <= lk) ? 1 : (k0 >= lk && k0 + XTK <= ltot) ? 2 : -1;
+        if (which >= 0) {   // the usual case: a wave-uniform base, no vector arithmetic on addresses
+            const long first = which == 0 ? (long)gh * p.Lp + k0 : which == 1 ? (long)gh * p.Tt + (k0 - p.Lp) : (long)gh * p.Q * p.S + (k0 - lk);
+            const char* kb = (const char*)(which == 0 ? p.kp : which == 1 ? p.kt : p.gk) + first * (D * 2);
+            const char* vb = (const char*)(which == 0 ? p.vp : which == 1 ? p.vt : p.gv) + first * (D * 2);
 #pragma unroll
-        for (int i = 0; i < IPW; i++) {
-            const int reg = w * IPW + i;
-            int which;
-            const long off = locate((long)tile * XTK + reg + GK::NREG * (lane / GK::CPR), which) + (lane % GK::CPR) * 8;
-            const char* kb = which == 0 ? kp_s : which == 1 ? kt_s : gk_s;
-            const char* vb = which == 0 ? vp_s : which == 1 ? vt_s : gv_s;
-            dma16_lane(kb + off * 2, buf + reg * GK::KRS);
-            dma16_lane(vb + off * 2, buf + KTILEB + reg * GK::VRS);
+            for (int i = 0; i < IPW; i++) {
+                const int reg = w * IPW + i;
+                dma16_uniform(kb + reg * (D * 2), lane_src, buf + reg * GK::KRS);
+                dma16_uniform(vb + reg * (D * 2), lane_src, buf + KTILEB + reg * GK::VRS);
+            }
+        } else {
+            // (the cache pointers as opaque scalar values: picking one per lane is then a register select; left as fields of
+            // the argument block, the compiler picks the FIELD per lane and loads the pointer from memory in front of every
+            // DMA, with a wait that also waits for the DMAs before it)
+            const char* const kp_s = uniform_ptr((const char*)p.kp); const char* const vp_s = uniform_ptr((const char*)p.vp);
+            const char* const kt_s = uniform_ptr((const char*)p.kt); const char* const vt_s = uniform_ptr((const char*)p.vt);
+            const char* const gk_s = uniform_ptr((const char*)p.gk); const char* const gv_s = uniform_ptr((const char*)p.gv);
+#pragma unroll
+            for (int i = 0; i < IPW; i++) {   // a tile across two caches, or the stream's last
+                const int reg = w * IPW + i;
+                int wh;
+                const long off = locate(k0 + reg + GK::NREG * (lane / GK::CPR), wh) + (lane % GK::CPR) * 8;
+                const char* kb = wh == 0 ? kp_s : wh == 1 ? kt_s : gk_s;
+                const char* vb = wh == 0 ? vp_s : wh == 1 ? vt_s : gv_s;
+                dma16_lane(kb + off * 2, buf + reg * GK::KRS);
+                dma16_lane(vb + off * 2, buf + KTILEB + reg * GK::VRS);
+            }
         }
+        const long key = k0 + (lane & (XTK - 1));
+        const bool pre = key < p.Lp, tem = !pre && key < lk;
+        const int* const pos_p_s = (const int*)uniform_ptr((const char*)p.pos_p); const int* const pos_t_s = (const int*)uniform_ptr((const char*)p.pos_t);
+        const int* const own_t_s = (const int*)uniform_ptr((const char*)p.own_t); const char* const step_s = uniform_ptr((const char*)p.step);
+        const int* a0 = pre ? pos_p_s + (long)g * p.Lp + key : tem ? own_t_s + (long)g * p.Tt + (key - p.Lp) : (const int*)step_s;
+        const int* a1 = tem ? pos_t_s + (long)g * p.Tt + (key - p.Lp) : (const int*)step_s;
+        dma4_lane(a0, buf + KTILEB + VTILEB);
+        dma4_lane(a1, buf + KTILEB + VTILEB + 256);
     };
-    // Key `lane` of a tile (lanes 0 .. 31 of wave 0): who may see it (queries lo .. hi, packed lo | hi << 16) and its position.
-    // The two values it needs from memory are loaded BEFORE the DMA of the tile ahead of it and turned into the LDS words one
-    // iteration later, after the loop's own wait: a wait for them between a DMA's issue and the end of the tile's
-    // arithmetic would wait for the DMA as well (one counter for all memory operations, in order).
-    auto load_raw = [&](const int tile, int& r0, int& r1) {
-        const long key = (long)tile * XTK + lane;
-        const bool pre = key < p.Lp, tem = !pre && key < (long)p.Lp + p.Tt;
-        const int* a0 = pre ? p.pos_p + (long)g * p.Lp + key : p.own_t + (long)g * p.Tt + (key - p.Lp);
-        const int* a1 = p.pos_t + (long)g * p.Tt + (key - p.Lp);
-        r0 = 0; r1 = 0;
-        if (pre || tem) r0 = *a0;
-        if (tem) r1 = *a1;
-    };
-    auto put_meta = [&](int* meta, const int tile, const int r0, const int r1) {
-        const long key = (long)tile * XTK + lane;
-        int range = RANGE_EMPTY, kpos = POS_ALWAYS;
+    // (range, position) of key m of a tile from its two words: who may see it (queries lo .. hi, packed lo | hi << 16)
+    auto derive = [&](const int tile, const int r0, const int r1, int& range, int& kpos) {
+        const long key = (long)tile * XTK + m;
+        range = RANGE_EMPTY;
+        kpos = POS_ALWAYS;
         if (key < p.Lp) {
             kpos = r0;
             if (kpos >= 0) range = (p.Q - 1) << 16;
@@ -193,47 +215,42 @@ __global__ __launch_bounds__(256) void xdec_kernel(const XdecParams p) {
             const int idx = (int)(key - p.Lp - p.Tt), qq = idx / p.S;
             if (idx - qq * p.S <= step) range = qq | (qq << 16);
         }
-        meta[lane] = range;
-        meta[XTK + lane] = kpos;
-        // a tile whose 32 keys every query sees needs no mask (sliding layers: not decided here)
-        const bool all = __builtin_amdgcn_ballot_w64(range != ((p.Q - 1) << 16)) == 0;
-        if (lane == 0) meta[2 * XTK] = !WIN && all;
     };
-    const bool meta_lane = w == 0 && lane < XTK;
-    int m_r0 = 0, m_r1 = 0;
 
+    // Everything loaded so far (queries, step, positions) is waited for HERE: left to the compiler, the waits would sit in front
+    // of the first uses inside the loop, where they would wait for the tile DMAs in flight as well, every iteration.
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+#pragma unroll
+    for (int s = 0; s < NS; s++) asm volatile("" : "+v"(qf[s]));
     const unsigned buf_base = lds_addr(bufs);
-    if (i0 < i1) {
-        if (meta_lane) {
-            load_raw(tl.tile(i0), m_r0, m_r1);
-            put_meta((int*)(bufs + KTILEB + VTILEB), tl.tile(i0), m_r0, m_r1);
-            if (i0 + 1 < i1) load_raw(tl.tile(i0 + 1), m_r0, m_r1);
-        }
-        issue(buf_base, tl.tile(i0));
-    }
+    for (int j = 0; j < NBUF - 1; j++)
+        if (i0 + j < i1) issue(buf_base + j * BUFB, tl.tile(i0 + j));
     for (int i = i0; i < i1; i++) {
-        __builtin_amdgcn_s_waitcnt(0x0f70);   // this wave's share of tile i has landed
+        // this wave's share of tile i has landed: all but the DMAs of the tiles issued after it
+        const int ahead = i1 - 1 - i;
+        if (ahead >= NBUF - 2) __builtin_amdgcn_s_waitcnt(vmcnt_imm((NBUF - 2) * DMAS));
+        else if (ahead == 1) __builtin_amdgcn_s_waitcnt(vmcnt_imm(DMAS));
+        else __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
         __syncthreads();                      // ... and everybody's; all waves are done with tile i - 1
-        const int b = (i - i0) & 1;
-        if (i + 1 < i1) {
-            if (meta_lane) {
-                put_meta((int*)(bufs + (b ^ 1) * BUFB + KTILEB + VTILEB), tl.tile(i + 1), m_r0, m_r1);
-                if (i + 2 < i1) load_raw(tl.tile(i + 2), m_r0, m_r1);
-            }
-            issue(buf_base + (b ^ 1) * BUFB, tl.tile(i + 1));
-        }
-#ifdef XDEC_NO_COMPUTE
-        continue;
-#endif
+        const int b = (i - i0) % NBUF;
+        if (i + NBUF - 1 < i1) issue(buf_base + ((i - i0 + NBUF - 1) % NBUF) * BUFB, tl.tile(i + NBUF - 1));
         const char* kb = bufs + b * BUFB;
         const char* vb = kb + KTILEB;
-        const int* meta = (const int*)(kb + KTILEB + VTILEB);
-        {   // does any key of the tile belong to a query of this wave?
-            const unsigned rg = (unsigned)meta[m];
-            const int lo = rg & 0xffff, hi = rg >> 16;
+        int* meta = (int*)(bufs + b * BUFB + KTILEB + VTILEB);
+        bool all_seen;
+        {   // who sees key m of the tile; does any key belong to a query of this wave, do all queries see all keys?
+            int range, kpos;
+            derive(tl.tile(i), meta[m], meta[64 + m], range, kpos);
+            const int lo = range & 0xffff, hi = (unsigned)range >> 16;
             const bool need = wave_on && lo <= hi && lo <= qhi_w && hi >= qlo_w;
             if (__builtin_amdgcn_ballot_w64(need) == 0) continue;
+            all_seen = !WIN && __builtin_amdgcn_ballot_w64(range != ((p.Q - 1) << 16)) == 0;
+            if (!all_seen) {   // every wave leaves the same values at the same place and reads back what it wrote itself
+                meta[128 + m] = range;
+                meta[128 + XTK + m] = kpos;
+            }
         }
+        meta += 128;
         const char* krow = kb + k_lane;
         const char* vrow = vb + v_lane;
         f32x16 s_acc;
@@ -253,7 +270,7 @@ __global__ __launch_bounds__(256) void xdec_kernel(const XdecParams p) {
             }
             return t * p.c;
         };
-        if (__builtin_amdgcn_readfirstlane(meta[2 * XTK])) {   // every row sees every key of the tile
+        if (all_seen) {   // every row sees every key of the tile: no mask
 #pragma unroll
             for (int i2 = 0; i2 < 16; i2++) {
                 s_acc[i2] = to_log2(s_acc[i2]);
@@ -421,7 +438,7 @@ extern "C" int spinf_xdecode_plan(const spinf_xdec_args* a, int32_t* nsplit, int
     *nsplit = 1;
     *workspace_bytes = 0;
     if (a->G == 0 || a->Q == 0) return SPINF_OK;
-    // 512 workgroups run at a time (two per CU of 256).  Take the split count with the fewest tile steps one after the other:
+    // One workgroup per CU of 256 runs at a time at head dim 256 (four tile buffers fill the LDS), two below.  Take the split count with the fewest tile steps one after the other:
     // rounds of workgroups x (tiles per split + 2 for a workgroup's start and end + what a split's partial results cost in
     // memory traffic, written and read back, in tiles), a split keeping at least 8 tiles.
     const long base = (long)a->G * a->h * n_chunks(a);
@@ -430,7 +447,8 @@ extern "C" int spinf_xdecode_plan(const spinf_xdec_args* a, int32_t* nsplit, int
     for (int ns = 1; ns <= 16; ns++) {
         const int per = (nt + ns - 1) / ns;
         if (ns > 1 && per < 8) break;
-        const long rounds = (base * ns + 511) / 512;
+        const long slots = a->d == 256 ? 256 : 512;
+        const long rounds = (base * ns + slots - 1) / slots;
         const int r = a->H / a->h;
         const long rows = (int64_t)a->Q * r < XROWS ? (int64_t)a->Q * r : XROWS;
         const long partial_tiles = ns > 1 ? (rows * (a->d + 2) * 8 + XTK * a->d * 4 - 1) / (XTK * a->d * 4) : 0;
