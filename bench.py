@@ -42,7 +42,8 @@ WORKLOADS = {
 # HBM bytes per launch of the dominant kernel(s), from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE runs of this file (KiB per
 # dispatch), each scaled by what the same counter reads for `--workload copy` (whose traffic is known).  The figures and the
 # commands are in profiles/*_counters.md; a workload without a counter run has None.
-TRAFFIC_BYTES = {"C2": 791_205_888, "C5": 8_716_861_440, "C5_prologue": 10_777_077_760, "C5_gate": 7_650_867_200}
+TRAFFIC_BYTES = {"C2": 791_205_888, "C5": 8_716_861_440, "C5_prologue": 10_777_077_760, "C5_gate": 7_650_867_200,
+                 "XDEC": 445_415_424, "XDEC_long": 2_324_865_024}
 
 
 def timed(fn, steps, warmup, torch):
@@ -172,7 +173,8 @@ def main():
                     ms_per_step=1e3 * wall / args.steps, dtype="bf16",
                     config={"workload": WORKLOADS[args.workload], "groups": G, "queries": G * Q, "nsplit": sa.decode.plan_splits(G, 16, 8, Q, 33, c.kp[0].shape[2], c.kt[0].shape[2], 256, 6)[0],
                             "way": "torch ops" if args.rows == "scatter" else "kernel"},
-                    roofline={"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS, "traffic": None,
+                    roofline={"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
+                              "traffic": TRAFFIC_BYTES[args.workload] if args.contents is None and args.rows != "scatter" else None,
                               "kernel_ms": ms, "algorithmic_bytes": nbytes},
                     cpu_baseline=cpu)
         print(json.dumps(line))

@@ -193,3 +193,34 @@ def test_the_interface_callable_and_the_cache_update(dev):
         decode._CURRENT[0] = None
     with pytest.raises(RuntimeError, match="outside a decoding step"):
         decode.x_attention(None, qs, ("x", 0), ("x", 0), None)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("nsplit", [1, 2])
+def test_step_replayed_from_a_graph(dev, nsplit):
+    """the reference replays a decoding step from a captured graph on static buffers (decode.py:82, 170-171): the step index, the
+    query positions and the generated K/V change between replays, the launch does not.  Every replay against the eager result."""
+    q, c = synth.xdecode_case(3, 8, 4, 128, 3, 6, 6, (50, 120), (3, 8), None, 0, seed=13, device=dev)
+    static_q = q.clone()
+    sa.xdecode_attn(static_q, c, 0, 0.09, nsplit=nsplit)   # the workspace exists before the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            static_out = sa.xdecode_attn(static_q, c, 0, 0.09, nsplit=nsplit)
+    torch.cuda.current_stream().wait_stream(side)
+    gen = torch.Generator().manual_seed(3)
+    base = c.qpos.clone()
+    for step in (0, 3, 5, 1):
+        c.step_t.fill_(step)
+        c.qpos.copy_(base + step)
+        c.gk[0][:, :, :, step] = (torch.randn(3, 4, 18, 128, generator=gen) * 0.5).to(torch.bfloat16).to(dev)
+        static_q.copy_(torch.randn(3, 8, 18, 128, generator=gen).to(torch.bfloat16).to(dev))
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = sa.xdecode_attn(static_q, c, 0, 0.09, nsplit=nsplit)
+        torch.cuda.synchronize()
+        assert torch.equal(static_out, eager)
+        assert np.abs(_np(static_out) - _oracle(static_q, c, 0.09)).max() <= TOL
