@@ -43,7 +43,7 @@ WORKLOADS = {
 # dispatch), each scaled by what the same counter reads for `--workload copy` (whose traffic is known).  The figures and the
 # commands are in profiles/*_counters.md; a workload without a counter run has None.
 TRAFFIC_BYTES = {"C2": 791_205_888, "C5": 8_716_861_440, "C5_prologue": 10_777_077_760, "C5_gate": 7_650_867_200,
-                 "XDEC": 445_415_424, "XDEC_long": 2_324_865_024}
+                 "XDEC": 525_321_216, "XDEC_long": 2_324_807_680}
 
 
 def timed(fn, steps, warmup, torch):

@@ -13,11 +13,12 @@
 // head) are its Q queries x r = H / h heads, row = q * r + head % r, so that the rows of one 32-row block are neighbouring
 // queries and their generated keys one contiguous piece of the stream.  A workgroup of four waves owns up to 128 rows (wave w the
 // rows 32 w ..) and a contiguous share of the key tiles (blockIdx: split); it visits the prefix / template tiles of its share and those generated
-// tiles that hold keys of its own queries.  K / V tiles go global -> LDS by DMA (global_load_lds) into a ring of four buffers, three
-// tiles ahead of the arithmetic, one barrier per tile, and are shared by the four waves, so every key is read from memory once
-// per 128 rows; padding behind a group's own prefix / template length is neither read nor scheduled.  The loop issues no memory
-// operation but these DMAs (the words that say who sees a key ride along), so its wait can count them: all but the two
-// youngest tiles' worth.  Scores are S^T = K Q^T with
+// tiles that hold keys of its own queries.  K / V tiles go global -> LDS by DMA (global_load_lds), double buffered (a ring of NBUF
+// buffers, NBUF - 1 tiles ahead of the arithmetic), one barrier per tile, and are shared by the four waves, so every key is read
+// from memory once per 128 rows; two workgroups share a CU, so one's arithmetic runs under the other's DMA and softmax.  Padding
+// behind a group's own prefix / template length is neither read nor scheduled.  The loop issues no memory operation but these
+// DMAs (the words that say who sees a key ride along), so its wait can count them: all but the tiles issued after the one
+// it is about to use.  Scores are S^T = K Q^T with
 // v_mfma_f32_32x32x16_bf16 (a lane owns one query row), classic online softmax with a lazily raised reference, O^T = V^T P^T
 // with V^T fragments read through ds_read_b64_tr_b16.  With more than one split every workgroup leaves (O, reference, sum)
 // per row in a workspace and xdec_combine_kernel merges them; with one split the workgroup writes the output itself.
@@ -39,7 +40,7 @@ namespace {
 constexpr int XTK = 32;            // keys per tile
 constexpr int XROWS = 128;         // rows per workgroup
 constexpr float XTAU = 8.f;        // the reference point is raised when a tile's maximum exceeds it by more than this (log2 units)
-constexpr int NBUF = 4;            // tile buffers in LDS: the DMA runs NBUF - 1 tiles ahead of the arithmetic
+constexpr int NBUF = 2;            // tile buffers in LDS: the DMA runs NBUF - 1 tiles ahead of the arithmetic (two workgroups share a CU)
 constexpr int RANGE_EMPTY = 1;     // lo = 1 > hi = 0: a key nobody sees
 constexpr int POS_ALWAYS = 0x3fffffff;   // position of a key the window never hides
 
@@ -88,7 +89,9 @@ __device__ __forceinline__ int group_len(const int* len, long g, int full) {
 constexpr int vmcnt_imm(int n) { return 0x0f70 | (n & 15) | ((n >> 4) << 14); }
 
 template <int D, bool WIN, bool CAP>
-__global__ __launch_bounds__(256) void xdec_kernel(const XdecParams p) {
+// (two waves per SIMD asked for: the compiler then stays inside 256 registers; allowed 512, it kept O^T in the accumulator half
+// of the file and spent 400 copy instructions per tile moving values between the halves)
+__global__ __launch_bounds__(256, 2) void xdec_kernel(const XdecParams p) {
     using GK = Geo<D, XTK>;
     constexpr int KTILEB = GK::KTILEB, VTILEB = GK::VTILEB, METAB = 2 * 256 + 2 * XTK * 4;   // two words per key as they lie in memory (by DMA), then (range, position) per key
     constexpr int BUFB = KTILEB + VTILEB + METAB;
@@ -438,7 +441,7 @@ extern "C" int spinf_xdecode_plan(const spinf_xdec_args* a, int32_t* nsplit, int
     *nsplit = 1;
     *workspace_bytes = 0;
     if (a->G == 0 || a->Q == 0) return SPINF_OK;
-    // One workgroup per CU of 256 runs at a time at head dim 256 (four tile buffers fill the LDS), two below.  Take the split count with the fewest tile steps one after the other:
+    // Two workgroups per CU of 256 run at a time.  Take the split count with the fewest tile steps one after the other:
     // rounds of workgroups x (tiles per split + 2 for a workgroup's start and end + what a split's partial results cost in
     // memory traffic, written and read back, in tiles), a split keeping at least 8 tiles.
     const long base = (long)a->G * a->h * n_chunks(a);
@@ -447,7 +450,7 @@ extern "C" int spinf_xdecode_plan(const spinf_xdec_args* a, int32_t* nsplit, int
     for (int ns = 1; ns <= 16; ns++) {
         const int per = (nt + ns - 1) / ns;
         if (ns > 1 && per < 8) break;
-        const long slots = a->d == 256 ? 256 : 512;
+        const long slots = 512;
         const long rounds = (base * ns + slots - 1) / slots;
         const int r = a->H / a->h;
         const long rows = (int64_t)a->Q * r < XROWS ? (int64_t)a->Q * r : XROWS;

@@ -102,8 +102,8 @@ def test_argument_checks_come_before_any_launch(lib):
 
 def test_split_suggestion():
     assert decode.plan_splits(64, 16, 8, 24, 17, 470, 40, 256, 6) == (1, 0)          # 512 workgroups already
-    ns, wb = decode.plan_splits(4, 16, 8, 24, 17, 4096, 40, 256, 6)                  # 32 (group, kv head) pairs for 256 CUs
-    assert ns == 8 and wb == 4 * 16 * 24 * ns * 258 * 4
+    ns, wb = decode.plan_splits(4, 16, 8, 24, 17, 4096, 40, 256, 6)                  # 32 (group, kv head) pairs for 512 places
+    assert ns == 16 and wb == 4 * 16 * 24 * ns * 258 * 4
     ns, _ = decode.plan_splits(4, 16, 8, 24, 17, 300, 40, 256, 6)                    # short stream: a split keeps 8 tiles
     assert 1 <= ns <= (300 + 40 + 24 * 17 + 31) // 32 // 8
 
