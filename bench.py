@@ -72,6 +72,7 @@ def main():
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--variant", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--nsplit", type=int, default=None, help="XDEC workloads: splits of a (group, kv head) key stream (default: the library's choice)")
     ap.add_argument("--rows", default="stream", choices=["stream", "compact", "scatter"],
                     help="attention workloads: stream layout (default); compact = real rows only, read through the kernel's row map; "
                          "scatter = real rows only, scattered into stream layout and gathered back around the call (the reference's way). "
@@ -155,7 +156,7 @@ def main():
                 out += torch.einsum("ghrqs,ghqsd->ghrqd", a[..., Lp + Lt :], gv).float()
                 return out.reshape(G, 16, Q, 256).transpose(1, 2).contiguous().to(q.dtype)
         else:
-            step = lambda: sa.xdecode_attn(q, c, 0, scale)  # noqa: E731
+            step = lambda: sa.xdecode_attn(q, c, 0, scale, nsplit=args.nsplit)  # noqa: E731
         wall, kern = timed(step, args.steps, args.warmup, torch)
         ms = float(np.mean(kern))
         nbytes = synth.xdecode_bytes(c, 0, H=16)
@@ -171,7 +172,7 @@ def main():
             cpu = {"value": ng * Q / dt, "unit": "queries/s", "cores": 1, "kind": "port", "sample": f"{ng} of {G} groups through the numpy float64 oracle"}
         line.update(metric="decoded queries/s, extraction-decode attention step (one layer)", value=G * Q * args.steps / wall, unit="queries/s",
                     ms_per_step=1e3 * wall / args.steps, dtype="bf16",
-                    config={"workload": WORKLOADS[args.workload], "groups": G, "queries": G * Q, "nsplit": sa.decode.plan_splits(G, 16, 8, Q, 33, c.kp[0].shape[2], c.kt[0].shape[2], 256, 6)[0],
+                    config={"workload": WORKLOADS[args.workload], "groups": G, "queries": G * Q, "nsplit": args.nsplit or sa.decode.plan_splits(G, 16, 8, Q, 33, c.kp[0].shape[2], c.kt[0].shape[2], 256, 6)[0],
                             "way": "torch ops" if args.rows == "scatter" else "kernel"},
                     roofline={"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
                               "traffic": TRAFFIC_BYTES[args.workload] if args.contents is None and args.rows != "scatter" else None,
