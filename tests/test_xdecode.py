@@ -224,3 +224,30 @@ def test_step_replayed_from_a_graph(dev, nsplit):
         torch.cuda.synchronize()
         assert torch.equal(static_out, eager)
         assert np.abs(_np(static_out) - _oracle(static_q, c, 0.09)).max() <= TOL
+
+
+@pytest.mark.gpu
+def test_seeded_random_shapes(dev):
+    """random geometries: head dims, GQA ratios, slots x beams (row chunks of 1 .. 3), ragged prefixes shorter than a tile or
+    thousands long, windows, soft caps, steps, forced split counts (more splits than some groups have tiles)"""
+    rng = np.random.default_rng(2024)
+    for case in range(24):
+        d = int(rng.choice([64, 128, 256]))
+        h = int(rng.choice([1, 2, 4]))
+        r = int(rng.choice([1, 2, 3, 6]))
+        slots, beam = int(rng.integers(1, 9)), int(rng.choice([1, 3, 6]))
+        S = int(rng.integers(1, 40))
+        G = int(rng.integers(1, 5))
+        lo = int(rng.integers(1, 200))
+        hi = lo + int(rng.choice([0, 30, 700, 2500]))
+        tl = int(rng.integers(1, 6))
+        window = int(rng.choice([0, 16, 300, 4096])) or None
+        softcap = float(rng.choice([0.0, 20.0])) or None
+        step = int(rng.integers(0, S))
+        nsplit = int(rng.choice([0, 1, 2, 5])) or None
+        print(f"case {case}: G={G} H={h * r} h={h} d={d} slots={slots} beam={beam} S={S} prefix=({lo},{hi}) window={window} softcap={softcap} step={step} nsplit={nsplit}", flush=True)
+        q, c = synth.xdecode_case(G, h * r, h, d, slots, beam, S, (lo, hi), (tl, tl + 9), window, step, seed=100 + case, device=dev)
+        scale = float(rng.choice([d**-0.5, 1 / 16]))
+        out = sa.xdecode_attn(q, c, 0, scale, window, softcap, nsplit=nsplit)
+        err = np.abs(_np(out) - _oracle(q, c, scale, window, softcap)).max()
+        assert err <= TOL, (case, err)
