@@ -35,6 +35,7 @@ WORKLOADS = {
     "C5_gate": "C5's stream through the Gated DeltaNet layer's output gate: per-head rms norm x norm_w x silu(z)",
     "XDEC": "extraction-decode attention step: 24 groups x (470-token prefix + 8 slots with templates of U{8..16} tokens) x 6 beams = 48 queries per group, 33 generated entries per query all written (step 32), 16 query / 8 KV heads, head_dim 256, scale 1/16, global layer",
     "XDEC_long": "extraction-decode attention step: 64 groups x (U{1024..4096}-token prefix + 8 slots with templates of U{8..16} tokens) x 6 beams, 33 generated entries (step 32), 16 / 8 heads, head_dim 256, global layer",
+    "XDEC_512": "XDEC's step at the head geometry of the Gemma-4 full-attention layers: 16 query heads / 1 KV head, head_dim 512 (output computed 256 head dims at a time, two launches)",
     "LM": "lm head read-out of one chunk of 1,024 read rows: soft-capping (30) + log-softmax over 262,144 fp32 logits + 8 option columns",
 }
 
@@ -129,12 +130,13 @@ def main():
         print(json.dumps(line))
         return
 
-    if args.workload in ("XDEC", "XDEC_long"):
+    if args.workload in ("XDEC", "XDEC_long", "XDEC_512"):
         from oracle import xdecode as ox
 
         long = args.workload == "XDEC_long"
         G = args.contents or (64 if long else 24)
-        q, c = synth.xdecode_case(G=G, H=16, h=8, d=256, slots=8, beam=6, S=33, prefix=(1024, 4096) if long else (470, 470), template=(8, 16),
+        xh, xd = (1, 512) if args.workload == "XDEC_512" else (8, 256)
+        q, c = synth.xdecode_case(G=G, H=16, h=xh, d=xd, slots=8, beam=6, S=33, prefix=(1024, 4096) if long else (470, 470), template=(8, 16),
                                   step=32, seed=args.seed, device=dev)
         Q, scale = q.shape[2], 1 / 16
         if args.rows == "scatter":   # the reference's own way (decode.py:81-103: three einsums, masks, one softmax, three einsums), for comparison
@@ -145,7 +147,7 @@ def main():
             ninf = torch.finfo(torch.float32).min
 
             def step():
-                qq = q.reshape(G, 8, 2, Q, 256)
+                qq = q.reshape(G, xh, 16 // xh, Q, xd)
                 sp = (torch.einsum("ghrqd,ghkd->ghrqk", qq, kp).float() * scale).masked_fill(~mp, ninf)
                 st = (torch.einsum("ghrqd,ghkd->ghrqk", qq, kt).float() * scale).masked_fill(~mt, ninf)
                 sg = (torch.einsum("ghrqd,ghqsd->ghrqs", qq, gk).float() * scale).masked_fill(mg, ninf)
@@ -154,7 +156,7 @@ def main():
                 out = torch.einsum("ghrqk,ghkd->ghrqd", a[..., :Lp], vp).float()
                 out += torch.einsum("ghrqk,ghkd->ghrqd", a[..., Lp : Lp + Lt], vt).float()
                 out += torch.einsum("ghrqs,ghqsd->ghrqd", a[..., Lp + Lt :], gv).float()
-                return out.reshape(G, 16, Q, 256).transpose(1, 2).contiguous().to(q.dtype)
+                return out.reshape(G, 16, Q, xd).transpose(1, 2).contiguous().to(q.dtype)
         else:
             step = lambda: sa.xdecode_attn(q, c, 0, scale, nsplit=args.nsplit)  # noqa: E731
         wall, kern = timed(step, args.steps, args.warmup, torch)
@@ -172,10 +174,10 @@ def main():
             cpu = {"value": ng * Q / dt, "unit": "queries/s", "cores": 1, "kind": "port", "sample": f"{ng} of {G} groups through the numpy float64 oracle"}
         line.update(metric="decoded queries/s, extraction-decode attention step (one layer)", value=G * Q * args.steps / wall, unit="queries/s",
                     ms_per_step=1e3 * wall / args.steps, dtype="bf16",
-                    config={"workload": WORKLOADS[args.workload], "groups": G, "queries": G * Q, "nsplit": args.nsplit or sa.decode.plan_splits(G, 16, 8, Q, 33, c.kp[0].shape[2], c.kt[0].shape[2], 256, 6)[0],
+                    config={"workload": WORKLOADS[args.workload], "groups": G, "queries": G * Q, "nsplit": args.nsplit or sa.decode.plan_splits(G, 16, xh, Q, 33, c.kp[0].shape[2], c.kt[0].shape[2], xd, 6)[0],
                             "way": "torch ops" if args.rows == "scatter" else "kernel"},
                     roofline={"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
-                              "traffic": TRAFFIC_BYTES[args.workload] if args.contents is None and args.rows != "scatter" else None,
+                              "traffic": TRAFFIC_BYTES.get(args.workload) if args.contents is None and args.rows != "scatter" and not args.nsplit else None,
                               "kernel_ms": ms, "algorithmic_bytes": nbytes},
                     cpu_baseline=cpu)
         print(json.dumps(line))

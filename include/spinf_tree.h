@@ -192,7 +192,7 @@ int spinf_lm_logprobs(const spinf_lm_args* args, void* stream);
  *   qpos - pos >= window (decode.py:88-89); window 0 = global layer.  softcap 0 = none (decode.py:86-87).
  *   len_p, len_t [G] int32 device, each may be NULL: a group's prefix holds keys (pos_p >= 0) only in its first len_p[g] entries,
  *   its template range (own_t >= 0) only in its first len_t[g]; the entries behind are padding and are not read.  NULL = Lp / Tt.
- * All caches contiguous, 16-byte aligned, d in {64, 128, 256}, H a multiple of h.  The key stream of a (group, kv head) can be
+ * All caches contiguous, 16-byte aligned, d in {64, 128, 256, 512}, H a multiple of h.  The key stream of a (group, kv head) can be
  * split over nsplit workgroups; nsplit > 1 needs a workspace of the size spinf_xdecode_plan reports (partial results, fp32),
  * which the caller owns.  Calls are stream-ordered; nothing is allocated.
  */

@@ -23,6 +23,8 @@
 // with V^T fragments read through ds_read_b64_tr_b16.  With more than one split every workgroup leaves (O, reference, sum)
 // per row in a workspace and xdec_combine_kernel merges them; with one split the workgroup writes the output itself.
 //
+// Head dim 512: the output is computed 256 head dims at a time, in two launches (see launch_d).
+//
 // A row's result depends on its own keys only (fixed tile order, masked entries are exact zeros), so a group's outputs do
 // not depend on which other groups share the call.
 #include <hip/hip_runtime.h>
@@ -54,6 +56,7 @@ struct XdecParams {
     float* part_o; float* part_ml;
     int G, H, h, r, Q, Lp, Tt, S, beam, window;
     int R, nchunk, nsplit, per;
+    int vcol;   // first of the DV value / output head dims this launch computes (head dim 512: two launches of 256)
     float c, cap_in, cap_out;
 };
 
@@ -88,16 +91,17 @@ __device__ __forceinline__ int group_len(const int* len, long g, int full) {
 // s_waitcnt immediate that waits for all but the n youngest vector memory operations (gfx9 encoding: vmcnt in bits 3:0 and 15:14)
 constexpr int vmcnt_imm(int n) { return 0x0f70 | (n & 15) | ((n >> 4) << 14); }
 
-template <int D, bool WIN, bool CAP>
+template <int D, int DV, bool WIN, bool CAP>
 // (two waves per SIMD asked for: the compiler then stays inside 256 registers; allowed 512, it kept O^T in the accumulator half
 // of the file and spent 400 copy instructions per tile moving values between the halves)
-__global__ __launch_bounds__(256, 2) void xdec_kernel(const XdecParams p) {
-    using GK = Geo<D, XTK>;
-    constexpr int KTILEB = GK::KTILEB, VTILEB = GK::VTILEB, METAB = 2 * 256 + 2 * XTK * 4;   // two words per key as they lie in memory (by DMA), then (range, position) per key
+__global__ __launch_bounds__(256, D <= 256 ? 2 : 1) void xdec_kernel(const XdecParams p) {
+    using GK = Geo<D, XTK>;    // K tile: 32 rows of D head dims
+    using GV = Geo<DV, XTK>;   // V tile: 32 rows of DV of the D head dims (DV = D but for head dim 512)
+    constexpr int KTILEB = GK::KTILEB, VTILEB = GV::VTILEB, METAB = 2 * 256 + 2 * XTK * 4;   // two words per key as they lie in memory (by DMA), then (range, position) per key
     constexpr int BUFB = KTILEB + VTILEB + METAB;
-    constexpr int NS = D / 16, NDT = D / 32;
-    constexpr int IPW = GK::NREG / 4;
-    static_assert(IPW >= 1 && IPW * 4 == GK::NREG, "the tile's regions must divide among the four waves");
+    constexpr int NS = D / 16, NDT = DV / 32;
+    constexpr int IPWK = GK::NREG / 4, IPWV = GV::NREG / 4;
+    static_assert(IPWK >= 1 && IPWK * 4 == GK::NREG && IPWV >= 1 && IPWV * 4 == GV::NREG, "the tile's regions must divide among the four waves");
     static_assert(NBUF * BUFB <= 160 * 1024, "LDS budget");
     __shared__ __attribute__((aligned(16))) char bufs[NBUF * BUFB];
 
@@ -144,7 +148,7 @@ __global__ __launch_bounds__(256, 2) void xdec_kernel(const XdecParams p) {
     // fragment addresses inside a tile (see Geo): K row m, 16-byte chunk g2 of each 32-byte step; V^T through the transposing read
     const int tr_a = lane & 3, tr_j = (lane >> 2) & 3, tr_mb = (lane >> 4) & 1;
     const int k_lane = GK::k_off(m) + 16 * g2;
-    const int v_lane = GK::v_off(4 * g2 + tr_j) + 32 * tr_mb + 8 * tr_a;
+    const int v_lane = GV::v_off(4 * g2 + tr_j) + 32 * tr_mb + 8 * tr_a;
 
     // element offset of key `key` of the stream inside its cache, and which cache (0 prefix, 1 templates, 2 generated)
     auto locate = [&](long key, int& which) -> long {
@@ -155,8 +159,9 @@ __global__ __launch_bounds__(256, 2) void xdec_kernel(const XdecParams p) {
         return ((long)gh * p.Q * p.S + (key - p.Lp - p.Tt)) * D;
     };
     // per-lane part of a DMA's source address when the tile's 32 keys are 32 consecutive rows of one cache
-    const unsigned lane_src = (unsigned)((lane / GK::CPR) * GK::NREG * D * 2 + (lane % GK::CPR) * 16);
-    constexpr int DMAS = 2 * IPW + 2;   // DMA instructions per wave and tile: its share of K and of V, two words per key
+    const unsigned lane_src_k = (unsigned)((lane / GK::CPR) * GK::NREG * D * 2 + (lane % GK::CPR) * 16);
+    const unsigned lane_src_v = (unsigned)((lane / GV::CPR) * GV::NREG * D * 2 + (lane % GV::CPR) * 16);
+    constexpr int DMAS = IPWK + IPWV + 2;   // DMA instructions per wave and tile: its share of K and of V, two words per key
     // Starts the DMA of a tile: K and V rows, and for every key the two words that say who sees it (prefix: position; template:
     // owning slot, position), which every wave copies to the same place (so that all waves have the same number of DMAs in
     // flight and the loop's wait can count them).  No other memory operation is issued inside the loop.
@@ -166,12 +171,16 @@ __global__ __launch_bounds__(256, 2) void xdec_kernel(const XdecParams p) {
         if (which >= 0) {   // the usual case: a wave-uniform base, no vector arithmetic on addresses
             const long first = which == 0 ? (long)gh * p.Lp + k0 : which == 1 ? (long)gh * p.Tt + (k0 - p.Lp) : (long)gh * p.Q * p.S + (k0 - lk);
             const char* kb = (const char*)(which == 0 ? p.kp : which == 1 ? p.kt : p.gk) + first * (D * 2);
-            const char* vb = (const char*)(which == 0 ? p.vp : which == 1 ? p.vt : p.gv) + first * (D * 2);
+            const char* vb = (const char*)(which == 0 ? p.vp : which == 1 ? p.vt : p.gv) + first * (D * 2) + p.vcol * 2;
 #pragma unroll
-            for (int i = 0; i < IPW; i++) {
-                const int reg = w * IPW + i;
-                dma16_uniform(kb + reg * (D * 2), lane_src, buf + reg * GK::KRS);
-                dma16_uniform(vb + reg * (D * 2), lane_src, buf + KTILEB + reg * GK::VRS);
+            for (int i = 0; i < IPWK; i++) {
+                const int reg = w * IPWK + i;
+                dma16_uniform(kb + reg * (D * 2), lane_src_k, buf + reg * GK::KRS);
+            }
+#pragma unroll
+            for (int i = 0; i < IPWV; i++) {
+                const int reg = w * IPWV + i;
+                dma16_uniform(vb + reg * (D * 2), lane_src_v, buf + KTILEB + reg * GV::VRS);
             }
         } else {
             // (the cache pointers as opaque scalar values: picking one per lane is then a register select; left as fields of
@@ -181,14 +190,18 @@ __global__ __launch_bounds__(256, 2) void xdec_kernel(const XdecParams p) {
             const char* const kt_s = uniform_ptr((const char*)p.kt); const char* const vt_s = uniform_ptr((const char*)p.vt);
             const char* const gk_s = uniform_ptr((const char*)p.gk); const char* const gv_s = uniform_ptr((const char*)p.gv);
 #pragma unroll
-            for (int i = 0; i < IPW; i++) {   // a tile across two caches, or the stream's last
-                const int reg = w * IPW + i;
+            for (int i = 0; i < IPWK; i++) {   // a tile across two caches, or the stream's last
+                const int reg = w * IPWK + i;
                 int wh;
                 const long off = locate(k0 + reg + GK::NREG * (lane / GK::CPR), wh) + (lane % GK::CPR) * 8;
-                const char* kb = wh == 0 ? kp_s : wh == 1 ? kt_s : gk_s;
-                const char* vb = wh == 0 ? vp_s : wh == 1 ? vt_s : gv_s;
-                dma16_lane(kb + off * 2, buf + reg * GK::KRS);
-                dma16_lane(vb + off * 2, buf + KTILEB + reg * GK::VRS);
+                dma16_lane((wh == 0 ? kp_s : wh == 1 ? kt_s : gk_s) + off * 2, buf + reg * GK::KRS);
+            }
+#pragma unroll
+            for (int i = 0; i < IPWV; i++) {
+                const int reg = w * IPWV + i;
+                int wh;
+                const long off = locate(k0 + reg + GV::NREG * (lane / GV::CPR), wh) + (lane % GV::CPR) * 8 + p.vcol;
+                dma16_lane((wh == 0 ? vp_s : wh == 1 ? vt_s : gv_s) + off * 2, buf + KTILEB + reg * GV::VRS);
             }
         }
         const long key = k0 + (lane & (XTK - 1));
@@ -322,9 +335,9 @@ __global__ __launch_bounds__(256, 2) void xdec_kernel(const XdecParams p) {
         l += sum;
 #pragma unroll
         for (int f = 0; f < 2 * NDT; f++) {
-            const char* vp = vrow + GK::v_off(16 * (f / NDT)) + 64 * (f % NDT);
+            const char* vp = vrow + GV::v_off(16 * (f / NDT)) + 64 * (f % NDT);
             const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)vp);
-            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vp + GK::v_off(8)));
+            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vp + GV::v_off(8)));
             const bf16x8 a = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
             o[f % NDT] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[f / NDT], o[f % NDT], 0, 0, 0);
         }
@@ -335,7 +348,7 @@ __global__ __launch_bounds__(256, 2) void xdec_kernel(const XdecParams p) {
     if (!valid) return;
     if (p.nsplit == 1) {
         const float inv = 1.0f / lsum;
-        __bf16* ob = p.out + (((long)g * p.Q + qi) * p.H + head) * D;
+        __bf16* ob = p.out + (((long)g * p.Q + qi) * p.H + head) * D + p.vcol;
 #pragma unroll
         for (int dt = 0; dt < NDT; dt++)
 #pragma unroll
@@ -347,7 +360,7 @@ __global__ __launch_bounds__(256, 2) void xdec_kernel(const XdecParams p) {
             }
     } else {
         const long prow = (((long)g * p.H + head) * p.Q + qi) * p.nsplit + split;
-        float* po = p.part_o + prow * D;
+        float* po = p.part_o + prow * DV;
 #pragma unroll
         for (int dt = 0; dt < NDT; dt++)
 #pragma unroll
@@ -358,11 +371,11 @@ __global__ __launch_bounds__(256, 2) void xdec_kernel(const XdecParams p) {
 }
 
 // out = sum_s 2^(M_s - M*) O_s / sum_s 2^(M_s - M*) l_s over the splits of a row, splits in ascending order; one thread per 4 head dims
-template <int D>
+template <int D, int DV>
 __global__ __launch_bounds__(256) void xdec_combine_kernel(const XdecParams p, const long n_rows) {
     const long idx = (long)blockIdx.x * 256 + threadIdx.x;
-    const long rowid = idx / (D / 4);
-    const int d4 = (int)(idx - rowid * (D / 4));
+    const long rowid = idx / (DV / 4);
+    const int d4 = (int)(idx - rowid * (DV / 4));
     if (rowid >= n_rows) return;
     const long gg = rowid / ((long)p.H * p.Q);
     const int head = (int)((rowid / p.Q) % p.H), qi = (int)(rowid % p.Q);
@@ -380,21 +393,21 @@ __global__ __launch_bounds__(256) void xdec_combine_kernel(const XdecParams p, c
         const float ms = ml[2 * s];
         if (ms == -INFINITY) continue;
         const float wgt = __builtin_amdgcn_exp2f(ms - mstar);
-        const float4 x = *(const float4*)(p.part_o + (rowid * p.nsplit + s) * D + 4 * d4);
+        const float4 x = *(const float4*)(p.part_o + (rowid * p.nsplit + s) * DV + 4 * d4);
         acc.x += wgt * x.x; acc.y += wgt * x.y; acc.z += wgt * x.z; acc.w += wgt * x.w;
         lsum += wgt * ml[2 * s + 1];
     }
     const float inv = 1.0f / lsum;
     bf16x4 r;
     r[0] = (__bf16)(acc.x * inv); r[1] = (__bf16)(acc.y * inv); r[2] = (__bf16)(acc.z * inv); r[3] = (__bf16)(acc.w * inv);
-    *(bf16x4*)(p.out + ((gg * p.Q + qi) * p.H + head) * D + 4 * d4) = r;
+    *(bf16x4*)(p.out + ((gg * p.Q + qi) * p.H + head) * D + p.vcol + 4 * d4) = r;
 }
 
 int check_args(const spinf_xdec_args* a) {
     if (!a) return spinf_fail(SPINF_E_ARG, "xdecode_attn: null args");
     if (a->G < 0 || a->H <= 0 || a->h <= 0 || a->H % a->h || a->Q < 0 || a->S <= 0 || a->Lp < 0 || a->Tt < 0 || a->beam <= 0)
         return spinf_fail(SPINF_E_ARG, "xdecode_attn: bad sizes (G %d H %d h %d Q %d S %d Lp %d Tt %d beam %d)", a->G, a->H, a->h, a->Q, a->S, a->Lp, a->Tt, a->beam);
-    if (a->d != 64 && a->d != 128 && a->d != 256) return spinf_fail(SPINF_E_ARG, "xdecode_attn: head dim %d not supported (64, 128, 256)", a->d);
+    if (a->d != 64 && a->d != 128 && a->d != 256 && a->d != 512) return spinf_fail(SPINF_E_ARG, "xdecode_attn: head dim %d not supported (64, 128, 256, 512)", a->d);
     if (a->Q > 32767 || (int64_t)a->Q * (a->H / a->h) > (1 << 20)) return spinf_fail(SPINF_E_ARG, "xdecode_attn: %d queries per group out of range", a->Q);
     if ((int64_t)a->Lp + a->Tt + (int64_t)a->Q * a->S > (1 << 30)) return spinf_fail(SPINF_E_ARG, "xdecode_attn: key stream too long");
     if ((int64_t)a->G * a->h > (1 << 24)) return spinf_fail(SPINF_E_ARG, "xdecode_attn: too many (group, kv head) pairs");
@@ -405,25 +418,30 @@ int check_args(const spinf_xdec_args* a) {
 
 int n_chunks(const spinf_xdec_args* a) { return (int)(((int64_t)a->Q * (a->H / a->h) + XROWS - 1) / XROWS); }
 
-template <int D>
-int launch_d(const XdecParams& p, bool cap, int blocks, hipStream_t s) {
+// Head dim 512 (the Gemma-4 full-attention layers): O^T for 32 rows x 512 head dims would be 256 accumulator registers per lane
+// next to 128 of queries, so the output is computed 256 head dims at a time, in two launches: each computes the scores over all
+// 512 head dims and P V for one half of V's columns (DV = 256, XdecParams::vcol), in one workgroup per CU.
+template <int D, int DV>
+int launch_d(XdecParams p, bool cap, int blocks, hipStream_t s) {
     const bool win = p.window > 0;
-    if (win && cap) hipLaunchKernelGGL((xdec_kernel<D, true, true>), dim3(blocks), dim3(256), 0, s, p);
-    else if (win) hipLaunchKernelGGL((xdec_kernel<D, true, false>), dim3(blocks), dim3(256), 0, s, p);
-    else if (cap) hipLaunchKernelGGL((xdec_kernel<D, false, true>), dim3(blocks), dim3(256), 0, s, p);
-    else hipLaunchKernelGGL((xdec_kernel<D, false, false>), dim3(blocks), dim3(256), 0, s, p);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "xdecode_attn: launch: %s", hipGetErrorString(e));
-    if (p.nsplit > 1) {
-        const long n_rows = (long)p.G * p.H * p.Q;
-        const long threads = n_rows * (D / 4);
-        hipLaunchKernelGGL((xdec_combine_kernel<D>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, p, n_rows);
-        e = hipGetLastError();
-        if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "xdecode_attn: launch (combine): %s", hipGetErrorString(e));
+    p.part_ml = p.part_o ? p.part_o + (long)p.G * p.H * p.Q * p.nsplit * DV : nullptr;
+    for (p.vcol = 0; p.vcol < D; p.vcol += DV) {
+        if (win && cap) hipLaunchKernelGGL((xdec_kernel<D, DV, true, true>), dim3(blocks), dim3(256), 0, s, p);
+        else if (win) hipLaunchKernelGGL((xdec_kernel<D, DV, true, false>), dim3(blocks), dim3(256), 0, s, p);
+        else if (cap) hipLaunchKernelGGL((xdec_kernel<D, DV, false, true>), dim3(blocks), dim3(256), 0, s, p);
+        else hipLaunchKernelGGL((xdec_kernel<D, DV, false, false>), dim3(blocks), dim3(256), 0, s, p);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "xdecode_attn: launch: %s", hipGetErrorString(e));
+        if (p.nsplit > 1) {
+            const long n_rows = (long)p.G * p.H * p.Q;
+            const long threads = n_rows * (DV / 4);
+            hipLaunchKernelGGL((xdec_combine_kernel<D, DV>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, p, n_rows);
+            e = hipGetLastError();
+            if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "xdecode_attn: launch (combine): %s", hipGetErrorString(e));
+        }
     }
     return SPINF_OK;
 }
-
 
 // tiles of the longest list of the call: the first row chunk of a group whose prefix and template ranges are full
 int max_tiles(const spinf_xdec_args* a) {
@@ -499,8 +517,9 @@ extern "C" int spinf_xdecode_attn_fwd(const spinf_xdec_args* a, void* stream) {
     const bool cap = a->softcap > 0.f;
     hipStream_t s = (hipStream_t)stream;
     switch (a->d) {
-        case 64: return launch_d<64>(p, cap, (int)blocks, s);
-        case 128: return launch_d<128>(p, cap, (int)blocks, s);
-        default: return launch_d<256>(p, cap, (int)blocks, s);
+        case 64: return launch_d<64, 64>(p, cap, (int)blocks, s);
+        case 128: return launch_d<128, 128>(p, cap, (int)blocks, s);
+        case 256: return launch_d<256, 256>(p, cap, (int)blocks, s);
+        default: return launch_d<512, 256>(p, cap, (int)blocks, s);
     }
 }

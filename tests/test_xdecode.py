@@ -119,6 +119,8 @@ CASES = [
     (2, 8, 8, 128, 3, 6, 33, (31, 33), (1, 2), None, 30.0, 20, 2),           # MHA, soft cap, keys end inside a tile
     (1, 4, 1, 64, 1, 1, 3, (1, 1), (1, 1), 1024, 50.0, 1, 1),                # one query, a handful of keys
     (5, 16, 8, 256, 2, 6, 65, (64, 1500), (10, 30), 512, None, 40, 4),       # ragged prefixes, window clips them
+    (2, 16, 1, 512, 4, 6, 9, (200, 600), (4, 12), None, None, 5, None),      # head dim 512, one kv head (Gemma-4 global layers): 384 rows
+    (2, 8, 2, 512, 2, 3, 5, (20, 90), (2, 6), 64, 25.0, 4, 2),               # head dim 512 with window, soft cap and splits
 ]
 
 
@@ -232,7 +234,7 @@ def test_seeded_random_shapes(dev):
     thousands long, windows, soft caps, steps, forced split counts (more splits than some groups have tiles)"""
     rng = np.random.default_rng(2024)
     for case in range(24):
-        d = int(rng.choice([64, 128, 256]))
+        d = int(rng.choice([64, 128, 256, 512]))
         h = int(rng.choice([1, 2, 4]))
         r = int(rng.choice([1, 2, 3, 6]))
         slots, beam = int(rng.integers(1, 9)), int(rng.choice([1, 3, 6]))
