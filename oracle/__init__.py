@@ -19,6 +19,11 @@ How each function is pinned (none relies on re-typing its own formula in a test)
                             rule (after one token the state maps k_t to v_t exactly when |k_t|=1); linearity in v
   gdn.chunked               equals gdn.recurrent in float64 (two different algorithms for the same function)
   gdn.tree_scan             branch from the trunk's state == one sequence trunk||branch (docs/QWEN.md:51-52)
+  gdn_layer.prologue/gate   torch's conv1d (one path = a depthwise causal convolution), silu, sigmoid, softplus, rms_norm
+  lm_head.logprobs          torch.tanh / torch.log_softmax
+  xdecode.x_attention       torch's scaled_dot_product_attention over the concatenated visible keys (the mask rebuilt key by
+                            key in the test), and attention.tree_attention: a decoding step is the last row of causal
+                            attention over prefix || own template || own generated tokens
   plan.tree_plan            the toy integer recurrence of the reference's tests/test_qwen_plan.py:27-94 and the
                             literal of tests/test_stacks.py:67-75
 
