@@ -194,7 +194,10 @@ int spinf_lm_logprobs(const spinf_lm_args* args, void* stream);
  *   its template range (own_t >= 0) only in its first len_t[g]; the entries behind are padding and are not read.  NULL = Lp / Tt.
  * All caches contiguous, 16-byte aligned, d in {64, 128, 256, 512}, H a multiple of h.  The key stream of a (group, kv head) can be
  * split over nsplit workgroups; nsplit > 1 needs a workspace of the size spinf_xdecode_plan reports (partial results, fp32),
- * which the caller owns.  Calls are stream-ordered; nothing is allocated.
+ * which the caller owns.  A split is tiles_per_split 32-key tiles of a (group, kv head, 128 rows) list, 0 = the longest list's
+ * tiles (spinf_xdecode_tiles) / nsplit, rounded up; nsplit x tiles_per_split must cover the longest list.  Lists that fit one
+ * split (short groups, once len_p / len_t are given) are computed by one workgroup and leave no partial results.
+ * Calls are stream-ordered; nothing is allocated.
  */
 typedef struct spinf_xdec_args {
     const void* q; int64_t q_g, q_h, q_q;
@@ -205,11 +208,14 @@ typedef struct spinf_xdec_args {
     const int64_t* qpos; const int64_t* step;
     void* out;
     void* workspace; int64_t workspace_bytes; int32_t nsplit;
+    int32_t tiles_per_split;
     int32_t G, H, h, Q, S, Lp, Tt, d, beam, window;
     float scale, softcap;
 } spinf_xdec_args;
 /* suggested nsplit for these sizes (enough workgroups to fill the GPU) and the workspace it needs (0 for nsplit 1) */
 int spinf_xdecode_plan(const spinf_xdec_args* args, int32_t* nsplit, int64_t* workspace_bytes);
+/* tiles of the longest list of these sizes (a group whose prefix and template ranges are full) */
+int spinf_xdecode_tiles(const spinf_xdec_args* args, int32_t* tiles);
 int spinf_xdecode_attn_fwd(const spinf_xdec_args* args, void* stream);
 
 #ifdef __cplusplus

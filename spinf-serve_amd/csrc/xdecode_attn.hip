@@ -346,7 +346,7 @@ __global__ __launch_bounds__(256, D <= 256 ? 2 : 1) void xdec_kernel(const XdecP
     // register i of O^T tile dt holds head dim 32 dt + 8 (i / 4) + 4 g2 + i % 4 of this lane's row
     const float lsum = lane32_sum(l);
     if (!valid) return;
-    if (p.nsplit == 1) {
+    if (tl.nt <= p.per) {   // the list's only split: the output itself (lists longer than p.per leave partial results)
         const float inv = 1.0f / lsum;
         __bf16* ob = p.out + (((long)g * p.Q + qi) * p.H + head) * D + p.vcol;
 #pragma unroll
@@ -384,6 +384,7 @@ __global__ __launch_bounds__(256) void xdec_combine_kernel(const XdecParams p, c
     const int last_row = chunk * XROWS + XROWS - 1 < p.R ? chunk * XROWS + XROWS - 1 : p.R - 1;
     const TileList tl(p.Lp, p.Tt, p.S, group_len(p.len_p, gg, p.Lp), group_len(p.len_t, gg, p.Tt), (chunk * XROWS) / p.r, last_row / p.r);
     const int ns = (tl.nt + p.per - 1) / p.per;
+    if (ns == 1) return;   // written by the one workgroup itself
     const float* ml = p.part_ml + rowid * p.nsplit * 2;
     float mstar = -INFINITY;
     for (int s = 0; s < ns; s++) mstar = fmaxf(mstar, ml[2 * s]);
@@ -480,6 +481,14 @@ extern "C" int spinf_xdecode_plan(const spinf_xdec_args* a, int32_t* nsplit, int
     return SPINF_OK;
 }
 
+extern "C" int spinf_xdecode_tiles(const spinf_xdec_args* a, int32_t* tiles) {
+    const int rc = check_args(a);
+    if (rc) return rc;
+    if (!tiles) return spinf_fail(SPINF_E_ARG, "xdecode_tiles: null output");
+    *tiles = a->G == 0 || a->Q == 0 ? 0 : max_tiles(a);
+    return SPINF_OK;
+}
+
 extern "C" int spinf_xdecode_attn_fwd(const spinf_xdec_args* a, void* stream) {
     const int rc = check_args(a);
     if (rc) return rc;
@@ -492,6 +501,8 @@ extern "C" int spinf_xdecode_attn_fwd(const spinf_xdec_args* a, void* stream) {
     for (const void* ptr : {a->q, (const void*)a->out, a->kp, a->vp, a->kt, a->vt, a->gk, a->gv})
         if ((uintptr_t)ptr % 16) return spinf_fail(SPINF_E_ARG, "xdecode_attn: q, out and the caches must be 16-byte aligned");
     if (a->nsplit < 1 || a->nsplit > 64) return spinf_fail(SPINF_E_ARG, "xdecode_attn: nsplit %d (1 .. 64)", a->nsplit);
+    if (a->tiles_per_split < 0 || (a->tiles_per_split > 0 && (int64_t)a->tiles_per_split * a->nsplit < max_tiles(a)))
+        return spinf_fail(SPINF_E_ARG, "xdecode_attn: %d splits of %d tiles do not cover the longest list (%d tiles)", a->nsplit, a->tiles_per_split, max_tiles(a));
     const int64_t need = a->nsplit > 1 ? (int64_t)a->G * a->H * a->Q * a->nsplit * (a->d + 2) * 4 : 0;
     if (need > 0 && (!a->workspace || a->workspace_bytes < need || (uintptr_t)a->workspace % 16))
         return spinf_fail(SPINF_E_ARG, "xdecode_attn: %d splits need a 16-byte aligned workspace of %lld bytes", a->nsplit, (long long)need);
@@ -507,7 +518,7 @@ extern "C" int spinf_xdecode_attn_fwd(const spinf_xdec_args* a, void* stream) {
     p.G = a->G; p.H = a->H; p.h = a->h; p.r = a->H / a->h; p.Q = a->Q; p.Lp = a->Lp; p.Tt = a->Tt; p.S = a->S; p.beam = a->beam;
     p.window = a->window;
     p.R = p.Q * p.r; p.nchunk = n_chunks(a); p.nsplit = a->nsplit;
-    p.per = (max_tiles(a) + p.nsplit - 1) / p.nsplit;
+    p.per = a->tiles_per_split > 0 ? a->tiles_per_split : (max_tiles(a) + p.nsplit - 1) / p.nsplit;
     const float log2e = 1.4426950408889634f;
     p.c = a->scale * log2e;
     p.cap_in = a->softcap > 0.f ? 2.0f * log2e * a->scale / a->softcap : 0.f;

@@ -62,7 +62,7 @@ class XdecArgs(C.Structure):
         ("gk", C.c_void_p), ("gv", C.c_void_p),
         ("qpos", C.c_void_p), ("step", C.c_void_p),
         ("out", C.c_void_p),
-        ("workspace", C.c_void_p), ("workspace_bytes", C.c_int64), ("nsplit", C.c_int32),
+        ("workspace", C.c_void_p), ("workspace_bytes", C.c_int64), ("nsplit", C.c_int32), ("tiles_per_split", C.c_int32),
         ("G", C.c_int32), ("H", C.c_int32), ("h", C.c_int32), ("Q", C.c_int32), ("S", C.c_int32), ("Lp", C.c_int32), ("Tt", C.c_int32),
         ("d", C.c_int32), ("beam", C.c_int32), ("window", C.c_int32),
         ("scale", C.c_float), ("softcap", C.c_float),
@@ -114,7 +114,8 @@ def load_library():
     lib.spinf_lm_logprobs.argtypes = [C.POINTER(LmArgs), C.c_void_p]
     lib.spinf_xdecode_plan.argtypes = [C.POINTER(XdecArgs), C.POINTER(C.c_int32), C.POINTER(C.c_int64)]
     lib.spinf_xdecode_attn_fwd.argtypes = [C.POINTER(XdecArgs), C.c_void_p]
-    for name in ("spinf_tileplan_build", "spinf_tileplan_build_groups", "spinf_tileplan_build_ktile", "spinf_tileplan_counts", "spinf_tileplan_export", "spinf_tileplan_schedule", "spinf_tileplan_row0", "spinf_tree_attn_fwd", "spinf_attn_exact_items", "spinf_gdn_fwd", "spinf_gdn_prologue", "spinf_gdn_gate", "spinf_lm_logprobs", "spinf_xdecode_plan", "spinf_xdecode_attn_fwd"):
+    lib.spinf_xdecode_tiles.argtypes = [C.POINTER(XdecArgs), C.POINTER(C.c_int32)]
+    for name in ("spinf_tileplan_build", "spinf_tileplan_build_groups", "spinf_tileplan_build_ktile", "spinf_tileplan_counts", "spinf_tileplan_export", "spinf_tileplan_schedule", "spinf_tileplan_row0", "spinf_tree_attn_fwd", "spinf_attn_exact_items", "spinf_gdn_fwd", "spinf_gdn_prologue", "spinf_gdn_gate", "spinf_lm_logprobs", "spinf_xdecode_plan", "spinf_xdecode_tiles", "spinf_xdecode_attn_fwd"):
         getattr(lib, name).restype = C.c_int
     _LIB = lib
     return lib

@@ -43,7 +43,9 @@ class XCaches:
     beam: int = 6
     len_p: dict = field(default_factory=dict)   # by layer: [G] int32, entries of each group's prefix that can hold keys (set_lengths)
     len_t: Optional[torch.Tensor] = None        # [G] int32, the same for the template range
-    _work: dict = field(default_factory=dict)   # workspace of the split launches, by (device, bytes needed)
+    _work: dict = field(default_factory=dict)   # workspace of the split launches, by device
+    _host_len: dict = field(default_factory=dict)   # by layer: (len_p, len_t) as host tuples (set_lengths)
+    _plans: dict = field(default_factory=dict)      # split plans by geometry and lengths (plan_ragged)
 
     def set_lengths(self) -> None:
         """once per decoder, after the caches are filled: how far each group's prefix (pos_p >= 0) and template range
@@ -57,6 +59,9 @@ class XCaches:
         for li, pos in self.pos_p.items():
             self.len_p[li] = reach(pos >= 0)
         self.len_t = reach(self.own_t >= 0)
+        lt = tuple(self.len_t.tolist())
+        self._host_len = {li: (tuple(n.tolist()), lt) for li, n in self.len_p.items()}
+        self._plans.clear()
 
     def workspace(self, device, nbytes: int) -> torch.Tensor:
         w = self._work.get(device)
@@ -94,7 +99,7 @@ def _i32(t: Optional[torch.Tensor], what: str) -> Optional[torch.Tensor]:
 @torch.library.custom_op("spinf::xdecode_attn", mutates_args=())
 def _xdecode_op(query: torch.Tensor, kp: torch.Tensor, vp: torch.Tensor, pos_p: torch.Tensor, kt: torch.Tensor, vt: torch.Tensor,
                 pos_t: torch.Tensor, own_t: torch.Tensor, gk: torch.Tensor, gv: torch.Tensor, qpos: torch.Tensor, step_t: torch.Tensor,
-                len_p: Optional[torch.Tensor], len_t: Optional[torch.Tensor], workspace: Optional[torch.Tensor], nsplit: int, beam: int, scale: float, window: int, softcap: float) -> torch.Tensor:
+                len_p: Optional[torch.Tensor], len_t: Optional[torch.Tensor], workspace: Optional[torch.Tensor], nsplit: int, tiles_per_split: int, beam: int, scale: float, window: int, softcap: float) -> torch.Tensor:
     if not query.is_cuda:
         raise RuntimeError("spinf::xdecode_attn runs on ROCm device tensors only (no CPU path)")
     G, H, Q, d = query.shape
@@ -124,7 +129,7 @@ def _xdecode_op(query: torch.Tensor, kp: torch.Tensor, vp: torch.Tensor, pos_p: 
                 raise ValueError(f"{name} must hold one length per group")
             setattr(a, name, _i32(t, name).data_ptr())
     a.out = out.data_ptr()
-    a.nsplit = nsplit
+    a.nsplit, a.tiles_per_split = nsplit, tiles_per_split
     if workspace is not None:
         a.workspace, a.workspace_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
     a.G, a.H, a.h, a.Q, a.S, a.Lp, a.Tt, a.d, a.beam, a.window = G, H, h, Q, S, Lp, Tt, d, beam, window
@@ -136,7 +141,7 @@ def _xdecode_op(query: torch.Tensor, kp: torch.Tensor, vp: torch.Tensor, pos_p: 
 
 
 @_xdecode_op.register_fake
-def _(query, kp, vp, pos_p, kt, vt, pos_t, own_t, gk, gv, qpos, step_t, len_p, len_t, workspace, nsplit, beam, scale, window, softcap):
+def _(query, kp, vp, pos_p, kt, vt, pos_t, own_t, gk, gv, qpos, step_t, len_p, len_t, workspace, nsplit, tiles_per_split, beam, scale, window, softcap):
     G, H, Q, d = query.shape
     return torch.empty((G, Q, H, d), dtype=torch.bfloat16, device=query.device)
 
@@ -150,19 +155,82 @@ def plan_splits(G: int, H: int, h: int, Q: int, S: int, Lp: int, Tt: int, d: int
     return ns.value, wb.value
 
 
+_TILE, _ROWS = 32, 128   # keys per tile, rows per workgroup (csrc/xdecode_attn.hip)
+
+
+def _list_tiles(Lp: int, Tt: int, S: int, len_p: int, len_t: int, qlo: int, qhi: int) -> int:
+    """tiles of the list of a workgroup that owns queries qlo .. qhi (TileList of csrc/xdecode_attn.hip)"""
+    lk = Lp + Tt
+    e0 = -(-len_p // _TILE)
+    s1 = max(Lp // _TILE if len_t > 0 else e0, e0)
+    e1 = max(-(-(Lp + len_t) // _TILE) if len_t > 0 else s1, s1)
+    s2 = max((lk + qlo * S) // _TILE, e1)
+    e2 = max(-(-(lk + (qhi + 1) * S) // _TILE), s2)
+    return e0 + (e1 - s1) + (e2 - s2)
+
+
+def plan_ragged(G: int, H: int, h: int, Q: int, S: int, Lp: int, Tt: int, d: int, beam: int, len_p, len_t) -> tuple[int, int]:
+    """-> (nsplit, tiles per split) for groups whose prefix / template ranges reach len_p[g] / len_t[g] entries: the split size
+    with the shortest simulated schedule (workgroups in launch order onto the places the GPU runs at a time; a workgroup costs
+    its tiles + 2, a list that is split also its partial results' traffic, 7 tiles a piece at 128 rows x 256 head dims)"""
+    import heapq
+
+    r = H // h
+    R = Q * r
+    a = _lib.XdecArgs()
+    a.G, a.H, a.h, a.Q, a.S, a.Lp, a.Tt, a.d, a.beam = G, H, h, Q, S, Lp, Tt, d, beam
+    nt_max = C.c_int32(0)
+    _lib.check(_lib.load_library().spinf_xdecode_tiles(C.byref(a), C.byref(nt_max)), "spinf_xdecode_tiles")
+    nt_max = nt_max.value
+    chunks = [(c * _ROWS // r, (min(c * _ROWS + _ROWS, R) - 1) // r, min(_ROWS, R - c * _ROWS)) for c in range(-(-R // _ROWS))]
+    lists = [[_list_tiles(Lp, Tt, S, min(len_p[g], Lp), min(len_t[g], Tt), lo, hi) for g in range(G)] for lo, hi, _ in chunks]
+    mean = sum(map(sum, lists)) / (G * len(chunks))
+    places = 256 if d == 512 else 512
+    cands = {nt_max} | {-(-nt_max // k) for k in range(2, 9)} | {int(mean * f) + 1 for f in (1.0, 1.15, 1.3, 1.5)}
+    best = None
+    for per in sorted(c for c in cands if 8 <= c <= nt_max or c == nt_max):
+        ns_max = -(-nt_max // per)
+        if ns_max > 16:
+            continue
+        free = [0.0] * places
+        heapq.heapify(free)
+        end = 0.0
+        for (lo, hi, rows), nts in zip(chunks, lists):
+            part = 7.0 * rows * (min(d, 256) + 2) / (_ROWS * 258)
+            for nt in nts:
+                ns = -(-nt // per)
+                for _ in range(h):
+                    for sp in range(ns_max):
+                        t = min(per, nt - sp * per)
+                        cost = 0.2 if t <= 0 else t + 2 + (part if ns > 1 else 0.0)
+                        t0 = heapq.heappop(free)
+                        heapq.heappush(free, t0 + cost)
+                        end = max(end, t0 + cost)
+        end += 3.0 if ns_max > 1 else 0.0   # the merge launch
+        if best is None or end < best[0]:
+            best = (end, ns_max, per)
+    return best[1], best[2]
+
+
 def xdecode_attn(query, caches: XCaches, layer_idx: int, scale=None, window=None, softcap=None, nsplit=None):
     """query [G, H, Q, d] bf16 -> [G, Q, H, d] bf16: softmax over (the group's prefix | the slot's own template | the beam's own
     generated tokens up to caches.step_t), see x_attention"""
     c = caches
     G, H, Q, d = query.shape
     kp, gk = c.kp[layer_idx], c.gk[layer_idx]
-    if nsplit is None:
-        nsplit, nbytes = plan_splits(G, H, gk.shape[1], Q, gk.shape[3], kp.shape[2], c.kt[layer_idx].shape[2], d, c.beam)
-    else:
-        nbytes = G * H * Q * nsplit * (d + 2) * 4 if nsplit > 1 else 0
+    per = 0
+    if nsplit is None and layer_idx in c._host_len:   # the groups' own lengths are known: split sizes that balance them
+        geo = (G, H, gk.shape[1], Q, gk.shape[3], kp.shape[2], c.kt[layer_idx].shape[2], d, c.beam)
+        key = geo + c._host_len[layer_idx]
+        if key not in c._plans:
+            c._plans[key] = plan_ragged(*geo, *c._host_len[layer_idx])
+        nsplit, per = c._plans[key]
+    elif nsplit is None:
+        nsplit, _ = plan_splits(G, H, gk.shape[1], Q, gk.shape[3], kp.shape[2], c.kt[layer_idx].shape[2], d, c.beam)
+    nbytes = G * H * Q * nsplit * (d + 2) * 4 if nsplit > 1 else 0
     work = c.workspace(query.device, nbytes) if nbytes else None
     return _xdecode_op(query, kp, c.vp[layer_idx], c.pos_p[layer_idx], c.kt[layer_idx], c.vt[layer_idx], c.pos_t, c.own_t, gk, c.gv[layer_idx],
-                       c.qpos, c.step_t, c.len_p.get(layer_idx), c.len_t, work, int(nsplit), int(c.beam), float(scale if scale is not None else d**-0.5), int(window or 0),
+                       c.qpos, c.step_t, c.len_p.get(layer_idx), c.len_t, work, int(nsplit), int(per), int(c.beam), float(scale if scale is not None else d**-0.5), int(window or 0),
                        float(softcap or 0.0))
 
 

@@ -108,6 +108,24 @@ def test_split_suggestion():
     assert 1 <= ns <= (300 + 40 + 24 * 17 + 31) // 32 // 8
 
 
+def test_split_sizes_for_ragged_groups():
+    """with the groups' own lengths known the split size comes from a simulated schedule: many groups fill the GPU unsplit, a
+    few ragged ones are cut into pieces of about the same size; nsplit x tiles per split always covers the longest list"""
+    rng = np.random.default_rng(0)
+    for G in (64, 12, 3):
+        P = [int(x) for x in rng.integers(1024, 4097, G)]
+        ns, per = decode.plan_ragged(G, 16, 8, 48, 33, max(P), 100, 256, 6, tuple(P), (100,) * G)
+        longest = decode._list_tiles(max(P), 100, 33, max(P), 100, 0, 47)
+        assert ns * per >= longest and per >= 8
+        assert (ns == 1) == (G == 64)
+    # the host's tile count is the library's
+    a = _lib.XdecArgs()
+    a.G, a.H, a.h, a.Q, a.S, a.Lp, a.Tt, a.d, a.beam = 2, 16, 8, 48, 33, 1000, 77, 256, 6
+    n = C.c_int32(0)
+    assert _lib.load_library().spinf_xdecode_tiles(C.byref(a), C.byref(n)) == 0
+    assert n.value == decode._list_tiles(1000, 77, 33, 1000, 77, 0, 47) == 84   # 96 rows: one chunk with all 48 queries
+
+
 # ------------------------------------------------------------------------------------------------ kernel parity (GPU)
 CASES = [
     # G, H, h, d, slots, beam, S, prefix, template, window, softcap, step, nsplit
