@@ -43,7 +43,7 @@ class XCaches:
     beam: int = 6
     len_p: dict = field(default_factory=dict)   # by layer: [G] int32, entries of each group's prefix that can hold keys (set_lengths)
     len_t: Optional[torch.Tensor] = None        # [G] int32, the same for the template range
-    _work: dict = field(default_factory=dict)   # workspace of the split launches, by device
+    _spaces: dict = field(default_factory=dict)   # workspace of the split launches, by device
     _host_len: dict = field(default_factory=dict)   # by layer: (len_p, len_t) as host tuples (set_lengths)
     _plans: dict = field(default_factory=dict)      # split plans by geometry and lengths (plan_ragged)
 
@@ -64,9 +64,9 @@ class XCaches:
         self._plans.clear()
 
     def workspace(self, device, nbytes: int) -> torch.Tensor:
-        w = self._work.get(device)
+        w = self._spaces.get(device)
         if w is None or w.numel() < nbytes:
-            w = self._work[device] = torch.empty(nbytes, dtype=torch.uint8, device=device)
+            w = self._spaces[device] = torch.empty(nbytes, dtype=torch.uint8, device=device)
         return w
 
 
@@ -96,7 +96,7 @@ def _i32(t: Optional[torch.Tensor], what: str) -> Optional[torch.Tensor]:
     return t
 
 
-@torch.library.custom_op("spinf::xdecode_attn", mutates_args=())
+@torch.library.custom_op("spinf::xdecode_attn", mutates_args=("workspace",))
 def _xdecode_op(query: torch.Tensor, kp: torch.Tensor, vp: torch.Tensor, pos_p: torch.Tensor, kt: torch.Tensor, vt: torch.Tensor,
                 pos_t: torch.Tensor, own_t: torch.Tensor, gk: torch.Tensor, gv: torch.Tensor, qpos: torch.Tensor, step_t: torch.Tensor,
                 len_p: Optional[torch.Tensor], len_t: Optional[torch.Tensor], workspace: Optional[torch.Tensor], nsplit: int, tiles_per_split: int, beam: int, scale: float, window: int, softcap: float) -> torch.Tensor:
