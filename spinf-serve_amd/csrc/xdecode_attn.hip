@@ -346,7 +346,7 @@ __global__ __launch_bounds__(256, D <= 256 ? 2 : 1) void xdec_kernel(const XdecP
     // register i of O^T tile dt holds head dim 32 dt + 8 (i / 4) + 4 g2 + i % 4 of this lane's row
     const float lsum = lane32_sum(l);
     if (!valid) return;
-    if (tl.nt <= p.per) {   // the list's only split: the output itself (lists longer than p.per leave partial results)
+    if (p.nsplit == 1 || tl.nt <= p.per) {   // the list's only split: the output itself (lists longer than p.per leave partial results)
         const float inv = 1.0f / lsum;
         __bf16* ob = p.out + (((long)g * p.Q + qi) * p.H + head) * D + p.vcol;
 #pragma unroll
@@ -444,11 +444,19 @@ int launch_d(XdecParams p, bool cap, int blocks, hipStream_t s) {
     return SPINF_OK;
 }
 
-// tiles of the longest list of the call: the first row chunk of a group whose prefix and template ranges are full
+// tiles of the longest list of the call: a group whose prefix and template ranges are full, the row chunk with the most tiles
+// (not always the first: the tile where the template range ends and the generated entries begin counts with the former, and
+// where a chunk's generated entries begin and end inside their tiles differs from chunk to chunk)
 int max_tiles(const spinf_xdec_args* a) {
     const int r = a->H / a->h;
-    const int first_hi = (int)(((int64_t)a->Q * r < XROWS ? (int64_t)a->Q * r : XROWS) - 1) / r;
-    return TileList(a->Lp, a->Tt, a->S, a->Lp, a->Tt, 0, first_hi).nt;
+    const long R = (long)a->Q * r;
+    int most = 0;
+    for (long row0 = 0; row0 < R; row0 += XROWS) {
+        const long last = row0 + XROWS - 1 < R ? row0 + XROWS - 1 : R - 1;
+        const int nt = TileList(a->Lp, a->Tt, a->S, a->Lp, a->Tt, (int)(row0 / r), (int)(last / r)).nt;
+        most = nt > most ? nt : most;
+    }
+    return most;
 }
 
 }  // namespace

@@ -126,6 +126,29 @@ def test_split_sizes_for_ragged_groups():
     assert n.value == decode._list_tiles(1000, 77, 33, 1000, 77, 0, 47) == 84   # 96 rows: one chunk with all 48 queries
 
 
+def test_longest_list_over_all_row_chunks():
+    """the library's tile count is the maximum over the row chunks (a later chunk can hold more tiles than the first: where its
+    generated entries begin and end inside their tiles), so that splits sized from it cover every list"""
+    rng = np.random.default_rng(5)
+    lib = _lib.load_library()
+    later = 0
+    for _ in range(300):
+        H, h = [(16, 1), (16, 8), (24, 4), (8, 8), (6, 2)][int(rng.integers(5))]
+        Q, S = int(rng.integers(1, 200)), int(rng.integers(1, 70))
+        Lp, Tt = int(rng.integers(0, 3000)), int(rng.integers(0, 300))
+        a = _lib.XdecArgs()
+        a.G, a.H, a.h, a.Q, a.S, a.Lp, a.Tt, a.d, a.beam = 3, H, h, Q, S, Lp, Tt, 128, 3
+        n = C.c_int32(0)
+        assert lib.spinf_xdecode_tiles(C.byref(a), C.byref(n)) == 0
+        r, R = H // h, Q * (H // h)
+        per_chunk = [decode._list_tiles(Lp, Tt, S, Lp, Tt, c * 128 // r, (min(c * 128 + 128, R) - 1) // r) for c in range(-(-R // 128))]
+        assert n.value == max(per_chunk)
+        later += max(per_chunk) > per_chunk[0]
+        ns, per = decode.plan_ragged(3, H, h, Q, S, Lp, Tt, 128, 3, (Lp,) * 3, (Tt,) * 3)
+        assert ns * per >= max(per_chunk)
+    assert later > 10   # the case exists
+
+
 # ------------------------------------------------------------------------------------------------ kernel parity (GPU)
 CASES = [
     # G, H, h, d, slots, beam, S, prefix, template, window, softcap, step, nsplit
@@ -139,6 +162,8 @@ CASES = [
     (5, 16, 8, 256, 2, 6, 65, (64, 1500), (10, 30), 512, None, 40, 4),       # ragged prefixes, window clips them
     (2, 16, 1, 512, 4, 6, 9, (200, 600), (4, 12), None, None, 5, None),      # head dim 512, one kv head (Gemma-4 global layers): 384 rows
     (2, 8, 2, 512, 2, 3, 5, (20, 90), (2, 6), 64, 25.0, 4, 2),               # head dim 512 with window, soft cap and splits
+    (24, 16, 1, 512, 8, 6, 33, (470, 470), (8, 16), None, None, 32, None),   # six row chunks, the later ones with longer tile lists than the first
+    (3, 16, 1, 256, 8, 6, 33, (470, 470), (8, 16), None, None, 32, 1),       # the same at head dim 256, one split
 ]
 
 
