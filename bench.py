@@ -176,7 +176,7 @@ def main():
             cpu = {"value": ng * Q / dt, "unit": "queries/s", "cores": 1, "kind": "port", "sample": f"{ng} of {G} groups through the numpy float64 oracle"}
         line.update(metric="decoded queries/s, extraction-decode attention step (one layer)", value=G * Q * args.steps / wall, unit="queries/s",
                     ms_per_step=1e3 * wall / args.steps, dtype="bf16",
-                    config={"workload": WORKLOADS[args.workload], "groups": G, "queries": G * Q, "nsplit": args.nsplit or sa.decode.plan_splits(G, 16, xh, Q, 33, c.kp[0].shape[2], c.kt[0].shape[2], xd, 6)[0],
+                    config={"workload": WORKLOADS[args.workload], "groups": G, "queries": G * Q, "nsplit": args.nsplit or (next(iter(c._plans.values()))[0] if c._plans else None),
                             "way": "torch ops" if args.rows == "scatter" else "kernel"},
                     roofline={"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
                               "traffic": TRAFFIC_BYTES.get(args.workload) if args.contents is None and args.rows != "scatter" and not args.nsplit else None,
