@@ -11,17 +11,17 @@
 // Layout of the work.  The three ranges are taken as ONE stream of keys per (group, kv head), cut into tiles of 32 keys:
 // prefix | templates | generated (row-major over (q, s), which is how gk / gv lie in memory).  The rows of a (group, kv
 // head) are its Q queries x r = H / h heads, row = q * r + head % r, so that the rows of one 32-row block are neighbouring
-// queries and their generated keys one contiguous piece of the stream.  A workgroup of four waves owns up to 128 rows (wave w the
-// rows 32 w ..) and a contiguous share of the key tiles (blockIdx: split); it visits the prefix / template tiles of its share and those generated
-// tiles that hold keys of its own queries.  K / V tiles go global -> LDS by DMA (global_load_lds), double buffered (a ring of NBUF
-// buffers, NBUF - 1 tiles ahead of the arithmetic), one barrier per tile, and are shared by the four waves, so every key is read
-// from memory once per 128 rows; two workgroups share a CU, so one's arithmetic runs under the other's DMA and softmax.  Padding
-// behind a group's own prefix / template length is neither read nor scheduled.  The loop issues no memory operation but these
-// DMAs (the words that say who sees a key ride along), so its wait can count them: all but the tiles issued after the one
-// it is about to use.  Scores are S^T = K Q^T with
-// v_mfma_f32_32x32x16_bf16 (a lane owns one query row), classic online softmax with a lazily raised reference, O^T = V^T P^T
-// with V^T fragments read through ds_read_b64_tr_b16.  With more than one split every workgroup leaves (O, reference, sum)
-// per row in a workspace and xdec_combine_kernel merges them; with one split the workgroup writes the output itself.
+// queries and their generated keys one contiguous piece of the stream.  A workgroup of four waves owns up to 128 rows (wave
+// w the rows 32 w ..) and a contiguous share of the key tiles (a split); it visits the prefix / template tiles of its share
+// and those generated tiles that hold keys of its own queries.  K / V tiles go global -> LDS by DMA (global_load_lds), double
+// buffered (a ring of NBUF buffers, NBUF - 1 tiles ahead of the arithmetic), one barrier per tile, and are shared by the four
+// waves, so every key is read from memory once per 128 rows; two workgroups share a CU, so one's arithmetic runs under the
+// other's DMA and softmax.  Padding behind a group's own prefix / template length is neither read nor scheduled.  The loop
+// issues no memory operation but these DMAs (the words that say who sees a key ride along), so its wait can count them: all
+// but the tiles issued after the one it is about to use.  Scores are S^T = K Q^T with v_mfma_f32_32x32x16_bf16 (a lane owns
+// one query row), classic online softmax with a lazily raised reference, O^T = V^T P^T with V^T fragments read through
+// ds_read_b64_tr_b16.  A list longer than one split (XdecParams::per tiles) leaves (O, reference, sum) per row and split in a
+// workspace and xdec_combine_kernel merges them; a list that fits one split is written out by its one workgroup.
 //
 // Head dim 512: the output is computed 256 head dims at a time, in two launches (see launch_d).
 //
