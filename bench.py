@@ -6,6 +6,7 @@ A step is one pass of the attention op (one layer's call through the C ABI) over
 resident in HBM; the tile plan is compiled once per stream, outside the timed region, as the reference builds its block
 masks once per forward for all layers.  Prints ONE JSON line: packed query tokens/s, the useful-FLOP roofline fraction of
 the kernel (events on the launch stream around every step) and the CPU baseline (dense-mask attention on the host cores).
+Before the W warm-up steps the step is run untimed for SPINUP_S seconds, so that the timed steps see the GPU's sustained clocks.
 """
 
 from __future__ import annotations
@@ -47,7 +48,14 @@ TRAFFIC_BYTES = {"C2": 791_205_888, "C5": 8_716_861_440, "C5_prologue": 10_777_0
                  "XDEC": 525_321_216, "XDEC_long": 2_324_807_680}
 
 
+SPINUP_S = 0.05   # untimed, before the warm-up steps: keeps the GPU busy until its clocks have come up from idle
+
+
 def timed(fn, steps, warmup, torch):
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < SPINUP_S:
+        fn()
+        torch.cuda.synchronize()
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -97,7 +105,7 @@ def main():
     torch.cuda.set_device(dev)
     line = {"metric": "packed query tokens/s + % bf16 MFMA peak (useful FLOPs), tree-mask attn", "unit": "tokens/s", "n_gpus": 1,
             "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-            "data": "synthetic (seeded, numpy default_rng / torch generator)", "seed": args.seed}
+            "data": "synthetic (seeded, numpy default_rng / torch generator)", "seed": args.seed, "spinup_s": SPINUP_S}
 
     if args.workload == "copy":
         n = 1 << 30
