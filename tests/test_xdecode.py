@@ -273,14 +273,14 @@ def test_step_replayed_from_a_graph(dev, nsplit):
 
 @pytest.mark.gpu
 def test_seeded_random_shapes(dev):
-    """random geometries: head dims, GQA ratios, slots x beams (row chunks of 1 .. 3), ragged prefixes shorter than a tile or
+    """random geometries: head dims, GQA ratios, slots x beams (one to nine row chunks), ragged prefixes shorter than a tile or
     thousands long, windows, soft caps, steps, forced split counts (more splits than some groups have tiles)"""
     rng = np.random.default_rng(2024)
-    for case in range(24):
+    for case in range(60):
         d = int(rng.choice([64, 128, 256, 512]))
         h = int(rng.choice([1, 2, 4]))
-        r = int(rng.choice([1, 2, 3, 6]))
-        slots, beam = int(rng.integers(1, 9)), int(rng.choice([1, 3, 6]))
+        r = int(rng.choice([1, 2, 3, 6, 16]))
+        slots, beam = int(rng.integers(1, 13)), int(rng.choice([1, 3, 6]))
         S = int(rng.integers(1, 40))
         G = int(rng.integers(1, 5))
         lo = int(rng.integers(1, 200))
