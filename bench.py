@@ -36,6 +36,7 @@ WORKLOADS = {
     "C5_gate": "C5's stream through the Gated DeltaNet layer's output gate: per-head rms norm x norm_w x silu(z)",
     "XDEC": "extraction-decode attention step: 24 groups x (470-token prefix + 8 slots with templates of U{8..16} tokens) x 6 beams = 48 queries per group, 33 generated entries per query all written (step 32), 16 query / 8 KV heads, head_dim 256, scale 1/16, global layer",
     "XDEC_long": "extraction-decode attention step: 64 groups x (U{1024..4096}-token prefix + 8 slots with templates of U{8..16} tokens) x 6 beams, 33 generated entries (step 32), 16 / 8 heads, head_dim 256, global layer",
+    "XDEC_qwen": "XDEC's step at the Qwen-hybrid attention geometry: 24 query heads / 4 KV heads, head_dim 256 (288 rows per (group, kv head): three row chunks)",
     "XDEC_512": "XDEC's step at the head geometry of the Gemma-4 full-attention layers: 16 query heads / 1 KV head, head_dim 512 (output computed 256 head dims at a time, two launches)",
     "LM": "lm head read-out of one chunk of 1,024 read rows: soft-capping (30) + log-softmax over 262,144 fp32 logits + 8 option columns",
 }
@@ -140,13 +141,13 @@ def main():
         print(json.dumps(line))
         return
 
-    if args.workload in ("XDEC", "XDEC_long", "XDEC_512"):
+    if args.workload in ("XDEC", "XDEC_long", "XDEC_512", "XDEC_qwen"):
         from oracle import xdecode as ox
 
         long = args.workload == "XDEC_long"
         G = args.contents or (64 if long else 24)
-        xh, xd = (1, 512) if args.workload == "XDEC_512" else (8, 256)
-        q, c = synth.xdecode_case(G=G, H=16, h=xh, d=xd, slots=8, beam=6, S=33, prefix=(1024, 4096) if long else (470, 470), template=(8, 16),
+        xH, xh, xd = {"XDEC_512": (16, 1, 512), "XDEC_qwen": (24, 4, 256)}.get(args.workload, (16, 8, 256))
+        q, c = synth.xdecode_case(G=G, H=xH, h=xh, d=xd, slots=8, beam=6, S=33, prefix=(1024, 4096) if long else (470, 470), template=(8, 16),
                                   step=32, seed=args.seed, device=dev)
         Q, scale = q.shape[2], 1 / 16
         if args.rows == "scatter":   # the reference's own way (decode.py:81-103: three einsums, masks, one softmax, three einsums), for comparison
@@ -157,7 +158,7 @@ def main():
             ninf = torch.finfo(torch.float32).min
 
             def step():
-                qq = q.reshape(G, xh, 16 // xh, Q, xd)
+                qq = q.reshape(G, xh, xH // xh, Q, xd)
                 sp = (torch.einsum("ghrqd,ghkd->ghrqk", qq, kp).float() * scale).masked_fill(~mp, ninf)
                 st = (torch.einsum("ghrqd,ghkd->ghrqk", qq, kt).float() * scale).masked_fill(~mt, ninf)
                 sg = (torch.einsum("ghrqd,ghqsd->ghrqs", qq, gk).float() * scale).masked_fill(mg, ninf)
@@ -166,12 +167,12 @@ def main():
                 out = torch.einsum("ghrqk,ghkd->ghrqd", a[..., :Lp], vp).float()
                 out += torch.einsum("ghrqk,ghkd->ghrqd", a[..., Lp : Lp + Lt], vt).float()
                 out += torch.einsum("ghrqs,ghqsd->ghrqd", a[..., Lp + Lt :], gv).float()
-                return out.reshape(G, 16, Q, xd).transpose(1, 2).contiguous().to(q.dtype)
+                return out.reshape(G, xH, Q, xd).transpose(1, 2).contiguous().to(q.dtype)
         else:
             step = lambda: sa.xdecode_attn(q, c, 0, scale, nsplit=args.nsplit)  # noqa: E731
         wall, kern = timed(step, args.steps, args.warmup, torch)
         ms = float(np.mean(kern))
-        nbytes = synth.xdecode_bytes(c, 0, H=16)
+        nbytes = synth.xdecode_bytes(c, 0, H=xH)
         gbs = nbytes / (ms * 1e-3) / 1e9
         cpu = None
         if not args.no_cpu and args.rows != "scatter":   # the float64 oracle on the first groups, one core
