@@ -171,8 +171,10 @@ def _list_tiles(Lp: int, Tt: int, S: int, len_p: int, len_t: int, qlo: int, qhi:
 
 def plan_ragged(G: int, H: int, h: int, Q: int, S: int, Lp: int, Tt: int, d: int, beam: int, len_p, len_t) -> tuple[int, int]:
     """-> (nsplit, tiles per split) for groups whose prefix / template ranges reach len_p[g] / len_t[g] entries: the split size
-    with the shortest simulated schedule (workgroups in launch order onto the places the GPU runs at a time; a workgroup costs
-    its tiles + 2, a list that is split also its partial results' traffic, 7 tiles a piece at 128 rows x 256 head dims)"""
+    with the shortest estimated step: the longer of (a) the simulated schedule (workgroups in launch order onto the places the
+    GPU runs at a time; a workgroup costs its tiles + 2, a list that is split also its partial results' traffic, 7 tiles a piece
+    at 128 rows x 256 head dims) at 2 us a tile and (b) all the tiles of the step at the rate the memory delivers them (6.5 ns a
+    tile), plus 10 us for the merge launch of a split step.  The two rates are measured ones (XDEC, XDEC_long, XDEC_qwen of bench.py)."""
     import heapq
 
     r = H // h
@@ -194,7 +196,7 @@ def plan_ragged(G: int, H: int, h: int, Q: int, S: int, Lp: int, Tt: int, d: int
             continue
         free = [0.0] * places
         heapq.heapify(free)
-        end = 0.0
+        end = total = 0.0
         for (lo, hi, rows), nts in zip(chunks, lists):
             part = 7.0 * rows * (min(d, 256) + 2) / (_ROWS * 258)
             for nt in nts:
@@ -206,9 +208,10 @@ def plan_ragged(G: int, H: int, h: int, Q: int, S: int, Lp: int, Tt: int, d: int
                         t0 = heapq.heappop(free)
                         heapq.heappush(free, t0 + cost)
                         end = max(end, t0 + cost)
-        end += 3.0 if ns_max > 1 else 0.0   # the merge launch
-        if best is None or end < best[0]:
-            best = (end, ns_max, per)
+                        total += cost
+        est = max(end * 2.0, total * 0.0065) + (10.0 if ns_max > 1 else 0.0)   # microseconds
+        if best is None or est < best[0]:
+            best = (est, ns_max, per)
     return best[1], best[2]
 
 
