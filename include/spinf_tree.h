@@ -108,6 +108,15 @@ typedef struct spinf_attn_args {
 /* query heads one work item covers for this geometry (1 or 2); 0 for an invalid geometry */
 int spinf_attn_heads_per_item(int32_t hq, int32_t hkv, int32_t d, int32_t variant);
 int spinf_tree_attn_fwd(const spinf_attn_args* args, void* stream);
+/* The same pass with nothing allocated.  No counterpart in the reference: it is for callers that cannot call hipMalloc (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid allocation).  spinf_tree_attn_fwd keeps its list cursors,
+ * counts and redo list in a buffer that the library allocates (and regrows) on the device; this entry point keeps them in a
+ * file-scope device array of 64 + 65,536 ints (256.25 KiB per GPU, held until the process ends) and calls no hipMalloc /
+ * hipFree nor any allocating routine.  Same arguments, same kernels, same results bit for bit.  Limit: n_items (query tiles x
+ * head groups) <= 65,536, more is SPINF_E_ARG.  The cursors and counts are cleared by a small kernel in front of every pass, so
+ * a call does not depend on what the previous one left.  Every call on a GPU shares that GPU's array: calls that overlap on
+ * one GPU (different streams or threads) race; order them on one stream. */
+int spinf_tree_attn_fwd_noalloc(const spinf_attn_args* args, void* stream);
 /* Diagnostics (no counterpart in the reference): *total = work items that the exact (rescaling) pass has recomputed on the
  * current device since the library was loaded, i.e. query tiles whose scores ranged too widely for the fast pass.
  * Synchronises the device. */

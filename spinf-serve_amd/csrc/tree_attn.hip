@@ -54,6 +54,7 @@ struct AttnParams {
     // kv_row0[entry] = row of the entry's first key if its 64 keys are 64 consecutive rows, else -1
     const int* row_of; const int* kv_row0;
     const int* grp;       // image groups (GRP kernels): -1 none; the tokens of a group see each other both ways
+    bool clear_first;     // host side only: zero the cursors and counts in front of the pass (the entry point that allocates nothing)
 };
 
 // Softmax reference point.  The fast pass fixes each row's reference at the maximum of the first 32-key block in which
@@ -756,6 +757,11 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
 }
 
 // ------------------------------------------------------------------------------------------------ host side
+// Scratch memory of the entry point that allocates nothing (spinf_tree_attn_fwd_noalloc): list cursors, counts and the redo
+// list.  In host code this name is a stand-in, not a device address: hipGetSymbolAddress gives the address, per device.
+constexpr long NOALLOC_MAX_ITEMS = 1 << 16;                            // work items (query tiles x head groups) of one call
+static __device__ __align__(256) int scratch[64 + NOALLOC_MAX_ITEMS];  // 256.25 KiB per GPU, held until the process ends
+
 namespace {
 
 struct DeviceState {
@@ -795,10 +801,49 @@ int device_state(DeviceState** out, long n_items) {
     return SPINF_OK;
 }
 
+// ---- the entry point that allocates nothing
+
+struct ScratchState {
+    int* ptr = nullptr;   // device address of `scratch` on this device (every GPU holds its own copy of the array)
+    int cus = 0;
+};
+ScratchState g_scratch[64];
+
+int scratch_state(ScratchState** out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= 64) return spinf_fail(SPINF_E_HIP, "tree_attn (no allocation): hipGetDevice: %s", hipGetErrorString(e));
+    std::lock_guard<std::mutex> lock(g_mu);
+    ScratchState& s = g_scratch[dev];
+    if (!s.ptr) {   // first call on this device (it is the current one)
+        hipDeviceProp_t prop;
+        e = hipGetDeviceProperties(&prop, dev);
+        if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn (no allocation): hipGetDeviceProperties: %s", hipGetErrorString(e));
+        int* ptr = nullptr;
+        e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) return spinf_fail(SPINF_E_HIP, "tree_attn (no allocation): hipGetSymbolAddress: %s", hipGetErrorString(e));
+        s.cus = prop.multiProcessorCount;
+        s.ptr = ptr;
+    }
+    *out = &s;
+    return SPINF_OK;
+}
+
+// cursors and counts of a call start at zero whatever the previous call on this GPU left behind (a fill kernel, not a memset
+// node: the call may be recorded into a graph); the running total of exact-pass items at [NLIST + 3] is kept
+__global__ void attn_clear_counters_kernel(int* counters) {
+    if (threadIdx.x < NLIST + 3) counters[threadIdx.x] = 0;
+}
+
 template <int D, int RT, bool WIN, int NHW, bool ROWS, int GRP = 0, int TK = 64, int DV = D>
 int launch(const AttnParams& p, int blocks, hipStream_t stream) {
     using G = TileGeo<D, TK, DV>;
     static_assert(2 * G::BUFB + 2 * ENT_CAP * 12 + ((NHW == 2 && D == 256) ? 16 : 4 * NHW * 32 * 144) + 64 <= 160 * 1024, "LDS budget");
+    if (p.clear_first) {
+        hipLaunchKernelGGL(attn_clear_counters_kernel, dim3(1), dim3(64), 0, stream, p.counters);
+        hipError_t e0 = hipGetLastError();
+        if (e0 != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: launch (clear): %s", hipGetErrorString(e0));
+    }
     hipLaunchKernelGGL((tree_attn_kernel<D, RT, WIN, NHW, ROWS, GRP, TK, DV>), dim3(blocks), dim3(256 * NHW), 0, stream, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: launch: %s", hipGetErrorString(e));
@@ -877,11 +922,13 @@ extern "C" int spinf_attn_exact_items(int64_t* total) {
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess || dev < 0 || dev >= 64) return spinf_fail(SPINF_E_HIP, "attn_exact_items: hipGetDevice: %s", hipGetErrorString(e));
     std::lock_guard<std::mutex> lock(g_mu);
-    if (!g_dev[dev].counters) return SPINF_OK;   // no attention launch on this device yet
-    int v = 0;
-    e = hipMemcpy(&v, g_dev[dev].counters + NLIST + 3, sizeof(int), hipMemcpyDeviceToHost);
-    if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "attn_exact_items: hipMemcpy: %s", hipGetErrorString(e));
-    *total = v;
+    for (const int* c : {(const int*)g_dev[dev].counters, (const int*)g_scratch[dev].ptr}) {
+        if (!c) continue;   // no attention launch of that kind on this device yet
+        int v = 0;
+        e = hipMemcpy(&v, c + NLIST + 3, sizeof(int), hipMemcpyDeviceToHost);
+        if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "attn_exact_items: hipMemcpy: %s", hipGetErrorString(e));
+        *total += v;
+    }
     return SPINF_OK;
 }
 
@@ -892,11 +939,13 @@ extern "C" int spinf_attn_heads_per_item(int32_t hq, int32_t hkv, int32_t d, int
     return rt * nhw;
 }
 
-extern "C" int spinf_tree_attn_fwd(const spinf_attn_args* a, void* stream) {
+static int attn_fwd(const spinf_attn_args* a, void* stream, bool no_alloc) {
     if (!a) return spinf_fail(SPINF_E_ARG, "tree_attn: null args");
     if (a->n <= 0 || a->n_items <= 0) return SPINF_OK;
     if (!a->q || !a->k || !a->v || !a->out || !a->art || !a->end || !a->pos || !a->kv_idx || !a->kv_bits || !a->items || !a->list_ptr)
         return spinf_fail(SPINF_E_ARG, "tree_attn: null pointer");
+    if (no_alloc && a->n_items > NOALLOC_MAX_ITEMS)
+        return spinf_fail(SPINF_E_ARG, "tree_attn (no allocation): %lld work items, at most %ld (query tiles x head groups)", (long long)a->n_items, NOALLOC_MAX_ITEMS);
     if (a->d != 64 && a->d != 128 && a->d != 256 && a->d != 512) return spinf_fail(SPINF_E_ARG, "tree_attn: head dim %d not in {64,128,256,512}", a->d);
     if (a->hq <= 0 || a->hkv <= 0 || a->hq % a->hkv) return spinf_fail(SPINF_E_ARG, "tree_attn: hq %d not a multiple of hkv %d", a->hq, a->hkv);
     if (a->n > INT32_MAX / 2) return spinf_fail(SPINF_E_ARG, "tree_attn: stream too long");
@@ -920,9 +969,21 @@ extern "C" int spinf_tree_attn_fwd(const spinf_attn_args* a, void* stream) {
     const uintptr_t ptrs[4] = {(uintptr_t)a->q, (uintptr_t)a->k, (uintptr_t)a->v, (uintptr_t)a->out};
     for (int i = 0; i < 4; i++)
         if (ptrs[i] % 16) return spinf_fail(SPINF_E_ARG, "tree_attn: tensors must be 16-byte aligned");
-    DeviceState* st = nullptr;
-    if (int rc = device_state(&st, (long)a->n_items)) return rc;
+    int* counters = nullptr;
+    int cus = 0;
+    if (no_alloc) {
+        ScratchState* st = nullptr;
+        if (int rc = scratch_state(&st)) return rc;
+        counters = st->ptr;
+        cus = st->cus;
+    } else {
+        DeviceState* st = nullptr;
+        if (int rc = device_state(&st, (long)a->n_items)) return rc;
+        counters = st->counters;
+        cus = st->cus;
+    }
     AttnParams p;
+    p.clear_first = no_alloc;
     p.q = (const __bf16*)a->q; p.k = (const __bf16*)a->k; p.v = (const __bf16*)a->v; p.o = (__bf16*)a->out;
     p.q_tok = a->q_tok; p.q_head = a->q_head; p.k_tok = a->k_tok; p.k_head = a->k_head;
     p.v_tok = a->v_tok; p.v_head = a->v_head; p.o_tok = a->o_tok; p.o_head = a->o_head;
@@ -934,9 +995,9 @@ extern "C" int spinf_tree_attn_fwd(const spinf_attn_args* a, void* stream) {
     p.items = (const int4*)a->items; p.list_ptr = a->list_ptr;
     p.row_of = a->row_of; p.kv_row0 = a->kv_row0;
     p.grp = a->grp;
-    p.counters = st->counters;
-    p.redo = st->counters + 64;
-    const int blocks = (int)(a->n_items < st->cus ? a->n_items : st->cus);
+    p.counters = counters;
+    p.redo = counters + 64;
+    const int blocks = (int)(a->n_items < cus ? a->n_items : cus);
     const bool win = p.window > 0;
     hipStream_t s = (hipStream_t)stream;
     switch (a->d) {
@@ -946,3 +1007,7 @@ extern "C" int spinf_tree_attn_fwd(const spinf_attn_args* a, void* stream) {
         default: return launch_d512(p, win, a->grp_mode, blocks, s);
     }
 }
+
+extern "C" int spinf_tree_attn_fwd(const spinf_attn_args* a, void* stream) { return attn_fwd(a, stream, false); }
+
+extern "C" int spinf_tree_attn_fwd_noalloc(const spinf_attn_args* a, void* stream) { return attn_fwd(a, stream, true); }

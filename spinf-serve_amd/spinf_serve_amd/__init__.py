@@ -15,7 +15,7 @@ compute entry points without the built library raises.
 from ._lib import load_library, library_path  # noqa: F401
 from .packer import BLOCK, Batch, GroupedTree, Owner, Packer, ReadPlan, Tree, build_grouped_tree, build_tree, split_grouped_trees, split_trees, trie_branches  # noqa: F401
 from .masks import TreeMask, TilePlan, block_masks  # noqa: F401
-from .attention import CAPTURE, register_tree_attention, tree_attention, tree_attn, tree_flex_forward  # noqa: F401
+from .attention import CAPTURE, register_tree_attention, tree_attention, tree_attn, tree_attn_noalloc, tree_flex_forward  # noqa: F401
 from .gdn import chunked, recurrent  # noqa: F401
 from .gdn_layer import gdn_gate, gdn_prologue  # noqa: F401
 from .lm_head import lm_logprobs  # noqa: F401

@@ -10,7 +10,7 @@ _LIB = None
 
 SYMBOLS = (
     "spinf_last_error", "spinf_version", "spinf_tileplan_build", "spinf_tileplan_counts", "spinf_tileplan_export",
-    "spinf_tileplan_schedule", "spinf_tileplan_free", "spinf_attn_heads_per_item", "spinf_tree_attn_fwd", "spinf_attn_exact_items", "spinf_gdn_fwd",
+    "spinf_tileplan_schedule", "spinf_tileplan_free", "spinf_attn_heads_per_item", "spinf_tree_attn_fwd", "spinf_tree_attn_fwd_noalloc", "spinf_attn_exact_items", "spinf_gdn_fwd",
 )
 
 
@@ -107,6 +107,7 @@ def load_library():
     lib.spinf_tileplan_free.argtypes = [C.c_void_p]
     lib.spinf_tileplan_free.restype = None
     lib.spinf_tree_attn_fwd.argtypes = [C.POINTER(AttnArgs), C.c_void_p]
+    lib.spinf_tree_attn_fwd_noalloc.argtypes = [C.POINTER(AttnArgs), C.c_void_p]
     lib.spinf_attn_exact_items.argtypes = [C.POINTER(C.c_int64)]
     lib.spinf_gdn_fwd.argtypes = [C.POINTER(GdnArgs), C.c_void_p]
     lib.spinf_gdn_prologue.argtypes = [C.POINTER(GdnPreArgs), C.c_void_p]
@@ -115,7 +116,7 @@ def load_library():
     lib.spinf_xdecode_plan.argtypes = [C.POINTER(XdecArgs), C.POINTER(C.c_int32), C.POINTER(C.c_int64)]
     lib.spinf_xdecode_attn_fwd.argtypes = [C.POINTER(XdecArgs), C.c_void_p]
     lib.spinf_xdecode_tiles.argtypes = [C.POINTER(XdecArgs), C.POINTER(C.c_int32)]
-    for name in ("spinf_tileplan_build", "spinf_tileplan_build_groups", "spinf_tileplan_build_ktile", "spinf_tileplan_counts", "spinf_tileplan_export", "spinf_tileplan_schedule", "spinf_tileplan_row0", "spinf_tree_attn_fwd", "spinf_attn_exact_items", "spinf_gdn_fwd", "spinf_gdn_prologue", "spinf_gdn_gate", "spinf_lm_logprobs", "spinf_xdecode_plan", "spinf_xdecode_tiles", "spinf_xdecode_attn_fwd"):
+    for name in ("spinf_tileplan_build", "spinf_tileplan_build_groups", "spinf_tileplan_build_ktile", "spinf_tileplan_counts", "spinf_tileplan_export", "spinf_tileplan_schedule", "spinf_tileplan_row0", "spinf_tree_attn_fwd", "spinf_tree_attn_fwd_noalloc", "spinf_attn_exact_items", "spinf_gdn_fwd", "spinf_gdn_prologue", "spinf_gdn_gate", "spinf_lm_logprobs", "spinf_xdecode_plan", "spinf_xdecode_tiles", "spinf_xdecode_attn_fwd"):
         getattr(lib, name).restype = C.c_int
     _LIB = lib
     return lib

@@ -24,6 +24,31 @@ from .masks import TreeMask
 VARIANT = int(os.environ.get("SPINF_ATTN_VARIANT", "0"))
 
 
+def _attn_args(q, k, v, out, n, art, end, pos, kv_idx, kv_bits, items, list_ptr, n_items, scale, window, variant, row_of, kv_row0, grp, grp_mode, ktile):
+    """the C ABI's argument block (spinf_attn_args) for these tensors"""
+    hq, d = q.shape[1], q.shape[2]
+    hkv = k.shape[1]
+    a = _lib.AttnArgs()
+    a.q, a.k, a.v, a.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
+    a.q_tok, a.q_head = q.stride(0), q.stride(1)
+    a.k_tok, a.k_head = k.stride(0), k.stride(1)
+    a.v_tok, a.v_head = v.stride(0), v.stride(1)
+    a.o_tok, a.o_head = out.stride(0), out.stride(1)
+    a.n, a.hq, a.hkv, a.d, a.scale, a.window = n, hq, hkv, d, scale, window
+    a.art, a.end, a.pos = art.data_ptr(), end.data_ptr(), pos.data_ptr()
+    a.kv_idx, a.kv_bits, a.items, a.list_ptr = kv_idx.data_ptr(), kv_bits.data_ptr(), items.data_ptr(), list_ptr.data_ptr()
+    a.n_items = n_items
+    a.variant = variant
+    a.ktile = ktile
+    if row_of is not None:
+        a.row_of, a.kv_row0 = row_of.data_ptr(), kv_row0.data_ptr()
+    if grp is not None:
+        if grp.dtype != torch.int32 or grp.numel() < n:
+            raise ValueError("grp must be int32 [n]")
+        a.grp, a.grp_mode = grp.data_ptr(), grp_mode
+    return a
+
+
 @torch.library.custom_op("spinf::tree_attn", mutates_args=())
 def _tree_attn_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, art: torch.Tensor, end: torch.Tensor, pos: torch.Tensor,
                   kv_idx: torch.Tensor, kv_bits: torch.Tensor, items: torch.Tensor, list_ptr: torch.Tensor, n_items: int,
@@ -56,24 +81,7 @@ def _tree_attn_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, art: torch.
         out[n_mapped:].zero_()
     else:
         out = torch.empty((rows, hq, d), dtype=torch.bfloat16, device=q.device)
-    a = _lib.AttnArgs()
-    a.q, a.k, a.v, a.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
-    a.q_tok, a.q_head = q.stride(0), q.stride(1)
-    a.k_tok, a.k_head = k.stride(0), k.stride(1)
-    a.v_tok, a.v_head = v.stride(0), v.stride(1)
-    a.o_tok, a.o_head = out.stride(0), out.stride(1)
-    a.n, a.hq, a.hkv, a.d, a.scale, a.window = n, hq, hkv, d, scale, window
-    a.art, a.end, a.pos = art.data_ptr(), end.data_ptr(), pos.data_ptr()
-    a.kv_idx, a.kv_bits, a.items, a.list_ptr = kv_idx.data_ptr(), kv_bits.data_ptr(), items.data_ptr(), list_ptr.data_ptr()
-    a.n_items = n_items
-    a.variant = variant
-    a.ktile = ktile
-    if row_of is not None:
-        a.row_of, a.kv_row0 = row_of.data_ptr(), kv_row0.data_ptr()
-    if grp is not None:
-        if grp.dtype != torch.int32 or grp.numel() < n:
-            raise ValueError("grp must be int32 [n]")
-        a.grp, a.grp_mode = grp.data_ptr(), grp_mode
+    a = _attn_args(q, k, v, out, n, art, end, pos, kv_idx, kv_bits, items, list_ptr, n_items, scale, window, variant, row_of, kv_row0, grp, grp_mode, ktile)
     lib = _lib.load_library()
     with torch.cuda.device(q.device):
         stream = torch.cuda.current_stream(q.device).cuda_stream
@@ -112,6 +120,32 @@ def tree_attn(q, k, v, mask: TreeMask, scale=None, variant=None, sidx=None):
     return _tree_attn_op(q, k, v, mask.art, mask.end, mask.pos, mask.kv_idx, mask.kv_bits, items, list_ptr, n_items,
                          scale, int(mask.window), variant, row_of, kv_row0, 0 if sidx is None else int(sidx.shape[0]),
                          mask.grp, int(mask.grp_mode), int(mask.plan.ktile))
+
+
+def tree_attn_noalloc(q, k, v, mask: TreeMask, out, scale=None):
+    """tree_attn into a caller-owned ``out`` [n, hq, d] through spinf_tree_attn_fwd_noalloc: the pass that allocates nothing on
+    the device (for callers under graph capture or in loops that must not allocate; no counterpart in the reference).  The
+    mask's schedule must already be on the device (any earlier call with this head geometry uploads it); stream layout only;
+    at most 65,536 work items.  Same bits as tree_attn."""
+    if not q.is_cuda or q.dtype != torch.bfloat16 or k.dtype != torch.bfloat16 or v.dtype != torch.bfloat16:
+        raise ValueError("tree_attn_noalloc takes bf16 device tensors")
+    n, hq, d = q.shape
+    hkv = k.shape[1]
+    if n != mask.n or out.shape != q.shape or out.dtype != torch.bfloat16 or not out.is_contiguous():
+        raise ValueError("out must be a contiguous bf16 tensor of q's shape, and the mask must describe q's rows")
+    mask = mask.for_head_dim(d)
+    per_item = _lib.load_library().spinf_attn_heads_per_item(hq, hkv, d, 0)
+    if per_item <= 0:
+        raise ValueError(f"{hq} query heads do not group over {hkv} key / value heads")
+    items, list_ptr, n_items = mask.schedule(hq // per_item)
+    scale = float(d ** -0.5 if scale is None else scale)
+    a = _attn_args(q, k, v, out, n, mask.art, mask.end, mask.pos, mask.kv_idx, mask.kv_bits, items, list_ptr, n_items, scale, int(mask.window), 0,
+                   None, None, mask.grp, int(mask.grp_mode), int(mask.plan.ktile))
+    lib = _lib.load_library()
+    with torch.cuda.device(q.device):
+        stream = torch.cuda.current_stream(q.device).cuda_stream
+        _lib.check(lib.spinf_tree_attn_fwd_noalloc(C.byref(a), C.c_void_p(stream)), "spinf_tree_attn_fwd_noalloc")
+    return out
 
 
 # K/V capture for extraction, as spinf_serve/models/gemma4.py:66-70: while CAPTURE[device] = {"window", "ranges": [(start, n, key)],

@@ -1,0 +1,75 @@
+"""The attention entry point that allocates nothing (spinf_tree_attn_fwd_noalloc: cursors, counts and redo list in a file-scope
+device array) against spinf_tree_attn_fwd, through the C ABI: the same bits, on two calls in a row, the second on a smaller
+stream; then a tile that needs the exact pass, and the size limit."""
+
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import spinf_serve_amd as sa
+from spinf_serve_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+
+def _pair(cfg, b, dev, seed, window=None, scale_keys=None):
+    q, k, v = synth.qkv(cfg, b, seed=seed, device=dev)
+    if scale_keys is not None:
+        k = k.clone()
+        k[scale_keys[0]:] *= scale_keys[1]
+    mask = sa.TreeMask.build(b.art, b.end, b.pos, window=window, device=dev)
+    want = sa.tree_attn(q, k, v, mask, cfg.scale)          # spinf_tree_attn_fwd (uploads the schedule, allocates its output)
+    torch.cuda.synchronize()
+    got = torch.full_like(want, float("nan"))
+    print(f"no-alloc case {cfg.name} n={b.length} hq={cfg.hq} hkv={cfg.hkv} d={cfg.d} window={window}", flush=True)
+    sa.tree_attn_noalloc(q, k, v, mask, got, cfg.scale)     # spinf_tree_attn_fwd_noalloc into the caller's tensor
+    torch.cuda.synchronize()
+    return want, got
+
+
+def test_noalloc_equals_the_allocating_entry_point_twice_in_a_row(dev):
+    big = synth.attention_config("C2", contents=5)
+    want, got = _pair(big, big.batches[0], dev, seed=1)
+    assert torch.equal(want, got)
+    small = synth.attention_config("C2", contents=2)       # the second call: a smaller stream on the same scratch array
+    want, got = _pair(small, small.batches[0], dev, seed=2)
+    assert torch.equal(want, got)
+    want, got = _pair(small, small.batches[0], dev, seed=3, window=200)
+    assert torch.equal(want, got)
+
+
+def test_noalloc_exact_pass_and_other_geometry(dev):
+    rng = np.random.default_rng(11)
+    trees = [synth._tree(rng, 300, [20, 9]), synth._tree(rng, 90, [7])]
+    cfg = synth.AttnConfig("wide", 4, 2, 128, 128 ** -0.5, 1.0, None, trees)
+    b = synth.pack(trees)[0]
+    total = ctypes.c_int64(0)
+    lib = sa.load_library()
+    assert lib.spinf_attn_exact_items(ctypes.byref(total)) == 0
+    before = total.value
+    want, got = _pair(cfg, b, dev, seed=3, scale_keys=(96, 60.0))   # scores far wider than the fast pass allows: redo list in use
+    assert torch.equal(want, got)
+    assert lib.spinf_attn_exact_items(ctypes.byref(total)) == 0
+    assert total.value >= before + 2, "both entry points hand the wide tiles to the exact pass"
+    c1 = synth.attention_config("C1")
+    want, got = _pair(c1, c1.batches[0], dev, seed=0)
+    assert torch.equal(want, got)
+
+
+def test_noalloc_rejects_more_items_than_its_array_holds(dev):
+    a = sa._lib.AttnArgs()
+    one = torch.zeros(8, dtype=torch.int32, device=dev)
+    t = torch.zeros((128, 2, 64), dtype=torch.bfloat16, device=dev)
+    for f in ("q", "k", "v", "out"):
+        setattr(a, f, t.data_ptr())
+    for f in ("art", "end", "pos", "kv_idx", "kv_bits", "items", "list_ptr"):
+        setattr(a, f, one.data_ptr())
+    a.q_tok = a.k_tok = a.v_tok = a.o_tok = 128
+    a.q_head = a.k_head = a.v_head = a.o_head = 64
+    a.n, a.hq, a.hkv, a.d, a.scale = 128, 2, 2, 64, 0.125
+    a.n_items = 65537
+    lib = sa.load_library()
+    assert lib.spinf_tree_attn_fwd_noalloc(ctypes.byref(a), None) == -1
+    assert b"at most" in lib.spinf_last_error()
