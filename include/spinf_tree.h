@@ -66,6 +66,10 @@ int spinf_tileplan_counts(const spinf_tileplan* plan, int64_t counts[5]);
 int spinf_tileplan_export(const spinf_tileplan* plan, int32_t* qt_ptr, int32_t* kv_idx, uint32_t* kv_bits, int32_t* order);
 /* items [4 * n_qtiles * head_groups], list_ptr [9]: caller-allocated host arrays */
 int spinf_tileplan_schedule(const spinf_tileplan* plan, int32_t head_groups, int32_t* items, int32_t* list_ptr);
+/* The same items dealt out to n_lists workgroups ahead of the launch (a simulation of "the workgroup that is free first takes the
+ * next item of its XCD's list" under a cost model): items [4 * n_qtiles * head_groups] regrouped list by list, list_ptr [n_lists + 1].
+ * For spinf_attn_args.n_lists > 0; n_lists = the number of workgroups to launch, normally the GPU's compute units.  Host arrays. */
+int spinf_tileplan_schedule_static(const spinf_tileplan* plan, int32_t head_groups, int32_t n_lists, int32_t* items, int32_t* list_ptr);
 /* Compact rows (tree_attention with sidx, spinf_serve/models/qwen35/qwen.py:613-622): row_of [n] = row of each stream
  * position in tensors that hold the real tokens only, -1 for a pad position.  kv_row0 [entries] (caller-allocated) receives,
  * per plan entry, the row of the entry's first key if its 64 keys are 64 consecutive rows, else -1.  Host arrays. */
@@ -102,7 +106,11 @@ typedef struct spinf_attn_args {
                           no compact rows) */
     const int32_t* row_of; const int32_t* kv_row0;
     const int32_t* grp; int32_t grp_mode;   /* image groups, as given to spinf_tileplan_build_groups (device copy of grp), or NULL */
-    int32_t ktile;                          /* keys per plan entry: 0 or 64; 32 with d = 512 (and only then) */
+    int32_t ktile;                          /* keys per plan entry: 0 or 64; 32 with d = 512, and with a static schedule */
+    int32_t n_lists;                        /* 0: items / list_ptr are the eight work lists of spinf_tileplan_schedule.  > 0: a static
+                                               schedule (spinf_tileplan_schedule_static) of n_lists item lists, list_ptr [n_lists + 1]; the
+                                               pass then runs as n_lists workgroups of decoupled waves, one list each (head dim 256, an even
+                                               number of query heads per key / value head, variant 0, ktile 32, stream layout, no groups) */
 } spinf_attn_args;
 
 /* query heads one work item covers for this geometry (1 or 2); 0 for an invalid geometry */
@@ -121,6 +129,10 @@ int spinf_tree_attn_fwd_noalloc(const spinf_attn_args* args, void* stream);
  * current device since the library was loaded, i.e. query tiles whose scores ranged too widely for the fast pass.
  * Synchronises the device. */
 int spinf_attn_exact_items(int64_t* total);
+/* Diagnostics (no counterpart in the reference): *total = waves of the static-schedule kernel that gave up a bounded wait on
+ * the current device since the library was loaded.  Always 0 unless the kernel has a bug; the results of such a pass are
+ * invalid.  Synchronises the device. */
+int spinf_attn_ring_aborts(int64_t* total);
 
 /* ------------------------------------------------------------------------------------------------ Gated DeltaNet
  * Replaces gdn.recurrent / gdn.chunked (spinf_serve/models/qwen35/gdn.py:197-235 and :109-133): the gated delta rule

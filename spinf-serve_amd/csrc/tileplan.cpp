@@ -304,6 +304,65 @@ extern "C" int spinf_tileplan_schedule(const spinf_tileplan* p, int32_t head_gro
     return SPINF_OK;
 }
 
+// Static schedule for the kernel with decoupled waves: the items of spinf_tileplan_schedule (same order, same eight lists, one per
+// XCD), dealt out to n_lists workgroups by simulating "the workgroup that is free first takes the next item of its XCD's list"
+// with a cost model, so that a workgroup's items are known before the launch.  Workgroup b serves list b % 8.  The model is a
+// fit to per-workgroup cycle counts of that kernel on the 24-content pass (residual 1.2 %): a workgroup moves through its key
+// tiles at about the same pace whatever the number of 32 x 32 blocks its waves compute in them, so an item costs its number of
+// key tiles, 0.3 per block that needs the per-element mask (of the busier SIMD pair: SIMDs 0 and 3 run the row groups 0 and 3 of
+// a query tile, SIMDs 1 and 2 the row groups 1 and 2) and 3.2 on top (queries, output rows).
+extern "C" int spinf_tileplan_schedule_static(const spinf_tileplan* p, int32_t head_groups, int32_t n_lists, int32_t* items, int32_t* list_ptr) {
+    if (!p || !list_ptr) return spinf_fail(SPINF_E_ARG, "tileplan_schedule_static: null argument");
+    if (n_lists <= 0 || n_lists > 65536) return spinf_fail(SPINF_E_ARG, "tileplan_schedule_static: %d lists out of range", n_lists);
+    const int64_t nqt = (int64_t)p->order.size();
+    try {
+        std::vector<int32_t> base((size_t)std::max<int64_t>(1, nqt * head_groups) * 4);
+        int32_t lp[9];
+        if (int rc = spinf_tileplan_schedule(p, head_groups, base.data(), lp)) return rc;
+        const int nsub = p->ktile / SPINF_SUB;
+        std::vector<float> cost(nqt, 0.f);
+        for (int64_t t = 0; t < nqt; t++) {
+            float tiles = 0.f, ma = 0.f, mb = 0.f;
+            for (int32_t e = p->qt_ptr[t]; e < p->qt_ptr[t + 1]; e++) {
+                const uint32_t bits = p->kv_bits[e];
+                for (int sb = 0; sb < nsub; sb++) {
+                    bool any = false;
+                    for (int w = 0; w < 4; w++) {
+                        if (!((bits >> (2 * w + sb)) & 1u)) continue;
+                        any = true;
+                        if ((bits >> (8 + 2 * w + sb)) & 1u) (w == 0 || w == 3 ? ma : mb) += 1.f;
+                    }
+                    if (any) tiles += 1.f;
+                }
+            }
+            cost[t] = 3.2f + tiles + 0.3f * std::max(ma, mb);
+        }
+        const int nl = std::min<int32_t>(8, n_lists);
+        std::vector<std::vector<int32_t>> mine((size_t)n_lists);
+        std::vector<float> load((size_t)n_lists, 0.f);
+        for (int l = 0; l < 8; l++)
+            for (int64_t i = lp[l]; i < lp[l + 1]; i++) {
+                int best = -1;
+                for (int w = l % nl; w < n_lists; w += nl)
+                    if (best < 0 || load[w] < load[best]) best = w;
+                mine[best].push_back((int32_t)i);
+                load[best] += cost[base[4 * i]];
+            }
+        int64_t k = 0;
+        for (int w = 0; w < n_lists; w++) {
+            list_ptr[w] = (int32_t)k;
+            for (int32_t i : mine[w]) {
+                std::memcpy(items + 4 * k, base.data() + 4 * (int64_t)i, 4 * sizeof(int32_t));
+                k++;
+            }
+        }
+        list_ptr[n_lists] = (int32_t)k;
+    } catch (const std::bad_alloc&) {
+        return spinf_fail(SPINF_E_NOMEM, "tileplan_schedule_static: out of memory");
+    }
+    return SPINF_OK;
+}
+
 extern "C" int spinf_tileplan_row0(const spinf_tileplan* p, const int32_t* row_of, int32_t* kv_row0) {
     if (!p || !row_of) return spinf_fail(SPINF_E_ARG, "tileplan_row0: null argument");
     if (!kv_row0 && !p->kv_idx.empty()) return spinf_fail(SPINF_E_ARG, "tileplan_row0: null kv_row0");

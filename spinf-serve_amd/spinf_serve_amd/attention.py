@@ -22,9 +22,21 @@ from .masks import TreeMask
 # kernel tuning variant handed to the library (0 = its default choice, 1 = one head per work item, 2 = eight waves per
 # workgroup where two heads share an item); results do not depend on it
 VARIANT = int(os.environ.get("SPINF_ATTN_VARIANT", "0"))
+# the kernel with decoupled waves over a static schedule, where the library has one for the geometry (0: the lockstep kernels only)
+RING = int(os.environ.get("SPINF_ATTN_RING", "1"))
 
 
-def _attn_args(q, k, v, out, n, art, end, pos, kv_idx, kv_bits, items, list_ptr, n_items, scale, window, variant, row_of, kv_row0, grp, grp_mode, ktile):
+def _ring_lists(q, hq, hkv, d, variant, sidx, mask) -> int:
+    """workgroups of the static schedule if this call goes to the kernel with decoupled waves, else 0"""
+    if not RING or variant != 0 or d != 256 or (hq // hkv) % 2 or sidx is not None or mask.grp is not None:
+        return 0
+    from .masks import _static_lists
+
+    return _static_lists(q.device)
+
+
+
+def _attn_args(q, k, v, out, n, art, end, pos, kv_idx, kv_bits, items, list_ptr, n_items, scale, window, variant, row_of, kv_row0, grp, grp_mode, ktile, n_lists=0):
     """the C ABI's argument block (spinf_attn_args) for these tensors"""
     hq, d = q.shape[1], q.shape[2]
     hkv = k.shape[1]
@@ -40,6 +52,7 @@ def _attn_args(q, k, v, out, n, art, end, pos, kv_idx, kv_bits, items, list_ptr,
     a.n_items = n_items
     a.variant = variant
     a.ktile = ktile
+    a.n_lists = n_lists
     if row_of is not None:
         a.row_of, a.kv_row0 = row_of.data_ptr(), kv_row0.data_ptr()
     if grp is not None:
@@ -53,7 +66,7 @@ def _attn_args(q, k, v, out, n, art, end, pos, kv_idx, kv_bits, items, list_ptr,
 def _tree_attn_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, art: torch.Tensor, end: torch.Tensor, pos: torch.Tensor,
                   kv_idx: torch.Tensor, kv_bits: torch.Tensor, items: torch.Tensor, list_ptr: torch.Tensor, n_items: int,
                   scale: float, window: int, variant: int, row_of: Optional[torch.Tensor], kv_row0: Optional[torch.Tensor],
-                  n_mapped: int, grp: Optional[torch.Tensor], grp_mode: int, ktile: int) -> torch.Tensor:
+                  n_mapped: int, grp: Optional[torch.Tensor], grp_mode: int, ktile: int, n_lists: int) -> torch.Tensor:
     """q [rows, hq, d], k / v [rows, hkv, d] (any token / head strides, d contiguous) -> out [rows, hq, d] contiguous, bf16.
     rows = the stream length, or with row_of / kv_row0 (compact rows) any number of rows: the kernel maps stream positions to
     rows through row_of; rows 0 .. n_mapped-1 are the rows row_of names (each written by the kernel), later rows come back zero."""
@@ -81,7 +94,7 @@ def _tree_attn_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, art: torch.
         out[n_mapped:].zero_()
     else:
         out = torch.empty((rows, hq, d), dtype=torch.bfloat16, device=q.device)
-    a = _attn_args(q, k, v, out, n, art, end, pos, kv_idx, kv_bits, items, list_ptr, n_items, scale, window, variant, row_of, kv_row0, grp, grp_mode, ktile)
+    a = _attn_args(q, k, v, out, n, art, end, pos, kv_idx, kv_bits, items, list_ptr, n_items, scale, window, variant, row_of, kv_row0, grp, grp_mode, ktile, n_lists)
     lib = _lib.load_library()
     with torch.cuda.device(q.device):
         stream = torch.cuda.current_stream(q.device).cuda_stream
@@ -90,7 +103,7 @@ def _tree_attn_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, art: torch.
 
 
 @_tree_attn_op.register_fake
-def _(q, k, v, art, end, pos, kv_idx, kv_bits, items, list_ptr, n_items, scale, window, variant, row_of, kv_row0, n_mapped, grp, grp_mode, ktile):
+def _(q, k, v, art, end, pos, kv_idx, kv_bits, items, list_ptr, n_items, scale, window, variant, row_of, kv_row0, n_mapped, grp, grp_mode, ktile, n_lists):
     return torch.empty(q.shape, dtype=torch.bfloat16, device=q.device)
 
 
@@ -111,15 +124,18 @@ def tree_attn(q, k, v, mask: TreeMask, scale=None, variant=None, sidx=None):
     if sidx is not None and mask.grp is not None:
         raise ValueError("image groups go with the stream layout (no sidx)")
     hq, hkv, d = q.shape[1], k.shape[1], q.shape[2]
-    mask = mask.for_head_dim(d)
+    if hkv <= 0 or hq % hkv:
+        raise ValueError(f"{hq} query heads do not group over {hkv} key / value heads")
+    n_lists = _ring_lists(q, hq, hkv, d, variant, sidx, mask)
+    mask = mask.for_head_dim(d, ring=n_lists > 0)
     per_item = _lib.load_library().spinf_attn_heads_per_item(hq, hkv, d, variant)
     if per_item <= 0:
         raise ValueError(f"{hq} query heads do not group over {hkv} key / value heads")
-    items, list_ptr, n_items = mask.schedule(hq // per_item)
+    items, list_ptr, n_items = mask.schedule(hq // per_item, n_lists)
     row_of, kv_row0 = mask.rows(sidx) if sidx is not None else (None, None)
     return _tree_attn_op(q, k, v, mask.art, mask.end, mask.pos, mask.kv_idx, mask.kv_bits, items, list_ptr, n_items,
                          scale, int(mask.window), variant, row_of, kv_row0, 0 if sidx is None else int(sidx.shape[0]),
-                         mask.grp, int(mask.grp_mode), int(mask.plan.ktile))
+                         mask.grp, int(mask.grp_mode), int(mask.plan.ktile), n_lists)
 
 
 def tree_attn_noalloc(q, k, v, mask: TreeMask, out, scale=None):
@@ -133,14 +149,17 @@ def tree_attn_noalloc(q, k, v, mask: TreeMask, out, scale=None):
     hkv = k.shape[1]
     if n != mask.n or out.shape != q.shape or out.dtype != torch.bfloat16 or not out.is_contiguous():
         raise ValueError("out must be a contiguous bf16 tensor of q's shape, and the mask must describe q's rows")
-    mask = mask.for_head_dim(d)
+    if hkv <= 0 or hq % hkv:
+        raise ValueError(f"{hq} query heads do not group over {hkv} key / value heads")
+    n_lists = _ring_lists(q, hq, hkv, d, 0, None, mask)
+    mask = mask.for_head_dim(d, ring=n_lists > 0)
     per_item = _lib.load_library().spinf_attn_heads_per_item(hq, hkv, d, 0)
     if per_item <= 0:
         raise ValueError(f"{hq} query heads do not group over {hkv} key / value heads")
-    items, list_ptr, n_items = mask.schedule(hq // per_item)
+    items, list_ptr, n_items = mask.schedule(hq // per_item, n_lists)
     scale = float(d ** -0.5 if scale is None else scale)
     a = _attn_args(q, k, v, out, n, mask.art, mask.end, mask.pos, mask.kv_idx, mask.kv_bits, items, list_ptr, n_items, scale, int(mask.window), 0,
-                   None, None, mask.grp, int(mask.grp_mode), int(mask.plan.ktile))
+                   None, None, mask.grp, int(mask.grp_mode), int(mask.plan.ktile), n_lists)
     lib = _lib.load_library()
     with torch.cuda.device(q.device):
         stream = torch.cuda.current_stream(q.device).cuda_stream

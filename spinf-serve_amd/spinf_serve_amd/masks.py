@@ -84,6 +84,25 @@ class TilePlan:
             got = self._schedules[head_groups] = (items[: self.n_qtiles * head_groups], list_ptr)
         return got
 
+    def schedule_static(self, head_groups: int, n_lists: int):
+        """-> (items [n_qtiles * head_groups, 4] int32, list_ptr [n_lists + 1] int32): the items dealt out to n_lists workgroups
+        ahead of the launch (the kernel with decoupled waves)"""
+        got = self._schedules.get((head_groups, n_lists))
+        if got is None:
+            items = np.zeros((max(self.n_qtiles * head_groups, 1), 4), np.int32)
+            list_ptr = np.zeros(n_lists + 1, np.int32)
+            _lib.check(_lib.load_library().spinf_tileplan_schedule_static(self._handle, head_groups, n_lists, items.ctypes.data, list_ptr.ctypes.data),
+                       "tileplan_schedule_static")
+            got = self._schedules[(head_groups, n_lists)] = (items[: self.n_qtiles * head_groups], list_ptr)
+        return got
+
+
+def _static_lists(device) -> int:
+    """workgroups of a static schedule on this device: one per compute unit"""
+    import torch
+
+    return int(torch.cuda.get_device_properties(device).multi_processor_count)
+
 
 def _upload(a, dtype, device):
     import torch
@@ -115,10 +134,10 @@ class TreeMask:
         self._sched = {}
         self._rows = None
 
-    def for_head_dim(self, d: int) -> "TreeMask":
-        """the mask with the plan granularity the kernel of this head dim takes: 32-key entries at 512, 64-key ones otherwise
-        (the second plan is compiled on first use and shares the device metadata)"""
-        ktile = 32 if d == 512 else 64
+    def for_head_dim(self, d: int, ring: bool = False) -> "TreeMask":
+        """the mask with the plan granularity the kernel takes: 32-key entries at head dim 512 and for the kernel with decoupled
+        waves (ring), 64-key ones otherwise (the second plan is compiled on first use and shares the device metadata)"""
+        ktile = 32 if d == 512 or ring else 64
         if ktile == self.plan.ktile:
             return self
         if self._other is None:
@@ -150,14 +169,15 @@ class TreeMask:
         self._rows = (sidx, row_of[:n].contiguous(), kv_row0)
         return self._rows[1], self._rows[2]
 
-    def schedule(self, head_groups: int):
-        """device copy of the work lists for this many head groups (built on first use, then kept)"""
-        got = self._sched.get(head_groups)
+    def schedule(self, head_groups: int, n_lists: int = 0):
+        """device copy of the work lists for this many head groups (built on first use, then kept); n_lists > 0: the static
+        schedule for that many workgroups"""
+        got = self._sched.get((head_groups, n_lists))
         if got is None:
-            items, list_ptr = self.plan.schedule(head_groups)
+            items, list_ptr = self.plan.schedule_static(head_groups, n_lists) if n_lists else self.plan.schedule(head_groups)
             if not len(items):
                 items = np.zeros((1, 4), np.int32)
-            got = self._sched[head_groups] = (_upload(items, np.int32, self.device), _upload(list_ptr, np.int32, self.device), self.plan.n_qtiles * head_groups)
+            got = self._sched[(head_groups, n_lists)] = (_upload(items, np.int32, self.device), _upload(list_ptr, np.int32, self.device), self.plan.n_qtiles * head_groups)
         return got
 
     @classmethod
