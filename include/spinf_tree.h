@@ -107,10 +107,11 @@ typedef struct spinf_attn_args {
     const int32_t* row_of; const int32_t* kv_row0;
     const int32_t* grp; int32_t grp_mode;   /* image groups, as given to spinf_tileplan_build_groups (device copy of grp), or NULL */
     int32_t ktile;                          /* keys per plan entry: 0 or 64; 32 with d = 512, and with a static schedule */
-    int32_t n_lists;                        /* 0: items / list_ptr are the eight work lists of spinf_tileplan_schedule.  > 0: a static
-                                               schedule (spinf_tileplan_schedule_static) of n_lists item lists, list_ptr [n_lists + 1]; the
-                                               pass then runs as n_lists workgroups of decoupled waves, one list each (head dim 256, an even
-                                               number of query heads per key / value head, variant 0, ktile 32, stream layout, no groups) */
+    int32_t n_lists;                        /* 0: items / list_ptr are the eight work lists of spinf_tileplan_schedule, shared by all
+                                               workgroups.  > 0: a static schedule (spinf_tileplan_schedule_static) of n_lists item lists,
+                                               list_ptr [n_lists + 1]; the pass runs as n_lists workgroups, each through its own list.  With
+                                               ktile 32 (and d = 256, an even number of query heads per key / value head, variant 0, stream
+                                               layout, no groups) that is the kernel with decoupled waves */
 } spinf_attn_args;
 
 /* query heads one work item covers for this geometry (1 or 2); 0 for an invalid geometry */

@@ -27,6 +27,7 @@ struct AttnParams {
     // kv_row0[entry] = row of the entry's first key if its 64 keys are 64 consecutive rows, else -1
     const int* row_of; const int* kv_row0;
     const int* grp;       // image groups (GRP kernels): -1 none; the tokens of a group see each other both ways
+    bool static_lists;    // list_ptr delimits one item list per workgroup (a static schedule) instead of the eight shared lists
     bool clear_first;     // host side only: zero the cursors and counts in front of the pass (the entry point that allocates nothing)
 };
 

@@ -335,7 +335,8 @@ extern "C" int spinf_tileplan_schedule_static(const spinf_tileplan* p, int32_t h
                     if (any) tiles += 1.f;
                 }
             }
-            cost[t] = 3.2f + tiles + 0.3f * std::max(ma, mb);
+            // 64-key entries: the lockstep kernels, whose items cost what spinf_tileplan_schedule weighs them with
+            cost[t] = p->ktile == SPINF_SUB ? 3.2f + tiles + 0.3f * std::max(ma, mb) : (float)(p->weight[t] + 15);
         }
         const int nl = std::min<int32_t>(8, n_lists);
         std::vector<std::vector<int32_t>> mine((size_t)n_lists);

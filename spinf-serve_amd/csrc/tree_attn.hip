@@ -292,9 +292,14 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
     unsigned xcc;
     asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
     int my_list = (int)(xcc & 7u), lists_done = 0;    // thread 0 only
+    int own_next = p.static_lists ? p.list_ptr[blockIdx.x] : 0;   // static schedule: this workgroup's own list, in order, nobody else's
     auto grab = [&](const int slot) __attribute__((always_inline)) {   // thread 0: next item index into s_next[slot], -1 when all lists are empty
         if (threadIdx.x == 0) {
             int idx = -1;
+            if (p.static_lists) {
+                if (own_next < p.list_ptr[blockIdx.x + 1]) idx = own_next++;
+                lists_done = NLIST;
+            }
             while (lists_done < NLIST) {
                 const int lo = p.list_ptr[my_list], hi = p.list_ptr[my_list + 1];
                 const int j = lo + atomicAdd(&p.counters[my_list], 1);
@@ -815,12 +820,12 @@ static int attn_fwd(const spinf_attn_args* a, void* stream, bool no_alloc) {
     pick_kernel(a->hq, a->hkv, a->d, a->variant, &rt, &nhw);
     if ((a->row_of != nullptr) != (a->kv_row0 != nullptr)) return spinf_fail(SPINF_E_ARG, "tree_attn: row_of and kv_row0 come together");
     if (a->row_of && rt != 1) return spinf_fail(SPINF_E_ARG, "tree_attn: variant %d does not take compact rows", a->variant);
-    const bool ring = a->n_lists > 0;   // static schedule: the ring kernel
+    if (a->n_lists < 0 || a->n_lists > 65536) return spinf_fail(SPINF_E_ARG, "tree_attn: %d item lists, at most 65,536", a->n_lists);
+    const bool ring = a->n_lists > 0 && a->ktile == 32 && a->d != 512;   // static schedule over 32-key entries: the ring kernel
     if (ring) {
-        if (a->d != 256 || nhw != 2 || rt != 1 || a->row_of || a->grp || a->ktile != 32)
-            return spinf_fail(SPINF_E_ARG, "tree_attn: a static schedule (n_lists > 0) goes with head dim 256, an even number of query heads per key / value head, "
-                                           "variant 0, plan entries of 32 keys, the stream layout and no image groups");
-        if (a->n_lists > 65536) return spinf_fail(SPINF_E_ARG, "tree_attn: %d item lists, at most 65,536", a->n_lists);
+        if (a->d != 256 || nhw != 2 || rt != 1 || a->row_of || a->grp)
+            return spinf_fail(SPINF_E_ARG, "tree_attn: a static schedule over 32-key entries goes with head dim 256, an even number of query heads per key / value head, "
+                                           "variant 0, the stream layout and no image groups");
     } else if ((a->d == 512) != (a->ktile == 32) || (a->ktile != 0 && a->ktile != 32 && a->ktile != 64))
         return spinf_fail(SPINF_E_ARG, "tree_attn: plan entries of %d keys with head dim %d (32 goes with 512, 64 with the others)", a->ktile ? a->ktile : 64, a->d);
     if (a->grp && (a->grp_mode != 1 && a->grp_mode != 2)) return spinf_fail(SPINF_E_ARG, "tree_attn: group mode %d not in {1, 2}", a->grp_mode);
@@ -851,6 +856,7 @@ static int attn_fwd(const spinf_attn_args* a, void* stream, bool no_alloc) {
     }
     AttnParams p;
     p.clear_first = no_alloc;
+    p.static_lists = a->n_lists > 0;
     p.q = (const __bf16*)a->q; p.k = (const __bf16*)a->k; p.v = (const __bf16*)a->v; p.o = (__bf16*)a->out;
     p.q_tok = a->q_tok; p.q_head = a->q_head; p.k_tok = a->k_tok; p.k_head = a->k_head;
     p.v_tok = a->v_tok; p.v_head = a->v_head; p.o_tok = a->o_tok; p.o_head = a->o_head;
@@ -864,7 +870,7 @@ static int attn_fwd(const spinf_attn_args* a, void* stream, bool no_alloc) {
     p.grp = a->grp;
     p.counters = counters;
     p.redo = counters + 64;
-    const int blocks = (int)(a->n_items < cus ? a->n_items : cus);
+    const int blocks = a->n_lists > 0 ? a->n_lists : (int)(a->n_items < cus ? a->n_items : cus);
     const bool win = p.window > 0;
     hipStream_t s = (hipStream_t)stream;
     if (ring) return launch_ring(p, a->d, win, a->n_lists, s);

@@ -415,7 +415,9 @@ __global__ __launch_bounds__(512) void tree_attn_ring_kernel(const AttnParams p)
         __bf16* ob = p.o + (long)h * p.o_head;
         char* const stage = stage_all + L.w * 32 * SROW;
         asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");   // the last MFMAs' results -> v_accvgpr_read
-        auto one = [&](auto dt_c) __attribute__((always_inline)) {
+        // tile dt is read back from the slice while tile dt + 1 is converted and written to it (the LDS takes a wave's requests
+        // in order, so the write behind the read is safe), and stored after that: no wait between a write and its read-back
+        auto put = [&](auto dt_c) __attribute__((always_inline)) {
             constexpr int dt = decltype(dt_c)::value;
             float r16[16];
             acc_read<dt>(r16);
@@ -426,17 +428,27 @@ __global__ __launch_bounds__(512) void tree_attn_ring_kernel(const AttnParams p)
                 for (int jj = 0; jj < 4; jj++) r[jj] = (__bf16)(r16[4 * i4 + jj] * inv);
                 *(bf16x4*)(stage + m * SROW + (8 * i4 + 4 * g) * 2) = r;
             }
+        };
+        auto round = [&](auto dt_c) __attribute__((always_inline)) {
+            constexpr int dt = decltype(dt_c)::value;
+            bf16x8 val[2];
+#pragma unroll
+            for (int jj = 0; jj < 2; jj++) {
+                const int c = jj * 64 + lane;
+                val[jj] = *(const bf16x8*)(stage + (c >> 2) * SROW + (c & 3) * 16);
+            }
+            if constexpr (dt + 1 < NDT) put(std::integral_constant<int, dt + 1>{});
 #pragma unroll
             for (int jj = 0; jj < 2; jj++) {
                 const int c = jj * 64 + lane, row = c >> 2, col = c & 3;
-                const bf16x8 val = *(const bf16x8*)(stage + row * SROW + col * 16);
-                if (tok0 + row < p.n) *(bf16x8*)(ob + (long)(tok0 + row) * p.o_tok + 32 * dt + col * 8) = val;
+                if (tok0 + row < p.n) *(bf16x8*)(ob + (long)(tok0 + row) * p.o_tok + 32 * dt + col * 8) = val[jj];
             }
         };
-        one(std::integral_constant<int, 0>{});
-        one(std::integral_constant<int, 1>{});
-        if constexpr (NDT > 2) { one(std::integral_constant<int, 2>{}); one(std::integral_constant<int, 3>{}); }
-        if constexpr (NDT > 4) { one(std::integral_constant<int, 4>{}); one(std::integral_constant<int, 5>{}); one(std::integral_constant<int, 6>{}); one(std::integral_constant<int, 7>{}); }
+        put(std::integral_constant<int, 0>{});
+        round(std::integral_constant<int, 0>{});
+        round(std::integral_constant<int, 1>{});
+        if constexpr (NDT > 2) { round(std::integral_constant<int, 2>{}); round(std::integral_constant<int, 3>{}); }
+        if constexpr (NDT > 4) { round(std::integral_constant<int, 4>{}); round(std::integral_constant<int, 5>{}); round(std::integral_constant<int, 6>{}); round(std::integral_constant<int, 7>{}); }
     };
 
     {   // the first item's queries
@@ -589,19 +601,22 @@ __global__ __launch_bounds__(512) void tree_attn_ring_kernel(const AttnParams p)
             j++;
         } while (!last);
         if (dead) break;
-        // this wave's rows of the item are complete: out they go (or the item goes to the exact pass), then the next item's queries
-        if (__builtin_amdgcn_ballot_w64(viol) != 0) {   // scores ranged too widely somewhere in these 32 rows
-            if (fresh_lane_id() == 0) {
-                const int was = __hip_atomic_fetch_max(&sy_redo[iseq & 15], iseq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                if (was < iseq) p.redo[atomicAdd(&p.counters[NLIST + 1], 1)] = d.w;
-            }
-        } else {
-            store_rows(d.z);
-        }
+        // this wave's rows of the item are complete: the next item's queries are requested (their registers are free), then the rows
+        // go out (or the item goes to the exact pass)
+        const bool hand_over = __builtin_amdgcn_ballot_w64(viol) != 0;   // scores ranged too widely somewhere in these 32 rows
+        const int tz_done = d.z, item_done = d.w;
         if (j < ntiles) {
             need_desc(j);
             if (dead) break;
             load_q(read_desc(j).z);
+        }
+        if (hand_over) {
+            if (fresh_lane_id() == 0) {
+                const int was = __hip_atomic_fetch_max(&sy_redo[iseq & 15], iseq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                if (was < iseq) p.redo[atomicAdd(&p.counters[NLIST + 1], 1)] = item_done;
+            }
+        } else {
+            store_rows(tz_done);
         }
     }
     if (dead && fresh_lane_id() == 0) atomicAdd(&p.counters[NLIST + 4], 1);

@@ -26,13 +26,18 @@ VARIANT = int(os.environ.get("SPINF_ATTN_VARIANT", "0"))
 RING = int(os.environ.get("SPINF_ATTN_RING", "1"))
 
 
-def _ring_lists(q, hq, hkv, d, variant, sidx, mask) -> int:
-    """workgroups of the static schedule if this call goes to the kernel with decoupled waves, else 0"""
-    if not RING or variant != 0 or d != 256 or (hq // hkv) % 2 or sidx is not None or mask.grp is not None:
-        return 0
+# a static schedule (items dealt out to the workgroups on the host) also for the lockstep kernels
+STATIC = int(os.environ.get("SPINF_ATTN_STATIC", "0"))
+
+
+def _ring_lists(q, hq, hkv, d, variant, sidx, mask):
+    """-> (workgroups of the static schedule or 0, whether the call goes to the kernel with decoupled waves)"""
     from .masks import _static_lists
 
-    return _static_lists(q.device)
+    ring = bool(RING) and variant == 0 and d == 256 and (hq // hkv) % 2 == 0 and sidx is None and mask.grp is None
+    if ring or (STATIC and d != 512):
+        return _static_lists(q.device), ring
+    return 0, False
 
 
 
@@ -126,8 +131,8 @@ def tree_attn(q, k, v, mask: TreeMask, scale=None, variant=None, sidx=None):
     hq, hkv, d = q.shape[1], k.shape[1], q.shape[2]
     if hkv <= 0 or hq % hkv:
         raise ValueError(f"{hq} query heads do not group over {hkv} key / value heads")
-    n_lists = _ring_lists(q, hq, hkv, d, variant, sidx, mask)
-    mask = mask.for_head_dim(d, ring=n_lists > 0)
+    n_lists, ring = _ring_lists(q, hq, hkv, d, variant, sidx, mask)
+    mask = mask.for_head_dim(d, ring=ring)
     per_item = _lib.load_library().spinf_attn_heads_per_item(hq, hkv, d, variant)
     if per_item <= 0:
         raise ValueError(f"{hq} query heads do not group over {hkv} key / value heads")
@@ -151,8 +156,8 @@ def tree_attn_noalloc(q, k, v, mask: TreeMask, out, scale=None):
         raise ValueError("out must be a contiguous bf16 tensor of q's shape, and the mask must describe q's rows")
     if hkv <= 0 or hq % hkv:
         raise ValueError(f"{hq} query heads do not group over {hkv} key / value heads")
-    n_lists = _ring_lists(q, hq, hkv, d, 0, None, mask)
-    mask = mask.for_head_dim(d, ring=n_lists > 0)
+    n_lists, ring = _ring_lists(q, hq, hkv, d, 0, None, mask)
+    mask = mask.for_head_dim(d, ring=ring)
     per_item = _lib.load_library().spinf_attn_heads_per_item(hq, hkv, d, 0)
     if per_item <= 0:
         raise ValueError(f"{hq} query heads do not group over {hkv} key / value heads")
