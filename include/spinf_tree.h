@@ -160,6 +160,34 @@ typedef struct spinf_gdn_args {
 
 int spinf_gdn_fwd(const spinf_gdn_args* args, void* stream);
 
+/* ------------------------------------------------------------------------------------------------ Gated DeltaNet plan
+ * Replaces tree_plan (spinf_serve/models/qwen35/qwen.py:158-276): from the path predecessors of a packed stream, the segments
+ * (maximal stream-consecutive runs one scan takes in one go: a segment begins where the predecessor is missing, is not the stream
+ * token right before, or has several children, qwen.py:185-187), their levels, and per level the calls spinf_gdn_fwd runs.
+ *
+ *   prev [n] int64: the token before each token on its path, -1 none; real [n] uint8: not a pad.  Host arrays.
+ *   path 0 ("indexed", qwen.py:220-241): a level's segments longer than short_len go to the chunked entry point, in calls of at most
+ *   call_tokens tokens (a call holds at least one segment), the others to the recurrent entry point in one call; segments that are
+ *   continued from (or that hold a token of `keep`) leave their state in a slot of their level.  path 1 ("levels"): per level the
+ *   keeping segments first, then the others, below the roots in calls of at most max_init segments.
+ *   rows >= 0: the tensors hold the real tokens first (compact rows, qwen.py:179-184,266-275): row indices are compact rows and
+ *   `rows` stands for "no row"; rows < 0: rows are stream positions and n stands for "no row".
+ * Export (host arrays, caller-allocated from spinf_gdn_plan_counts: [0] segments, [1] levels, [2] calls, [3] call segments in all,
+ * [4] rows in all calls, [5] conv rows):
+ *   level_ptr [levels + 1] -> calls; call_kind [calls] (1 chunked, 0 recurrent); call_keep [calls] (some segment leaves its state);
+ *   call_seg_ptr / call_row_ptr [calls + 1] -> seg_len, h0_idx, ht_idx [call segments] (length; slot of the start state in the level
+ *   above, -1 zero state; slot of the final state in this level, -1 not kept) and idx [rows] (the segments' rows back to back);
+ *   n_keep [levels] slots per level; conv [conv rows, 4]: rows of the three path predecessors (oldest first) and of the token itself
+ *   (qwen.py:260-265); seg_of_row [conv rows] (-1 pad); seg_level, seg_slot [segments]. */
+typedef struct spinf_gdn_plan spinf_gdn_plan;
+int spinf_gdn_plan_build(const int64_t* prev, const uint8_t* real, int64_t n, int32_t path, int32_t short_len, int64_t call_tokens,
+                         int32_t max_init, int64_t rows, const int64_t* keep, int64_t n_keep, spinf_gdn_plan** out);
+int spinf_gdn_plan_counts(const spinf_gdn_plan* plan, int64_t counts[6]);
+int spinf_gdn_plan_export(const spinf_gdn_plan* plan, int64_t* level_ptr, int32_t* call_kind, int32_t* call_keep, int64_t* call_seg_ptr,
+                          int64_t* call_row_ptr, int64_t* seg_len, int64_t* h0_idx, int64_t* ht_idx, int64_t* idx, int64_t* n_keep,
+                          int64_t* conv, int64_t* seg_of_row, int64_t* seg_level, int64_t* seg_slot);
+void spinf_gdn_plan_free(spinf_gdn_plan* plan);
+
 /* ------------------------------------------------------------------------------------------------ Gated DeltaNet layer, around the scan
  * spinf_gdn_prologue replaces the element-wise work of GatedDeltaNet.forward before the scan
  * (spinf_serve/models/qwen35/qwen.py:657-668): the 4-tap convolution along each token's path (conv [T, 4]: rows of the

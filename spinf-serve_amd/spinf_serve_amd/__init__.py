@@ -1,6 +1,6 @@
 """MI355X-native tree-mask packed-prefill attention and Gated DeltaNet scan behind the reference's call boundary.
 
-  packer      Tree / GroupedTree / Packer / Batch: the stream metadata producer (spinf_serve/packer.py)
+  layout      TokenTree / Batch / pack_stream: the stream layout of packed token trees (spinf_serve/packer.py:352-423)
   masks       TreeMask, block_masks: the mask side of the boundary (spinf_serve/scorer.py:163-238)
   attention   tree_attn custom op, tree_flex_forward, tree_attention (gemma4.py:98-119, qwen.py:604-623)
   gdn         recurrent, chunked (spinf_serve/models/qwen35/gdn.py)
@@ -13,7 +13,7 @@ compute entry points without the built library raises.
 """
 
 from ._lib import load_library, library_path  # noqa: F401
-from .packer import BLOCK, Batch, GroupedTree, Owner, Packer, ReadPlan, Tree, build_grouped_tree, build_tree, split_grouped_trees, split_trees, trie_branches  # noqa: F401
+from .layout import BLOCK, Batch, TokenTree, pack_stream, pack_streams  # noqa: F401
 from .masks import TreeMask, TilePlan, block_masks  # noqa: F401
 from .attention import CAPTURE, register_tree_attention, tree_attention, tree_attn, tree_attn_noalloc, tree_flex_forward  # noqa: F401
 from .gdn import chunked, recurrent  # noqa: F401

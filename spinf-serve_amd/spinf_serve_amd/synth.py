@@ -1,7 +1,7 @@
 """Seeded synthetic workloads: the benchmark configurations of the tree-mask attention path and of the Gated DeltaNet scan.
 
-Each attention config is a set of contents (trunk + question branches, optionally two-level) packed by the package's own
-Packer with aligned jobs (every content starts on a 128-token boundary, spinf_serve/packer.py:421-422), plus the head
+Each attention config is a set of contents (trunk + question branches, optionally two-level) laid out by the package's own
+layout module with aligned jobs (every content starts on a 128-token boundary, spinf_serve/packer.py:421-422), plus the head
 geometry and value distribution.  Everything derives from numpy.random.default_rng(seed).
 
   C1     2 x (64 + 4 x 8), 4/2 heads, d 64, scale d^-0.5, N(0,1)           (the CPU plumbing case)
@@ -18,7 +18,7 @@ from dataclasses import dataclass, field
 
 import numpy as np
 
-from .packer import BLOCK, GroupedTree, Packer
+from .layout import BLOCK, TokenTree, pack_stream, pack_streams
 
 
 @dataclass
@@ -56,20 +56,14 @@ class AttnConfig:
 
 def _tree(rng, trunk, branch_lens, parents=None):
     ids = lambda n: rng.integers(5, 32000, int(n)).tolist()  # noqa: E731
-    return GroupedTree(ids(trunk), [ids(n) for n in branch_lens], [], [], parents=list(parents) if parents is not None else [])
+    return TokenTree(ids(trunk), [ids(n) for n in branch_lens], list(parents) if parents is not None else [])
 
 
 def pack(trees, budget=None, align=True):
     """-> batches.  budget None: one stream in the given order; else first-fit-decreasing streams of <= budget tokens"""
     if budget is None:
-        total = sum((t.n_tokens + BLOCK - 1) // BLOCK * BLOCK if align else t.n_tokens for t in trees)
-        pk = Packer(max(total, BLOCK), align=align)
-        return [pk._pack(list(enumerate(trees)), pk._length(total))]
-    pk = Packer(budget, budget, align=align)
-    out = []
-    for i, t in enumerate(trees):
-        out += list(pk.push(i, t, window=len(trees) + 1))
-    return out + list(pk.flush())
+        return [pack_stream(trees, align=align)]
+    return pack_streams(trees, budget, align=align)
 
 
 def attention_config(name: str, seed: int = 0, contents: int | None = None) -> AttnConfig:

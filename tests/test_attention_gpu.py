@@ -11,7 +11,7 @@ import spinf_serve_amd as sa
 from oracle import attention as oattn
 from oracle import mask as omask
 from spinf_serve_amd import synth
-from spinf_serve_amd.packer import GroupedTree
+from spinf_serve_amd.layout import TokenTree
 
 pytestmark = pytest.mark.gpu
 TOL = 2e-2
@@ -148,7 +148,7 @@ def test_unaligned_packing_and_ragged_length(dev):
 def test_aligned_query_groups_leave_gaps(dev):
     """a branch group that starts on a block boundary leaves pads inside the job (spinf_serve/packer.py:390-391)"""
     rng = np.random.default_rng(4)
-    t = GroupedTree(rng.integers(5, 99, 300).tolist(), [rng.integers(5, 99, n).tolist() for n in (9, 12, 7, 30)], [], [], parents=[-1, -1, -1, -1], aligned=[2])
+    t = TokenTree(rng.integers(5, 99, 300).tolist(), [rng.integers(5, 99, n).tolist() for n in (9, 12, 7, 30)], [-1, -1, -1, -1], aligned=(2,))
     cfg = synth.AttnConfig("gaps", 8, 4, 128, 128 ** -0.5, 1.0, None, [t])
     b = synth.pack([t])[0]
     assert (b.art[300:] == -1).any()
@@ -171,13 +171,13 @@ def test_batch_invariance_bit_exact(dev):
         k = torch.zeros((n, cfg.hkv, cfg.d), dtype=torch.bfloat16)
         v = torch.zeros((n, cfg.hkv, cfg.d), dtype=torch.bfloat16)
         for slot, i in enumerate(order):
-            s0 = b.owners[slot].start
+            s0 = b.jobs[slot][0]
             q[s0 : s0 + trees[i].n_tokens] = qs[i]
             k[s0 : s0 + trees[i].n_tokens] = ks[i]
             v[s0 : s0 + trees[i].n_tokens] = vs[i]
         mask = sa.TreeMask.build(b.art, b.end, b.pos, window=window, device=dev)
         out = sa.tree_attn(q.to(dev), k.to(dev), v.to(dev), mask, cfg.scale).cpu()
-        return {i: out[b.owners[slot].start : b.owners[slot].start + trees[i].n_tokens] for slot, i in enumerate(order)}
+        return {i: out[b.jobs[slot][0] : b.jobs[slot][0] + trees[i].n_tokens] for slot, i in enumerate(order)}
 
     for window in (None, 256):
         packed = run([0, 1, 2, 3], window)
@@ -222,7 +222,7 @@ def _compact_case(name):
         cfg = synth.attention_config("C2", contents=3)
         return cfg, cfg.batches[0], None
     if name == "gaps":        # pads INSIDE a job (aligned branch group), head dim 128
-        t = GroupedTree(rng.integers(5, 99, 300).tolist(), [rng.integers(5, 99, n).tolist() for n in (9, 12, 7, 30)], [], [], parents=[-1, -1, -1, -1], aligned=[2])
+        t = TokenTree(rng.integers(5, 99, 300).tolist(), [rng.integers(5, 99, n).tolist() for n in (9, 12, 7, 30)], [-1, -1, -1, -1], aligned=(2,))
         cfg = synth.AttnConfig("gaps", 8, 4, 128, 128 ** -0.5, 1.0, None, [t])
         return cfg, synth.pack([t])[0], None
     if name == "dense":       # no alignment: pads only at the end of the stream, head dim 64
@@ -294,7 +294,7 @@ def test_compact_rows_through_the_exact_pass(dev):
 def _image_stream(seed=8):
     """two jobs with image placeholders: groups that straddle tile borders, two in one block, one inside a branch"""
     rng = np.random.default_rng(seed)
-    t1 = GroupedTree(rng.integers(5, 99, 700).tolist(), [rng.integers(5, 99, n).tolist() for n in (40, 9, 70)], [], [], parents=[-1, -1, -1])
+    t1 = TokenTree(rng.integers(5, 99, 700).tolist(), [rng.integers(5, 99, n).tolist() for n in (40, 9, 70)], [-1, -1, -1])
     t2 = synth._tree(rng, 150, [20])
     trees = [t1, t2]
     b = synth.pack(trees)[0]
@@ -370,14 +370,14 @@ def test_head_dim_512(dev, hq, hkv):
     q, k, v = synth.qkv(cfg, b, device=dev)
     mask = sa.TreeMask.build(b.art, b.end, b.pos, device=dev)
     packed = sa.tree_attn(q, k, v, mask, cfg.scale)
-    o = b.owners[1]
+    start, length, *_ = b.jobs[1]
     b1 = synth.pack([trees[1]])[0]
     m1 = sa.TreeMask.build(b1.art, b1.end, b1.pos, device=dev)
-    sl = slice(o.start, o.start + o.n_tokens)
-    pad = b1.length - o.n_tokens
+    sl = slice(start, start + length)
+    pad = b1.length - length
     ext = lambda t: torch.cat([t[sl], t.new_zeros(pad, *t.shape[1:])])  # noqa: E731
     alone = sa.tree_attn(ext(q), ext(k), ext(v), m1, cfg.scale)
-    assert torch.equal(alone[: o.n_tokens], packed[sl])
+    assert torch.equal(alone[:length], packed[sl])
     # compact rows
     real = np.flatnonzero(b.art >= 0)
     sidx = torch.from_numpy(real).to(dev)
@@ -397,8 +397,7 @@ def test_random_forests_against_the_oracle(dev, seed):
         parents = [p_ if p_ < 0 or parents[p_] < 0 else -1 for p_ in parents]
         aligned = [i for i in range(nb) if parents[i] < 0 and rng.random() < 0.2]
         trunk = int(rng.integers(0 if nb else 1, 400))
-        trees.append(GroupedTree(rng.integers(5, 99, trunk).tolist(), [rng.integers(5, 99, n).tolist() for n in lens], [], [],
-                                 parents=parents, aligned=aligned))
+        trees.append(TokenTree(rng.integers(5, 99, trunk).tolist(), [rng.integers(5, 99, n).tolist() for n in lens], parents, tuple(aligned)))
     b = synth.pack(trees, align=bool(rng.integers(0, 2)))[0]
     hq, hkv, d = [(4, 2, 64), (8, 2, 128), (3, 3, 128), (4, 2, 256), (2, 1, 256), (4, 1, 512)][int(rng.integers(0, 6))]
     window = [None, 23, 150][int(rng.integers(0, 3))]

@@ -29,7 +29,7 @@ def test_c2_full_pack_is_invariant_and_matches_the_oracle(dev):
     out = sa.tree_attn(q, k, v, masks["full_attention"], cfg.scale)
     torch.cuda.synchronize()
     for slot in (0, 11, 23):
-        s0, n = b.owners[slot].start, cfg.trees[slot].n_tokens
+        s0, n = b.jobs[slot][0], cfg.trees[slot].n_tokens
         one = synth.pack([cfg.trees[slot]])[0]
         m1 = sa.TreeMask.build(one.art, one.end, one.pos, window=None, device=dev)
         pad = one.length - n
@@ -41,7 +41,7 @@ def test_c2_full_pack_is_invariant_and_matches_the_oracle(dev):
         alone = sa.tree_attn(z(q), z(k), z(v), m1, cfg.scale)
         assert torch.equal(alone[:n], out[s0 : s0 + n]), slot
     # one content against the dense float64 oracle
-    s0 = b.owners[5].start
+    s0 = b.jobs[5][0]
     one = synth.pack([cfg.trees[5]])[0]
     n = cfg.trees[5].n_tokens
     want = oattn.tree_attention(_np(q[s0 : s0 + n]), _np(k[s0 : s0 + n]), _np(v[s0 : s0 + n]), one.art[:n], one.end[:n], pos=one.pos[:n], scale=cfg.scale)
@@ -64,7 +64,7 @@ def test_c5_full_stream_properties(dev):
     del o2
     b = cfg.batch
     for slot in (0, 77, 127):
-        s0 = b.owners[slot].start
+        s0 = b.jobs[slot][0]
         n = cfg.trees[slot].n_tokens
         one = synth.GdnConfig("one", cfg.h, cfg.hv, cfg.dk, cfg.dv, [cfg.trees[slot]])
         one.batch = synth.pack([cfg.trees[slot]])[0]
@@ -105,7 +105,7 @@ def _check_pack(cfg, b, trees, slots, oracle_slot, oracle_heads, window, dev, se
     out = sa.tree_attn(q, k, v, masks["sliding_attention" if window else "full_attention"], cfg.scale)
     torch.cuda.synchronize()
     for slot in slots:
-        s0, n = b.owners[slot].start, trees[slot].n_tokens
+        s0, n = b.jobs[slot][0], trees[slot].n_tokens
         one = synth.pack([trees[slot]])[0]
         m1 = sa.TreeMask.build(one.art, one.end, one.pos, window=window, device=dev)
         pad = one.length - n
@@ -117,7 +117,7 @@ def _check_pack(cfg, b, trees, slots, oracle_slot, oracle_heads, window, dev, se
         alone = sa.tree_attn(z(q), z(k), z(v), m1, cfg.scale)
         assert torch.equal(alone[:n], out[s0 : s0 + n]), (slot, window)
     # one content, the first `oracle_heads` query heads of it, against the dense float64 oracle
-    s0, n = b.owners[oracle_slot].start, trees[oracle_slot].n_tokens
+    s0, n = b.jobs[oracle_slot][0], trees[oracle_slot].n_tokens
     one = synth.pack([trees[oracle_slot]])[0]
     hk = max(1, oracle_heads * cfg.hkv // cfg.hq)
     want = oattn.tree_attention(_np(q[s0 : s0 + n, :oracle_heads]), _np(k[s0 : s0 + n, :hk]), _np(v[s0 : s0 + n, :hk]), one.art[:n], one.end[:n],
@@ -134,7 +134,7 @@ def test_c3_largest_pass_is_invariant_and_matches_the_oracle(dev, window):
     cfg = synth.attention_config("C3")
     assert len(cfg.trees) == 512 and len(cfg.batches) >= 12
     b = max(cfg.batches, key=lambda x: x.length)
-    trees = [cfg.trees[o.job_id] for o in b.owners]
+    trees = [cfg.trees[k] for *_, k in b.jobs]
     small = min(range(len(trees)), key=lambda i: trees[i].n_tokens)
     _check_pack(cfg, b, trees, (0, len(trees) // 2, len(trees) - 1), small, cfg.hq, window, dev, seed=3)
 
@@ -144,4 +144,4 @@ def test_c4_full_pack_is_invariant_and_matches_the_oracle(dev):
     cfg = synth.attention_config("C4")
     assert len(cfg.trees) == 64 and len(cfg.batches) == 1
     b = cfg.batches[0]
-    _check_pack(cfg, b, [cfg.trees[o.job_id] for o in b.owners], (0, 37, 63), 5, 2, None, dev, seed=4)
+    _check_pack(cfg, b, [cfg.trees[k] for *_, k in b.jobs], (0, 37, 63), 5, 2, None, dev, seed=4)

@@ -1,4 +1,4 @@
-"""Host side of the path (no GPU): the packer mirror, the tile-plan compiler (C ABI, host code), the recurrent-layer planner,
+"""Host side of the path (no GPU): the stream layout, the tile-plan compiler (C ABI, host code), the recurrent-layer planner,
 and that the shared library loads and exports every symbol include/spinf_tree.h declares."""
 
 import ctypes
@@ -15,7 +15,8 @@ from oracle import mask as omask
 from oracle import plan as oplan
 from oracle.layout import Job, pack_stream
 from spinf_serve_amd import synth
-from spinf_serve_amd.packer import BLOCK, GroupedTree, Packer, ReadPlan, build_grouped_tree, build_tree, split_trees, trie_branches
+from spinf_serve_amd import layout as lay
+from spinf_serve_amd.layout import TokenTree
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
@@ -107,107 +108,78 @@ def test_ops_have_no_cpu_path(lib):
         sa.tree_attn(q, k, k, mask, cfg.scale)
 
 
-# ------------------------------------------------------------------------------------------------ packer mirror
-def test_build_tree_and_trie_literals(golden):
-    # spinf_serve/packer.py:38-64 via the reference's tests/test_packer.py:11-39
-    t = build_tree([[1, 5, 6, 7], [1, 5, 6, 8, 9]], [[[10], [11]], [[12], [13]]])
-    assert t.prefix == [1, 5, 6] and t.branches == [[7], [8, 9]]
-    assert t.reads == [(0, 0, 10, 0, 0), (0, 0, 11, 0, 1), (1, 1, 12, 1, 0), (1, 1, 13, 1, 1)] and t.n_tokens == 6
-    t = build_tree([[1, 2, 3], [1, 2, 3]], [[[4]], [[5]]])
-    assert t.prefix == [1, 2] and t.branches == [[3], [3]]
-    t = build_tree([[1, 2, 3]], [[[20], [21, 22], [21, 23]]])
-    assert t.branches == [[3], [3, 21]] and t.n_options == [3]
-    assert sorted(t.reads) == sorted([(0, 0, 20, 0, 0), (0, 0, 21, 0, 1), (1, 1, 22, 0, 1), (0, 0, 21, 0, 2), (1, 1, 23, 0, 2)])
-    with pytest.raises(ValueError):
-        build_tree([[1, 2]], [[[]]])
-    with pytest.raises(ValueError):
-        build_tree([], [])
-    g = golden["build_tree"]
-    t = build_tree([[1, 5, 6, 7], [1, 5, 6, 8, 9]], [[[10], [11]], [[12], [13, 14]]])
-    assert (t.prefix, t.branches, [list(r) for r in t.reads], t.n_options) == (g["prefix"], g["branches"], g["reads"], g["n_options"])
-    # tests/test_packer.py:191-206
-    plans = [ReadPlan.build([[30], [31]]), ReadPlan.build([[30], [31]]), ReadPlan.build([[20], [21, 22], [21, 23]])]
-    t = build_grouped_tree([[1, 2, 5, 6, 7, 8], [1, 2, 5, 6, 7, 9], [1, 2, 4]], plans)
-    gg = golden["build_grouped_tree"]
-    assert (t.prefix, t.branches, t.parents) == (gg["prefix"], gg["branches"], gg["parents"]) == ([1, 2], [[5, 6, 7], [8], [9], [4, 21]], [-1, 0, 0, -1])
-    assert [[list(x) for x in r] for r in t.prompt_rows] == gg["prompt_rows"] and t.n_tokens == 9
-    br, pa, rows = trie_branches([[3], [3]], [ReadPlan.build([[9]]), ReadPlan.build([[4, 5, 6], [4, 5, 7], [4, 8]])])
-    assert br == [[3, 4, 5]] and pa == [-1] and rows == [[(0, 0)], [(0, 0), (0, 1), (0, 2), (0, 1)]]
+# ------------------------------------------------------------------------------------------------ stream layout
+def _golden_trees(case):
+    return [TokenTree(t["prefix"], t["branches"], list(t["parents"]), tuple(t["aligned"])) for t in case["trees"]]
 
 
-def test_split_trees_halves_until_each_run_fits():
-    prompts = [[1] * 50 + [i] * 30 for i in range(2, 10)]
-    options = [[[100], [101]]] * len(prompts)
-    assert build_tree(prompts, options).n_tokens == 50 + 8 * 30
-    runs = split_trees(prompts, options, 110)
-    assert [a for a, _ in runs] == [0, 2, 4, 6] and all(t.n_tokens <= 110 for _, t in runs)
-    with pytest.raises(ValueError):
-        split_trees(prompts, options, 60)
-
-
-def test_packer_reproduces_reference_streams(golden):
-    """same trees pushed the same way -> the same batches, field by field (Packer.push / _flush / _pack)"""
+def test_layout_reproduces_reference_streams(golden):
+    """the jobs the reference's packer put into a stream (its owners say which, in which order), laid out by pack_stream: the same
+    ids / pos / seg / art / end / prev, field by field (Packer._pack, spinf_serve/packer.py:352-423)"""
     for case in golden["cases"]:
-        trees = [GroupedTree(t["prefix"], t["branches"], [], [], parents=t["parents"], aligned=t["aligned"]) for t in case["trees"]]
-        pk = Packer(case["budget"], case["max_tokens"], align=case["align"], min_stream=case["min_stream"])
-        batches = []
-        for k, t in enumerate(trees):
-            batches += list(pk.push(k, t, window=case["push_window"]))
-        batches += list(pk.flush())
-        assert len(batches) == len(case["batches"])
-        for b, want in zip(batches, case["batches"]):
+        trees = _golden_trees(case)
+        for want in case["batches"]:
+            members = [trees[job_id] for job_id, *_ in want["owners"]]
+            b = lay.pack_stream(members, align=case["align"], length=len(want["ids"]))
             for key in ("ids", "pos", "seg", "art", "end", "prev"):
                 assert getattr(b, key).tolist() == want[key], key
             assert b.n_tokens == want["n_tokens"]
-            assert [[o.job_id, o.start, o.n_tokens, o.prefix_len] for o in b.owners] == want["owners"]
+            assert [[s0, n, P] for s0, n, P, _ in b.jobs] == [o[1:] for o in want["owners"]]
 
 
-def test_packer_budget_rows_alignment_and_cost():
-    packer = Packer(256)
-    trees = [build_tree([[1] + [i] * n, [1] + [i] * n + [7]], [[[9], [8]], [[9], [8]]]) for i, n in ((2, 100), (3, 90), (4, 80))]
-    batches = [b for i, t in enumerate(trees) for b in packer.push(i, t, window=2)] + list(packer.flush())
-    assert sorted(o.job_id for b in batches for o in b.owners) == [0, 1, 2]
-    for b in batches:
-        assert b.length % BLOCK == 0 and b.length <= 256
-        assert b.n_tokens == sum(o.n_tokens for o in b.owners) and len(b.sel) == sum(o.n_rows for o in b.owners)
-        assert all(len(o.plan) == 4 and o.n_rows == 2 for o in b.owners)
+def test_layout_literals_and_invariants():
+    # two-level tree (spinf_serve/packer.py:382-408): depth on the path, subtree ends, the path predecessor
+    t = TokenTree([1, 2], [[5, 6, 7], [8], [9], [4, 21]], [-1, 0, 0, -1])
+    b = lay.pack_stream([t], align=True)
+    assert b.length == 128 and b.n_tokens == 9 and t.n_tokens == 9
+    assert b.pos[:9].tolist() == [0, 1, 2, 3, 4, 5, 5, 2, 3] and b.seg[:9].tolist() == [0, 0, 1, 1, 1, 2, 3, 4, 4]
+    assert b.end[:9].tolist() == [9, 9, 7, 7, 7, 6, 7, 9, 9] and b.prev[:9].tolist() == [-1, 0, 1, 2, 3, 4, 4, 1, 7]
+    assert (b.art[9:] == -1).all() and (b.end[9:] == -1).all() and (b.prev[9:] == -1).all() and (b.pos[9:] == 0).all()
+    # aligned branches start on a block boundary relative to the job, the gap is padding (packer.py:390-391)
+    t = TokenTree(list(range(100)), [[1] * 10, [2] * 10], [-1, -1], aligned=(1,))
+    b = lay.pack_stream([TokenTree([7] * 130, []), t], align=True)
+    assert t.n_tokens == 138 and b.jobs == [(0, 130, 130, 0), (256, 138, 100, 1)]
+    assert (b.art[256 + 110 : 256 + 128] == -1).all() and b.seg[256 + 128] == 2 and b.prev[256 + 128] == 256 + 99
+    # unaligned packing, stream length, a job that does not fit
+    b = lay.pack_stream([TokenTree([7] * 130, []), t], align=False, min_stream=512)
+    assert b.length == 512 and b.jobs[1][0] == 130
     with pytest.raises(ValueError):
-        list(Packer(128, 256).push("x", build_tree([[1] * 600], [[[2]]])))
-    (b,) = list(Packer(128, 1024).push("long", build_tree([[1] * 600], [[[2]]])))   # over the budget: runs alone, at once
-    assert b.length == 640
-    # second packing dimension (tests/test_packer.py:262-283)
-    def tree(n, costly):
-        t = build_grouped_tree([list(range(5, 5 + n)) + [3]], [ReadPlan.build([[4]])])
-        if costly:
-            t.xbranches = [(0, object())]
-        return t
-    cost = lambda t: 100 if t.xbranches else 0  # noqa: E731
-    pk = Packer(4096, cost=cost, cost_budget=250)
-    batches = [b for k, t in enumerate([tree(300, True) for _ in range(4)]) for b in pk.push(k, t)] + list(pk.flush())
-    assert sorted(len(b.owners) for b in batches) == [2, 2]
+        lay.pack_stream([t], length=128)
+    with pytest.raises(ValueError):
+        TokenTree([1], [[2], [3]], [1, -1])
+    # first-fit-decreasing streams: every job once, none over the budget
+    rng = np.random.default_rng(3)
+    trees = [TokenTree(rng.integers(1, 9, int(n)).tolist(), [[1, 2]]) for n in rng.integers(50, 900, 40)]
+    streams = lay.pack_streams(trees, 2048)
+    assert sorted(k for s in streams for *_, k in s.jobs) == list(range(40)) and all(s.length <= 2048 for s in streams)
+    with pytest.raises(ValueError):
+        lay.pack_streams([TokenTree([1] * 3000, [])], 2048)
 
 
-def test_reads_see_exactly_their_prompt():
-    """tests/test_packer.py:209-239 with the mirror packer and the oracle mask"""
+def test_every_token_sees_exactly_its_path():
+    """the invariant behind tests/test_packer.py:209-239: under the mask rule a token sees one token per position 0 .. pos, and they
+    spell its root-to-leaf path"""
     rng = np.random.default_rng(0)
     for _ in range(10):
-        stem = [1] + rng.integers(2, 6, 3).tolist()
-        prompts = [stem + rng.integers(2, 6, int(rng.integers(1, 6))).tolist() for _ in range(int(rng.integers(1, 9)))]
-        plans = [ReadPlan.build([rng.integers(6, 9, int(rng.integers(1, 4))).tolist() for _ in range(int(rng.integers(1, 6)))]) for _ in prompts]
-        t = build_grouped_tree(prompts, plans)
-        pk = Packer(1024)
-        list(pk.push("o", build_grouped_tree([[1, 7, 7, 2], [1, 7, 7, 3]], [ReadPlan.build([[9]])] * 2)))
-        list(pk.push("t", t))
-        (b,) = list(pk.flush())
-        o = next(o for o in b.owners if o.job_id == "t")
-        k0 = sum(x.n_rows for x in b.owners[: b.owners.index(o)])
+        nb = int(rng.integers(1, 9))
+        parents = []
+        for b in range(nb):   # pre-order: a branch hangs on the trunk, on the branch before it or on one of that branch's ancestors
+            chain, a = [-1], b - 1
+            while a >= 0:
+                chain.append(a)
+                a = parents[a]
+            parents.append(int(rng.choice(chain)))
+        t = TokenTree(rng.integers(2, 6, 4).tolist(), [rng.integers(2, 9, int(rng.integers(1, 6))).tolist() for _ in range(nb)], parents)
+        b = lay.pack_stream([TokenTree([1, 7, 7, 2], [[9], [3, 9]]), t], align=bool(rng.integers(0, 2)))
         m = omask.dense_tree_mask(b.art, b.end)
-        for c, (x, plan) in enumerate(zip(prompts, plans)):
-            want = [x] + [x + list(lead[:j]) for lead in plan.leadins for j in range(1, len(lead) + 1)]
-            for r, wseq in enumerate(want):
-                qpos = int(b.sel[k0 + o.row_start[c] + r])
-                ks = np.flatnonzero(m[qpos])
-                assert b.ids[ks].tolist() == wseq and b.pos[ks].tolist() == list(range(len(wseq)))
+        for q in np.flatnonzero(b.art >= 0):
+            ks = np.flatnonzero(m[q])
+            assert b.pos[ks].tolist() == list(range(b.pos[q] + 1))
+            path, i = [], int(q)
+            while i >= 0:
+                path.append(i)
+                i = int(b.prev[i])
+            assert path[::-1] == ks.tolist()
 
 
 # ------------------------------------------------------------------------------------------------ tile plan
@@ -246,7 +218,7 @@ def _check_plan(art, end, pos, window, grp=None, grp_windowed=False):
 def _image_stream(seed=8):
     """two jobs with image placeholders: groups that straddle tile borders, two in one block, one in a branch"""
     rng = np.random.default_rng(seed)
-    t1 = GroupedTree(rng.integers(5, 99, 700).tolist(), [rng.integers(5, 99, n).tolist() for n in (40, 9, 70)], [], [], parents=[-1, -1, -1])
+    t1 = TokenTree(rng.integers(5, 99, 700).tolist(), [rng.integers(5, 99, n).tolist() for n in (40, 9, 70)], [-1, -1, -1])
     t2 = synth._tree(rng, 150, [20])
     b = synth.pack([t1, t2])[0]
     grp = np.full(b.length, -1, np.int32)
@@ -337,9 +309,9 @@ def test_schedule_covers_every_tile_and_head_group_once():
         # a list is a body followed by a tail.  Body: the items of one (job, head group) are contiguous (they share keys).
         # Tail: the list's lightest items, at most 128 of them, heaviest first, so that the workgroups finish close together.
         job_of_tile = {}
-        for o in b.owners:
-            for t in range(o.start // 128, -(-(o.start + o.n_tokens) // 128)):
-                job_of_tile[t] = o.job_id
+        for start, length, _, k in b.jobs:
+            for t in range(start // 128, -(-(start + length) // 128)):
+                job_of_tile[t] = k
         for l in range(8):
             rows = items[list_ptr[l] : list_ptr[l + 1]].tolist()
             # cost of an item: per key tile, the most 32-key blocks any of the four row groups sees (they move in step)
@@ -358,7 +330,7 @@ def test_row_map_of_a_plan_names_the_tiles_that_are_consecutive_rows():
     import ctypes as C
 
     rng = np.random.default_rng(5)
-    t = GroupedTree(rng.integers(5, 99, 300).tolist(), [rng.integers(5, 99, n).tolist() for n in (9, 12, 7, 30)], [], [], parents=[-1, -1, -1, -1], aligned=[2])
+    t = TokenTree(rng.integers(5, 99, 300).tolist(), [rng.integers(5, 99, n).tolist() for n in (9, 12, 7, 30)], [-1, -1, -1, -1], aligned=(2,))
     trees = [t, synth._tree(rng, 200, [20, 9]), synth._tree(rng, 64, [])]
     b = synth.pack(trees)[0]
     plan = sa.TilePlan.build(b.art, b.end, b.pos, None)
@@ -390,8 +362,8 @@ def test_a_jobs_plan_does_not_depend_on_its_neighbours():
     def rel(trees, which, window):
         b = synth.pack(trees)[0]
         plan = sa.TilePlan.build(b.art, b.end, b.pos, window)
-        o = b.owners[which]
-        t0, t1 = o.start // 128, -(-(o.start + o.n_tokens) // 128)
+        start, length, *_ = b.jobs[which]
+        t0, t1 = start // 128, -(-(start + length) // 128)
         return [[(int(plan.kv_idx[e]) - 2 * t0, int(plan.kv_bits[e])) for e in range(plan.qt_ptr[t], plan.qt_ptr[t + 1])] for t in range(t0, t1)]
 
     for window in (None, 256):
@@ -486,8 +458,7 @@ def test_tileplan_is_exact_on_random_forests():
             parents = [p if p < 0 or parents[p] < 0 else -1 for p in parents]          # at most two levels, parents first
             aligned = [i for i in range(nb) if parents[i] < 0 and rng.random() < 0.2]
             trunk = int(rng.integers(0 if nb else 1, 300))
-            trees.append(GroupedTree(rng.integers(5, 99, trunk).tolist(), [rng.integers(5, 99, n).tolist() for n in lens], [], [],
-                                     parents=parents, aligned=aligned))
+            trees.append(TokenTree(rng.integers(5, 99, trunk).tolist(), [rng.integers(5, 99, n).tolist() for n in lens], parents, tuple(aligned)))
         b = synth.pack(trees, align=bool(rng.integers(0, 2)))[0]
         window = [None, 17, 100][int(rng.integers(0, 3))]
         grp = None
