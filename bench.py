@@ -1,6 +1,6 @@
 """Benchmark of the tree-mask packed-prefill attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K=200] [--warmup W=100] [--workload C2|C3|C4|C5|XDEC|LM|copy ...] [--seed S] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K=200] [--warmup W=100] [--workload C2|C3|C4|C5|XDEC|LM|LM_head|copy|mfma_peak ...] [--seed S] [--no-cpu]
 
 A step is one pass of the attention op (one layer's call through the C ABI) over one packed synthetic stream already
 resident in HBM; the tile plan is compiled once per stream, outside the timed region, as the reference builds its block
@@ -38,6 +38,8 @@ WORKLOADS = {
     "XDEC_long": "extraction-decode attention step: 64 groups x (U{1024..4096}-token prefix + 8 slots with templates of U{8..16} tokens) x 6 beams, 33 generated entries (step 32), 16 / 8 heads, head_dim 256, global layer",
     "XDEC_qwen": "XDEC's step at the Qwen-hybrid attention geometry: 24 query heads / 4 KV heads, head_dim 256 (288 rows per (group, kv head): three row chunks)",
     "XDEC_512": "XDEC's step at the head geometry of the Gemma-4 full-attention layers: 16 query heads / 1 KV head, head_dim 512 (output computed 256 head dims at a time, two launches)",
+    "mfma_peak": "pure v_mfma_f32_32x32x16_bf16 loop, one workgroup of eight waves on every compute unit, operands in registers: the yardstick for what the matrix cores sustain on this part",
+    "LM_head": "lm head of one chunk of 1,024 read rows gathered from a 65,536-row stream: h[sel] W^T (hidden 2,560, vocabulary 262,144, bf16 MFMA, fp32 logits) + soft-capping (30) + log-softmax + 8 option columns in one pass, no logits matrix",
     "LM": "lm head read-out of one chunk of 1,024 read rows: soft-capping (30) + log-softmax over 262,144 fp32 logits + 8 option columns",
 }
 
@@ -70,6 +72,43 @@ def timed(fn, steps, warmup, torch):
     wall = time.perf_counter() - t0
     kern = [a.elapsed_time(b) for a, b in ev]
     return wall, kern
+
+
+def mfma_rate(torch, steps=20, warmup=5, iters=4000):
+    """-> (TFLOP/s, ms per launch) of the library's pure MFMA loop, events on the launch stream"""
+    import ctypes as C
+
+    import numpy as np
+
+    from spinf_serve_amd import _lib
+
+    lib = _lib.load_library()
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    out = torch.empty(cus * 512, dtype=torch.float32, device="cuda:0")
+    flops = C.c_double()
+
+    def fn():
+        _lib.check(lib.spinf_diag_mfma_rate(iters, out.data_ptr(), out.numel(), C.byref(flops), C.c_void_p(torch.cuda.current_stream().cuda_stream)), "spinf_diag_mfma_rate")
+
+    _, kern = timed(fn, steps, warmup, torch)
+    ms = float(np.mean(kern))
+    return flops.value / (ms * 1e-3) / 1e12, ms
+
+
+def gdn_record(sa, synth, torch, np, args, steps, warmup):
+    """C5 through the Gated DeltaNet tree scan -> (record, cfg, tensors)"""
+    cfg = synth.gdn_config("C5", seed=args.seed, contents=args.contents if args.workload == "C5" else None)
+    t = synth.gdn_inputs(cfg, seed=args.seed, device=torch.device("cuda:0"))
+    plan = cfg.plan(torch.device("cuda:0"))
+    wall, kern = timed(lambda: sa.gdn_tree(t["q"], t["k"], t["v"], t["g"], t["beta"], plan), steps, warmup, torch)
+    ms = float(np.mean(kern))
+    gbs = cfg.bytes() / (ms * 1e-3) / 1e9
+    whole = args.workload != "C5" or args.contents is None
+    rec = {"metric": "packed tokens/s, Gated DeltaNet tree scan", "value": cfg.n_real * steps / wall, "unit": "tokens/s", "ms_per_step": 1e3 * wall / steps,
+           "steps": steps, "warmup": warmup, "dtype": "bf16 (fp32 state)", "config": {"workload": WORKLOADS["C5"], "contents": len(cfg.trees), "tokens": cfg.n_real},
+           "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
+                        "traffic": TRAFFIC_BYTES["C5"] if whole else None, "kernel_ms": ms, "algorithmic_bytes": cfg.bytes()}}
+    return rec, cfg, t
 
 
 def main():
@@ -118,6 +157,40 @@ def main():
                     config={"workload": WORKLOADS["copy"], "bytes_read": n, "bytes_written": n},
                     roofline={"bound": "hbm", "achieved": 2 * n / (ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                               "frac": 2 * n / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": 2 * n, "kernel_ms": ms})
+        print(json.dumps(line))
+        return
+
+    if args.workload == "mfma_peak":
+        tfl, ms = mfma_rate(torch, args.steps, args.warmup)
+        line.update(metric="bf16 MFMA rate, pure loop", unit="TFLOP/s", value=tfl, ms_per_step=ms, dtype="bf16", config={"workload": WORKLOADS["mfma_peak"]},
+                    roofline={"bound": "mfma", "achieved": tfl, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": tfl / PEAK_BF16_TFLOPS, "traffic": None,
+                              "kernel_ms": ms, "reachable_peak": tfl})
+        print(json.dumps(line))
+        return
+
+    if args.workload == "LM_head":
+        rows, stream, hidden, vocab, cap = 1024, 65536, 2560, 262144, 30.0
+        gen = torch.Generator(device=dev).manual_seed(args.seed)
+        h = torch.randn((stream, hidden), generator=gen, device=dev).to(torch.bfloat16)
+        w = (torch.randn((vocab, hidden), generator=gen, device=dev) * 0.05).to(torch.bfloat16)
+        sel = torch.randperm(stream, generator=gen, device=dev)[:rows].sort().values
+        cols = torch.randint(0, vocab, (8,), generator=gen, device=dev)
+        if args.rows == "scatter":   # the reference's own lines (scorer.py:247-254, :345-353), for comparison
+            step = lambda: torch.log_softmax(torch.tanh(torch.mm(h[sel], w.t(), out_dtype=torch.float32) / cap) * cap, dim=-1)[:, cols]  # noqa: E731
+        else:
+            step = lambda: sa.lm_head_logprobs(h, sel, w, cols, cap)  # noqa: E731
+        wall, kern = timed(step, args.steps, args.warmup, torch)
+        ms = float(np.mean(kern))
+        flops = 2.0 * rows * vocab * hidden
+        nbytes = (vocab + rows) * hidden * 2 + rows * 8 * 4
+        tfl = flops / (ms * 1e-3) / 1e12
+        peak_now, _ = mfma_rate(torch)
+        line.update(metric="read rows/s, lm head (GEMM + read-out in one pass)", value=rows * args.steps / wall, unit="rows/s", ms_per_step=1e3 * wall / args.steps,
+                    dtype="bf16 (fp32 accumulation and read-out)",
+                    config={"workload": WORKLOADS["LM_head"], "rows": rows, "vocab": vocab, "hidden": hidden, "way": "torch ops" if args.rows == "scatter" else "kernel"},
+                    roofline={"bound": "mfma", "achieved": tfl, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": tfl / PEAK_BF16_TFLOPS, "traffic": None,
+                              "kernel_ms": ms, "useful_flops": flops, "reachable_peak": peak_now, "algorithmic_bytes": nbytes,
+                              "hbm_frac_at_algorithmic_bytes": nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS})
         print(json.dumps(line))
         return
 
@@ -227,20 +300,8 @@ def main():
         return
 
     if args.workload == "C5":
-        cfg = synth.gdn_config("C5", seed=args.seed, contents=args.contents)
-        t = synth.gdn_inputs(cfg, seed=args.seed, device=dev)
-        plan = cfg.plan(dev)
-
-        def step():
-            return sa.gdn_tree(t["q"], t["k"], t["v"], t["g"], t["beta"], plan)
-
-        wall, kern = timed(step, args.steps, args.warmup, torch)
-        ms = float(np.mean(kern))
-        gbs = cfg.bytes() / (ms * 1e-3) / 1e9
-        line.update(metric="packed tokens/s, Gated DeltaNet tree scan", value=cfg.n_real * args.steps / wall, ms_per_step=1e3 * wall / args.steps,
-                    dtype="bf16 (fp32 state)", config={"workload": WORKLOADS["C5"], "contents": len(cfg.trees), "tokens": cfg.n_real},
-                    roofline={"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
-                              "traffic": TRAFFIC_BYTES["C5"] if args.contents is None else None, "kernel_ms": ms, "algorithmic_bytes": cfg.bytes()})
+        rec, cfg, t = gdn_record(sa, synth, torch, np, args, args.steps, args.warmup)
+        line.update({k: rec[k] for k in ("metric", "value", "ms_per_step", "dtype", "config", "roofline")})
         if not args.no_cpu:
             from oracle import cpu_baseline
 
@@ -306,6 +367,9 @@ def main():
                           "kernel_ms_min": float(np.min(kern)), "useful_flops": flops,
                           "algorithmic_bytes": cfg.bytes() * len(layers), "hbm_frac_at_algorithmic_bytes": cfg.bytes() * len(layers) / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS},
                 plan_build_ms_host=plan_ms, setup_s=setup_s)
+    # what a pure MFMA loop sustains on this part right now, next to the published constant the fraction is priced against
+    line["roofline"]["reachable_peak"] = mfma_rate(torch)[0]
+    line["roofline"]["frac_of_reachable_peak"] = tfl / line["roofline"]["reachable_peak"]
     if not args.no_cpu:
         from oracle import cpu_baseline
 
@@ -324,6 +388,10 @@ def main():
         line["cpu_baseline"] = {"value": tps, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
                                 "sample": f"{done} of {len(cfg.trees) if len(cfg.batches) == 1 else 'the first pass'} contents x {reps} repeats ({done_tok} packed tokens), fp32 torch scaled_dot_product_attention with an explicit dense tree mask per content, {dt:.1f} s; os.cpu_count()={os.cpu_count()}",
                                 "max_abs_err_gpu_vs_cpu_fp32": err}
+    if args.workload == "C2" and args.contents is None and args.rows == "stream":
+        # the other half of the hot path, timed in the same run: C5 through the Gated DeltaNet tree scan
+        work = None
+        line["gdn"] = gdn_record(sa, synth, torch, np, args, max(10, args.steps // 4), max(5, args.warmup // 4))[0]
     print(json.dumps(line))
 
 

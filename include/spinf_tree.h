@@ -219,7 +219,7 @@ int spinf_gdn_gate(const spinf_gdn_gate_args* args, void* stream);
  * (spinf_serve/scorer.py:351-353 and :254): out[r, c] = log_softmax(softcap * tanh(logits[r] / softcap))[cols[c]], or the whole
  * row with cols == NULL (the extraction rows, scorer.py:260).  softcap 0 = none.
  *   logits [rows, ld >= vocab]: fp32 (dtype 0) or bf16 (dtype 1) device matrix, rows 16-byte aligned; cols [n_cols] int64
- *   device array of column indices in 0 .. vocab-1; out [rows, out_ld] fp32.
+ *   device array of column indices in 0 .. vocab-1 (any other is not read and gives NaN); out [rows, out_ld] fp32.
  */
 typedef struct spinf_lm_args {
     const void* logits; int64_t ld; int32_t dtype;
@@ -228,6 +228,32 @@ typedef struct spinf_lm_args {
     float* out; int64_t out_ld;
 } spinf_lm_args;
 int spinf_lm_logprobs(const spinf_lm_args* args, void* stream);
+
+/* The whole read-out in one pass: replaces the row gather Hf[sel], the chunked logits GEMM, the soft-capping, the log-softmax and
+ * the column selection of Scorer._forward / Scorer._logprobs (spinf_serve/scorer.py:247-261 and :340-355).  The logits matrix is
+ * never stored: out[r, c] = log_softmax(cap(h[sel[r]] . W^T))[cols[c]], or the whole row with cols == NULL (scorer.py:260).
+ *   h [*, h_ld >= hidden] bf16: the final hidden states (after the final norm); sel [rows] int64 device: their rows to read,
+ *   NULL = rows 0 .. rows-1; w [vocab, w_ld >= hidden] bf16: the lm head's weight (nn.Linear layout); hidden a multiple of 64;
+ *   rows of h and w 16-byte aligned.
+ *   logits_dtype 0: the logits stay fp32 (the reference's "f32out" and "fp32" modes, scorer.py:345-348); 1: they are rounded to
+ *   bf16 and soft-capped in bf16 steps, as `h @ W.t()` on bf16 tensors gives them (scorer.py:349-352).
+ *   cols [n_cols] int64 device: columns in 0 .. vocab-1 (any other gives NaN); out [rows, out_ld] fp32.
+ *   workspace: device memory of the size spinf_lm_head_workspace reports (the per-tile log-sum-exp partials), owned by the caller.
+ * A row's results do not depend on which rows it is computed with (the reference pads chunks to lm_rows for that,
+ * spinf_serve/config.py:56-57).  Stream-ordered; nothing is allocated.
+ */
+typedef struct spinf_lm_head_args {
+    const void* h; int64_t h_ld;
+    const int64_t* sel; int64_t rows;
+    const void* w; int64_t w_ld;
+    int64_t vocab, hidden;
+    float softcap; int32_t logits_dtype;
+    const int64_t* cols; int64_t n_cols;
+    float* out; int64_t out_ld;
+    void* workspace; int64_t workspace_bytes;
+} spinf_lm_head_args;
+int spinf_lm_head_workspace(const spinf_lm_head_args* args, int64_t* bytes);
+int spinf_lm_head_fwd(const spinf_lm_head_args* args, void* stream);
 
 /* ------------------------------------------------------------------------------------------------ extraction-decode attention
  * Replaces _x_attention of spinf_serve/decode.py:71-104 (the attention interface "x_decode"): one decoding step for the
@@ -267,6 +293,14 @@ int spinf_xdecode_plan(const spinf_xdec_args* args, int32_t* nsplit, int64_t* wo
 /* tiles of the longest list of these sizes (a group whose prefix and template ranges are full) */
 int spinf_xdecode_tiles(const spinf_xdec_args* args, int32_t* tiles);
 int spinf_xdecode_attn_fwd(const spinf_xdec_args* args, void* stream);
+
+/* ------------------------------------------------------------------------------------------------ yardstick
+ * No counterpart in the reference: one launch of a pure v_mfma_f32_32x32x16_bf16 loop on every compute unit (one workgroup of eight
+ * waves per CU, iters x 8 MFMAs per wave, operands in registers), for the benchmark's "what do the matrix cores sustain on this
+ * part" figure, as a plain device copy is the yardstick for HBM.  out: device scratch of at least 512 floats per compute unit;
+ * *flops receives the floating-point operations of the launch.  Timing is the caller's (events on the stream).
+ */
+int spinf_diag_mfma_rate(int64_t iters, float* out, int64_t out_floats, double* flops, void* stream);
 
 #ifdef __cplusplus
 }

@@ -111,7 +111,10 @@ __global__ __launch_bounds__(256) void lm_logprobs_kernel(const LmParams p) {
     const float lse = m + logf(s);
     float* out = p.out + (long)row * p.out_ld;
     if (p.cols) {
-        for (int c = threadIdx.x; c < p.n_cols; c += 256) out[c] = softcap(load1<BF16>(base, p.cols[c]), p.cap, p.inv_cap) - lse;
+        for (int c = threadIdx.x; c < p.n_cols; c += 256) {   // a column outside the vocabulary is not read: NaN
+            const long col = p.cols[c];
+            out[c] = col >= 0 && col < p.vocab ? softcap(load1<BF16>(base, col), p.cap, p.inv_cap) - lse : __builtin_nanf("");
+        }
     } else {
         for (int i = threadIdx.x; i < p.vocab; i += 256) out[i] = softcap(load1<BF16>(base, i), p.cap, p.inv_cap) - lse;
     }

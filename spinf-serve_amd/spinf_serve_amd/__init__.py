@@ -18,6 +18,6 @@ from .masks import TreeMask, TilePlan, block_masks  # noqa: F401
 from .attention import CAPTURE, register_tree_attention, tree_attention, tree_attn, tree_attn_noalloc, tree_flex_forward  # noqa: F401
 from .gdn import chunked, recurrent  # noqa: F401
 from .gdn_layer import gdn_gate, gdn_prologue  # noqa: F401
-from .lm_head import lm_logprobs  # noqa: F401
+from .lm_head import lm_head_logprobs, lm_logprobs  # noqa: F401
 from .decode import GroupKV, XCaches, x_attention, xdecode_attn  # noqa: F401
 from .qwen_plan import Call, TreePlan, gdn_tree, tree_plan  # noqa: F401
