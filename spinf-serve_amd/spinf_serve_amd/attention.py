@@ -23,22 +23,36 @@ from .masks import TreeMask
 # workgroup where two heads share an item); results do not depend on it
 VARIANT = int(os.environ.get("SPINF_ATTN_VARIANT", "0"))
 # the kernel with decoupled waves over a static schedule, where the library has one for the geometry (0: the lockstep kernels only)
-RING = int(os.environ.get("SPINF_ATTN_RING", "1"))
+RING = int(os.environ.get("SPINF_ATTN_RING", "-1"))      # -1 = auto
 
 
 # a static schedule (items dealt out to the workgroups on the host) also for the lockstep kernels
-STATIC = int(os.environ.get("SPINF_ATTN_STATIC", "0"))
+STATIC = int(os.environ.get("SPINF_ATTN_STATIC", "-1"))  # -1 = auto
+
+
+RING_MAX_ITEMS_PER_WG = 8
 
 
 def _ring_lists(q, hq, hkv, d, variant, sidx, mask):
-    """-> (workgroups of the static schedule or 0, whether the call goes to the kernel with decoupled waves)"""
+    """-> (workgroups of the static schedule or 0, whether the call goes to the kernel with decoupled waves).
+
+    Measured on MI355X: the decoupled kernel wins where a workgroup gets only a handful of items (C2: 6.75 per workgroup), since
+    its waves run through the item boundaries; with many items per workgroup (C3's 65,536-token passes: 16) the lockstep kernel
+    is 6 - 10 % faster.  The lockstep kernel takes the static lists on sliding layers (5 % faster there than its queue) and its
+    queue on global layers (4 % faster).  SPINF_ATTN_RING / SPINF_ATTN_STATIC = 0 / 1 switch the two for every call where the
+    geometry allows, "auto" (the default) follows the measurements."""
     from .masks import _static_lists
 
-    ring = bool(RING) and variant == 0 and d == 256 and (hq // hkv) % 2 == 0 and sidx is None and mask.grp is None
-    if ring or (STATIC and d != 512):
-        return _static_lists(q.device), ring
+    n_wg = _static_lists(q.device)
+    ring = variant == 0 and d == 256 and (hq // hkv) % 2 == 0 and sidx is None and mask.grp is None
+    if ring and RING < 0:
+        ring = mask.plan.n_qtiles * (hq // 2) <= RING_MAX_ITEMS_PER_WG * n_wg
+    elif not RING:
+        ring = False
+    static = d != 512 and (int(mask.window) > 0 if STATIC < 0 else bool(STATIC))
+    if ring or static:
+        return n_wg, ring
     return 0, False
-
 
 
 def _attn_args(q, k, v, out, n, art, end, pos, kv_idx, kv_bits, items, list_ptr, n_items, scale, window, variant, row_of, kv_row0, grp, grp_mode, ktile, n_lists=0):
@@ -131,6 +145,8 @@ def tree_attn(q, k, v, mask: TreeMask, scale=None, variant=None, sidx=None):
     hq, hkv, d = q.shape[1], k.shape[1], q.shape[2]
     if hkv <= 0 or hq % hkv:
         raise ValueError(f"{hq} query heads do not group over {hkv} key / value heads")
+    if not q.is_cuda:
+        raise RuntimeError("spinf::tree_attn runs on ROCm device tensors only (no CPU path)")
     n_lists, ring = _ring_lists(q, hq, hkv, d, variant, sidx, mask)
     mask = mask.for_head_dim(d, ring=ring)
     per_item = _lib.load_library().spinf_attn_heads_per_item(hq, hkv, d, variant)

@@ -439,3 +439,27 @@ def test_argument_errors(dev):
         sa.tree_attn(q.float(), k, v, mask, cfg.scale)
     with pytest.raises(RuntimeError):
         sa.tree_attn(q.cpu(), k.cpu(), v.cpu(), mask, cfg.scale)  # no CPU path
+
+
+@pytest.mark.parametrize("window", [None, 256])
+def test_kernel_and_schedule_choices_give_the_same_bits(dev, window, monkeypatch):
+    """the lockstep kernel on its queue, the lockstep kernel on the static lists and the kernel with decoupled waves: one result,
+    and no wave of the decoupled kernel gave up a wait"""
+    import ctypes
+
+    from spinf_serve_amd import attention
+
+    cfg = synth.attention_config("C2", contents=5)
+    b = cfg.batches[0]
+    q, k, v = synth.qkv(cfg, b, seed=4, device=dev)
+    mask = sa.TreeMask.build(b.art, b.end, b.pos, window=window, device=dev)
+    outs = []
+    for ring, static in ((0, 0), (0, 1), (1, 0)):
+        monkeypatch.setattr(attention, "RING", ring)
+        monkeypatch.setattr(attention, "STATIC", static)
+        print(f"case ring={ring} static={static} window={window}", flush=True)
+        outs.append(sa.tree_attn(q, k, v, mask, cfg.scale))
+        torch.cuda.synchronize()
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+    aborts = ctypes.c_int64(-1)
+    assert sa.load_library().spinf_attn_ring_aborts(ctypes.byref(aborts)) == 0 and aborts.value == 0
