@@ -51,7 +51,7 @@ TRAFFIC_BYTES = {"C2": 791_205_888, "C5": 8_716_861_440, "C5_prologue": 10_777_0
                  "XDEC": 525_321_216, "XDEC_long": 2_324_807_680}
 
 
-SPINUP_S = 0.05   # untimed, before the warm-up steps: keeps the GPU busy until its clocks have come up from idle
+SPINUP_S = 0.3    # untimed, before the warm-up steps: keeps the GPU busy until its clocks have come up from idle
 
 
 def timed(fn, steps, warmup, torch):

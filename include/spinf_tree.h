@@ -91,8 +91,13 @@ void spinf_tileplan_free(spinf_tileplan* plan);
  *   scatters and the gather of qwen.py:617-622.  Pad positions write nothing.  Results equal the scattered call's bit for bit.
  *   grp, grp_mode: the image groups the plan was built with (spinf_tileplan_build_groups); stream layout, variant 0 / 1.
  *
- * The kernel is persistent (one workgroup per CU pulling items from the lists) and keeps its list cursors in a small
- * per-device buffer of the library: launches that overlap on one device (different streams) are not supported.
+ * The kernel is persistent (one workgroup per CU pulling items from the lists).  Every call takes a cursor block of its own from
+ * a per-device pool of the library (grown with hipMalloc when all are in flight, never freed) and clears it on the stream first:
+ * calls may overlap on different streams and come from different host threads.  Under stream capture the call needs an idle
+ * block of sufficient size from an earlier call (nothing can be allocated then) and keeps it for good; callers that record
+ * graphs or must not allocate take spinf_tree_attn_fwd_noalloc.
+ * Image groups: grp_mode 1 goes with every layer, grp_mode 2 with sliding layers only (window > 0; a global layer of that
+ * checkpoint passes grp = NULL, anything else is rejected).
  */
 typedef struct spinf_attn_args {
     const void* q; const void* k; const void* v; void* out;

@@ -28,6 +28,7 @@
 #include <hip/hip_runtime.h>
 
 #include <mutex>
+#include <vector>
 
 #include "spinf_tree.h"
 #include "common.h"
@@ -575,18 +576,6 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
         gslot ^= 1;
         if (grab_step(item_ne(cur)) < 0) grab(gslot);   // short item: fetch its successor now; read at the next tile step's barrier
     }
-    // ---- the last workgroup to finish resets the counters for the next launch
-    __builtin_amdgcn_s_waitcnt(0x0f70);
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        __threadfence();
-        const int done = atomicAdd(&p.counters[NLIST], 1);
-        if (done == (int)gridDim.x - 1) {
-            for (int k = 0; k < NLIST; k++) p.counters[k] = 0;
-            p.counters[NLIST] = 0;
-            __threadfence();
-        }
-    }
 }
 
 // ------------------------------------------------------------------------------------------------ host side
@@ -597,15 +586,28 @@ static __device__ __align__(256) int scratch[64 + NOALLOC_MAX_ITEMS];  // 256.25
 
 namespace {
 
+// Cursor blocks of the allocating entry point.  Every call takes a block of its own (64 ints of list cursors and counts, then
+// the redo list) from a per-device pool and clears it on the stream before its kernels run, so calls on different streams or
+// from different host threads never share cursors, and what an earlier call left behind does not matter.  A block returns to the
+// pool when the event recorded after its call's last kernel has completed.  Blocks are never freed before the process ends: a
+// bigger schedule gets a new block, and a launch recorded into a graph keeps the block it was recorded with for good.
+struct CursorBlock {
+    int* ptr = nullptr;
+    long cap = 0;               // redo entries
+    hipEvent_t done = nullptr;
+    bool recorded = false;      // `done` was recorded at least once
+    bool taken = false;         // between acquire and release on some host thread
+    bool pinned = false;        // handed to a call under stream capture: replays may run at any time
+};
 struct DeviceState {
-    int* counters = nullptr;   // 64 ints of cursors and counts, then the redo list
-    long redo_cap = 0;
+    std::vector<CursorBlock> blocks;
     int cus = 0;
 };
+constexpr size_t MAX_CURSOR_BLOCKS = 256;
 std::mutex g_mu;
 DeviceState g_dev[64];
 
-int device_state(DeviceState** out, long n_items) {
+int device_cus(int* cus) {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess || dev < 0 || dev >= 64) return spinf_fail(SPINF_E_HIP, "tree_attn: hipGetDevice: %s", hipGetErrorString(e));
@@ -617,21 +619,53 @@ int device_state(DeviceState** out, long n_items) {
         if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: hipGetDeviceProperties: %s", hipGetErrorString(e));
         s.cus = prop.multiProcessorCount;
     }
-    if (!s.counters || n_items > s.redo_cap) {   // first call on this device, or a bigger schedule than ever before
-        if (s.counters) {
-            e = hipFree(s.counters);   // waits for the device to drain
-            if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: hipFree: %s", hipGetErrorString(e));
-            s.counters = nullptr;
-        }
-        const long cap = n_items < (1 << 16) ? (1 << 16) : 2 * n_items;
-        e = hipMalloc((void**)&s.counters, (64 + cap) * sizeof(int));
-        if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: hipMalloc: %s", hipGetErrorString(e));
-        e = hipMemset(s.counters, 0, 64 * sizeof(int));
-        if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: hipMemset: %s", hipGetErrorString(e));
-        s.redo_cap = cap;
-    }
-    *out = &s;
+    *cus = s.cus;
     return SPINF_OK;
+}
+
+// -> a block no call in flight uses, with room for n_items redo entries; *slot names it for release_block
+int acquire_block(long n_items, bool capturing, int** ptr, int* slot) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= 64) return spinf_fail(SPINF_E_HIP, "tree_attn: hipGetDevice: %s", hipGetErrorString(e));
+    std::lock_guard<std::mutex> lock(g_mu);
+    DeviceState& s = g_dev[dev];
+    for (size_t i = 0; i < s.blocks.size(); i++) {
+        CursorBlock& b = s.blocks[i];
+        if (b.taken || b.pinned || b.cap < n_items) continue;
+        if (b.recorded && hipEventQuery(b.done) != hipSuccess) continue;   // its last call has not finished
+        b.taken = true;
+        b.pinned = capturing;
+        *ptr = b.ptr;
+        *slot = (int)i;
+        return SPINF_OK;
+    }
+    if (capturing)
+        return spinf_fail(SPINF_E_ARG, "tree_attn: no idle cursor block to record into the graph and none can be allocated during capture: "
+                                       "run one call of this size before the capture, or record spinf_tree_attn_fwd_noalloc");
+    if (s.blocks.size() >= MAX_CURSOR_BLOCKS) return spinf_fail(SPINF_E_NOMEM, "tree_attn: %zu attention calls in flight on one device", s.blocks.size());
+    CursorBlock b;
+    b.cap = n_items < (1 << 16) ? (1 << 16) : 2 * n_items;
+    e = hipMalloc((void**)&b.ptr, (64 + b.cap) * sizeof(int));
+    if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: hipMalloc: %s", hipGetErrorString(e));
+    e = hipMemset(b.ptr, 0, 64 * sizeof(int));   // the running totals at [NLIST + 3], [NLIST + 4] start at zero; the rest is cleared per call
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&b.done, hipEventDisableTiming);
+    if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: cursor block: %s", hipGetErrorString(e));
+    b.taken = true;
+    s.blocks.push_back(b);
+    *ptr = b.ptr;
+    *slot = (int)s.blocks.size() - 1;
+    return SPINF_OK;
+}
+
+// after the call's kernels are on the stream (or failed to get there)
+void release_block(int slot, hipStream_t stream, bool capturing) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return;
+    std::lock_guard<std::mutex> lock(g_mu);
+    CursorBlock& b = g_dev[dev].blocks[slot];
+    if (!capturing && hipEventRecord(b.done, stream) == hipSuccess) b.recorded = true;
+    b.taken = false;
 }
 
 // ---- the entry point that allocates nothing
@@ -771,7 +805,9 @@ extern "C" int spinf_attn_exact_items(int64_t* total) {
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess || dev < 0 || dev >= 64) return spinf_fail(SPINF_E_HIP, "attn_exact_items: hipGetDevice: %s", hipGetErrorString(e));
     std::lock_guard<std::mutex> lock(g_mu);
-    for (const int* c : {(const int*)g_dev[dev].counters, (const int*)g_scratch[dev].ptr}) {
+    std::vector<const int*> blocks{(const int*)g_scratch[dev].ptr};
+    for (const CursorBlock& b : g_dev[dev].blocks) blocks.push_back(b.ptr);
+    for (const int* c : blocks) {
         if (!c) continue;   // no attention launch of that kind on this device yet
         int v = 0;
         e = hipMemcpy(&v, c + NLIST + 3, sizeof(int), hipMemcpyDeviceToHost);
@@ -788,7 +824,9 @@ extern "C" int spinf_attn_ring_aborts(int64_t* total) {
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess || dev < 0 || dev >= 64) return spinf_fail(SPINF_E_HIP, "attn_ring_aborts: hipGetDevice: %s", hipGetErrorString(e));
     std::lock_guard<std::mutex> lock(g_mu);
-    for (const int* c : {(const int*)g_dev[dev].counters, (const int*)g_scratch[dev].ptr}) {
+    std::vector<const int*> blocks{(const int*)g_scratch[dev].ptr};
+    for (const CursorBlock& b : g_dev[dev].blocks) blocks.push_back(b.ptr);
+    for (const int* c : blocks) {
         if (!c) continue;
         int v = 0;
         e = hipMemcpy(&v, c + NLIST + 4, sizeof(int), hipMemcpyDeviceToHost);
@@ -829,6 +867,8 @@ static int attn_fwd(const spinf_attn_args* a, void* stream, bool no_alloc) {
     } else if ((a->d == 512) != (a->ktile == 32) || (a->ktile != 0 && a->ktile != 32 && a->ktile != 64))
         return spinf_fail(SPINF_E_ARG, "tree_attn: plan entries of %d keys with head dim %d (32 goes with 512, 64 with the others)", a->ktile ? a->ktile : 64, a->d);
     if (a->grp && (a->grp_mode != 1 && a->grp_mode != 2)) return spinf_fail(SPINF_E_ARG, "tree_attn: group mode %d not in {1, 2}", a->grp_mode);
+    if (a->grp && a->grp_mode == 2 && a->window <= 0)
+        return spinf_fail(SPINF_E_ARG, "tree_attn: group mode 2 widens the mask inside the window only; a global layer takes no groups (pass grp = NULL)");
     if (a->grp && (rt != 1 || a->row_of)) return spinf_fail(SPINF_E_ARG, "tree_attn: image groups go with variant 0 / 1 and the stream layout only");
     const int hpi = rt * nhw;
     const int64_t nqt = (a->n + SPINF_QTILE - 1) / SPINF_QTILE;
@@ -841,21 +881,24 @@ static int attn_fwd(const spinf_attn_args* a, void* stream, bool no_alloc) {
     const uintptr_t ptrs[4] = {(uintptr_t)a->q, (uintptr_t)a->k, (uintptr_t)a->v, (uintptr_t)a->out};
     for (int i = 0; i < 4; i++)
         if (ptrs[i] % 16) return spinf_fail(SPINF_E_ARG, "tree_attn: tensors must be 16-byte aligned");
+    hipStream_t s = (hipStream_t)stream;
     int* counters = nullptr;
-    int cus = 0;
+    int cus = 0, slot = -1;
+    bool capturing = false;
     if (no_alloc) {
         ScratchState* st = nullptr;
         if (int rc = scratch_state(&st)) return rc;
         counters = st->ptr;
         cus = st->cus;
     } else {
-        DeviceState* st = nullptr;
-        if (int rc = device_state(&st, (long)a->n_items)) return rc;
-        counters = st->counters;
-        cus = st->cus;
+        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(s, &cs) != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: hipStreamIsCapturing failed");
+        capturing = cs != hipStreamCaptureStatusNone;
+        if (int rc = device_cus(&cus)) return rc;
+        if (int rc = acquire_block((long)a->n_items, capturing, &counters, &slot)) return rc;
     }
     AttnParams p;
-    p.clear_first = no_alloc;
+    p.clear_first = true;   // the cursors start at zero whatever the block held
     p.static_lists = a->n_lists > 0;
     p.q = (const __bf16*)a->q; p.k = (const __bf16*)a->k; p.v = (const __bf16*)a->v; p.o = (__bf16*)a->out;
     p.q_tok = a->q_tok; p.q_head = a->q_head; p.k_tok = a->k_tok; p.k_head = a->k_head;
@@ -872,14 +915,16 @@ static int attn_fwd(const spinf_attn_args* a, void* stream, bool no_alloc) {
     p.redo = counters + 64;
     const int blocks = a->n_lists > 0 ? a->n_lists : (int)(a->n_items < cus ? a->n_items : cus);
     const bool win = p.window > 0;
-    hipStream_t s = (hipStream_t)stream;
-    if (ring) return launch_ring(p, a->d, win, a->n_lists, s);
-    switch (a->d) {
-        case 64: return launch_d<64>(p, rt, nhw, win, a->grp_mode, blocks, s);
-        case 128: return launch_d<128>(p, rt, nhw, win, a->grp_mode, blocks, s);
-        case 256: return launch_d<256>(p, rt, nhw, win, a->grp_mode, blocks, s);
-        default: return launch_d512(p, win, a->grp_mode, blocks, s);
+    int rc;
+    if (ring) rc = launch_ring(p, a->d, win, a->n_lists, s);
+    else switch (a->d) {
+        case 64: rc = launch_d<64>(p, rt, nhw, win, a->grp_mode, blocks, s); break;
+        case 128: rc = launch_d<128>(p, rt, nhw, win, a->grp_mode, blocks, s); break;
+        case 256: rc = launch_d<256>(p, rt, nhw, win, a->grp_mode, blocks, s); break;
+        default: rc = launch_d512(p, win, a->grp_mode, blocks, s);
     }
+    if (slot >= 0) release_block(slot, s, capturing);
+    return rc;
 }
 
 extern "C" int spinf_tree_attn_fwd(const spinf_attn_args* a, void* stream) { return attn_fwd(a, stream, false); }

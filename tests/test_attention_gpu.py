@@ -10,7 +10,7 @@ import torch
 import spinf_serve_amd as sa
 from oracle import attention as oattn
 from oracle import mask as omask
-from spinf_serve_amd import synth
+from spinf_serve_amd import attention, synth
 from spinf_serve_amd.layout import TokenTree
 
 pytestmark = pytest.mark.gpu
@@ -463,3 +463,41 @@ def test_kernel_and_schedule_choices_give_the_same_bits(dev, window, monkeypatch
     assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
     aborts = ctypes.c_int64(-1)
     assert sa.load_library().spinf_attn_ring_aborts(ctypes.byref(aborts)) == 0 and aborts.value == 0
+
+
+def test_calls_on_two_streams_do_not_share_cursors(dev):
+    """calls interleaved on two streams, not synchronised with each other, give the bits of the same calls one after the other"""
+    cfgs = [synth.attention_config("C2", seed=s, contents=4 + 3 * s) for s in range(2)]
+    work = []
+    for cfg in cfgs:
+        b = cfg.batches[0]
+        work.append((synth.qkv(cfg, b, seed=9, device=dev), sa.TreeMask.build(b.art, b.end, b.pos, device=dev), cfg.scale))
+    serial = [sa.tree_attn(*qkv, mask, scale) for qkv, mask, scale in work]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(device=dev) for _ in range(2)]
+    outs = [[], []]
+    for rep in range(6):
+        for i, st in enumerate(streams):
+            with torch.cuda.stream(st):
+                qkv, mask, scale = work[i]
+                outs[i].append(sa.tree_attn(*qkv, mask, scale))
+    torch.cuda.synchronize()
+    for i in range(2):
+        assert all(torch.equal(o, serial[i]) for o in outs[i])
+
+
+def test_groups_of_the_windowed_checkpoint_are_rejected_on_a_global_layer(dev):
+    import ctypes as C
+
+    from spinf_serve_amd import _lib
+
+    cfg = synth.attention_config("smoke")
+    b = cfg.batches[0]
+    q, k, v = synth.qkv(cfg, b, device=dev)
+    mask = sa.TreeMask.build(b.art, b.end, b.pos, device=dev)
+    items, list_ptr, n_items = mask.schedule(cfg.hq // 2)
+    grp = torch.full((b.length,), -1, dtype=torch.int32, device=dev)
+    out = torch.empty_like(q)
+    a = attention._attn_args(q, k, v, out, b.length, mask.art, mask.end, mask.pos, mask.kv_idx, mask.kv_bits, items, list_ptr, n_items, cfg.scale, 0, 0, None, None, grp, 2, 64)
+    lib = sa.load_library()
+    assert lib.spinf_tree_attn_fwd(C.byref(a), None) == -1 and b"global layer takes no groups" in lib.spinf_last_error()
