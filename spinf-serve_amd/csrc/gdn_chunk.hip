@@ -44,8 +44,15 @@ namespace {
 
 constexpr int KD = 128;        // key head dim
 constexpr int VD = 128;        // value head dim
-constexpr int LD = 136;        // row stride (elements) of the K / Q / V tiles
-constexpr int LW = 132;        // row stride of the -W tile
+// Row strides of the LDS tiles, chosen by how a tile is read most.  A tile read row-wise in 8- or 16-byte pieces (Q, -W: lane c
+// takes row c) wants a stride of 4 banks (mod 64): 16 rows then start in 16 different groups of four banks.  A tile read through
+// ds_read_b64_tr_b16 (K, V: 16 lanes take a 4 rows x 32 bytes block, the next 16 lanes the four rows below) wants 8 banks
+// (mod 64): eight rows x 32 bytes then cover the 64 banks once.  Measured LDS clocks per instruction of a workgroup (stride in
+// banks mod 64): 8-byte row reads 2.8 at 4 or 20, 4.0 at 2, 8, 18; transposing reads 2.9 at 8 or 24, 4.0 at 4, 12, 16, 20;
+// 16-byte row reads 4.0 at 8, 8.0 at 4, 20, 36.
+constexpr int LD = 136;        // row stride (elements) of the Q tile: 68 banks
+constexpr int LDT = 144;       // row stride of the K and V tiles: 72 banks
+constexpr int LW = 136;        // row stride of the -W tile
 constexpr int LP = 40;         // row stride of the token x token bf16 tiles (P, T diag(beta), -T diag(beta e^G))
 constexpr int LA = 36;         // row stride (floats) of A
 constexpr int LX = 20;         // row stride (floats) of the 16 x 16 blocks of T and of the merge scratch
@@ -64,13 +71,14 @@ template <bool PAIRS>
 __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
     constexpr int NT = 2;                           // 16-token tiles per chunk
     constexpr int CH = 16 * NT;
-    constexpr int LO = CH;                          // row stride (elements) of a wave's transposed output tile [32 values][CH tokens]
+    constexpr int LO = CH + 4;                      // row stride (elements) of a wave's transposed output tile [32 values][CH tokens]; 64-byte rows
+                                                    // put the 8-byte stores of 16 lanes into four banks (32 clocks per store instead of 7)
     constexpr int NTILES = NT * (NT + 1) / 2;       // 16 x 16 tiles of A / P on or below the diagonal
     typedef bf16x8 tok_op;                          // operand of a product that contracts over the chunk's 32 tokens
-    __shared__ __attribute__((aligned(16))) __bf16 Ks[CH * LD];
+    __shared__ __attribute__((aligned(16))) __bf16 Ks[CH * LDT];
     __shared__ __attribute__((aligned(16))) __bf16 Qs[CH * LD];
-    __shared__ __attribute__((aligned(16))) __bf16 Vs[CH * LD];      // V; later the waves' output tiles
-    __shared__ __attribute__((aligned(16))) char solve[32 * LA * 4 + 32 * LX * 4 + 16 * LX * 4];   // A, T blocks, merge scratch; later -W
+    __shared__ __attribute__((aligned(16))) __bf16 Vs[CH * LDT];     // V; later the waves' output tiles
+    __shared__ __attribute__((aligned(16))) char solve[32 * LA * 4 + 32 * LX * 4 + 16 * LX * 4 + 256];   // A, T blocks, merge scratch; later -W
     __shared__ __attribute__((aligned(16))) __bf16 Ps[CH * LP];
     __shared__ __attribute__((aligned(16))) __bf16 Tus[CH * LP];
     __shared__ __attribute__((aligned(16))) __bf16 Tws[CH * LP];
@@ -82,7 +90,7 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
     float* Xs = Ts + 32 * LX;
     __bf16* Wn = (__bf16*)solve;       // -W [CH][LW], written when A and T are dead
     static_assert(32 * LW * 2 <= (int)sizeof(solve), "-W must fit the region it shares");
-    static_assert(4 * 32 * LO <= CH * LD, "the output tiles must fit the V tile");
+    static_assert(4 * 32 * LO <= CH * LDT, "the output tiles must fit the V tile");
 
     const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6), c = lane & 15, q4 = lane >> 4;
     // Workgroups go round the 8 XCDs (each with its own L2) in launch order.  Two value heads that share a key head read the
@@ -242,9 +250,9 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
 #pragma unroll
             for (int cc = 0; cc < NT; cc++) {
                 const int row = (tid >> 4) + 16 * cc;
-                *(bf16x8*)(Ks + row * LD + col) = pk[cc];
+                *(bf16x8*)(Ks + row * LDT + col) = pk[cc];
                 *(bf16x8*)(Qs + row * LD + col) = pq[cc];
-                *(bf16x8*)(Vs + row * LD + col) = pv[cc];
+                *(bf16x8*)(Vs + row * LDT + col) = pv[cc];
             }
         }
         lds_barrier();
@@ -259,8 +267,8 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
             f32x4 kk = zero4(), qk = zero4();
 #pragma unroll
             for (int s = 0; s < KD / 32; s++) {
-                const bf16x8 kj = *(const bf16x8*)(Ks + (16 * jt + c) * LD + 32 * s + 8 * q4);
-                const bf16x8 ki = *(const bf16x8*)(Ks + (16 * it + c) * LD + 32 * s + 8 * q4);
+                const bf16x8 kj = *(const bf16x8*)(Ks + (16 * jt + c) * LDT + 32 * s + 8 * q4);
+                const bf16x8 ki = *(const bf16x8*)(Ks + (16 * it + c) * LDT + 32 * s + 8 * q4);
                 const bf16x8 qi = *(const bf16x8*)(Qs + (16 * it + c) * LD + 32 * s + 8 * q4);
                 kk = mfma32(kj, ki, kk);
                 qk = mfma32(kj, qi, qk);
@@ -358,7 +366,7 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
             }
 #pragma unroll
             for (int vt = 0; vt < 2; vt++) {
-                const tok_op vB = join(frag_tr4(Vs, LD, 0, 32 * w + 16 * vt, lane), frag_tr4(Vs, LD, 16, 32 * w + 16 * vt, lane));
+                const tok_op vB = join(frag_tr4(Vs, LDT, 0, 32 * w + 16 * vt, lane), frag_tr4(Vs, LDT, 16, 32 * w + 16 * vt, lane));
 #pragma unroll
                 for (int it = 0; it < NT; it++) {
                     vp[it][vt] = mfma32(tu[it], vB, zero4());
@@ -368,7 +376,7 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
 #pragma unroll
             for (int h = 0; h < 2; h++) {
                 const int kt = 2 * w + h;
-                const tok_op kT = join(frag_tr4(Ks, LD, 0, 16 * kt, lane), frag_tr4(Ks, LD, 16, 16 * kt, lane));
+                const tok_op kT = join(frag_tr4(Ks, LDT, 0, 16 * kt, lane), frag_tr4(Ks, LDT, 16, 16 * kt, lane));
 #pragma unroll
                 for (int it = 0; it < NT; it++) *(bf16x4*)(Wn + (16 * it + c) * LW + 16 * kt + 4 * q4) = round4(mfma32(kT, tw[it], zero4()));
             }
@@ -454,7 +462,7 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
             }
 #pragma unroll
             for (int kt = 0; kt < 8; kt++) {
-                const tok_op kT = join(frag_tr4(Ks, LD, 0, 16 * kt, lane), frag_tr4(Ks, LD, 16, 16 * kt, lane));
+                const tok_op kT = join(frag_tr4(Ks, LDT, 0, 16 * kt, lane), frag_tr4(Ks, LDT, 16, 16 * kt, lane));
 #pragma unroll
                 for (int vt = 0; vt < 2; vt++) {
 #pragma unroll
