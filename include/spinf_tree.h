@@ -92,7 +92,7 @@ void spinf_tileplan_free(spinf_tileplan* plan);
  *   grp, grp_mode: the image groups the plan was built with (spinf_tileplan_build_groups); stream layout, variant 0 / 1.
  *
  * The kernel is persistent (one workgroup per CU pulling items from the lists).  Every call takes a cursor block of its own from
- * a per-device pool of the library (grown with hipMalloc when all are in flight, never freed) and clears it on the stream first:
+ * a per-device pool of the library (grown with hipMalloc when all are in flight on other streams, never freed):
  * calls may overlap on different streams and come from different host threads.  Under stream capture the call needs an idle
  * block of sufficient size from an earlier call (nothing can be allocated then) and keeps it for good; callers that record
  * graphs or must not allocate take spinf_tree_attn_fwd_noalloc.

@@ -219,6 +219,8 @@ __global__ __launch_bounds__(256) void tree_attn_exact_kernel(const AttnParams p
     __shared__ __attribute__((aligned(16))) char stage_all[4 * 32 * 144];
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int n_redo = p.counters[NLIST + 1];
+    // the fast pass is over (stream order): its list cursors and its count of finished workgroups go back to zero for the block's next call
+    if (blockIdx.x == 0 && threadIdx.x <= NLIST) p.counters[threadIdx.x] = 0;
     if (n_redo == 0) return;   // the normal case: the fast pass handed nothing on (every workgroup reads the same count)
     for (int j = blockIdx.x; j < n_redo; j += gridDim.x) {
         const int4 it = p.items[p.redo[j]];
@@ -587,23 +589,25 @@ static __device__ __align__(256) int scratch[64 + NOALLOC_MAX_ITEMS];  // 256.25
 namespace {
 
 // Cursor blocks of the allocating entry point.  Every call takes a block of its own (64 ints of list cursors and counts, then
-// the redo list) from a per-device pool and clears it on the stream before its kernels run, so calls on different streams or
-// from different host threads never share cursors, and what an earlier call left behind does not matter.  A block returns to the
-// pool when the event recorded after its call's last kernel has completed.  Blocks are never freed before the process ends: a
-// bigger schedule gets a new block, and a launch recorded into a graph keeps the block it was recorded with for good.
+// the redo list) from a per-device pool, so calls on different streams or from different host threads never share cursors.  A block returns to the
+// pool when the event recorded after its call's last kernel has completed; the next call on the SAME stream takes it back at once
+// (stream order keeps the two apart), so a single-stream caller lives on one block.  Blocks are never freed before the process
+// ends: a bigger schedule gets a new block, and a launch recorded into a graph keeps the block it was recorded with for good.
 struct CursorBlock {
     int* ptr = nullptr;
     long cap = 0;               // redo entries
     hipEvent_t done = nullptr;
+    hipStream_t last = nullptr; // stream of the block's last call
     bool recorded = false;      // `done` was recorded at least once
     bool taken = false;         // between acquire and release on some host thread
     bool pinned = false;        // handed to a call under stream capture: replays may run at any time
+    bool dirty = false;         // a call on it failed to get all its kernels onto the stream: clear it before the next use
 };
 struct DeviceState {
     std::vector<CursorBlock> blocks;
     int cus = 0;
 };
-constexpr size_t MAX_CURSOR_BLOCKS = 256;
+constexpr size_t MAX_CURSOR_BLOCKS = 64;
 std::mutex g_mu;
 DeviceState g_dev[64];
 
@@ -624,7 +628,7 @@ int device_cus(int* cus) {
 }
 
 // -> a block no call in flight uses, with room for n_items redo entries; *slot names it for release_block
-int acquire_block(long n_items, bool capturing, int** ptr, int* slot) {
+int acquire_block(long n_items, bool capturing, hipStream_t stream, int** ptr, int* slot, bool* dirty) {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess || dev < 0 || dev >= 64) return spinf_fail(SPINF_E_HIP, "tree_attn: hipGetDevice: %s", hipGetErrorString(e));
@@ -633,17 +637,31 @@ int acquire_block(long n_items, bool capturing, int** ptr, int* slot) {
     for (size_t i = 0; i < s.blocks.size(); i++) {
         CursorBlock& b = s.blocks[i];
         if (b.taken || b.pinned || b.cap < n_items) continue;
-        if (b.recorded && hipEventQuery(b.done) != hipSuccess) continue;   // its last call has not finished
+        if (b.recorded && b.last != stream && hipEventQuery(b.done) != hipSuccess) continue;   // its last call, on another stream, has not finished
         b.taken = true;
         b.pinned = capturing;
         *ptr = b.ptr;
         *slot = (int)i;
+        *dirty = b.dirty;
         return SPINF_OK;
     }
     if (capturing)
         return spinf_fail(SPINF_E_ARG, "tree_attn: no idle cursor block to record into the graph and none can be allocated during capture: "
                                        "run one call of this size before the capture, or record spinf_tree_attn_fwd_noalloc");
-    if (s.blocks.size() >= MAX_CURSOR_BLOCKS) return spinf_fail(SPINF_E_NOMEM, "tree_attn: %zu attention calls in flight on one device", s.blocks.size());
+    if (s.blocks.size() >= MAX_CURSOR_BLOCKS) {   // wait for a call in flight rather than grow without bound
+        for (size_t i = 0; i < s.blocks.size(); i++) {
+            CursorBlock& b = s.blocks[i];
+            if (b.taken || b.pinned || b.cap < n_items || !b.recorded) continue;
+            e = hipEventSynchronize(b.done);
+            if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: hipEventSynchronize: %s", hipGetErrorString(e));
+            b.taken = true;
+            *ptr = b.ptr;
+            *slot = (int)i;
+            *dirty = b.dirty;
+            return SPINF_OK;
+        }
+        return spinf_fail(SPINF_E_NOMEM, "tree_attn: %zu cursor blocks on one device and none can be waited for", s.blocks.size());
+    }
     CursorBlock b;
     b.cap = n_items < (1 << 16) ? (1 << 16) : 2 * n_items;
     e = hipMalloc((void**)&b.ptr, (64 + b.cap) * sizeof(int));
@@ -655,16 +673,19 @@ int acquire_block(long n_items, bool capturing, int** ptr, int* slot) {
     s.blocks.push_back(b);
     *ptr = b.ptr;
     *slot = (int)s.blocks.size() - 1;
+    *dirty = false;
     return SPINF_OK;
 }
 
 // after the call's kernels are on the stream (or failed to get there)
-void release_block(int slot, hipStream_t stream, bool capturing) {
+void release_block(int slot, hipStream_t stream, bool capturing, bool failed) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return;
     std::lock_guard<std::mutex> lock(g_mu);
     CursorBlock& b = g_dev[dev].blocks[slot];
     if (!capturing && hipEventRecord(b.done, stream) == hipSuccess) b.recorded = true;
+    b.last = stream;
+    b.dirty = failed;
     b.taken = false;
 }
 
@@ -884,7 +905,7 @@ static int attn_fwd(const spinf_attn_args* a, void* stream, bool no_alloc) {
     hipStream_t s = (hipStream_t)stream;
     int* counters = nullptr;
     int cus = 0, slot = -1;
-    bool capturing = false;
+    bool capturing = false, dirty = false;
     if (no_alloc) {
         ScratchState* st = nullptr;
         if (int rc = scratch_state(&st)) return rc;
@@ -895,10 +916,13 @@ static int attn_fwd(const spinf_attn_args* a, void* stream, bool no_alloc) {
         if (hipStreamIsCapturing(s, &cs) != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: hipStreamIsCapturing failed");
         capturing = cs != hipStreamCaptureStatusNone;
         if (int rc = device_cus(&cus)) return rc;
-        if (int rc = acquire_block((long)a->n_items, capturing, &counters, &slot)) return rc;
+        if (int rc = acquire_block((long)a->n_items, capturing, s, &counters, &slot, &dirty)) return rc;
     }
     AttnParams p;
-    p.clear_first = true;   // the cursors start at zero whatever the block held
+    // A block's cursors are zero: it was cleared when allocated, and every call's exact-pass kernel, which runs after the fast pass,
+    // puts them back.  Only a block whose last call failed to get its kernels onto the stream is cleared first; so is the scratch
+    // array of the entry point that allocates nothing, which every caller on the GPU shares.
+    p.clear_first = no_alloc || dirty;
     p.static_lists = a->n_lists > 0;
     p.q = (const __bf16*)a->q; p.k = (const __bf16*)a->k; p.v = (const __bf16*)a->v; p.o = (__bf16*)a->out;
     p.q_tok = a->q_tok; p.q_head = a->q_head; p.k_tok = a->k_tok; p.k_head = a->k_head;
@@ -923,7 +947,7 @@ static int attn_fwd(const spinf_attn_args* a, void* stream, bool no_alloc) {
         case 256: rc = launch_d<256>(p, rt, nhw, win, a->grp_mode, blocks, s); break;
         default: rc = launch_d512(p, win, a->grp_mode, blocks, s);
     }
-    if (slot >= 0) release_block(slot, s, capturing);
+    if (slot >= 0) release_block(slot, s, capturing, rc != SPINF_OK);
     return rc;
 }
 
