@@ -91,11 +91,11 @@ void spinf_tileplan_free(spinf_tileplan* plan);
  *   scatters and the gather of qwen.py:617-622.  Pad positions write nothing.  Results equal the scattered call's bit for bit.
  *   grp, grp_mode: the image groups the plan was built with (spinf_tileplan_build_groups); stream layout, variant 0 / 1.
  *
- * The kernel is persistent (one workgroup per CU pulling items from the lists).  Every call takes a cursor block of its own from
- * a per-device pool of the library (grown with hipMalloc when all are in flight on other streams, never freed):
- * calls may overlap on different streams and come from different host threads.  Under stream capture the call needs an idle
- * block of sufficient size from an earlier call (nothing can be allocated then) and keeps it for good; callers that record
- * graphs or must not allocate take spinf_tree_attn_fwd_noalloc.
+ * The kernel is persistent (one workgroup per CU pulling items from the lists).  Its list cursors live in a block that the
+ * library keeps per stream (allocated with hipMalloc at a stream's first call, or when a bigger schedule comes; never freed):
+ * calls on one stream follow each other, calls on different streams may overlap, from any host thread.  Under stream capture
+ * the stream's block is recorded into the graph and stays with it (nothing can be allocated then: the stream must have made
+ * one call of that size before); callers that record graphs or must not allocate take spinf_tree_attn_fwd_noalloc.
  * Image groups: grp_mode 1 goes with every layer, grp_mode 2 with sliding layers only (window > 0; a global layer of that
  * checkpoint passes grp = NULL, anything else is rejected).
  */

@@ -588,26 +588,24 @@ static __device__ __align__(256) int scratch[64 + NOALLOC_MAX_ITEMS];  // 256.25
 
 namespace {
 
-// Cursor blocks of the allocating entry point.  Every call takes a block of its own (64 ints of list cursors and counts, then
-// the redo list) from a per-device pool, so calls on different streams or from different host threads never share cursors.  A block returns to the
-// pool when the event recorded after its call's last kernel has completed; the next call on the SAME stream takes it back at once
-// (stream order keeps the two apart), so a single-stream caller lives on one block.  Blocks are never freed before the process
-// ends: a bigger schedule gets a new block, and a launch recorded into a graph keeps the block it was recorded with for good.
+// Cursor blocks of the allocating entry point (64 ints of list cursors and counts, then the redo list).  A block belongs to the
+// stream it was first used on: calls on one stream follow each other in stream order and share it, calls on different streams
+// (or from host threads that use different streams) never share cursors, and no event or query is needed to tell when a block is
+// free.  Blocks are never freed before the process ends: a bigger schedule gets a new block for its stream, and a launch
+// recorded into a graph keeps the block it was recorded with for good (replays may run at any time).
 struct CursorBlock {
     int* ptr = nullptr;
     long cap = 0;               // redo entries
-    hipEvent_t done = nullptr;
-    hipStream_t last = nullptr; // stream of the block's last call
-    bool recorded = false;      // `done` was recorded at least once
+    hipStream_t owner = nullptr;
     bool taken = false;         // between acquire and release on some host thread
-    bool pinned = false;        // handed to a call under stream capture: replays may run at any time
+    bool pinned = false;        // recorded into a graph
     bool dirty = false;         // a call on it failed to get all its kernels onto the stream: clear it before the next use
 };
 struct DeviceState {
     std::vector<CursorBlock> blocks;
     int cus = 0;
 };
-constexpr size_t MAX_CURSOR_BLOCKS = 64;
+constexpr size_t MAX_CURSOR_BLOCKS = 1024;
 std::mutex g_mu;
 DeviceState g_dev[64];
 
@@ -627,7 +625,7 @@ int device_cus(int* cus) {
     return SPINF_OK;
 }
 
-// -> a block no call in flight uses, with room for n_items redo entries; *slot names it for release_block
+// -> the stream's block with room for n_items redo entries; *slot names it for release_block
 int acquire_block(long n_items, bool capturing, hipStream_t stream, int** ptr, int* slot, bool* dirty) {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
@@ -636,8 +634,7 @@ int acquire_block(long n_items, bool capturing, hipStream_t stream, int** ptr, i
     DeviceState& s = g_dev[dev];
     for (size_t i = 0; i < s.blocks.size(); i++) {
         CursorBlock& b = s.blocks[i];
-        if (b.taken || b.pinned || b.cap < n_items) continue;
-        if (b.recorded && b.last != stream && hipEventQuery(b.done) != hipSuccess) continue;   // its last call, on another stream, has not finished
+        if (b.taken || b.pinned || b.owner != stream || b.cap < n_items) continue;
         b.taken = true;
         b.pinned = capturing;
         *ptr = b.ptr;
@@ -646,28 +643,15 @@ int acquire_block(long n_items, bool capturing, hipStream_t stream, int** ptr, i
         return SPINF_OK;
     }
     if (capturing)
-        return spinf_fail(SPINF_E_ARG, "tree_attn: no idle cursor block to record into the graph and none can be allocated during capture: "
-                                       "run one call of this size before the capture, or record spinf_tree_attn_fwd_noalloc");
-    if (s.blocks.size() >= MAX_CURSOR_BLOCKS) {   // wait for a call in flight rather than grow without bound
-        for (size_t i = 0; i < s.blocks.size(); i++) {
-            CursorBlock& b = s.blocks[i];
-            if (b.taken || b.pinned || b.cap < n_items || !b.recorded) continue;
-            e = hipEventSynchronize(b.done);
-            if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: hipEventSynchronize: %s", hipGetErrorString(e));
-            b.taken = true;
-            *ptr = b.ptr;
-            *slot = (int)i;
-            *dirty = b.dirty;
-            return SPINF_OK;
-        }
-        return spinf_fail(SPINF_E_NOMEM, "tree_attn: %zu cursor blocks on one device and none can be waited for", s.blocks.size());
-    }
+        return spinf_fail(SPINF_E_ARG, "tree_attn: this stream has no cursor block of this size yet and none can be allocated during capture: "
+                                       "run one call of this size on the stream before the capture, or record spinf_tree_attn_fwd_noalloc");
+    if (s.blocks.size() >= MAX_CURSOR_BLOCKS) return spinf_fail(SPINF_E_NOMEM, "tree_attn: %zu cursor blocks on one device (one per stream in use)", s.blocks.size());
     CursorBlock b;
     b.cap = n_items < (1 << 16) ? (1 << 16) : 2 * n_items;
+    b.owner = stream;
     e = hipMalloc((void**)&b.ptr, (64 + b.cap) * sizeof(int));
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: hipMalloc: %s", hipGetErrorString(e));
-    e = hipMemset(b.ptr, 0, 64 * sizeof(int));   // the running totals at [NLIST + 3], [NLIST + 4] start at zero; the rest is cleared per call
-    if (e == hipSuccess) e = hipEventCreateWithFlags(&b.done, hipEventDisableTiming);
+    e = hipMemset(b.ptr, 0, 64 * sizeof(int));   // cursors, counts and the running totals at [NLIST + 3], [NLIST + 4] start at zero
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: cursor block: %s", hipGetErrorString(e));
     b.taken = true;
     s.blocks.push_back(b);
@@ -678,13 +662,11 @@ int acquire_block(long n_items, bool capturing, hipStream_t stream, int** ptr, i
 }
 
 // after the call's kernels are on the stream (or failed to get there)
-void release_block(int slot, hipStream_t stream, bool capturing, bool failed) {
+void release_block(int slot, bool failed) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return;
     std::lock_guard<std::mutex> lock(g_mu);
     CursorBlock& b = g_dev[dev].blocks[slot];
-    if (!capturing && hipEventRecord(b.done, stream) == hipSuccess) b.recorded = true;
-    b.last = stream;
     b.dirty = failed;
     b.taken = false;
 }
@@ -947,7 +929,7 @@ static int attn_fwd(const spinf_attn_args* a, void* stream, bool no_alloc) {
         case 256: rc = launch_d<256>(p, rt, nhw, win, a->grp_mode, blocks, s); break;
         default: rc = launch_d512(p, win, a->grp_mode, blocks, s);
     }
-    if (slot >= 0) release_block(slot, s, capturing, rc != SPINF_OK);
+    if (slot >= 0) release_block(slot, rc != SPINF_OK);
     return rc;
 }
 
