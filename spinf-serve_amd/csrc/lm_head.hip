@@ -1,13 +1,16 @@
 // The lm head over the read rows, for gfx950 (MI355X): row gather, logits GEMM, final soft-capping, log-softmax over the
 // vocabulary and column selection in one pass (spinf_serve/scorer.py:247-261 and :340-355).  The reference gathers h[sel],
 // multiplies 1,024 rows at a time by W^T into a [1024, vocab] logits matrix (1 GiB in fp32 at a 262k vocabulary), writes the
-// capped logits and the log-probs (two more such matrices) and keeps a handful of columns.  Here the logits exist only as
-// 128 x 128 tiles in LDS: a tile's contribution to its rows' log-sum-exp and the selected columns leave it, nothing else.
+// capped logits and the log-probs (two more such matrices) and keeps a handful of columns.  Here the logits exist only in the
+// accumulator registers of the GEMM: a tile's contribution to its rows' log-sum-exp and the selected columns leave it, nothing else.
 //
-// Kernel 1 (lm_head_tile_kernel): a workgroup of four waves computes L^T = W h^T for 128 vocabulary rows x 128 read rows with
-// v_mfma_f32_32x32x16_bf16 (W and the gathered h rows staged through LDS, 64 hidden dims per step, double buffered), caps the tile,
-// leaves it in LDS, and writes per read row two (reference, sum of exponentials) pairs (one per 64 vocabulary rows) and the
-// selected columns' capped logits (or, for the extraction rows, the whole tile).
+// Kernel 1 (lm_head_tile_kernel): a workgroup of four waves, one per SIMD, computes L^T = W h^T for 256 vocabulary rows x 256 read
+// rows with v_mfma_f32_32x32x16_bf16, each wave a 128 x 128 quarter (256 accumulator registers: with smaller wave tiles the
+// fragment reads ask more of the LDS than it delivers).  W and the gathered h rows are staged through LDS, 64 hidden dims per
+// step, double buffered.  The epilogue stays in registers: a lane owns one read row per 32 x 32 block, so the (reference, sum of
+// exponentials) pair of a read row over the wave's 128 vocabulary rows is an in-lane reduction and one exchange with the other
+// half of the wave; only blocks that hold a selected column (or, for the extraction rows, all blocks) pass through a small LDS
+// tile to be written out.
 // Kernel 2 (lm_head_finish_kernel): per read row, the pairs are merged into the log-sum-exp, which is subtracted in place.
 //
 // A read row's numbers depend on nothing but that row and W: every logit is one dot product accumulated in the fixed order of the
@@ -23,10 +26,11 @@ typedef __attribute__((ext_vector_type(16))) float f32x16;
 
 namespace {
 
-constexpr int TV = 128, TR = 128, BK = 64;      // tile: vocabulary rows, read rows, hidden dims per step
+constexpr int TV = 256, TR = 256, BK = 64;      // tile: vocabulary rows, read rows, hidden dims per step
+constexpr int WT = 128;                         // a wave's quarter: 128 vocabulary rows x 128 read rows
 constexpr int PITCH = BK * 2 + 16;              // bytes of a staged row (padded: the fragment reads of 32 rows spread over the banks)
 constexpr int STAGE = (TV + TR) * PITCH;        // one buffer: W rows then h rows
-constexpr int LPITCH = TR + 1;                  // floats of a logits-tile row in LDS ([vocabulary][read row])
+constexpr int BP = 33;                          // floats of a row of a wave's 32 x 32 output block in LDS ([vocabulary][read row])
 constexpr float LOG2E = 1.4426950408889634f;
 
 struct HeadParams {
@@ -38,6 +42,7 @@ struct HeadParams {
     const long* cols; int n_cols;
     float* out; long out_ld;
     float2* part; int n_part;   // [rows, n_part] pairs; n_part = 2 * vocabulary tiles
+    int row_tiles;
 };
 
 __device__ __forceinline__ float to_bf16(float x) { return (float)(__bf16)x; }
@@ -57,120 +62,209 @@ __device__ __forceinline__ float softcap(float x, float cap, float inv_cap) {
 }
 
 template <bool CAPPED, bool BF16>
-__global__ __launch_bounds__(256) void lm_head_tile_kernel(const HeadParams p) {
-    static_assert(TV * LPITCH * 4 <= 2 * STAGE, "the logits tile reuses the staging buffers");
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void lm_head_tile_kernel(const HeadParams p) {
     __shared__ __attribute__((aligned(16))) char lds[2 * STAGE];
     const int tid = threadIdx.x, lane = tid & 63, m = lane & 31, g = lane >> 5;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6), wv = w & 1, wr = w >> 1;
-    const int r0 = blockIdx.x * TR, v0 = blockIdx.y * TV;   // read-row tiles fastest: the tiles that share W rows run together
+    // Workgroups go round the 8 XCDs (each with its own L2) in launch order.  The read-row tiles of one vocabulary tile share its
+    // W rows, so they take consecutive launch slots of ONE XCD: W then comes from HBM once and from that L2 for the others (with
+    // the tiles of a vocabulary tile spread over the XCDs every one of them fetched W from HBM: 4 x 1.3 GB at 1,024 read rows).
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int vtile = (slot / p.row_tiles) * 8 + xcd, rtile = slot % p.row_tiles;
+    if (vtile * TV >= p.vocab) return;
+    const int r0 = rtile * TR, v0 = vtile * TV;
 
-    // ---- loader: a staged tile row is 64 hidden dims = 8 chunks of 16 bytes; thread t copies chunks t, t + 256, ... of W and of h
-    const __bf16* src_w[4];
-    const __bf16* src_h[4];
-    int dst[4];
+    // ---- loader: a staged tile row is 64 hidden dims = 8 chunks of 16 bytes; thread t copies chunk t % 8 of rows t / 8 + 32 i
+    const int kc = tid & 7;
+    int row_h[8];   // this thread's rows of h (through the row list); its rows of W are v0 + t / 8 + 32 i, clamped to the vocabulary
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const int c = tid + 256 * i, row = c >> 3, kc = c & 7;
-        const int vr = v0 + row < p.vocab ? v0 + row : p.vocab - 1;
-        int rr = r0 + row < p.rows ? r0 + row : p.rows - 1;
-        const long hr = p.sel ? p.sel[rr] : (long)rr;
-        src_w[i] = p.w + (long)vr * p.w_ld + kc * 8;
-        src_h[i] = p.h + hr * p.h_ld + kc * 8;
-        dst[i] = row * PITCH + kc * 16;
+    for (int i = 0; i < 8; i++) {
+        const int row = (tid >> 3) + 32 * i;
+        const int rr = r0 + row < p.rows ? r0 + row : p.rows - 1;
+        row_h[i] = p.sel ? (int)p.sel[rr] : rr;
     }
-    bf16x8 rw[4], rh[4];
-    auto fetch = [&](const int k0) __attribute__((always_inline)) {
+    // The row list's loads end here: a value that still counts as "in flight" when the loop is entered makes the compiler wait
+    // for it at every use, and such a wait also waits for every tile load issued before it.
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            rw[i] = *(const bf16x8*)(src_w[i] + k0);
-            rh[i] = *(const bf16x8*)(src_h[i] + k0);
-        }
+    for (int i = 0; i < 8; i++) asm volatile("" : "+v"(row_h[i]));
+    const int row_w0 = v0 + (tid >> 3), last_w = p.vocab - 1;
+    auto src_w = [&](const int i, const int k0) __attribute__((always_inline)) {
+        const int r = row_w0 + 32 * i < last_w ? row_w0 + 32 * i : last_w;
+        return p.w + (long)r * p.w_ld + (kc * 8 + k0);
     };
-    auto stash = [&](char* buf) __attribute__((always_inline)) {
+    auto src_h = [&](const int i, const int k0) __attribute__((always_inline)) { return p.h + (long)row_h[i] * p.h_ld + (kc * 8 + k0); };
+    const int dst = (tid >> 3) * PITCH + kc * 16;
+    const int nk = p.hidden / BK;
+    // Two register sets: the rows of step kt + 2 are requested while step kt is computed and are written to LDS during step
+    // kt + 1, so a load has a step and a half (about 3 k cycles of MFMA work) to arrive.  The loads and the waits for them are
+    // inline assembly: the compiler's own wait insertion, unsure across the loop's back edge which registers still have a load
+    // in flight, waited for the set just requested whenever it touched a register of the other one.  Loads complete in order, so
+    // "the older set has landed" is vmcnt(16) while a younger set is in flight and vmcnt(0) otherwise; the registers of the set
+    // pass through the waiting asm, which keeps their uses behind it.
+    bf16x8 rw[2][8], rh[2][8];
+    auto request = [&](const int set, const int i, const int k0) __attribute__((always_inline)) {
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(rw[set][i]) : "v"(src_w(i, k0)) : "memory");
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(rh[set][i]) : "v"(src_h(i, k0)) : "memory");
+    };
+    auto zero_set = [&](const int set) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            *(bf16x8*)(buf + dst[i]) = rw[i];
-            *(bf16x8*)(buf + TV * PITCH + dst[i]) = rh[i];
-        }
+        for (int i = 0; i < 8; i++)
+#pragma unroll
+            for (int j = 0; j < 8; j++) { rw[set][i][j] = (__bf16)0.f; rh[set][i][j] = (__bf16)0.f; }
+    };
+    auto landed = [&](const int set, const bool younger_in_flight) __attribute__((always_inline)) {
+        if (younger_in_flight) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        asm volatile("" : "+v"(rw[set][0]), "+v"(rw[set][1]), "+v"(rw[set][2]), "+v"(rw[set][3]), "+v"(rw[set][4]), "+v"(rw[set][5]), "+v"(rw[set][6]), "+v"(rw[set][7]));
+        asm volatile("" : "+v"(rh[set][0]), "+v"(rh[set][1]), "+v"(rh[set][2]), "+v"(rh[set][3]), "+v"(rh[set][4]), "+v"(rh[set][5]), "+v"(rh[set][6]), "+v"(rh[set][7]));
     };
 
-    f32x16 acc[2][2];
+    f32x16 acc[4][4];   // [vocabulary block a][read-row block b]
 #pragma unroll
-    for (int a = 0; a < 2; a++)
+    for (int a = 0; a < 4; a++)
 #pragma unroll
-        for (int b = 0; b < 2; b++)
+        for (int b = 0; b < 4; b++)
 #pragma unroll
             for (int i = 0; i < 16; i++) acc[a][b][i] = 0.f;
 
-    const int nk = p.hidden / BK;
-    fetch(0);
-    stash(lds);
-    __syncthreads();
-    for (int kt = 0; kt < nk; kt++) {
+    // One step, with the memory work dealt out between the MFMAs.  The wave is alone on its SIMD: whatever it issues in one piece
+    // (16 global loads, 16 LDS stores, 8 fragment reads) is time the matrix core waits, while an instruction placed between two
+    // MFMAs runs in their shadow.  Sixteen groups of four MFMAs per step; groups 0 - 7 each request one W and one h piece of step
+    // kt + 2 into `set`, groups 8 - 15 each move one pair of step kt + 1 (the other set) to the other LDS buffer, and every group
+    // of the first three quarters reads two fragments of the next quarter.  The steps come in pairs with no branch around the
+    // MFMAs (accumulators that are live across a merge of two paths cost the register allocator hundreds of copies): an odd
+    // number of steps is rounded up and the extra step multiplies zeros; what the last steps move to LDS is never read.
+    const int nk2 = (nk + 1) & ~1;
+    auto step = [&](const int kt, const int set) __attribute__((always_inline)) {
         const char* buf = lds + (kt & 1) * STAGE;
-        if (kt + 1 < nk) fetch((kt + 1) * BK);
-        const char* fa = buf + (wv * 64 + m) * PITCH + 16 * g;
-        const char* fb = buf + (TV + wr * 64 + m) * PITCH + 16 * g;
+        char* nbuf = lds + ((kt + 1) & 1) * STAGE;
+        const char* fa = buf + (wv * WT + m) * PITCH + 16 * g;
+        const char* fb = buf + (TV + wr * WT + m) * PITCH + 16 * g;
+        const int k0 = (kt + 2) * BK;
+        const bool more = kt + 2 < nk;   // wave-uniform
+        if (!more) zero_set(set);
+        bf16x8 av[2][4], bv[2][4];
 #pragma unroll
-        for (int ks = 0; ks < BK / 16; ks++) {
-            bf16x8 av[2], bv[2];
-#pragma unroll
-            for (int a = 0; a < 2; a++) av[a] = *(const bf16x8*)(fa + 32 * a * PITCH + 32 * ks);
-#pragma unroll
-            for (int b = 0; b < 2; b++) bv[b] = *(const bf16x8*)(fb + 32 * b * PITCH + 32 * ks);
-#pragma unroll
-            for (int a = 0; a < 2; a++)
-#pragma unroll
-                for (int b = 0; b < 2; b++) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[a], bv[b], acc[a][b], 0, 0, 0);
+        for (int a = 0; a < 4; a++) {
+            av[0][a] = *(const bf16x8*)(fa + 32 * a * PITCH);
+            bv[0][a] = *(const bf16x8*)(fb + 32 * a * PITCH);
         }
-        if (kt + 1 < nk) {
-            stash(lds + ((kt + 1) & 1) * STAGE);
-            __syncthreads();
-        }
-    }
-    __syncthreads();   // everyone is done with the staging buffers: the logits tile goes there
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++)
+#pragma unroll
+            for (int a = 0; a < 4; a++) {
+                const int grp = 4 * ks + a;
+                if (grp < 8) {
+                    if (more) request(set, grp, k0);
+                } else {
+                    if (grp == 8) landed(set ^ 1, more);
+                    *(bf16x8*)(nbuf + dst + 32 * (grp - 8) * PITCH) = rw[set ^ 1][grp - 8];
+                    *(bf16x8*)(nbuf + TV * PITCH + dst + 32 * (grp - 8) * PITCH) = rh[set ^ 1][grp - 8];
+                }
+                if (ks < 3) {
+                    av[(ks + 1) & 1][a] = *(const bf16x8*)(fa + 32 * a * PITCH + 32 * (ks + 1));
+                    bv[(ks + 1) & 1][a] = *(const bf16x8*)(fb + 32 * a * PITCH + 32 * (ks + 1));
+                }
+#pragma unroll
+                for (int b = 0; b < 4; b++) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[ks & 1][a], bv[ks & 1][b], acc[a][b], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        __syncthreads();
+    };
 
-    // ---- the capped logits tile in LDS, [vocabulary row][read row].  Register i of a 32 x 32 block holds vocabulary row
-    // 8 (i / 4) + 4 g + i % 4 of the block for read row m.
-    float* tile = (float*)lds;
 #pragma unroll
-    for (int a = 0; a < 2; a++)
+    for (int i = 0; i < 8; i++) request(0, i, 0);
+    if (nk > 1) {
 #pragma unroll
-        for (int b = 0; b < 2; b++)
+        for (int i = 0; i < 8; i++) request(1, i, BK);
+    } else zero_set(1);
+    landed(0, nk > 1);
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        *(bf16x8*)(lds + dst + 32 * i * PITCH) = rw[0][i];
+        *(bf16x8*)(lds + TV * PITCH + dst + 32 * i * PITCH) = rh[0][i];
+    }
+    __syncthreads();
+    for (int kt = 0; kt < nk2; kt += 2) {
+        step(kt, 0);
+        step(kt + 1, 1);
+    }
+    __syncthreads();   // everyone is done with the staging buffers: the waves' output blocks go there
+
+    // ---- the capped logits, in place.  Register i of block (a, b) holds vocabulary row vw0 + 32 a + 8 (i / 4) + 4 g + i % 4
+    // for read row rw0 + 32 b + m.
+    const int vw0 = v0 + wv * WT, rw0 = r0 + wr * WT;
+#pragma unroll
+    for (int a = 0; a < 4; a++)
+#pragma unroll
+        for (int b = 0; b < 4; b++)
 #pragma unroll
             for (int i = 0; i < 16; i++) {
                 float x = acc[a][b][i];
                 if (BF16) x = to_bf16(x);
                 if (CAPPED) x = softcap<BF16>(x, p.cap, p.inv_cap);
-                tile[(wv * 64 + 32 * a + 8 * (i >> 2) + 4 * g + (i & 3)) * LPITCH + wr * 64 + 32 * b + m] = x;
+                acc[a][b][i] = x;
             }
-    __syncthreads();
-
-    // ---- per read row, two (reference, sum) pairs: thread t takes read row t % 128 and vocabulary rows 64 (t / 128) .. + 63
-    {
-        const int row = tid & (TR - 1), half = tid >> 7;
-        const int nv = p.vocab - (v0 + 64 * half) < 64 ? p.vocab - (v0 + 64 * half) : 64;   // rows of the vocabulary that exist
-        const float* col = tile + 64 * half * LPITCH + row;
-        float ref = CAPPED ? p.cap : -INFINITY, sum = 0.f;
-        if (!CAPPED)
-            for (int j = 0; j < nv; j++) ref = fmaxf(ref, col[j * LPITCH]);
-        for (int j = 0; j < nv; j++) sum += __builtin_amdgcn_exp2f((col[j * LPITCH] - ref) * LOG2E);
-        if (r0 + row < p.rows) p.part[(long)(r0 + row) * p.n_part + 2 * blockIdx.y + half] = make_float2(ref, sum);
+    // ---- per read row one (reference, sum) pair over the wave's 128 vocabulary rows: 64 values in this lane, 64 in lane ^ 32
+    const bool tail = vw0 + WT > p.vocab;   // wave-uniform: some of the wave's vocabulary rows do not exist
+#pragma unroll
+    for (int b = 0; b < 4; b++) {
+        float ref = CAPPED ? p.cap : -INFINITY;
+        if (!CAPPED) {
+#pragma unroll
+            for (int a = 0; a < 4; a++)
+#pragma unroll
+                for (int i = 0; i < 16; i++)
+                    if (!tail || vw0 + 32 * a + 8 * (i >> 2) + 4 * g + (i & 3) < p.vocab) ref = fmaxf(ref, acc[a][b][i]);
+            ref = fmaxf(ref, __shfl_xor(ref, 32));
+        }
+        float sum = 0.f;
+        if (ref != -INFINITY) {
+#pragma unroll
+            for (int a = 0; a < 4; a++)
+#pragma unroll
+                for (int i = 0; i < 16; i++)
+                    if (!tail || vw0 + 32 * a + 8 * (i >> 2) + 4 * g + (i & 3) < p.vocab) sum += __builtin_amdgcn_exp2f((acc[a][b][i] - ref) * LOG2E);
+        }
+        const float other = __shfl_xor(sum, 32);
+        sum = g == 0 ? sum + other : other + sum;   // both halves add in the same order
+        const int row = rw0 + 32 * b + m;
+        if (g == 0 && row < p.rows) p.part[(long)row * p.n_part + 2 * vtile + wv] = make_float2(ref, sum);
     }
-    // ---- what leaves the tile
-    if (p.cols) {   // the selected columns: wave w looks at columns w, w + 4, ...
-        for (int c = w; c < p.n_cols; c += 4) {
+    // ---- what leaves the tile: a 32 x 32 block goes through the wave's LDS tile, vocabulary-major
+    float* blk = (float*)lds + w * 32 * BP;
+    auto put = [&](const f32x16& x) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 16; i++) blk[(8 * (i >> 2) + 4 * g + (i & 3)) * BP + m] = x[i];
+    };
+    if (p.cols) {   // the selected columns: rarely one of them lies in this wave's 128 vocabulary rows
+        for (int c = 0; c < p.n_cols; c++) {
             const long col = p.cols[c];
-            if (col < v0 || col >= v0 + TV) continue;
-            for (int row = lane; row < TR; row += 64)
-                if (r0 + row < p.rows) p.out[(long)(r0 + row) * p.out_ld + c] = tile[(col - v0) * LPITCH + row];
+            if (col < vw0 || col >= vw0 + WT) continue;   // wave-uniform
+            const int ca = (int)(col - vw0) >> 5, cv = (int)(col - vw0) & 31;
+#pragma unroll
+            for (int a = 0; a < 4; a++) {
+                if (a != ca) continue;
+#pragma unroll
+                for (int b = 0; b < 4; b++) {
+                    put(acc[a][b]);
+                    const int row = rw0 + 32 * b + m;
+                    if (g == 0 && row < p.rows) p.out[(long)row * p.out_ld + c] = blk[cv * BP + m];
+                }
+            }
         }
-    } else {        // the extraction rows: the whole tile, a read row's 128 values as two runs of 64
-        for (int row = w; row < TR; row += 4) {
-            if (r0 + row >= p.rows) break;
-            for (int v = lane; v < TV; v += 64)
-                if (v0 + v < p.vocab) p.out[(long)(r0 + row) * p.out_ld + v0 + v] = tile[v * LPITCH + row];
-        }
+    } else {        // the extraction rows: every block, a read row's 32 values of the block as one 128-byte run
+#pragma unroll
+        for (int a = 0; a < 4; a++)
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+                put(acc[a][b]);
+                const int vb = vw0 + 32 * a + m;
+                for (int r = g; r < 32; r += 2) {
+                    const int row = rw0 + 32 * b + r;
+                    if (row < p.rows && vb < p.vocab) p.out[(long)row * p.out_ld + vb] = blk[m * BP + r];
+                }
+            }
     }
 }
 
@@ -182,7 +276,7 @@ __global__ __launch_bounds__(256) void lm_head_finish_kernel(const HeadParams p)
     float m = -INFINITY, s = 0.f;
     for (int i = threadIdx.x; i < p.n_part; i += 256) {
         const float2 q = part[i];
-        if (q.y <= 0.f) continue;   // a half tile past the end of the vocabulary
+        if (q.y <= 0.f) continue;   // a wave's quarter past the end of the vocabulary
         const float mn = fmaxf(m, q.x);
         s = (m == -INFINITY ? 0.f : s * __builtin_amdgcn_exp2f((m - mn) * LOG2E)) + q.y * __builtin_amdgcn_exp2f((q.x - mn) * LOG2E);
         m = mn;
@@ -247,7 +341,9 @@ extern "C" int spinf_lm_head_fwd(const spinf_lm_head_args* a, void* stream) {
     p.cap = a->softcap; p.inv_cap = a->softcap > 0.f ? 1.0f / a->softcap : 0.f;
     p.cols = a->cols; p.n_cols = (int)a->n_cols; p.out = a->out; p.out_ld = a->out_ld;
     p.part = (float2*)a->workspace; p.n_part = (int)parts_of(a);
-    const dim3 grid((unsigned)((a->rows + TR - 1) / TR), (unsigned)((a->vocab + TV - 1) / TV));
+    p.row_tiles = (int)((a->rows + TR - 1) / TR);
+    const int64_t vtiles = (a->vocab + TV - 1) / TV;
+    const dim3 grid((unsigned)(p.row_tiles * ((vtiles + 7) / 8 * 8)));
     hipStream_t s = (hipStream_t)stream;
     const bool capped = a->softcap > 0.f, bf = a->logits_dtype == 1;
     if (capped && bf) hipLaunchKernelGGL((lm_head_tile_kernel<true, true>), grid, dim3(256), 0, s, p);
