@@ -112,8 +112,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
             for (int j = 0; j < 8; j++) { rw[set][i][j] = (__bf16)0.f; rh[set][i][j] = (__bf16)0.f; }
     };
-    auto landed = [&](const int set, const bool younger_in_flight) __attribute__((always_inline)) {
-        if (younger_in_flight) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    auto landed = [&](const int set, const bool younger_in_flight, const int younger) __attribute__((always_inline)) {
+        if (younger_in_flight && younger == 9) asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+        else if (younger_in_flight) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
         else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         asm volatile("" : "+v"(rw[set][0]), "+v"(rw[set][1]), "+v"(rw[set][2]), "+v"(rw[set][3]), "+v"(rw[set][4]), "+v"(rw[set][5]), "+v"(rw[set][6]), "+v"(rw[set][7]));
         asm volatile("" : "+v"(rh[set][0]), "+v"(rh[set][1]), "+v"(rh[set][2]), "+v"(rh[set][3]), "+v"(rh[set][4]), "+v"(rh[set][5]), "+v"(rh[set][6]), "+v"(rh[set][7]));
@@ -154,10 +155,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
             for (int a = 0; a < 4; a++) {
                 const int grp = 4 * ks + a;
-                if (grp < 8) {
-                    if (more) request(set, grp, k0);
-                } else {
-                    if (grp == 8) landed(set ^ 1, more);
+                if (more) {   // one request per group: W pieces in the even groups, h pieces in the odd ones
+                    if (grp & 1) asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(rh[set][grp >> 1]) : "v"(src_h(grp >> 1, k0)) : "memory");
+                    else asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(rw[set][grp >> 1]) : "v"(src_w(grp >> 1, k0)) : "memory");
+                }
+                if (grp >= 8) {
+                    if (grp == 8) landed(set ^ 1, more, 9);   // nine of this step's requests are younger
                     *(bf16x8*)(nbuf + dst + 32 * (grp - 8) * PITCH) = rw[set ^ 1][grp - 8];
                     *(bf16x8*)(nbuf + TV * PITCH + dst + 32 * (grp - 8) * PITCH) = rh[set ^ 1][grp - 8];
                 }
@@ -178,7 +181,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
         for (int i = 0; i < 8; i++) request(1, i, BK);
     } else zero_set(1);
-    landed(0, nk > 1);
+    landed(0, nk > 1, 16);
 #pragma unroll
     for (int i = 0; i < 8; i++) {
         *(bf16x8*)(lds + dst + 32 * i * PITCH) = rw[0][i];
