@@ -202,7 +202,7 @@ __global__ __launch_bounds__(512) void tree_attn_ring_kernel(const AttnParams p)
     constexpr int NDT = D / 32;    // 32-wide slices of the head dimension in O^T
     constexpr int NVF = 2 * NDT;   // V^T fragments of one 32-key block
     constexpr int PFD = D >= 256 ? 2 : 8;   // fragment read-ahead: at head dim 256 one more spills a query fragment inside the tile loop
-    constexpr int PF = NS < PFD ? NS : PFD;
+    constexpr int PF = D >= 256 ? 4 : (NS < PFD ? NS : PFD);   // K fragments are live in the score phase only, where registers are free
     constexpr int VPF = NVF < PFD ? NVF : PFD;
     static_assert(NSLOT * G::BUFB + 8 * 32 * SROW + NDESC * 16 + 256 <= 160 * 1024, "LDS budget");
     __shared__ __attribute__((aligned(16))) char ring[NSLOT * G::BUFB];
