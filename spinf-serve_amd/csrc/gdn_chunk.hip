@@ -24,22 +24,6 @@
 
 using namespace gdn_tiles;
 
-#ifdef SPINF_TRACE
-#ifndef SPINF_TRACE_THREAD
-#define SPINF_TRACE_THREAD 64
-#endif
-__device__ long g_gdn_trace[16];
-extern "C" int spinf_debug_gdn_trace(long* out) { return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_gdn_trace), sizeof(long) * 16, 0, hipMemcpyDeviceToHost); }
-#define GT_CLK(v) const long v = clock64()
-#ifndef SPINF_TRACE_PAIRS
-#define SPINF_TRACE_PAIRS false
-#endif
-#define GT_ADD(slot, val) do { if (PAIRS == SPINF_TRACE_PAIRS && threadIdx.x == SPINF_TRACE_THREAD && blockIdx.x == 7) g_gdn_trace[slot] += (val); } while (0)
-#else
-#define GT_CLK(v) do { } while (0)
-#define GT_ADD(slot, val) do { } while (0)
-#endif
-
 namespace {
 
 constexpr int KD = 128;        // key head dim
@@ -234,7 +218,6 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
     fetch_rows(1);
 
     for (int j = 0; j < n_chunks; j++) {
-        GT_CLK(g0);
         lds_barrier();   // every wave is done with the previous chunk's tiles
         // ---- stage the chunk from the prefetch registers (rows >= L are zero): cumulative g, beta, stream rows, K / Q / V
         if (tid < CH) {
@@ -256,7 +239,6 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
             }
         }
         lds_barrier();
-        GT_CLK(g1);
 
         // Token tiles: tile t = chunk rows 16 t .. 16 t + 15.  In a transposed token x token result the lane owns row
         // i = 16 it + c and its registers hold columns j = 16 jt + 4 q4 + r.
@@ -290,7 +272,6 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
             *(bf16x4*)(Ps + i * LP + 16 * jt + 4 * q4) = p4;
         }
         lds_barrier();
-        GT_CLK(g2);
 
         // ---- T = (I - A)^-1 on wave 0: rows of the diagonal blocks by substitution in registers (lane groups 0 and 2 the
         // upper-left block, 1 and 3 the lower-right one, in the same instructions), then the lower-left block
@@ -350,7 +331,6 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
             }
         }
         lds_barrier();   // T visible; A and the T blocks are dead, -W may take their place
-        GT_CLK(g3);
 
         // ---- U[i][v] = sum_j Tu[i][j] V[j][v] for this wave's columns (lane = column v, registers = rows i), and this wave's
         // share of -W^T[k][i] = sum_j K[j][k] Tw[i][j]: key tiles 2w and 2w + 1, stored as -W[i][k]
@@ -382,7 +362,6 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
             }
         }
         lds_barrier();   // -W visible; every wave has read its V columns
-        GT_CLK(g4);
 
         // ---- V' = U + (-W) S and Q S over the 128 key rows, 32 at a time (the state tiles 2s and 2s + 1 are the B operand)
 #pragma unroll
@@ -405,11 +384,9 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
                 }
             }
         }
-        GT_CLK(g5);
         // the next chunk's rows are requested here, where few registers are live; they arrive during the state update
         fetch_data();          // chunk j + 1, whose rows are known since the previous chunk
         fetch_rows(j + 2);
-        GT_CLK(g5a);
         // ---- O[i][v] = s e^{G_i} (Q S)[i][v] + sum_j P[i][j] V'[j][v], rows i = 16 it + 4 q4 + r; through LDS for 16-byte stores
         f32x4 Gj[NT];
 #pragma unroll
@@ -434,7 +411,6 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
             }
         }
         wave_lds_order();
-        GT_CLK(g5b);
         // row i = 16 it + lane%16, values 8 (lane/16) ..+7 of this wave's 32: two transposing reads, one 16-byte store
 #pragma unroll
         for (int it = 0; it < NT; it++) {
@@ -445,7 +421,6 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
             const int orow = Rs[row];      // -1: no such row in this chunk
             if (orow >= 0) *(bf16x8*)(p.o + row_offset(orow, p.o_tok) + hv * VD + 32 * w + 8 * q4) = join(lo, hi);
         }
-        GT_CLK(g6);
         // ---- S[k][v] = e^{G_L} S[k][v] + sum_j K[j][k] (V' e^{G_L - G_j})[j][v]; skipped when nothing reads the state again
         if (!run_mode && (j + 1 < n_chunks || keep)) {
             const float GL = Gs[CH - 1];
@@ -471,8 +446,6 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
                 }
             }
         }
-        GT_CLK(g7);
-        GT_ADD(0, g1 - g0); GT_ADD(1, g2 - g1); GT_ADD(2, g3 - g2); GT_ADD(3, g4 - g3); GT_ADD(4, g5 - g4); GT_ADD(5, g6 - g5); GT_ADD(6, g7 - g6); GT_ADD(8, 1); GT_ADD(9, g5a - g5); GT_ADD(10, g5b - g5a); GT_ADD(11, g6 - g5b);
     }
 
     if (keep) {

@@ -243,20 +243,6 @@ __global__ __launch_bounds__(256) void tree_attn_exact_kernel(const AttnParams p
 }
 
 // ------------------------------------------------------------------------------------------------ fast pass, persistent
-#ifdef SPINF_TRACE
-__device__ long g_trace[16 * 4096];
-extern "C" int spinf_debug_trace(long* out, int n) { return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_trace), sizeof(long) * n, 0, hipMemcpyDeviceToHost); }
-#define TRACE_ADD(slot, val) do { if (threadIdx.x == 64 && blockIdx.x < 4096) g_trace[blockIdx.x * 16 + (slot)] += (val); } while (0)
-#define TRACE_CLK(var) const long var = clock64()
-#define TRACE_WALL(var) const long var = wall_clock64()
-#define TRACE_SET(slot, val) do { if (threadIdx.x == 64 && blockIdx.x < 4096) g_trace[blockIdx.x * 16 + (slot)] = (val); } while (0)
-#else
-#define TRACE_ADD(slot, val) do { } while (0)
-#define TRACE_CLK(var) do { } while (0)
-#define TRACE_WALL(var) do { } while (0)
-#define TRACE_SET(slot, val) do { } while (0)
-#endif
-
 // NHW = 1: four waves, each with RT heads of the item.  NHW = 2: eight waves, waves 4..7 take the item's second set of RT heads
 // on the same K / V tiles (two waves per SIMD: one wave's softmax runs under the other's MFMAs).
 // ROWS: q, k, v, o hold the real tokens only (compact rows); the stream positions of the plan are mapped through row_of.
@@ -286,8 +272,6 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
     __shared__ __attribute__((aligned(16))) char stage_all[STAGE_IN_TILE ? 16 : 4 * NHW * 32 * 144];
     __shared__ int s_next[2];         // item grabbed by thread 0 for the whole workgroup, double buffered
 
-    TRACE_CLK(tk0);
-    TRACE_WALL(tw0);
     const Lane<D, TK, DV> L(p);
     char* const stage_own = stage_all + (STAGE_IN_TILE ? 0 : L.w * 32 * 144);
 
@@ -502,19 +486,11 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
         base = 0;
         pstage = 0;
         nxt_ok = false;
-        TRACE_WALL(twi);
-        TRACE_SET(5, twi);
-        TRACE_SET(6, (long)ne);
-        TRACE_SET(4, (long)cur_idx);
-        TRACE_SET(3, (long)xcc);
         for (i = 0; i < ne; i++, par ^= 1) {
             const char* buf = bufs + par * G::BUFB;
             const unsigned oth = lds_addr(bufs + (par ^ 1) * G::BUFB);
-            TRACE_CLK(tc0);
             __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's DMA into buf (and its other loads) have landed
             __syncthreads();                     // ... and everyone's; the other buffer is free; s_next[gslot] is visible
-            TRACE_CLK(tc1);
-            TRACE_ADD(8, tc1 - tc0);
             // next-item prefetch, one stage per step
             if (i < grab_at) {
             } else if (i == grab_at) {
@@ -544,14 +520,9 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
             }
             const int2 en = ent_cur[i - base];
             compute_tile(buf, __builtin_amdgcn_readfirstlane(en.x), (unsigned)__builtin_amdgcn_readfirstlane(en.y) >> (2 * L.wr));
-            TRACE_CLK(tc2);
-            TRACE_ADD(9, tc2 - tc1);
         }
         // ---- item finished: output (or hand the item to the exact pass), switch to the next item
-        TRACE_CLK(tc3);
         const int any_viol = __builtin_amdgcn_readfirstlane(__syncthreads_or(viol));
-        TRACE_CLK(tc3b);
-        TRACE_ADD(12, tc3b - tc3);
         if (any_viol) {
             if (threadIdx.x == 0) p.redo[atomicAdd(&p.counters[NLIST + 1], 1)] = cur_idx;
         } else {
@@ -559,13 +530,6 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
             char* const stage = STAGE_IN_TILE ? bufs + (par ^ 1) * G::BUFB + L.w * 32 * 144 : stage_own;
             store_rows<DV, RT, ROWS>(p, L, stage, o, l, item_t(cur), item_hp(cur) * HPI + L.wh * RT);
         }
-        TRACE_CLK(tc4);
-        TRACE_ADD(10, tc4 - tc3);
-        TRACE_ADD(11, 1);
-        TRACE_WALL(twe);
-        TRACE_SET(13, tw0);
-        TRACE_SET(7, twe);
-        TRACE_SET(14, tc4 - tk0);
         cur_ok = nxt_ok;
         if (!cur_ok) break;
         // finish whatever of the next item's prefetch has not happened yet (one-tile items), then switch
