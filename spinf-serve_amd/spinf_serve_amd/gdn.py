@@ -10,23 +10,42 @@ q and k arrive l2-normalised; g is the log decay (fp32), beta the write strength
 from __future__ import annotations
 
 import ctypes as C
+from typing import Optional
 
 import torch
 
 from . import _lib
 
 
+@torch.library.custom_op("spinf::gdn_scan", mutates_args=("o", "ht"))
+def _gdn_scan_op(mode: int, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor, beta: torch.Tensor, scale: float,
+                 cu: torch.Tensor, n: int, h0: Optional[torch.Tensor], h0_idx: Optional[torch.Tensor], ht: Optional[torch.Tensor],
+                 ht_idx: Optional[torch.Tensor], idx: Optional[torch.Tensor], o: torch.Tensor, max_len: int) -> None:
+    """the registered op over spinf_gdn_fwd: mode 0 = recurrent, 1 = chunked; writes the call's rows of `o` and the kept states
+    into `ht` (inductor sees one opaque node that mutates the two, as it sees the reference's @torch.compiler.disable call)"""
+    _launch(mode, q, k, v, g, beta, scale, cu, n, h0, h0_idx, ht, ht_idx, idx, o, max_len)
+
+
 def _run(mode, q, k, v, g, beta, scale, cu, n, h0, h0_idx, ht, ht_idx, idx, o, max_len):
+    if not q.is_cuda:
+        raise RuntimeError("the Gated DeltaNet scan runs on ROCm device tensors only (no CPU path)")
+    g = g if g.dtype == torch.float32 else g.float()
+    beta = beta if beta.dtype == torch.bfloat16 else beta.to(torch.bfloat16)
+    if o is None:
+        o = torch.zeros_like(v) if idx is not None else torch.empty_like(v)
+    _gdn_scan_op(mode, q, k, v, g, beta, float(scale), cu, int(n), h0, h0_idx, ht, ht_idx, idx, o, int(max_len))
+    return o
+
+
+def _launch(mode, q, k, v, g, beta, scale, cu, n, h0, h0_idx, ht, ht_idx, idx, o, max_len):
     if not q.is_cuda:
         raise RuntimeError("the Gated DeltaNet scan runs on ROCm device tensors only (no CPU path)")
     _, rows, H, K = k.shape
     HV, V = v.shape[2], v.shape[3]
     if q.dtype != torch.bfloat16 or k.dtype != torch.bfloat16 or v.dtype != torch.bfloat16:
         raise ValueError("q, k, v must be bf16")
-    g = g if g.dtype == torch.float32 else g.float()
-    beta = beta if beta.dtype == torch.bfloat16 else beta.to(torch.bfloat16)
-    if o is None:
-        o = torch.zeros_like(v) if idx is not None else torch.empty_like(v)
+    if g.dtype != torch.float32 or beta.dtype != torch.bfloat16:
+        raise ValueError("g must be fp32 and beta bf16")
     if not (o.is_contiguous() or (o.stride(-1) == 1 and o.stride(-2) == V)):
         raise ValueError("o must be dense per row")
     if q.stride(1) != k.stride(1) or g.stride(1) != beta.stride(1):

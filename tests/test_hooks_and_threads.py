@@ -29,6 +29,17 @@ def test_registration_with_transformers():
     assert AttentionInterface()["tree_flex_test"] is sa.tree_flex_forward
 
 
+def test_ops_are_registered_with_torch_library():
+    """the kernels are opaque torch.library ops (inductor never traces into them); the scan mutates its output and state tensors"""
+    for name in ("tree_attn", "gdn_scan", "lm_logprobs", "lm_head_logprobs"):
+        assert hasattr(torch.ops.spinf, name), name
+    schema = str(torch.ops.spinf.gdn_scan.default._schema)
+    assert "Tensor(a" in schema and "o" in schema and "-> ()" in schema, schema
+    with pytest.raises(RuntimeError):   # no CPU path
+        sa.gdn.recurrent(torch.zeros(1, 4, 1, 128, dtype=torch.bfloat16), torch.zeros(1, 4, 1, 128, dtype=torch.bfloat16), torch.zeros(1, 4, 2, 128, dtype=torch.bfloat16),
+                         torch.zeros(1, 4, 2), torch.zeros(1, 4, 2, dtype=torch.bfloat16), 1.0, torch.tensor([0, 4]), 1)
+
+
 def test_plan_compilers_from_two_threads():
     """tile plans, their schedules and recurrent-layer plans built at the same time on different streams equal the ones built
     one after the other"""
