@@ -487,7 +487,10 @@ __global__ __launch_bounds__(512) void tree_attn_ring_kernel(const AttnParams p)
                 flag = __builtin_amdgcn_readfirstlane(fv);
             }
             have_pf = false;
-            claim(n0, n1, n2, n3);
+            // The waves of the second head set run behind those of the first (a SIMD's arbiter favours its older wave), and the
+            // kernel ends when they do: they leave the recycling to the first set, which is ahead and mostly waiting for
+            // flags anyway, and lend a hand only from inside a wait.
+            if (L.w < 4) claim(n0, n1, n2, n3);
             if (dead) break;
             const unsigned bits = (unsigned)d.y;
             last = (bits & DESC_LAST) != 0;
