@@ -365,7 +365,9 @@ def main():
                 roofline={"bound": "mfma", "achieved": tfl, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": tfl / PEAK_BF16_TFLOPS,
                           "traffic": TRAFFIC_BYTES.get(args.workload) if args.contents is None and args.rows == "stream" else None, "kernel_ms": ms,
                           "kernel_ms_min": float(np.min(kern)), "useful_flops": flops,
-                          "algorithmic_bytes": cfg.bytes() * len(layers), "hbm_frac_at_algorithmic_bytes": cfg.bytes() * len(layers) / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS},
+                          "algorithmic_bytes": cfg.bytes() * len(layers), "hbm_frac_at_algorithmic_bytes": cfg.bytes() * len(layers) / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                          # the two roofs at the published peaks: whichever floor is higher binds the workload
+                          "mfma_floor_ms": flops / (PEAK_BF16_TFLOPS * 1e12) * 1e3, "hbm_floor_ms": cfg.bytes() * len(layers) / (PEAK_HBM_GBS * 1e9) * 1e3},
                 plan_build_ms_host=plan_ms, setup_s=setup_s)
     # what a pure MFMA loop sustains on this part right now, next to the published constant the fraction is priced against
     line["roofline"]["reachable_peak"] = mfma_rate(torch)[0]
