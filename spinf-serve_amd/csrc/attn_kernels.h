@@ -33,11 +33,13 @@ struct AttnParams {
 
 // Softmax reference point.  The fast pass fixes each row's reference at the maximum of the first 32-key block in which
 // the row sees a key and never rescales the accumulators: probabilities are exp2(t - ref) and stay below 2^TAU_FAST, well
-// inside fp32 / bf16 range.  If any row of a tile meets a score more than TAU_FAST above its reference, the whole tile is
+// inside fp32 / bf16 range.  If any row of a tile meets scores so far above its reference that a lane's 16 probabilities of a
+// block sum to more than 2^TAU_FAST (at the latest when one score lies TAU_FAST above the reference), the whole tile is
 // recomputed by the exact pass: classic online softmax, reference raised and accumulators rescaled whenever a block
 // maximum exceeds the reference by more than TAU_LAZY.  Which pass produced a row depends on the rows of its own
 // 128-token tile only, so it does not depend on what the job is packed with.
 constexpr float TAU_FAST = 60.f;
+constexpr float VIOL_SUM = 1152921504606846976.f;   // 2^TAU_FAST: a lane's 16 probabilities of a block summing above it send the tile to the exact pass
 constexpr float TAU_LAZY = 8.f;
 
 

@@ -363,14 +363,17 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
 
     // ---- compute pieces
     auto sm_head = [&](const int rt, const f32x16& sv) __attribute__((always_inline)) -> float {
-        float mx = sv[0];
-#pragma unroll
-        for (int i2 = 1; i2 < 16; i2++) mx = fmaxf(mx, sv[i2]);
-        mx = lane32_max(mx);
-        const float tm = mx * p.c;
+        // the block's maximum is needed only where a row meets its first keys (it becomes the row's reference): in the steady state
+        // no row of the wave does, and the 16 maxima and the lane exchange are skipped.  Whether a score lies too far above the
+        // reference shows in the probabilities (the caller checks their sum against 2^TAU_FAST).
         const bool first = M[rt] == -INFINITY;
-        viol = viol | (!first & (tm > M[rt] + TAU_FAST));
-        M[rt] = first ? tm : M[rt];
+        if (__builtin_amdgcn_ballot_w64(first) != 0) {
+            float mx = sv[0];
+#pragma unroll
+            for (int i2 = 1; i2 < 16; i2++) mx = fmaxf(mx, sv[i2]);
+            mx = lane32_max(mx);
+            M[rt] = first ? mx * p.c : M[rt];
+        }
         return M[rt] == -INFINITY ? 0.f : M[rt];
     };
     auto sm_elem = [&](const f32x16& sv, const int i2, const float ms, float& sum, bf16x8 (&pb)[2]) __attribute__((always_inline)) {
@@ -438,6 +441,7 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
 #pragma unroll
                 for (int i2 = 0; i2 < 16; i2++) sm_elem(sa[rt], i2, ms, sum, pa[rt]);
                 l[rt] += sum;
+                viol = viol | !(sum <= VIOL_SUM);   // (a NaN counts as too far as well)
             }
             pv_phase(vb + sub * G::VSUB, pa);
         };

@@ -530,14 +530,14 @@ __global__ __launch_bounds__(512) void tree_attn_ring_kernel(const AttnParams p)
                 // softmax against the row's fixed reference (the maximum of the first block it sees a key in)
                 bf16x8 pb[2];
                 {
-                    float mx = sa[0];
-#pragma unroll
-                    for (int i2 = 1; i2 < 16; i2++) mx = fmaxf(mx, sa[i2]);
-                    mx = lane32_max(mx);
-                    const float tm = mx * p.c;
                     const bool first = M == -INFINITY;
-                    viol = viol | (!first & (tm > M + TAU_FAST));
-                    M = first ? tm : M;
+                    if (__builtin_amdgcn_ballot_w64(first) != 0) {   // only where a row meets its first keys (see the lockstep kernel)
+                        float mx = sa[0];
+#pragma unroll
+                        for (int i2 = 1; i2 < 16; i2++) mx = fmaxf(mx, sa[i2]);
+                        mx = lane32_max(mx);
+                        M = first ? mx * p.c : M;
+                    }
                     const float ms = M == -INFINITY ? 0.f : M;
                     float sum = 0.f;
 #pragma unroll
@@ -547,6 +547,7 @@ __global__ __launch_bounds__(512) void tree_attn_ring_kernel(const AttnParams p)
                         pb[i2 >> 3][i2 & 7] = (__bf16)pr;
                     }
                     l += sum;
+                    viol = viol | !(sum <= VIOL_SUM);
                 }
                 // O^T += V^T P^T, with what the next tile's top needs fetched meanwhile; once the last fragment read is on its way,
                 // count this wave through with the tile
