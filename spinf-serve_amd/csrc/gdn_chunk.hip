@@ -362,6 +362,11 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
             }
         }
         lds_barrier();   // -W visible; every wave has read its V columns
+        // The next chunk's rows are requested here: the registers they land in are free since the staging, and from here no phase
+        // needs more registers than there are (one phase earlier the solve spills).  They have the three value-column phases
+        // (about 4 k cycles) to arrive; requested after the V' phase (2 k cycles) the next chunk's staging waited for them.
+        fetch_data();          // chunk j + 1, whose rows are known since the previous chunk
+        fetch_rows(j + 2);
 
         // ---- V' = U + (-W) S and Q S over the 128 key rows, 32 at a time (the state tiles 2s and 2s + 1 are the B operand)
 #pragma unroll
@@ -384,9 +389,6 @@ __device__ __forceinline__ void gdn_wy_body(const GdnParams& p) {
                 }
             }
         }
-        // the next chunk's rows are requested here, where few registers are live; they arrive during the state update
-        fetch_data();          // chunk j + 1, whose rows are known since the previous chunk
-        fetch_rows(j + 2);
         // ---- O[i][v] = s e^{G_i} (Q S)[i][v] + sum_j P[i][j] V'[j][v], rows i = 16 it + 4 q4 + r; through LDS for 16-byte stores
         f32x4 Gj[NT];
 #pragma unroll
