@@ -485,3 +485,64 @@ def test_tileplan_is_exact_on_random_forests():
             assert got == want, t
 
     run()
+
+
+def test_static_schedule_deals_every_item_out_once():
+    """the static schedule: the same items as the queue's lists, regrouped into one list per workgroup; workgroup b serves XCD
+    b % 8 (its items come from that XCD's list, in that list's order); lists are balanced under the cost model"""
+    cfg = synth.attention_config("C2", contents=7)
+    b = cfg.batches[0]
+    for ktile in (64, 32):
+        plan = sa.TilePlan.build(b.art, b.end, b.pos, None, ktile=ktile)
+        for head_groups, n_lists in ((8, 64), (8, 256), (3, 40), (1, 8)):
+            items, list_ptr = plan.schedule(head_groups)
+            sitems, sptr = plan.schedule_static(head_groups, n_lists)
+            assert sitems.shape == items.shape and len(sptr) == n_lists + 1
+            assert sptr[0] == 0 and sptr[-1] == len(items) and (np.diff(sptr) >= 0).all()
+            key = lambda rows: sorted(map(tuple, rows.tolist()))
+            assert key(sitems) == key(items)
+            xcd_of = {}
+            for l in range(8):
+                for pos_in_list, row in enumerate(items[list_ptr[l] : list_ptr[l + 1]].tolist()):
+                    xcd_of[tuple(row)] = (l, pos_in_list)
+            weights = []
+            for w in range(n_lists):
+                rows = [tuple(r) for r in sitems[sptr[w] : sptr[w + 1]].tolist()]
+                where = [xcd_of[r] for r in rows]
+                assert all(l == w % 8 for l, _ in where)
+                assert [p for _, p in where] == sorted(p for _, p in where)   # a workgroup takes its XCD's items in list order
+                weights.append(sum(r[2] & 0xFFFFF for r in rows))
+            if n_lists * 4 <= len(items):
+                assert max(weights) <= 1.6 * (sum(weights) / n_lists) + 40
+    lib = sa.load_library()
+    assert lib.spinf_tileplan_schedule_static(plan._handle, 1, 0, None, None) == -1 and b"null argument" in lib.spinf_last_error()
+
+
+def test_gdn_plan_compiler_edge_cases():
+    """the C ABI of the recurrent-layer plan compiler on the degenerate inputs: an empty stream, pads only, one token, bad arguments"""
+    import ctypes as C
+
+    from spinf_serve_amd import qwen_plan
+
+    lib = sa.load_library()
+    empty = qwen_plan._compile(np.zeros(0, np.int64), np.zeros(0, np.uint8), "indexed", 64, 8192, 96, None, None)
+    assert empty["n_segments"] == 0 and len(empty["idx"]) == 0 and len(empty["level_ptr"]) == 1
+    pads = qwen_plan._compile(np.full(5, -1, np.int64), np.zeros(5, np.uint8), "indexed", 64, 8192, 96, None, None)
+    assert pads["n_segments"] == 0 and (pads["seg_of_row"] == -1).all()
+    one = sa.tree_plan(np.array([-1]), np.array([True]), "cpu")
+    assert one.n_segments == 1 and len(one.levels) == 1 and one.levels[0][0].cu_cpu.tolist() == [0, 1]
+    assert one.conv.tolist() == [[1, 1, 1, 0]]   # no predecessors: the zero row, then the token itself
+    handle = C.c_void_p()
+    prev = np.array([-1, 0, 5], np.int64)   # token 2 names a later token
+    real = np.ones(3, np.uint8)
+    assert lib.spinf_gdn_plan_build(prev.ctypes.data, real.ctypes.data, 3, 0, 64, 8192, 96, -1, None, 0, C.byref(handle)) == -1
+    assert b"does not point backwards" in lib.spinf_last_error()
+    prev = np.array([-1, 0, 1], np.int64)
+    assert lib.spinf_gdn_plan_build(prev.ctypes.data, real.ctypes.data, 3, 7, 64, 8192, 96, -1, None, 0, C.byref(handle)) == -1
+    assert lib.spinf_gdn_plan_build(prev.ctypes.data, real.ctypes.data, 3, 0, 64, 8192, 96, 2, None, 0, C.byref(handle)) == -1
+    assert b"compact rows" in lib.spinf_last_error()
+    assert lib.spinf_gdn_plan_build(prev.ctypes.data, real.ctypes.data, 3, 0, 64, 8192, 96, -1, None, 0, None) == -1
+    with pytest.raises(ValueError):
+        sa.tree_plan(prev, real[:2].astype(bool), "cpu")
+    with pytest.raises(ValueError):
+        sa.tree_plan(prev, real.astype(bool), "cpu", path="sideways")
