@@ -501,3 +501,38 @@ def test_groups_of_the_windowed_checkpoint_are_rejected_on_a_global_layer(dev):
     a = attention._attn_args(q, k, v, out, b.length, mask.art, mask.end, mask.pos, mask.kv_idx, mask.kv_bits, items, list_ptr, n_items, cfg.scale, 0, 0, None, None, grp, 2, 64)
     lib = sa.load_library()
     assert lib.spinf_tree_attn_fwd(C.byref(a), None) == -1 and b"global layer takes no groups" in lib.spinf_last_error()
+
+
+def test_allocating_entry_point_under_graph_capture(dev):
+    """a stream that has made one call can record the call into a graph: the stream's cursor block goes with the graph, replays give
+    the eager result every time (with eager calls on the same stream in between, which take a new block), and a capture on a stream
+    that never made a call is refused with a message instead of allocating"""
+    cfg = synth.attention_config("C2", contents=3)
+    b = cfg.batches[0]
+    q, k, v = synth.qkv(cfg, b, seed=12, device=dev)
+    mask = sa.TreeMask.build(b.art, b.end, b.pos, device=dev)
+    want = sa.tree_attn(q, k, v, mask, cfg.scale)
+    torch.cuda.synchronize()
+    s = torch.cuda.Stream(device=dev)
+    with torch.cuda.stream(s):
+        warm = sa.tree_attn(q, k, v, mask, cfg.scale)   # the stream's block exists from here on
+    s.synchronize()
+    assert torch.equal(warm, want)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=s):
+        out = sa.tree_attn(q, k, v, mask, cfg.scale)
+    for rep in range(3):
+        out.zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), rep
+        with torch.cuda.stream(s):   # eager work on the same stream between the replays
+            again = sa.tree_attn(q, k, v, mask, cfg.scale)
+        s.synchronize()
+        assert torch.equal(again, want)
+    fresh = torch.cuda.Stream(device=dev)
+    g2 = torch.cuda.CUDAGraph()
+    with pytest.raises(ValueError, match="before the capture"):
+        with torch.cuda.graph(g2, stream=fresh):
+            sa.tree_attn(q, k, v, mask, cfg.scale)
+    torch.cuda.synchronize()
