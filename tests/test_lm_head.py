@@ -184,3 +184,19 @@ def test_fused_head_at_the_reference_vocabulary(dev):
     got = sa.lm_head_logprobs(h, sel, w, cols, 30.0)
     want = sa.lm_logprobs(torch.mm(h[sel], w.t(), out_dtype=torch.float32), cols, 30.0)
     assert (got - want).abs().max().item() <= 1e-4
+
+
+@pytest.mark.gpu
+def test_fused_head_columns_at_tile_and_wave_boundaries(dev):
+    """selected columns on both sides of every 32 / 128 / 256 boundary of the vocabulary tiling, read rows across the 256-row tile
+    boundary, a vocabulary that ends inside a wave's quarter: the same bits as the whole row's"""
+    rng = np.random.default_rng(21)
+    rows, vocab, hidden = 259, 700, 128
+    h, w = _bf16_values(rng, (rows, hidden), 1.0), _bf16_values(rng, (vocab, hidden), 1.0)
+    cols = np.array([0, 31, 32, 127, 128, 129, 255, 256, 257, 383, 384, 511, 512, 639, 640, 699, 1, 698])
+    whole = sa.lm_head_logprobs(h.to(dev), None, w.to(dev), None, 30.0)
+    part = sa.lm_head_logprobs(h.to(dev), None, w.to(dev), torch.from_numpy(cols).to(dev), 30.0)
+    assert torch.equal(part, whole[:, torch.from_numpy(cols).to(dev)])
+    want = olm.head_logprobs(h.float().numpy(), w.float().numpy(), None, None, 30.0)
+    assert np.abs(whole.cpu().numpy() - want).max() <= TOL
+    assert np.abs(np.exp(whole.double().cpu().numpy()).sum(1) - 1.0).max() < 1e-5
