@@ -29,6 +29,7 @@ struct AttnParams {
     const int* grp;       // image groups (GRP kernels): -1 none; the tokens of a group see each other both ways
     bool static_lists;    // list_ptr delimits one item list per workgroup (a static schedule) instead of the eight shared lists
     bool clear_first;     // host side only: zero the cursors and counts in front of the pass (the entry point that allocates nothing)
+    bool keep_redo;       // exact pass: leave the redo list and its count as they are (the first of two launches over one list)
 };
 
 // Softmax reference point.  The fast pass fixes each row's reference at the maximum of the first 32-key block in which

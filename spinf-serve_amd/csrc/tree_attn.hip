@@ -234,8 +234,10 @@ __global__ __launch_bounds__(256) void tree_attn_exact_kernel(const AttnParams p
     if (threadIdx.x == 0) {
         __threadfence();
         if (atomicAdd(&p.counters[NLIST + 2], 1) == (int)gridDim.x - 1) {
-            p.counters[NLIST + 3] += n_redo;   // running total, for spinf_attn_exact_items
-            p.counters[NLIST + 1] = 0;
+            if (!p.keep_redo) {
+                p.counters[NLIST + 3] += n_redo;   // running total, for spinf_attn_exact_items
+                p.counters[NLIST + 1] = 0;
+            }
             p.counters[NLIST + 2] = 0;
             __threadfence();
         }
@@ -751,6 +753,19 @@ int launch_ring(const AttnParams& p, int d, bool win, int n_wg, hipStream_t stre
     }
     if (int rc = spinf_launch_ring(p, d, win, n_wg, stream)) return rc;
     const int blocks = n_wg < 64 ? n_wg : 64;
+    if (d == 512) {   // the exact pass computes the output 256 dims at a time: twice over the same redo list, which the second launch clears
+        for (int half = 0; half < 2; half++) {
+            AttnParams ph = p;
+            ph.v = p.v + 256 * half;
+            ph.o = p.o + 256 * half;
+            ph.keep_redo = half == 0;
+            if (win) hipLaunchKernelGGL((tree_attn_exact_kernel<512, 1, true, 1, false, 0, 32, 256>), dim3(blocks), dim3(256), 0, stream, ph);
+            else hipLaunchKernelGGL((tree_attn_exact_kernel<512, 1, false, 1, false, 0, 32, 256>), dim3(blocks), dim3(256), 0, stream, ph);
+            const hipError_t e = hipGetLastError();
+            if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: launch (exact pass): %s", hipGetErrorString(e));
+        }
+        return SPINF_OK;
+    }
     if (win) hipLaunchKernelGGL((tree_attn_exact_kernel<256, 1, true, 2, false, 0, 32, 256>), dim3(blocks), dim3(256), 0, stream, p);
     else hipLaunchKernelGGL((tree_attn_exact_kernel<256, 1, false, 2, false, 0, 32, 256>), dim3(blocks), dim3(256), 0, stream, p);
     const hipError_t e = hipGetLastError();
@@ -830,11 +845,11 @@ static int attn_fwd(const spinf_attn_args* a, void* stream, bool no_alloc) {
     if ((a->row_of != nullptr) != (a->kv_row0 != nullptr)) return spinf_fail(SPINF_E_ARG, "tree_attn: row_of and kv_row0 come together");
     if (a->row_of && rt != 1) return spinf_fail(SPINF_E_ARG, "tree_attn: variant %d does not take compact rows", a->variant);
     if (a->n_lists < 0 || a->n_lists > 65536) return spinf_fail(SPINF_E_ARG, "tree_attn: %d item lists, at most 65,536", a->n_lists);
-    const bool ring = a->n_lists > 0 && a->ktile == 32 && a->d != 512;   // static schedule over 32-key entries: the ring kernel
+    const bool ring = a->n_lists > 0 && a->ktile == 32;   // static schedule over 32-key entries: the ring kernel
     if (ring) {
-        if (a->d != 256 || nhw != 2 || rt != 1 || a->row_of || a->grp)
-            return spinf_fail(SPINF_E_ARG, "tree_attn: a static schedule over 32-key entries goes with head dim 256, an even number of query heads per key / value head, "
-                                           "variant 0, the stream layout and no image groups");
+        if (!((a->d == 256 && nhw == 2 && rt == 1) || a->d == 512) || a->row_of || a->grp)
+            return spinf_fail(SPINF_E_ARG, "tree_attn: a static schedule over 32-key entries goes with head dim 512, or head dim 256 with an even number of query heads "
+                                           "per key / value head and variant 0; with the stream layout and no image groups");
     } else if ((a->d == 512) != (a->ktile == 32) || (a->ktile != 0 && a->ktile != 32 && a->ktile != 64))
         return spinf_fail(SPINF_E_ARG, "tree_attn: plan entries of %d keys with head dim %d (32 goes with 512, 64 with the others)", a->ktile ? a->ktile : 64, a->d);
     if (a->grp && (a->grp_mode != 1 && a->grp_mode != 2)) return spinf_fail(SPINF_E_ARG, "tree_attn: group mode %d not in {1, 2}", a->grp_mode);
@@ -873,6 +888,7 @@ static int attn_fwd(const spinf_attn_args* a, void* stream, bool no_alloc) {
     // puts them back.  Only a block whose last call failed to get its kernels onto the stream is cleared first; so is the scratch
     // array of the entry point that allocates nothing, which every caller on the GPU shares.
     p.clear_first = no_alloc || dirty;
+    p.keep_redo = false;
     p.static_lists = a->n_lists > 0;
     p.q = (const __bf16*)a->q; p.k = (const __bf16*)a->k; p.v = (const __bf16*)a->v; p.o = (__bf16*)a->out;
     p.q_tok = a->q_tok; p.q_head = a->q_head; p.k_tok = a->k_tok; p.k_head = a->k_head;

@@ -32,7 +32,7 @@
 
 namespace {
 
-constexpr int NSLOT = 4;            // tile ring depth (32-key tiles)
+constexpr int MAX_SLOT = 4;         // tile ring depth (32-key tiles): 4, at head dim 512 (69 KB a tile) 2
 constexpr int NDESC = 128;          // tile descriptors kept in LDS
 constexpr int GEN_AHEAD = 48;       // wave 0 keeps the descriptors this far ahead of its own tile
 constexpr int SPIN_LIMIT = 1 << 18; // polls of one wait before the workgroup gives up (a healthy wait takes a handful)
@@ -93,6 +93,14 @@ __device__ __forceinline__ void acc_op(const bf16x8 a, const bf16x8 b, float (&r
     ACC_TILE_OPS(5, 80, 95, 80, 81, 82, 83, 84, 85, 86, 87, 88, 89, 90, 91, 92, 93, 94, 95)
     ACC_TILE_OPS(6, 96, 111, 96, 97, 98, 99, 100, 101, 102, 103, 104, 105, 106, 107, 108, 109, 110, 111)
     ACC_TILE_OPS(7, 112, 127, 112, 113, 114, 115, 116, 117, 118, 119, 120, 121, 122, 123, 124, 125, 126, 127)
+    ACC_TILE_OPS(8, 128, 143, 128, 129, 130, 131, 132, 133, 134, 135, 136, 137, 138, 139, 140, 141, 142, 143)
+    ACC_TILE_OPS(9, 144, 159, 144, 145, 146, 147, 148, 149, 150, 151, 152, 153, 154, 155, 156, 157, 158, 159)
+    ACC_TILE_OPS(10, 160, 175, 160, 161, 162, 163, 164, 165, 166, 167, 168, 169, 170, 171, 172, 173, 174, 175)
+    ACC_TILE_OPS(11, 176, 191, 176, 177, 178, 179, 180, 181, 182, 183, 184, 185, 186, 187, 188, 189, 190, 191)
+    ACC_TILE_OPS(12, 192, 207, 192, 193, 194, 195, 196, 197, 198, 199, 200, 201, 202, 203, 204, 205, 206, 207)
+    ACC_TILE_OPS(13, 208, 223, 208, 209, 210, 211, 212, 213, 214, 215, 216, 217, 218, 219, 220, 221, 222, 223)
+    ACC_TILE_OPS(14, 224, 239, 224, 225, 226, 227, 228, 229, 230, 231, 232, 233, 234, 235, 236, 237, 238, 239)
+    ACC_TILE_OPS(15, 240, 255, 240, 241, 242, 243, 244, 245, 246, 247, 248, 249, 250, 251, 252, 253, 254, 255)
 }
 template <int TILE>
 __device__ __forceinline__ void acc_mfma(const bf16x8 a, const bf16x8 b) {
@@ -195,8 +203,11 @@ __device__ __forceinline__ void pv_steps(Fn& fn) {
 }
 
 template <int D, bool WIN>
-__global__ __launch_bounds__(512) void tree_attn_ring_kernel(const AttnParams p) {
+__global__ __launch_bounds__(D == 512 ? 256 : 512) void tree_attn_ring_kernel(const AttnParams p) {
     constexpr int TK = 32;
+    constexpr int NW = D == 512 ? 4 : 8;      // waves: four row groups x HPI heads of the item
+    constexpr int HPI = NW / 4;
+    constexpr int NSLOT = D == 512 ? 2 : MAX_SLOT;
     using G = TileGeo<D, TK, D>;
     constexpr int NS = D / 16;     // contraction steps of K Q^T
     constexpr int NDT = D / 32;    // 32-wide slices of the head dimension in O^T
@@ -204,12 +215,12 @@ __global__ __launch_bounds__(512) void tree_attn_ring_kernel(const AttnParams p)
     constexpr int PFD = D >= 256 ? 2 : 8;   // fragment read-ahead: at head dim 256 one more spills a query fragment inside the tile loop
     constexpr int PF = D >= 256 ? 4 : (NS < PFD ? NS : PFD);   // K fragments are live in the score phase only, where registers are free
     constexpr int VPF = NVF < PFD ? NVF : PFD;
-    static_assert(NSLOT * G::BUFB + 8 * 32 * SROW + NDESC * 16 + 256 <= 160 * 1024, "LDS budget");
+    static_assert(NSLOT * G::BUFB + NW * 32 * SROW + NDESC * 16 + 256 <= 160 * 1024, "LDS budget");
     __shared__ __attribute__((aligned(16))) char ring[NSLOT * G::BUFB];
-    __shared__ __attribute__((aligned(16))) char stage_all[8 * 32 * SROW];   // output staging, one slice per wave
+    __shared__ __attribute__((aligned(16))) char stage_all[NW * 32 * SROW];   // output staging, one slice per wave
     __shared__ int4 desc[NDESC];       // {key tile, bits | DESC_FIRST | DESC_LAST, query tile | head group << 20, item index}
-    __shared__ __attribute__((aligned(16))) int sy_done[NSLOT];   // waves through with the tile in the slot; 8 = the slot waits for somebody to recycle it
-    __shared__ int sy_issued[NSLOT];   // tile the slot was last recycled for (its DMA requested)
+    __shared__ __attribute__((aligned(16))) int sy_done[MAX_SLOT];   // waves through with the tile in the slot; NW = the slot waits for somebody to recycle it (words past NSLOT stay 0)
+    __shared__ int sy_issued[MAX_SLOT];   // tile the slot was last recycled for (its DMA requested)
     __shared__ int sy_gen;             // descriptors written so far
     __shared__ int sy_abort;
     __shared__ int sy_ntiles;
@@ -233,9 +244,9 @@ __global__ __launch_bounds__(512) void tree_attn_ring_kernel(const AttnParams p)
                  "s_mov_b32 %8, 2\n\ts_cmp_lg_u32 %7, 0\n\ts_cbranch_scc1 2f\n\ts_sub_u32 %9, %9, 1\n\ts_cmp_eq_u32 %9, 0\n\ts_cbranch_scc1 2f\n\t" \
                  WATCH "s_sleep 1\n\ts_branch 1b\n2:"                                                                                               \
                  : "=&v"(t0), "=&v"(t1), "=&v"(n0), "=&v"(n1), "=&v"(n2), "=&v"(n3), "=&s"(v), "=&s"(ab), "=&s"(code), "+s"(cnt)                     \
-                 : "v"(a_word), "v"(a_abort), "v"(a_next), "s"(want)                                                                                \
+                 : "v"(a_word), "v"(a_abort), "v"(a_next), "s"(want), "n"(NW)                                                                       \
                  : "memory", "scc", "vcc")
-#define SPIN_WATCH "s_mov_b32 %8, 1\n\tv_cmp_eq_u32_e32 vcc, 8, %2\n\ts_cbranch_vccnz 2f\n\tv_cmp_eq_u32_e32 vcc, 8, %3\n\ts_cbranch_vccnz 2f\n\tv_cmp_eq_u32_e32 vcc, 8, %4\n\ts_cbranch_vccnz 2f\n\tv_cmp_eq_u32_e32 vcc, 8, %5\n\ts_cbranch_vccnz 2f\n\t"
+#define SPIN_WATCH "s_mov_b32 %8, 1\n\tv_cmp_eq_u32_e32 vcc, %c14, %2\n\ts_cbranch_vccnz 2f\n\tv_cmp_eq_u32_e32 vcc, %c14, %3\n\ts_cbranch_vccnz 2f\n\tv_cmp_eq_u32_e32 vcc, %c14, %4\n\ts_cbranch_vccnz 2f\n\tv_cmp_eq_u32_e32 vcc, %c14, %5\n\ts_cbranch_vccnz 2f\n\t"
         if (at_least) {
             if (watch) SPIN_ASM("s_cmp_ge_i32", SPIN_WATCH); else SPIN_ASM("s_cmp_ge_i32", "");
         } else {
@@ -257,10 +268,10 @@ __global__ __launch_bounds__(512) void tree_attn_ring_kernel(const AttnParams p)
     };
 
     // ---- prologue: sync words, the workgroup's tile count, the first descriptors
-    if (threadIdx.x < NSLOT) {
+    if (threadIdx.x < MAX_SLOT) {
         sy_done[threadIdx.x] = 0;
         sy_issued[threadIdx.x] = (int)threadIdx.x;
-        *(int*)(ring + threadIdx.x * G::BUFB + G::KTILEB + G::VTILEB + 768) = -1;   // the slot's flag: no generation yet
+        if (threadIdx.x < NSLOT) *(int*)(ring + threadIdx.x * G::BUFB + G::KTILEB + G::VTILEB + 768) = -1;   // the slot's flag: no generation yet
     }
     if (threadIdx.x < 16) sy_redo[threadIdx.x] = 0;
     if (threadIdx.x == 0) { sy_gen = 0; sy_abort = 0; sy_ntiles = 0; }
@@ -330,7 +341,7 @@ __global__ __launch_bounds__(512) void tree_attn_ring_kernel(const AttnParams p)
         if (j >= gen_seen) gen_seen = wait_gen(j + 1);
     };
     auto issue = [&](const int j, const int4& d) __attribute__((always_inline)) {
-        const int kvh = (int)((unsigned)d.z >> 20) * 2 / p.group;
+        const int kvh = (int)((unsigned)d.z >> 20) * HPI / p.group;
         // the per-lane parts of the source addresses are recomputed here: kept in registers they are spilled across the tile loop
         using GK = Geo<D, TK>;
         const int lane = fresh_lane_id();
@@ -343,11 +354,11 @@ __global__ __launch_bounds__(512) void tree_attn_ring_kernel(const AttnParams p)
     // it takes the count back to 0 (compare-and-swap: one winner) and requests the tile NSLOT places further on.  Not the last
     // wave through by design: that one is the wave the others are waiting for.  n0..n3 = sy_done as read a moment ago.
     auto claim = [&](const int n0, const int n1, const int n2, const int n3) __attribute__((always_inline)) {
-        if (n0 == 8 || n1 == 8 || n2 == 8 || n3 == 8) {
-            const int sl = n0 == 8 ? 0 : n1 == 8 ? 1 : n2 == 8 ? 2 : 3;
+        if (n0 == NW || n1 == NW || n2 == NW || n3 == NW) {
+            const int sl = n0 == NW ? 0 : n1 == NW ? 1 : n2 == NW ? 2 : 3;
             int got = 0;
             if (fresh_lane_id() == 0) {
-                int expect = 8;
+                int expect = NW;
                 got = __hip_atomic_compare_exchange_strong(&sy_done[sl], &expect, 0, __ATOMIC_ACQ_REL, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             }
             if (__builtin_amdgcn_readfirstlane(got)) {
@@ -392,7 +403,7 @@ __global__ __launch_bounds__(512) void tree_attn_ring_kernel(const AttnParams p)
         const int lane = fresh_lane_id();
         const int tok = (tz & 0xfffff) * SPINF_QTILE + 32 * L.wr + (lane & 31);
         const int tok_c = tok < p.n ? tok : p.n - 1;
-        const int h = (int)((unsigned)tz >> 20) * 2 + L.wh;
+        const int h = (int)((unsigned)tz >> 20) * HPI + L.wh;
         const __bf16* qp = p.q + (long)tok_c * p.q_tok + (long)h * p.q_head + 8 * (lane >> 5);
 #pragma unroll
         for (int s = 0; s < NS; s++) qf[s] = *(const bf16x8*)(qp + 16 * s);
@@ -410,7 +421,7 @@ __global__ __launch_bounds__(512) void tree_attn_ring_kernel(const AttnParams p)
     auto store_rows = [&](const int tz) __attribute__((always_inline)) {
         const int lane = fresh_lane_id(), m = lane & 31, g = lane >> 5;
         const int tok0 = (tz & 0xfffff) * SPINF_QTILE + 32 * L.wr;
-        const int h = (int)((unsigned)tz >> 20) * 2 + L.wh;
+        const int h = (int)((unsigned)tz >> 20) * HPI + L.wh;
         const float inv = 1.0f / lane32_sum(l);
         __bf16* ob = p.o + (long)h * p.o_head;
         char* const stage = stage_all + L.w * 32 * SROW;
@@ -445,10 +456,7 @@ __global__ __launch_bounds__(512) void tree_attn_ring_kernel(const AttnParams p)
             }
         };
         put(std::integral_constant<int, 0>{});
-        round(std::integral_constant<int, 0>{});
-        round(std::integral_constant<int, 1>{});
-        if constexpr (NDT > 2) { round(std::integral_constant<int, 2>{}); round(std::integral_constant<int, 3>{}); }
-        if constexpr (NDT > 4) { round(std::integral_constant<int, 4>{}); round(std::integral_constant<int, 5>{}); round(std::integral_constant<int, 6>{}); round(std::integral_constant<int, 7>{}); }
+        pv_steps<NDT>(round);
     };
 
     {   // the first item's queries
@@ -629,7 +637,7 @@ __global__ __launch_bounds__(512) void tree_attn_ring_kernel(const AttnParams p)
 
 template <int D, bool WIN>
 int launch_ring_t(const AttnParams& p, int n_wg, hipStream_t stream) {
-    hipLaunchKernelGGL((tree_attn_ring_kernel<D, WIN>), dim3(n_wg), dim3(512), 0, stream, p);
+    hipLaunchKernelGGL((tree_attn_ring_kernel<D, WIN>), dim3(n_wg), dim3(D == 512 ? 256 : 512), 0, stream, p);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: launch (ring kernel): %s", hipGetErrorString(e));
     return SPINF_OK;
@@ -639,5 +647,6 @@ int launch_ring_t(const AttnParams& p, int n_wg, hipStream_t stream) {
 
 int spinf_launch_ring(const AttnParams& p, int d, bool win, int n_wg, hipStream_t stream) {
     if (d == 256) return win ? launch_ring_t<256, true>(p, n_wg, stream) : launch_ring_t<256, false>(p, n_wg, stream);
-    return spinf_fail(SPINF_E_ARG, "tree_attn: the ring kernel takes head dim 256, not %d", d);
+    if (d == 512) return win ? launch_ring_t<512, true>(p, n_wg, stream) : launch_ring_t<512, false>(p, n_wg, stream);
+    return spinf_fail(SPINF_E_ARG, "tree_attn: the ring kernel takes head dim 256 or 512, not %d", d);
 }

@@ -44,9 +44,9 @@ def _ring_lists(q, hq, hkv, d, variant, sidx, mask):
     from .masks import _static_lists
 
     n_wg = _static_lists(q.device)
-    ring = variant == 0 and d == 256 and (hq // hkv) % 2 == 0 and sidx is None and mask.grp is None
+    ring = (d == 512 or (variant == 0 and d == 256 and (hq // hkv) % 2 == 0)) and sidx is None and mask.grp is None
     if ring and RING < 0:
-        ring = mask.plan.n_qtiles * (hq // 2) <= RING_MAX_ITEMS_PER_WG * n_wg
+        ring = d == 512 or mask.plan.n_qtiles * (hq // 2) <= RING_MAX_ITEMS_PER_WG * n_wg
     elif not RING:
         ring = False
     static = d != 512 and (int(mask.window) > 0 if STATIC < 0 else bool(STATIC))
