@@ -465,6 +465,38 @@ def test_kernel_and_schedule_choices_give_the_same_bits(dev, window, monkeypatch
     assert sa.load_library().spinf_attn_ring_aborts(ctypes.byref(aborts)) == 0 and aborts.value == 0
 
 
+@pytest.mark.parametrize("window", [None, 300])
+def test_head_dim_512_kernel_choices_give_the_same_bits(dev, window, monkeypatch):
+    """head dim 512: the kernel with decoupled waves (one launch, the whole output row in accumulation registers) and the lockstep
+    kernel (two launches of 256 value dims) give one result, on a stream long enough for several items per workgroup and with
+    its last query tile cut off by the end of the stream; no wave of the decoupled kernel gave up a wait"""
+    import ctypes
+
+    from spinf_serve_amd import attention
+
+    cfg = synth.attention_config("C2_512", contents=6)
+    b = cfg.batches[0]
+    q, k, v = synth.qkv(cfg, b, seed=5, device=dev)
+    n = b.length - 37   # a stream that ends inside a query tile and inside a key tile
+    q, k, v = q[:n].contiguous(), k[:n].contiguous(), v[:n].contiguous()
+    mask = sa.TreeMask.build(b.art[:n], b.end[:n], b.pos[:n], window=window, device=dev)
+    outs = []
+    for ring in (0, 1):
+        monkeypatch.setattr(attention, "RING", ring)
+        print(f"case d512 ring={ring} window={window} n={n}", flush=True)
+        outs.append(sa.tree_attn(q, k, v, mask, cfg.scale))
+        torch.cuda.synchronize()
+    assert torch.equal(outs[0], outs[1])
+    aborts = ctypes.c_int64(-1)
+    assert sa.load_library().spinf_attn_ring_aborts(ctypes.byref(aborts)) == 0 and aborts.value == 0
+    # and both against the oracle on one content
+    start, length, *_ = b.jobs[0]
+    sl = slice(start, start + length)
+    dense = omask.dense_tree_mask(b.art[sl], b.end[sl] - start, b.pos[sl], window)
+    ref = oattn.masked_attention(q[sl].float().cpu().numpy(), k[sl].float().cpu().numpy(), v[sl].float().cpu().numpy(), dense, cfg.scale)
+    assert float(np.abs(outs[1][sl].float().cpu().numpy() - ref).max()) <= TOL
+
+
 def test_calls_on_two_streams_do_not_share_cursors(dev):
     """calls interleaved on two streams, not synchronised with each other, give the bits of the same calls one after the other"""
     cfgs = [synth.attention_config("C2", seed=s, contents=4 + 3 * s) for s in range(2)]
