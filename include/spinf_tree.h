@@ -115,8 +115,9 @@ typedef struct spinf_attn_args {
     int32_t n_lists;                        /* 0: items / list_ptr are the eight work lists of spinf_tileplan_schedule, shared by all
                                                workgroups.  > 0: a static schedule (spinf_tileplan_schedule_static) of n_lists item lists,
                                                list_ptr [n_lists + 1]; the pass runs as n_lists workgroups, each through its own list.  With
-                                               ktile 32 (and d = 256, an even number of query heads per key / value head, variant 0, stream
-                                               layout, no groups) that is the kernel with decoupled waves */
+                                               ktile 32 (and d = 512, or d = 256 with an even number of query heads per key / value head and
+                                               variant 0; stream layout, no groups) that is the kernel with decoupled waves, which at
+                                               d = 512 computes the pass in one launch instead of two */
 } spinf_attn_args;
 
 /* query heads one work item covers for this geometry (1 or 2); 0 for an invalid geometry */

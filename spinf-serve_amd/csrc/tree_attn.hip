@@ -728,7 +728,9 @@ int launch_d(const AttnParams& p, int rt, int nhw, bool win, int grp_mode, int b
     return win ? launch<D, 1, true, 1, false>(p, blocks, s) : launch<D, 1, false, 1, false>(p, blocks, s);
 }
 
-// Head dim 512 (the full-attention layers of the Gemma-4 checkpoints, one key / value head).  O^T for 32 rows x 512 dims is 256
+// Head dim 512 (the full-attention layers of the Gemma-4 checkpoints, one key / value head) for compact rows and image groups
+// (the stream layout without groups goes to the ring kernel, which keeps the accumulators in registers of its own choosing).
+// O^T for 32 rows x 512 dims is 256
 // accumulator registers per lane, which with the score tile and the 128 query registers leaves the register allocator no way
 // out but scratch memory.  So the output is computed 256 dims at a time, in two launches over the same plan: each computes the
 // scores over all 512 dims (that part is done twice) and P V for one half of V's columns.  Tiles are 32 keys (the plan is

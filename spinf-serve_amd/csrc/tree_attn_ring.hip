@@ -1,8 +1,10 @@
 // Tree-mask packed-prefill attention for gfx950, the ring kernel: the same arithmetic as tree_attn.hip's fast pass (same 32-key
-// blocks in the same order, same softmax reference, same bits), with the eight waves of a workgroup decoupled.
+// blocks in the same order, same softmax reference, same bits), with the waves of a workgroup decoupled.
 //
 // Replaces the flex_attention call of spinf_serve/models/gemma4.py:107-118 and spinf_serve/models/qwen35/qwen.py:614,620 for
-// head dim 256 / 128 / 64 with an even number of query heads per key / value head.
+// head dim 256 with an even number of query heads per key / value head (eight waves: four row groups x the two heads of an
+// item) and for head dim 512 (four waves, one head per item, one wave per SIMD: the 32 x 512 outputs of a wave are all 256
+// accumulation registers, which no kernel that leaves its accumulators to the compiler gets allocated; a ring of two slots).
 //
 // Why.  With a workgroup barrier at every key tile the eight waves move in lockstep: a wave whose 32 rows see nothing of a tile
 // (the diagonal of a branch region) idles, all waves start their MFMA phases and their softmax phases together, and nothing
@@ -12,8 +14,8 @@
 //
 //   * K / V tiles of 32 keys live in a ring of NSLOT slots.  Every wave walks the workgroup's tile sequence (all the tiles of
 //     its work items, item after item) and skips the tiles its rows see nothing of.  When a wave is through with a tile it
-//     counts itself in (`done`); the last of the eight to do so recycles the slot: it requests, by itself, the DMA of the tile
-//     NSLOT places further on (`issued`); the last request of the batch writes the slot's flag, so the DMA engine itself
+//     counts itself in (`done`); once all have, whichever wave comes by first recycles the slot: it requests, by itself, the
+//     DMA of the tile NSLOT places further on (`issued`); the last request of the batch writes the slot's flag, so the DMA engine itself
 //     reports the tile as landed.  A wave needs the flag before it reads a tile and `issued` before it skips one, so the
 //     waves stay within NSLOT - 1 tiles of each other.
 //   * Work items are assigned to workgroups on the host (spinf_tileplan_schedule_static: a simulation of "the workgroup that
