@@ -55,6 +55,10 @@ SPINUP_S = 0.3    # untimed, before the warm-up steps: keeps the GPU busy until 
 
 
 def timed(fn, steps, warmup, torch):
+    """-> (wall seconds of the `steps` timed steps, [event milliseconds per step] * steps).  The timed steps follow each other
+    with nothing between them: ONE pair of events around all of them, on the stream they are launched on (an event recorded
+    between two launches costs the GPU ~5 us of idling, which is 4 % of a C2 step if every step is bracketed).  The shortest
+    single step, from a second, untimed pass that does bracket every step, is left in timed.min_ms."""
     t0 = time.perf_counter()
     while time.perf_counter() - t0 < SPINUP_S:
         fn()
@@ -62,16 +66,23 @@ def timed(fn, steps, warmup, torch):
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
-    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
+    a.record()
+    for _ in range(steps):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    per_step = a.elapsed_time(b) / steps
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(min(steps, 20))]
     for a, b in ev:
         a.record()
         fn()
         b.record()
     torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    kern = [a.elapsed_time(b) for a, b in ev]
-    return wall, kern
+    timed.min_ms = min(a.elapsed_time(b) for a, b in ev)
+    return wall, [per_step] * steps
 
 
 def mfma_rate(torch, steps=20, warmup=5, iters=4000):
@@ -364,7 +375,7 @@ def main():
                         "visible_pairs": [cfg.pairs(w) for w in layers], "variant": args.variant, "rows": args.rows},
                 roofline={"bound": "mfma", "achieved": tfl, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": tfl / PEAK_BF16_TFLOPS,
                           "traffic": TRAFFIC_BYTES.get(args.workload) if args.contents is None and args.rows == "stream" else None, "kernel_ms": ms,
-                          "kernel_ms_min": float(np.min(kern)), "useful_flops": flops,
+                          "kernel_ms_min": float(timed.min_ms), "useful_flops": flops,
                           "algorithmic_bytes": cfg.bytes() * len(layers), "hbm_frac_at_algorithmic_bytes": cfg.bytes() * len(layers) / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
                           # the two roofs at the published peaks: whichever floor is higher binds the workload
                           "mfma_floor_ms": flops / (PEAK_BF16_TFLOPS * 1e12) * 1e3, "hbm_floor_ms": cfg.bytes() * len(layers) / (PEAK_HBM_GBS * 1e9) * 1e3},

@@ -22,14 +22,14 @@ struct AttnParams {
     const int* list_ptr;  // [NLIST + 1] offsets of the lists in items
     int* counters;        // [0..NLIST) next item of each list, [NLIST] workgroups done, [NLIST+1] items awaiting the exact pass,
                           // [NLIST+2] exact-pass workgroups done; each kernel's last workgroup resets what it used
-    int* redo;            // indices (into items) of the work items the fast pass handed to the exact pass
+    int* redo;            // indices (into items) of the work items the fast pass handed to the exact pass (the ring kernel: entries
+                          // list_ptr[b] .. of workgroup b's own hand-overs, which it recomputes itself)
     // compact rows (ROWS kernels): q, k, v, o hold the real tokens only; row_of[stream position] = row, -1 for a pad position;
     // kv_row0[entry] = row of the entry's first key if its 64 keys are 64 consecutive rows, else -1
     const int* row_of; const int* kv_row0;
     const int* grp;       // image groups (GRP kernels): -1 none; the tokens of a group see each other both ways
     bool static_lists;    // list_ptr delimits one item list per workgroup (a static schedule) instead of the eight shared lists
     bool clear_first;     // host side only: zero the cursors and counts in front of the pass (the entry point that allocates nothing)
-    bool keep_redo;       // exact pass: leave the redo list and its count as they are (the first of two launches over one list)
 };
 
 // Softmax reference point.  The fast pass fixes each row's reference at the maximum of the first 32-key block in which
@@ -184,6 +184,6 @@ __device__ __forceinline__ int fresh_lane_id() {
     return lane;
 }
 
-// tree_attn_ring.hip: the fast pass with decoupled waves over a static schedule (p.list_ptr delimits n_wg item lists, one per
-// workgroup; plan entries of 32 keys).  Stream-ordered launch on `stream`; the caller launches the exact pass behind it.
+// tree_attn_ring.hip: the pass with decoupled waves over a static schedule (p.list_ptr delimits n_wg item lists, one per
+// workgroup; plan entries of 32 keys), the exact recomputation of the items that need it included.  Stream-ordered launch on `stream`.
 int spinf_launch_ring(const AttnParams& p, int d, bool win, int n_wg, hipStream_t stream);

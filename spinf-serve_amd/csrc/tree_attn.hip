@@ -234,10 +234,8 @@ __global__ __launch_bounds__(256) void tree_attn_exact_kernel(const AttnParams p
     if (threadIdx.x == 0) {
         __threadfence();
         if (atomicAdd(&p.counters[NLIST + 2], 1) == (int)gridDim.x - 1) {
-            if (!p.keep_redo) {
-                p.counters[NLIST + 3] += n_redo;   // running total, for spinf_attn_exact_items
-                p.counters[NLIST + 1] = 0;
-            }
+            atomicAdd(&p.counters[NLIST + 3], n_redo);   // running total, for spinf_attn_exact_items
+            p.counters[NLIST + 1] = 0;
             p.counters[NLIST + 2] = 0;
             __threadfence();
         }
@@ -746,33 +744,15 @@ int launch_512(const AttnParams& p, int blocks, hipStream_t s) {
     return SPINF_OK;
 }
 
-// The ring kernel (tree_attn_ring.hip) over a static schedule, then the exact pass over what it handed on.
+// The ring kernel (tree_attn_ring.hip) over a static schedule: one launch.  It takes no item from a shared list and recomputes
+// the items that need the exact arithmetic itself, so the call uses none of the block's cursors and no second kernel.
 int launch_ring(const AttnParams& p, int d, bool win, int n_wg, hipStream_t stream) {
     if (p.clear_first) {
         hipLaunchKernelGGL(attn_clear_counters_kernel, dim3(1), dim3(64), 0, stream, p.counters);
         hipError_t e0 = hipGetLastError();
         if (e0 != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: launch (clear): %s", hipGetErrorString(e0));
     }
-    if (int rc = spinf_launch_ring(p, d, win, n_wg, stream)) return rc;
-    const int blocks = n_wg < 64 ? n_wg : 64;
-    if (d == 512) {   // the exact pass computes the output 256 dims at a time: twice over the same redo list, which the second launch clears
-        for (int half = 0; half < 2; half++) {
-            AttnParams ph = p;
-            ph.v = p.v + 256 * half;
-            ph.o = p.o + 256 * half;
-            ph.keep_redo = half == 0;
-            if (win) hipLaunchKernelGGL((tree_attn_exact_kernel<512, 1, true, 1, false, 0, 32, 256>), dim3(blocks), dim3(256), 0, stream, ph);
-            else hipLaunchKernelGGL((tree_attn_exact_kernel<512, 1, false, 1, false, 0, 32, 256>), dim3(blocks), dim3(256), 0, stream, ph);
-            const hipError_t e = hipGetLastError();
-            if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: launch (exact pass): %s", hipGetErrorString(e));
-        }
-        return SPINF_OK;
-    }
-    if (win) hipLaunchKernelGGL((tree_attn_exact_kernel<256, 1, true, 2, false, 0, 32, 256>), dim3(blocks), dim3(256), 0, stream, p);
-    else hipLaunchKernelGGL((tree_attn_exact_kernel<256, 1, false, 2, false, 0, 32, 256>), dim3(blocks), dim3(256), 0, stream, p);
-    const hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: launch (exact pass): %s", hipGetErrorString(e));
-    return SPINF_OK;
+    return spinf_launch_ring(p, d, win, n_wg, stream);
 }
 
 int launch_d512(const AttnParams& p, bool win, int grp_mode, int blocks, hipStream_t s) {
@@ -889,8 +869,8 @@ static int attn_fwd(const spinf_attn_args* a, void* stream, bool no_alloc) {
     // A block's cursors are zero: it was cleared when allocated, and every call's exact-pass kernel, which runs after the fast pass,
     // puts them back.  Only a block whose last call failed to get its kernels onto the stream is cleared first; so is the scratch
     // array of the entry point that allocates nothing, which every caller on the GPU shares.
-    p.clear_first = no_alloc || dirty;
-    p.keep_redo = false;
+    // (the ring kernel uses no cursors: only a block left dirty is cleared in front of it, for the calls that follow)
+    p.clear_first = ring ? dirty : no_alloc || dirty;
     p.static_lists = a->n_lists > 0;
     p.q = (const __bf16*)a->q; p.k = (const __bf16*)a->k; p.v = (const __bf16*)a->v; p.o = (__bf16*)a->out;
     p.q_tok = a->q_tok; p.q_head = a->q_head; p.k_tok = a->k_tok; p.k_head = a->k_head;

@@ -75,6 +75,14 @@ __device__ __forceinline__ void lds_store(int* p, int v) { __hip_atomic_store(p,
                          "v_accvgpr_write_b32 a" #C8 ", 0\n\tv_accvgpr_write_b32 a" #C9 ", 0\n\tv_accvgpr_write_b32 a" #C10 ", 0\n\tv_accvgpr_write_b32 a" #C11 ", 0\n\t" \
                          "v_accvgpr_write_b32 a" #C12 ", 0\n\tv_accvgpr_write_b32 a" #C13 ", 0\n\tv_accvgpr_write_b32 a" #C14 ", 0\n\tv_accvgpr_write_b32 a" #C15 ", 0" :: \
                              : ACC16_CLOBBERS(C0, C1, C2, C3, C4, C5, C6, C7, C8, C9, C10, C11, C12, C13, C14, C15));                                 \
+        else if constexpr (OP == 3)                                                                                                                    \
+            asm volatile("v_accvgpr_write_b32 a" #C0 ", %0\n\tv_accvgpr_write_b32 a" #C1 ", %1\n\tv_accvgpr_write_b32 a" #C2 ", %2\n\tv_accvgpr_write_b32 a" #C3 ", %3\n\t"     \
+                         "v_accvgpr_write_b32 a" #C4 ", %4\n\tv_accvgpr_write_b32 a" #C5 ", %5\n\tv_accvgpr_write_b32 a" #C6 ", %6\n\tv_accvgpr_write_b32 a" #C7 ", %7\n\t"     \
+                         "v_accvgpr_write_b32 a" #C8 ", %8\n\tv_accvgpr_write_b32 a" #C9 ", %9\n\tv_accvgpr_write_b32 a" #C10 ", %10\n\tv_accvgpr_write_b32 a" #C11 ", %11\n\t" \
+                         "v_accvgpr_write_b32 a" #C12 ", %12\n\tv_accvgpr_write_b32 a" #C13 ", %13\n\tv_accvgpr_write_b32 a" #C14 ", %14\n\tv_accvgpr_write_b32 a" #C15 ", %15" :: \
+                             "v"(r[0]), "v"(r[1]), "v"(r[2]), "v"(r[3]), "v"(r[4]), "v"(r[5]), "v"(r[6]), "v"(r[7]), "v"(r[8]), "v"(r[9]), "v"(r[10]),            \
+                         "v"(r[11]), "v"(r[12]), "v"(r[13]), "v"(r[14]), "v"(r[15])                                                                      \
+                         : ACC16_CLOBBERS(C0, C1, C2, C3, C4, C5, C6, C7, C8, C9, C10, C11, C12, C13, C14, C15));                                     \
         else                                                                                                                                           \
             asm volatile("v_accvgpr_read_b32 %0, a" #C0 "\n\tv_accvgpr_read_b32 %1, a" #C1 "\n\tv_accvgpr_read_b32 %2, a" #C2 "\n\tv_accvgpr_read_b32 %3, a" #C3 "\n\t"     \
                          "v_accvgpr_read_b32 %4, a" #C4 "\n\tv_accvgpr_read_b32 %5, a" #C5 "\n\tv_accvgpr_read_b32 %6, a" #C6 "\n\tv_accvgpr_read_b32 %7, a" #C7 "\n\t"     \
@@ -84,7 +92,7 @@ __device__ __forceinline__ void lds_store(int* p, int v) { __hip_atomic_store(p,
                            "=v"(r[11]), "=v"(r[12]), "=v"(r[13]), "=v"(r[14]), "=v"(r[15]));                                                        \
     }
 
-// OP 0: acc[TILE] += a * b (MFMA 32x32x16 bf16); OP 1: acc[TILE] = 0; OP 2: r[0..15] = acc[TILE]
+// OP 0: acc[TILE] += a * b (MFMA 32x32x16 bf16); OP 1: acc[TILE] = 0; OP 2: r[0..15] = acc[TILE]; OP 3: acc[TILE] = r[0..15]
 template <int TILE, int OP>
 __device__ __forceinline__ void acc_op(const bf16x8 a, const bf16x8 b, float (&r)[16]) {
     ACC_TILE_OPS(0, 0, 15, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15)
@@ -122,6 +130,19 @@ __device__ __forceinline__ void acc_zero() {
 template <int TILE>
 __device__ __forceinline__ void acc_read(float (&r)[16]) {
     acc_op<TILE, 2>(bf16x8{}, bf16x8{}, r);
+}
+// acc[0 .. N-1] *= alpha (the exact recomputation's rescaling; the caller brackets it with the wait states that acc_read and
+// acc_zero need)
+template <int N, int TILE = 0>
+__device__ __forceinline__ void acc_scale(const float alpha) {
+    if constexpr (TILE < N) {
+        float r[16];
+        acc_op<TILE, 2>(bf16x8{}, bf16x8{}, r);
+#pragma unroll
+        for (int i = 0; i < 16; i++) r[i] *= alpha;
+        acc_op<TILE, 3>(bf16x8{}, bf16x8{}, r);
+        acc_scale<N, TILE + 1>(alpha);
+    }
 }
 // S^T chain on ordinary registers, as assembly as well (a kernel that mixes MFMA builtins with the fixed accumulation registers
 // above would let the compiler pick accumulation registers of its own for them)
@@ -226,7 +247,8 @@ __global__ __launch_bounds__(D == 512 ? 256 : 512) void tree_attn_ring_kernel(co
     __shared__ int sy_gen;             // descriptors written so far
     __shared__ int sy_abort;
     __shared__ int sy_ntiles;
-    __shared__ int sy_redo[16];        // item sequence number + 1 of the last hand-over to the exact pass, per sequence number mod 16
+    __shared__ int sy_redo[16];        // item sequence number + 1 of the last hand-over to the exact recomputation, per sequence number mod 16
+    __shared__ int sy_nredo;           // items of this workgroup handed over so far (their indices: p.redo[lo ..])
 
     const Lane<D, TK, D> L(p);
     const int lo = p.list_ptr[blockIdx.x], hi = p.list_ptr[blockIdx.x + 1];
@@ -276,7 +298,7 @@ __global__ __launch_bounds__(D == 512 ? 256 : 512) void tree_attn_ring_kernel(co
         if (threadIdx.x < NSLOT) *(int*)(ring + threadIdx.x * G::BUFB + G::KTILEB + G::VTILEB + 768) = -1;   // the slot's flag: no generation yet
     }
     if (threadIdx.x < 16) sy_redo[threadIdx.x] = 0;
-    if (threadIdx.x == 0) { sy_gen = 0; sy_abort = 0; sy_ntiles = 0; }
+    if (threadIdx.x == 0) { sy_gen = 0; sy_abort = 0; sy_ntiles = 0; sy_nredo = 0; }
     __syncthreads();
 
     // descriptor generator (wave 0): items lo .. hi - 1, each item's plan entries in chunks of at most 64
@@ -627,13 +649,117 @@ __global__ __launch_bounds__(D == 512 ? 256 : 512) void tree_attn_ring_kernel(co
         if (hand_over) {
             if (fresh_lane_id() == 0) {
                 const int was = __hip_atomic_fetch_max(&sy_redo[iseq & 15], iseq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                if (was < iseq) p.redo[atomicAdd(&p.counters[NLIST + 1], 1)] = item_done;
+                if (was < iseq) {   // first wave of the item to say so: the workgroup recomputes the item after its list (below)
+                    const int k = __hip_atomic_fetch_add(&sy_nredo, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    __hip_atomic_store(&p.redo[lo + k], item_done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
             }
         } else {
             store_rows(tz_done);
         }
     }
     if (dead && fresh_lane_id() == 0) atomicAdd(&p.counters[NLIST + 4], 1);
+    __builtin_amdgcn_s_waitcnt(0x0f70);
+
+    // ---- the exact recomputation.  Items in which some row met scores too far above its reference (normally none) are done
+    // again here, by the workgroup that owns them, after its list: classic online softmax over the same 32-key blocks in the same
+    // order (the reference is raised, and the accumulators rescaled, whenever a block maximum exceeds it by more than TAU_LAZY),
+    // the arithmetic of tree_attn_exact_kernel (tree_attn.hip) step for step, so the two give the same bits.  Nothing is
+    // overlapped: one tile at a time into slot 0, a workgroup barrier on either side of its request.  Whether an item comes here
+    // depends on its own rows only, so a job's output does not depend on what it is packed with.
+    __syncthreads();   // every wave is through with its list: the ring is free, the hand-overs are all in
+    const int n_redo = __builtin_amdgcn_readfirstlane(lds_load(&sy_nredo));
+    if (n_redo == 0 || __builtin_amdgcn_readfirstlane(lds_load(&sy_abort)) != 0) return;
+#pragma unroll 1
+    for (int r = 0; r < n_redo; r++) {
+        const int idx = __builtin_amdgcn_readfirstlane(__hip_atomic_load(&p.redo[lo + r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+        const int4 itv = p.items[idx];
+        const int it_t = __builtin_amdgcn_readfirstlane(itv.x), it_e0 = __builtin_amdgcn_readfirstlane(itv.y), it_z = __builtin_amdgcn_readfirstlane(itv.z);
+        const int ne = it_z & 0xfffff;
+        const int tz = it_t | (int)((unsigned)it_z >> 20 << 20);
+        const int kvh = (int)((unsigned)it_z >> 20) * HPI / p.group;
+        load_q(tz);
+        reset_acc();
+#pragma unroll 1
+        for (int e = 0; e < ne; e++) {
+            const int kt = __builtin_amdgcn_readfirstlane(p.kv_idx[it_e0 + e]);
+            const unsigned bits = (unsigned)__builtin_amdgcn_readfirstlane((int)p.kv_bits[it_e0 + e]);
+            __syncthreads();   // everyone is through with the slot
+            if (L.w == 0) {
+                using GK = Geo<D, TK>;
+                const int lane = fresh_lane_id();
+                const unsigned lane_k = (unsigned)((lane / GK::CPR) * GK::NREG * p.k_tok * 2 + (lane % GK::CPR) * 16);
+                const unsigned lane_v = (unsigned)((lane / GK::CPR) * GK::NREG * p.v_tok * 2 + (lane % GK::CPR) * 16);
+                issue_tile_wave<D, WIN>(p, lds_addr(ring), kt, kvh, 0, lane, lane_k, lane_v);
+            }
+            __builtin_amdgcn_s_waitcnt(0x0f70);   // the tile has landed (and this wave's queries)
+            __syncthreads();
+            if (!((bits >> (2 * L.wr)) & 1u)) continue;   // (wave-uniform; the barriers above are passed by every wave)
+            const int ln = fresh_lane_id();
+            const char* krow = ring + G::K::k_off(ln & 31) + 16 * (ln >> 5);
+            const char* vrow = ring + G::KTILEB + G::V::v_off(4 * (ln >> 5) + ((ln >> 2) & 3)) + 32 * ((ln >> 4) & 1) + 8 * (ln & 3);
+            // (the scheduling barriers keep the three kinds of LDS reads apart: the transposing reads of V and the 16-byte reads
+            // of K and of the keys' metadata do not complete in the order they were issued, which the compiler's counting assumes)
+            f32x16 sa;
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int x = 0; x < NS; x++) {
+                const bf16x8 kf = *(const bf16x8*)(krow + 32 * x);
+                if (x == 0) qk_first(sa, kf, qf[x]);
+                else if (x == NS - 1) qk_last(sa, kf, qf[x]);
+                else qk_next(sa, kf, qf[x]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if ((bits >> (8 + 2 * L.wr)) & 1u) {
+                f32x16 sm[1] = {sa};
+                const int tok = (tz & 0xfffff) * SPINF_QTILE + 32 * L.wr + (ln & 31);
+                apply_mask<1, WIN, 0, TK>(sm, (const int*)(ring + G::KTILEB + G::VTILEB), kt, 0, ln >> 5, tok, art_q, pos_q, p.window);
+                sa = sm[0];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            bf16x8 pb[2];
+            {
+                float mx = sa[0];
+#pragma unroll
+                for (int i2 = 1; i2 < 16; i2++) mx = fmaxf(mx, sa[i2]);
+                mx = lane32_max(mx);
+                const float tm = mx * p.c;
+                const bool up = tm > M + TAU_LAZY;
+                const float mn = up ? tm : M;
+                const float alpha = up ? __builtin_amdgcn_exp2f(M - mn) : 1.0f;
+                if (__builtin_amdgcn_ballot_w64(up && M != -INFINITY) != 0) {   // rows without a key so far hold zeros
+                    asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");   // the last MFMAs' results -> v_accvgpr_read
+                    acc_scale<NDT>(alpha);
+                    asm volatile("s_nop 3" ::: "memory");                // v_accvgpr_write -> MFMA srcC
+                }
+                l *= alpha;
+                M = mn;
+                const float ms = mn == -INFINITY ? 0.f : mn;
+                float sum = 0.f;
+#pragma unroll
+                for (int i2 = 0; i2 < 16; i2++) {
+                    const float pr = __builtin_amdgcn_exp2f(__builtin_fmaf(sa[i2], p.c, -ms));
+                    sum += pr;
+                    pb[i2 >> 3][i2 & 7] = (__bf16)pr;
+                }
+                l += sum;
+            }
+            __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): no 16-byte read in flight when the transposing reads begin
+            __builtin_amdgcn_sched_barrier(0);
+            auto step = [&](auto f_c) __attribute__((always_inline)) {
+                constexpr int f = decltype(f_c)::value;
+                const char* vp = vrow + G::V::v_off(16 * (f / NDT)) + 64 * (f % NDT);
+                const s16x4 lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)vp);
+                const s16x4 hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vp + G::V::v_off(8)));
+                const bf16x8 a = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo4, hi4, 0, 1, 2, 3, 4, 5, 6, 7));
+                acc_mfma<f % NDT>(a, pb[f / NDT]);
+                __builtin_amdgcn_sched_barrier(0);
+            };
+            pv_steps<NVF>(step);
+        }
+        store_rows(tz);
+    }
+    if (threadIdx.x == 0) atomicAdd(&p.counters[NLIST + 3], n_redo);   // running total, for spinf_attn_exact_items
     __builtin_amdgcn_s_waitcnt(0x0f70);
 }
 

@@ -63,7 +63,7 @@ def _exact_items():
     return total.value
 
 
-@pytest.mark.parametrize("d,hq,hkv", [(64, 4, 2), (128, 4, 2), (256, 2, 1), (128, 3, 3)])
+@pytest.mark.parametrize("d,hq,hkv", [(64, 4, 2), (128, 4, 2), (256, 2, 1), (128, 3, 3), (512, 4, 1)])
 def test_wide_score_range_takes_the_exact_pass(dev, d, hq, hkv):
     """scores that grow by far more than the fast pass allows for (2^60 above a row's first block maximum) send the query tile
     to the exact pass, which rescales its accumulators like a classic online softmax; the result must still match"""
@@ -91,6 +91,38 @@ def test_wide_score_range_takes_the_exact_pass(dev, d, hq, hkv):
     torch.cuda.synchronize()
     assert _exact_items() == mid
     assert float(np.abs(out2.float().cpu().numpy() - _oracle(q, k2, v, b, cfg.scale)).max()) <= TOL
+
+
+@pytest.mark.parametrize("d,hq,hkv", [(256, 4, 2), (512, 4, 1)])
+@pytest.mark.parametrize("window", [None, 150])
+def test_exact_recomputation_is_the_same_in_both_kernels(dev, d, hq, hkv, window, monkeypatch):
+    """the kernel with decoupled waves recomputes the items with too wide a score range itself, after its list; the lockstep
+    kernels leave them to a second kernel: the same arithmetic, so the same bits, on a stream where some items take it and
+    others do not; each run counts its items"""
+    from spinf_serve_amd import attention
+
+    rng = np.random.default_rng(21)
+    trees = [synth._tree(rng, 400, [30, 11, 64]), synth._tree(rng, 150, [9, 40]), synth._tree(rng, 260, [])]
+    cfg = synth.AttnConfig("wide2", hq, hkv, d, d ** -0.5, 1.0, None, trees)
+    b = synth.pack(trees)[0]
+    q, k, v = synth.qkv(cfg, b, seed=6, device=dev)
+    k = k.clone()
+    k[200:330] *= 60.0      # a stretch in the middle of the first trunk: the tiles of the first content that see it are redone
+    mask = sa.TreeMask.build(b.art, b.end, b.pos, window=window, device=dev)
+    outs, counts = [], []
+    for ring in (0, 1):
+        monkeypatch.setattr(attention, "RING", ring)
+        print(f"case wide d={d} ring={ring} window={window}", flush=True)
+        before = _exact_items()
+        outs.append(sa.tree_attn(q, k, v, mask, cfg.scale))
+        torch.cuda.synchronize()
+        counts.append(_exact_items() - before)
+    assert counts[0] > 0 and counts[1] > 0, counts
+    assert counts[0] == counts[1] * (2 if d == 512 else 1), counts   # (the lockstep kernels take head dim 512 in two launches)
+    assert torch.equal(outs[0], outs[1])
+    got = outs[1].float().cpu().numpy()
+    assert np.isfinite(got).all()
+    assert float(np.abs(got - _oracle(q, k, v, b, cfg.scale, window)).max()) <= TOL
 
 
 @pytest.mark.parametrize("variant", [0, 1, 2])
