@@ -128,8 +128,9 @@ int spinf_tree_attn_fwd(const spinf_attn_args* args, void* stream);
  * counts and redo list in a buffer that the library allocates (and regrows) on the device; this entry point keeps them in a
  * file-scope device array of 64 + 65,536 ints (256.25 KiB per GPU, held until the process ends) and calls no hipMalloc /
  * hipFree nor any allocating routine.  Same arguments, same kernels, same results bit for bit.  Limit: n_items (query tiles x
- * head groups) <= 65,536, more is SPINF_E_ARG.  The cursors and counts are cleared by a small kernel in front of every pass, so
- * a call does not depend on what the previous one left.  Every call on a GPU shares that GPU's array: calls that overlap on
+ * head groups) <= 65,536, more is SPINF_E_ARG.  The cursors and counts are cleared by a small kernel in front of every pass that
+ * uses them (the kernel with decoupled waves uses none: such a call is one launch), so a call does not depend on what the
+ * previous one left.  Every call on a GPU shares that GPU's array: calls that overlap on
  * one GPU (different streams or threads) race; order them on one stream. */
 int spinf_tree_attn_fwd_noalloc(const spinf_attn_args* args, void* stream);
 /* Diagnostics (no counterpart in the reference): *total = work items that the exact (rescaling) pass has recomputed on the
