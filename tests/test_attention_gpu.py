@@ -125,6 +125,46 @@ def test_exact_recomputation_is_the_same_in_both_kernels(dev, d, hq, hkv, window
     assert float(np.abs(got - _oracle(q, k, v, b, cfg.scale, window)).max()) <= TOL
 
 
+def test_exact_recomputation_with_several_items_per_workgroup(dev, monkeypatch):
+    """a stream with more work items than workgroups (some workgroups own two or three, of which one or more are redone after the
+    list), wide scores in two of its contents: decoupled kernel == lockstep kernels + exact-pass kernel, bit for bit, and every
+    content that has no wide scores is bit-identical to the same stream without any"""
+    from spinf_serve_amd import attention
+
+    cfg = synth.attention_config("C2", contents=9)
+    b = cfg.batches[0]
+    q, k, v = synth.qkv(cfg, b, seed=8, device=dev)
+    k_wide = k.clone()
+    for slot in (1, 4):
+        start, length, *_ = b.jobs[slot]
+        k_wide[start + length // 3 : start + length // 2] *= 50.0
+    mask = sa.TreeMask.build(b.art, b.end, b.pos, device=dev)
+    n_items = mask.for_head_dim(cfg.d, ring=True).plan.n_qtiles * (cfg.hq // 2)
+    assert n_items > torch.cuda.get_device_properties(dev).multi_processor_count
+    outs, counts = [], []
+    for ring in (0, 1):
+        monkeypatch.setattr(attention, "RING", ring)
+        print(f"case several items per workgroup ring={ring}", flush=True)
+        before = _exact_items()
+        outs.append(sa.tree_attn(q, k_wide, v, mask, cfg.scale))
+        torch.cuda.synchronize()
+        counts.append(_exact_items() - before)
+    assert counts[0] == counts[1] and counts[1] >= 4, counts
+    assert torch.equal(outs[0], outs[1])
+    assert torch.isfinite(outs[1].float()).all()
+    plain = sa.tree_attn(q, k, v, mask, cfg.scale)
+    for slot in range(len(b.jobs)):
+        if slot in (1, 4):
+            continue
+        start, length, *_ = b.jobs[slot]
+        assert torch.equal(plain[start : start + length], outs[1][start : start + length]), slot
+    start, length, *_ = b.jobs[1]
+    sl = slice(start, start + length)
+    dense = omask.dense_tree_mask(b.art[sl], b.end[sl] - start, b.pos[sl], None)
+    ref = oattn.masked_attention(q[sl].float().cpu().numpy(), k_wide[sl].float().cpu().numpy(), v[sl].float().cpu().numpy(), dense, cfg.scale)
+    assert float(np.abs(outs[1][sl].float().cpu().numpy() - ref).max()) <= TOL
+
+
 @pytest.mark.parametrize("variant", [0, 1, 2])
 def test_c4_shape_two_level_tree(dev, variant):
     """variant 0: eight waves, heads of a pair on different waves; 1: one head per item; 2: four waves with two heads each"""
