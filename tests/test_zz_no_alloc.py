@@ -58,6 +58,42 @@ def test_noalloc_exact_pass_and_other_geometry(dev):
     assert torch.equal(want, got)
 
 
+def test_noalloc_head_dim_512_one_launch_and_graph_replay(dev):
+    """head dim 512 through the entry point that allocates nothing: the kernel with decoupled waves, ONE launch per call (it takes
+    no item from a shared list and redoes its wide-range items itself, their indices in the scratch array), so the call can be
+    recorded into a graph as it is; replays, with eager calls in between, give the allocating entry point's bits every time"""
+    cfg = synth.attention_config("C2_512", contents=3)
+    b = cfg.batches[0]
+    want, got = _pair(cfg, b, dev, seed=4)
+    assert torch.equal(want, got)
+    lib = sa.load_library()
+    total = ctypes.c_int64(0)
+    assert lib.spinf_attn_exact_items(ctypes.byref(total)) == 0
+    before = total.value
+    want_w, got_w = _pair(cfg, b, dev, seed=4, scale_keys=(200, 50.0))   # wide scores: items redone inside the launch
+    assert torch.equal(want_w, got_w)
+    assert lib.spinf_attn_exact_items(ctypes.byref(total)) == 0
+    assert total.value > before
+    q, k, v = synth.qkv(cfg, b, seed=4, device=dev)
+    mask = sa.TreeMask.build(b.art, b.end, b.pos, device=dev)
+    sa.tree_attn(q, k, v, mask, cfg.scale)     # uploads the schedule of this mask
+    torch.cuda.synchronize()
+    out = torch.zeros_like(want)
+    side = torch.cuda.Stream(device=dev)
+    g = torch.cuda.CUDAGraph()
+    print("no-alloc case d512 under capture", flush=True)
+    with torch.cuda.graph(g, stream=side):
+        sa.tree_attn_noalloc(q, k, v, mask, out, cfg.scale)
+    for rep in range(3):
+        out.zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), rep
+        again = sa.tree_attn(q, k, v, mask, cfg.scale)   # eager work between the replays
+        torch.cuda.synchronize()
+        assert torch.equal(again, want)
+
+
 def test_noalloc_rejects_more_items_than_its_array_holds(dev):
     a = sa._lib.AttnArgs()
     one = torch.zeros(8, dtype=torch.int32, device=dev)
