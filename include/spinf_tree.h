@@ -118,6 +118,10 @@ typedef struct spinf_attn_args {
                                                ktile 32 (and d = 512, or d = 256 with an even number of query heads per key / value head and
                                                variant 0; stream layout, no groups) that is the kernel with decoupled waves, which at
                                                d = 512 computes the pass in one launch instead of two */
+    int32_t debug_expire;                   /* 0 in production.  Test hook of the kernel with decoupled waves (no counterpart in the reference):
+                                               k > 0 makes wave 0 of every workgroup treat its wait at its k-th tile as run out, which takes the
+                                               workgroup through the landing that a real time-out would take (the rest of its list computed one
+                                               tile at a time between barriers).  Same results bit for bit; spinf_attn_ring_aborts counts it */
 } spinf_attn_args;
 
 /* query heads one work item covers for this geometry (1 or 2); 0 for an invalid geometry */
@@ -138,8 +142,9 @@ int spinf_tree_attn_fwd_noalloc(const spinf_attn_args* args, void* stream);
  * Synchronises the device. */
 int spinf_attn_exact_items(int64_t* total);
 /* Diagnostics (no counterpart in the reference): *total = waves of the static-schedule kernel that gave up a bounded wait on
- * the current device since the library was loaded.  Always 0 unless the kernel has a bug; the results of such a pass are
- * invalid.  Synchronises the device. */
+ * the current device since the library was loaded.  Always 0 unless the kernel has a bug (or debug_expire asked for it).  The
+ * results of such a pass are still complete and the same bit for bit: the workgroup finishes its list one tile at a time between
+ * barriers; the count says that time was lost.  Synchronises the device. */
 int spinf_attn_ring_aborts(int64_t* total);
 
 /* ------------------------------------------------------------------------------------------------ Gated DeltaNet

@@ -30,6 +30,7 @@ struct AttnParams {
     const int* grp;       // image groups (GRP kernels): -1 none; the tokens of a group see each other both ways
     bool static_lists;    // list_ptr delimits one item list per workgroup (a static schedule) instead of the eight shared lists
     bool clear_first;     // host side only: zero the cursors and counts in front of the pass (the entry point that allocates nothing)
+    int debug_expire;     // ring kernel, test hook: > 0 makes wave 0 of every workgroup give up at its tile debug_expire - 1, as if a wait had run out
 };
 
 // Softmax reference point.  The fast pass fixes each row's reference at the maximum of the first 32-key block in which
@@ -145,11 +146,14 @@ struct Lane {
 
 // mask of one 32-key block: register i of the S^T tile holds key 8*(i/4) + 4g + i%4 of the block
 // GRP 1: a key of the row's image group is visible whatever the rest says; GRP 2: if it also lies within the window
-template <int RT, bool WIN, int GRP = 0, int TK = 64>
+// STEPWISE: the four groups of four keys one after the other (a scheduling barrier between them), so that only one group's
+// metadata is in registers at a time; otherwise the compiler requests all of it up front (up to 64 registers)
+template <int RT, bool WIN, int GRP = 0, int TK = 64, bool STEPWISE = false>
 __device__ __forceinline__ void apply_mask(f32x16 (&s_acc)[RT], const int* meta, int kt, int sub, int g, int tok, int art_q, int pos_q, int window,
                                            int grp_q = -1) {
 #pragma unroll
     for (int i4 = 0; i4 < 4; i4++) {
+        if (STEPWISE && i4 > 0) __builtin_amdgcn_sched_barrier(0);
         const int ko = 32 * sub + 8 * i4 + 4 * g;
         const int4 ka = *(const int4*)(meta + ko);
         const int4 ke = *(const int4*)(meta + 64 + ko);

@@ -888,6 +888,7 @@ static int attn_fwd(const spinf_attn_args* a, void* stream, bool no_alloc) {
     p.row_of = a->row_of; p.kv_row0 = a->kv_row0;
     p.grp = a->grp;
     p.counters = counters;
+    p.debug_expire = ring ? a->debug_expire : 0;
     p.redo = counters + 64;
     const int blocks = a->n_lists > 0 ? a->n_lists : (int)(a->n_items < cus ? a->n_items : cus);
     const bool win = p.window > 0;

@@ -40,6 +40,7 @@ constexpr int GEN_AHEAD = 48;       // wave 0 keeps the descriptors this far ahe
 constexpr int SPIN_LIMIT = 1 << 18; // polls of one wait before the workgroup gives up (a healthy wait takes a handful)
 constexpr int SROW = 64 + 16;       // output staging: 32 rows x 32 head dims, 80-byte rows
 constexpr unsigned DESC_FIRST = 1u << 16, DESC_LAST = 1u << 17;
+constexpr unsigned DESC_EXPIRE = 1u << 18;   // test hook: wave 0 treats its wait for this tile as run out
 
 __device__ __forceinline__ int lds_load(const int* p) { return __hip_atomic_load(p, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP); }
 // plain (non-atomic) reads of words other waves write, as LDS instructions: a volatile access through a generic pointer becomes a
@@ -145,15 +146,34 @@ __device__ __forceinline__ void acc_scale(const float alpha) {
     }
 }
 // S^T chain on ordinary registers, as assembly as well (a kernel that mixes MFMA builtins with the fixed accumulation registers
-// above would let the compiler pick accumulation registers of its own for them)
-__device__ __forceinline__ void qk_first(f32x16& sa, const bf16x8 k, const bf16x8 q) {
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(sa) : "v"(k), "v"(q));
-}
-__device__ __forceinline__ void qk_next(f32x16& sa, const bf16x8 k, const bf16x8 q) {
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(sa) : "v"(k), "v"(q));
-}
-__device__ __forceinline__ void qk_last(f32x16& sa, const bf16x8 k, const bf16x8 q) {   // + the wait states before the vector ALU reads the result
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0\n\ts_nop 15" : "+v"(sa) : "v"(k), "v"(q));
+// above would let the compiler pick accumulation registers of its own for them).
+// Where the queries live.  At head dim 256 the 16 query fragments of a wave (64 registers, constant over a work item) sit in
+// a[128:191], behind the compiler's back like the accumulators: as compiler-visible values they are what the register allocator
+// spills whenever anything else in the tile loop changes (the loop then reloads them from scratch memory in front of the first
+// MFMAs, and such a reload waits for every tile request in flight).  The kernel is limited to 60 ordinary registers
+// (amdgpu_num_vgpr), 196 accumulation registers: a[0:127] O^T, a[128:191] queries, a192 / a193 art / pos of the wave's rows.
+// At head dim 512 the accumulators take all 256 accumulation registers and the queries stay compiler-visible (205 ordinary
+// registers, one wave per SIMD: nothing is spilled there).
+template <int D>
+constexpr bool Q_IN_ACC = D == 256;
+constexpr int QBASE = 128, ROW_ART = 192, ROW_POS = 193;
+
+// step S of NS of S^T = K Q^T: sa (+)= k * q fragment S; the last step carries the wait states before the vector ALU reads the result
+template <int D, int S>
+__device__ __forceinline__ void qk_step(f32x16& sa, const bf16x8 k, const bf16x8 (&qf)[Q_IN_ACC<D> ? 1 : D / 16]) {
+    constexpr int NS = D / 16;
+    if constexpr (Q_IN_ACC<D>) {
+        if constexpr (S == 0)
+            asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, a[%c2:%c3], 0" : "=&v"(sa) : "v"(k), "n"(QBASE + 4 * S), "n"(QBASE + 4 * S + 3));
+        else if constexpr (S == NS - 1)
+            asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, a[%c2:%c3], %0\n\ts_nop 15" : "+v"(sa) : "v"(k), "n"(QBASE + 4 * S), "n"(QBASE + 4 * S + 3));
+        else
+            asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, a[%c2:%c3], %0" : "+v"(sa) : "v"(k), "n"(QBASE + 4 * S), "n"(QBASE + 4 * S + 3));
+    } else {
+        if constexpr (S == 0) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(sa) : "v"(k), "v"(qf[S]));
+        else if constexpr (S == NS - 1) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0\n\ts_nop 15" : "+v"(sa) : "v"(k), "v"(qf[S]));
+        else asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(sa) : "v"(k), "v"(qf[S]));
+    }
 }
 
 // A tile's "landed" flag is written by the DMA engine itself: the last request of a tile copies ring_seq[generation % 64] from
@@ -217,6 +237,75 @@ __device__ __forceinline__ void issue_tile_wave(const AttnParams& p, unsigned bu
     dma4_lane(ring_seq + (gen & 63), buf + KTILEB + VTILEB + 768);   // every lane the same word: 64 copies of the flag
 }
 
+// A wave's place in the workgroup: four row groups x HPI heads of the item.
+template <int D>
+struct RingShape {
+    static constexpr int TK = 32;
+    static constexpr int NW = D == 512 ? 4 : 8;      // waves: four row groups x HPI heads of the item
+    static constexpr int HPI = NW / 4;
+    static constexpr int NSLOT = D == 512 ? 2 : MAX_SLOT;
+    static constexpr int NS = D / 16;     // contraction steps of K Q^T
+    static constexpr int NDT = D / 32;    // 32-wide slices of the head dimension in O^T
+    static constexpr int NVF = 2 * NDT;   // V^T fragments of one 32-key block
+};
+
+// Requests the queries of rows 32 wr .. of query tile tz & 0xfffff, head (tz >> 20) * HPI + wh (the B operands of K Q^T), and art / pos
+// of the wave's rows.  Head dim 256: into the accumulation registers, by assembly; nothing the compiler sees depends on them, so
+// the caller waits (ring_wait_q) before the item's first MFMA and before ring_row_meta.  Head dim 512: ordinary loads into qf, art_q, pos_q.
+#define RING_Q_LOAD(S) "global_load_dwordx4 a[" #S "*4+128:" #S "*4+131], %0, off offset:" #S "*32\n\t"
+#define RING_Q_CLOB(B) "a" #B
+template <int D, bool WIN>
+__device__ __forceinline__ void ring_load_q(const AttnParams& p, const int wr, const int wh, const int tz, bf16x8 (&qf)[Q_IN_ACC<D> ? 1 : D / 16], int& art_q,
+                                            int& pos_q) {
+    const int lane = fresh_lane_id();
+    const int tok = (tz & 0xfffff) * SPINF_QTILE + 32 * wr + (lane & 31);
+    const int tok_c = tok < p.n ? tok : p.n - 1;
+    const int h = (int)((unsigned)tz >> 20) * RingShape<D>::HPI + wh;
+    const __bf16* qp = p.q + (long)tok_c * p.q_tok + (long)h * p.q_head + 8 * (lane >> 5);
+    if constexpr (Q_IN_ACC<D>) {
+        asm volatile(RING_Q_LOAD(0) RING_Q_LOAD(1) RING_Q_LOAD(2) RING_Q_LOAD(3) RING_Q_LOAD(4) RING_Q_LOAD(5) RING_Q_LOAD(6) RING_Q_LOAD(7)
+                     RING_Q_LOAD(8) RING_Q_LOAD(9) RING_Q_LOAD(10) RING_Q_LOAD(11) RING_Q_LOAD(12) RING_Q_LOAD(13) RING_Q_LOAD(14) RING_Q_LOAD(15)
+                     "global_load_dword a192, %1, off"
+                     :: "v"(qp), "v"(p.art + tok_c)
+                     : "memory", RING_Q_CLOB(128), RING_Q_CLOB(129), RING_Q_CLOB(130), RING_Q_CLOB(131), RING_Q_CLOB(132), RING_Q_CLOB(133), RING_Q_CLOB(134),
+                       RING_Q_CLOB(135), RING_Q_CLOB(136), RING_Q_CLOB(137), RING_Q_CLOB(138), RING_Q_CLOB(139), RING_Q_CLOB(140), RING_Q_CLOB(141), RING_Q_CLOB(142),
+                       RING_Q_CLOB(143), RING_Q_CLOB(144), RING_Q_CLOB(145), RING_Q_CLOB(146), RING_Q_CLOB(147), RING_Q_CLOB(148), RING_Q_CLOB(149), RING_Q_CLOB(150),
+                       RING_Q_CLOB(151), RING_Q_CLOB(152), RING_Q_CLOB(153), RING_Q_CLOB(154), RING_Q_CLOB(155), RING_Q_CLOB(156), RING_Q_CLOB(157), RING_Q_CLOB(158),
+                       RING_Q_CLOB(159), RING_Q_CLOB(160), RING_Q_CLOB(161), RING_Q_CLOB(162), RING_Q_CLOB(163), RING_Q_CLOB(164), RING_Q_CLOB(165), RING_Q_CLOB(166),
+                       RING_Q_CLOB(167), RING_Q_CLOB(168), RING_Q_CLOB(169), RING_Q_CLOB(170), RING_Q_CLOB(171), RING_Q_CLOB(172), RING_Q_CLOB(173), RING_Q_CLOB(174),
+                       RING_Q_CLOB(175), RING_Q_CLOB(176), RING_Q_CLOB(177), RING_Q_CLOB(178), RING_Q_CLOB(179), RING_Q_CLOB(180), RING_Q_CLOB(181), RING_Q_CLOB(182),
+                       RING_Q_CLOB(183), RING_Q_CLOB(184), RING_Q_CLOB(185), RING_Q_CLOB(186), RING_Q_CLOB(187), RING_Q_CLOB(188), RING_Q_CLOB(189), RING_Q_CLOB(190),
+                       RING_Q_CLOB(191), RING_Q_CLOB(192));
+        if (WIN) asm volatile("global_load_dword a193, %0, off" :: "v"(p.pos + tok_c) : "memory", RING_Q_CLOB(193));
+    } else {
+#pragma unroll
+        for (int s = 0; s < D / 16; s++) qf[s] = *(const bf16x8*)(qp + 16 * s);
+        art_q = tok < p.n ? p.art[tok_c] : -1;
+        pos_q = WIN ? p.pos[tok_c] : 0;
+    }
+}
+#undef RING_Q_LOAD
+#undef RING_Q_CLOB
+// Head dim 256: waits until every request of the wave has returned, the queries with them.  (Loads and stores do not return in one
+// order, so "all but the n youngest" says nothing once stores are in flight: the wait stands in front of the item's stores, which
+// then drain while the next item is computed.)
+template <int D>
+__device__ __forceinline__ void ring_wait_q() {
+    if constexpr (Q_IN_ACC<D>) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+// art / pos of this lane's query row (head dim 256: out of the accumulation registers the requests went to; the caller has waited)
+template <int D, bool WIN>
+__device__ __forceinline__ void ring_row_meta(const AttnParams& p, const int wr, const int tz, int& art_q, int& pos_q) {
+    if constexpr (Q_IN_ACC<D>) {
+        const int tok = (tz & 0xfffff) * SPINF_QTILE + 32 * wr + (fresh_lane_id() & 31);
+        int a, ps = 0;
+        asm volatile("v_accvgpr_read_b32 %0, a192" : "=v"(a));
+        if (WIN) asm volatile("v_accvgpr_read_b32 %0, a193" : "=v"(ps));
+        art_q = tok < p.n ? a : -1;
+        pos_q = ps;
+    }
+}
+
 template <int N, int F = 0, class Fn>
 __device__ __forceinline__ void pv_steps(Fn& fn) {
     if constexpr (F < N) {
@@ -225,23 +314,227 @@ __device__ __forceinline__ void pv_steps(Fn& fn) {
     }
 }
 
+// normalise O^T and store it as rows: 32 rows x 32 head dims at a time through the wave's own LDS slice `stage`, 16-byte pieces out
+// (pieces of 8 bytes straight from the registers were measured slower: twice the requests for the same bytes)
+template <int D>
+__device__ __forceinline__ void ring_store_rows(const AttnParams& p, const int wr, const int wh, char* const stage, const int tz, const float l) {
+    constexpr int NDT = D / 32;
+    const int lane = fresh_lane_id(), m = lane & 31, g = lane >> 5;
+    const int tok0 = (tz & 0xfffff) * SPINF_QTILE + 32 * wr;
+    const int h = (int)((unsigned)tz >> 20) * RingShape<D>::HPI + wh;
+    const float inv = 1.0f / lane32_sum(l);
+    __bf16* ob = p.o + (long)h * p.o_head;
+    asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");   // the last MFMAs' results -> v_accvgpr_read
+    // tile dt is read back from the slice while tile dt + 1 is converted and written to it (the LDS takes a wave's requests
+    // in order, so the write behind the read is safe), and stored after that: no wait between a write and its read-back
+    auto put = [&](auto dt_c) __attribute__((always_inline)) {
+        constexpr int dt = decltype(dt_c)::value;
+        float r16[16];
+        acc_read<dt>(r16);
+#pragma unroll
+        for (int i4 = 0; i4 < 4; i4++) {
+            bf16x4 r;
+#pragma unroll
+            for (int jj = 0; jj < 4; jj++) r[jj] = (__bf16)(r16[4 * i4 + jj] * inv);
+            *(bf16x4*)(stage + m * SROW + (8 * i4 + 4 * g) * 2) = r;
+        }
+    };
+    auto round = [&](auto dt_c) __attribute__((always_inline)) {
+        constexpr int dt = decltype(dt_c)::value;
+        bf16x8 val[2];
+#pragma unroll
+        for (int jj = 0; jj < 2; jj++) {
+            const int c = jj * 64 + lane;
+            val[jj] = *(const bf16x8*)(stage + (c >> 2) * SROW + (c & 3) * 16);
+        }
+        if constexpr (dt + 1 < NDT) put(std::integral_constant<int, dt + 1>{});
+#pragma unroll
+        for (int jj = 0; jj < 2; jj++) {
+            const int c = jj * 64 + lane, row = c >> 2, col = c & 3;
+            if (tok0 + row < p.n) *(bf16x8*)(ob + (long)(tok0 + row) * p.o_tok + 32 * dt + col * 8) = val[jj];
+        }
+    };
+    put(std::integral_constant<int, 0>{});
+    pv_steps<NDT>(round);
+}
+
+// ---- after the list: the barrier-paced pass over single items.  One tile at a time into slot 0 of the ring, a workgroup barrier on
+// either side of its request, nothing overlapped, no spin anywhere.  Two users:
+//   * the exact recomputation.  Items in which some row met scores too far above its reference (normally none) are done again by the
+//     workgroup that owns them: classic online softmax over the same 32-key blocks in the same order (the reference is raised, and
+//     the accumulators rescaled, whenever a block maximum exceeds it by more than TAU_LAZY), the arithmetic of tree_attn_exact_kernel
+//     (tree_attn.hip) step for step, so the two give the same bits.  Whether an item comes here depends on its own rows only, so a
+//     job's output does not depend on what it is packed with.
+//   * the landing after an abort.  If a wave gave up a wait, every wave has left the ring; the items li .. hi - 1 of the list (from
+//     the first one that some wave had not completed) are then computed here with the ring pass's own arithmetic (fixed reference, no
+//     rescaling: the same bits), handing items to the exact recomputation by the same rule.  An abort costs time, never rows.
+// Every wave of the workgroup calls it together: li < hi only after an abort; *sy_nredo = entries of the workgroup's redo list
+// p.redo[lo ..]; *sy_vote = 0.
 template <int D, bool WIN>
-__global__ __launch_bounds__(D == 512 ? 256 : 512) void tree_attn_ring_kernel(const AttnParams p) {
-    constexpr int TK = 32;
-    constexpr int NW = D == 512 ? 4 : 8;      // waves: four row groups x HPI heads of the item
-    constexpr int HPI = NW / 4;
-    constexpr int NSLOT = D == 512 ? 2 : MAX_SLOT;
+__device__ __forceinline__ void ring_paced_pass(const AttnParams& p, char* const ring, char* const stage_all, int* const sy_nredo, int* const sy_vote,
+                                                          const int lo, const int hi, int li) {
+    using S = RingShape<D>;
+    constexpr int TK = S::TK, HPI = S::HPI, NS = S::NS, NDT = S::NDT, NVF = S::NVF;
     using G = TileGeo<D, TK, D>;
-    constexpr int NS = D / 16;     // contraction steps of K Q^T
-    constexpr int NDT = D / 32;    // 32-wide slices of the head dimension in O^T
-    constexpr int NVF = 2 * NDT;   // V^T fragments of one 32-key block
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wh = w >> 2, wr = wh ? 3 - (w & 3) : (w & 3);   // as Lane (attn_kernels.h)
+    char* const stage = stage_all + w * 32 * SROW;
+    bf16x8 qf[Q_IN_ACC<D> ? 1 : NS];
+    int art_q = -1, pos_q = 0;
+    int ri = 0;   // next entry of the redo list
+#pragma unroll 1
+    while (true) {
+        const bool exact = li >= hi;   // first the landing's items, if any, then the recomputations
+        int idx = li;
+        if (exact) {
+            if (ri >= __builtin_amdgcn_readfirstlane(lds_load(sy_nredo))) break;
+            idx = __builtin_amdgcn_readfirstlane(__hip_atomic_load(&p.redo[lo + ri], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+        }
+        const int4 itv = p.items[idx];
+        const int it_t = __builtin_amdgcn_readfirstlane(itv.x), it_e0 = __builtin_amdgcn_readfirstlane(itv.y), it_z = __builtin_amdgcn_readfirstlane(itv.z);
+        const int ne = it_z & 0xfffff;
+        const int tz = it_t | (int)((unsigned)it_z >> 20 << 20);
+        const int kvh = (int)((unsigned)it_z >> 20) * HPI / p.group;
+        ring_load_q<D, WIN>(p, wr, wh, tz, qf, art_q, pos_q);
+        float M = -INFINITY, l = 0.f;
+        bool viol = false;
+        acc_zero<NDT>();
+        ring_wait_q<D>();
+        ring_row_meta<D, WIN>(p, wr, tz, art_q, pos_q);
+#pragma unroll 1
+        for (int e = 0; e < ne; e++) {
+            const int kt = __builtin_amdgcn_readfirstlane(p.kv_idx[it_e0 + e]);
+            const unsigned bits = (unsigned)__builtin_amdgcn_readfirstlane((int)p.kv_bits[it_e0 + e]);
+            __syncthreads();   // everyone is through with the slot
+            if (w == 0) {
+                using GK = Geo<D, TK>;
+                const int lane = fresh_lane_id();
+                const unsigned lane_k = (unsigned)((lane / GK::CPR) * GK::NREG * p.k_tok * 2 + (lane % GK::CPR) * 16);
+                const unsigned lane_v = (unsigned)((lane / GK::CPR) * GK::NREG * p.v_tok * 2 + (lane % GK::CPR) * 16);
+                issue_tile_wave<D, WIN>(p, lds_addr(ring), kt, kvh, 0, lane, lane_k, lane_v);
+            }
+            __builtin_amdgcn_s_waitcnt(0x0f70);   // the tile has landed (and this wave's queries)
+            __syncthreads();
+            if (!((bits >> (2 * wr)) & 1u)) continue;   // (wave-uniform; the barriers above are passed by every wave)
+            const int ln = fresh_lane_id();
+            const char* krow = ring + G::K::k_off(ln & 31) + 16 * (ln >> 5);
+            const char* vrow = ring + G::KTILEB + G::V::v_off(4 * (ln >> 5) + ((ln >> 2) & 3)) + 32 * ((ln >> 4) & 1) + 8 * (ln & 3);
+            // (the scheduling barriers keep the three kinds of LDS reads apart, and every read of one kind has returned before the
+            // first of the next kind is issued: the MFMAs are assembly, so nothing else orders the loads that feed them)
+            f32x16 sa;
+            __builtin_amdgcn_sched_barrier(0);
+            auto score = [&](auto x_c) __attribute__((always_inline)) {
+                constexpr int x = decltype(x_c)::value;
+                const bf16x8 kf = *(const bf16x8*)(krow + 32 * x);
+                qk_step<D, x>(sa, kf, qf);
+            };
+            pv_steps<NS>(score);
+            __builtin_amdgcn_sched_barrier(0);
+            if ((bits >> (8 + 2 * wr)) & 1u) {
+                f32x16 sm[1] = {sa};
+                const int tok = (tz & 0xfffff) * SPINF_QTILE + 32 * wr + (ln & 31);
+                apply_mask<1, WIN, 0, TK>(sm, (const int*)(ring + G::KTILEB + G::VTILEB), kt, 0, ln >> 5, tok, art_q, pos_q, p.window);
+                sa = sm[0];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            bf16x8 pb[2];
+            // (each branch is written out in full, statement for statement as in tree_attn_exact_kernel and in the ring loop: the
+            // compiler contracts `l *= alpha; l += sum` into one fused multiply-add where it sees them together, and the bits follow)
+            if (exact) {
+                float mx = sa[0];
+#pragma unroll
+                for (int i2 = 1; i2 < 16; i2++) mx = fmaxf(mx, sa[i2]);
+                mx = lane32_max(mx);
+                const float tm = mx * p.c;
+                const bool up = tm > M + TAU_LAZY;
+                const float mn = up ? tm : M;
+                const float alpha = up ? __builtin_amdgcn_exp2f(M - mn) : 1.0f;
+                if (__builtin_amdgcn_ballot_w64(up && M != -INFINITY) != 0) {   // rows without a key so far hold zeros
+                    asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");   // the last MFMAs' results -> v_accvgpr_read
+                    acc_scale<NDT>(alpha);
+                    asm volatile("s_nop 3" ::: "memory");                // v_accvgpr_write -> MFMA srcC
+                }
+                l *= alpha;
+                M = mn;
+                const float ms = mn == -INFINITY ? 0.f : mn;
+                float sum = 0.f;
+#pragma unroll
+                for (int i2 = 0; i2 < 16; i2++) {
+                    const float pr = __builtin_amdgcn_exp2f(__builtin_fmaf(sa[i2], p.c, -ms));
+                    sum += pr;
+                    pb[i2 >> 3][i2 & 7] = (__bf16)pr;
+                }
+                l += sum;
+            } else {   // the ring pass's arithmetic: the row's reference is the maximum of the first block it sees a key in
+                const bool first = M == -INFINITY;
+                if (__builtin_amdgcn_ballot_w64(first) != 0) {
+                    float mx = sa[0];
+#pragma unroll
+                    for (int i2 = 1; i2 < 16; i2++) mx = fmaxf(mx, sa[i2]);
+                    mx = lane32_max(mx);
+                    M = first ? mx * p.c : M;
+                }
+                const float ms = M == -INFINITY ? 0.f : M;
+                float sum = 0.f;
+#pragma unroll
+                for (int i2 = 0; i2 < 16; i2++) {
+                    const float pr = __builtin_amdgcn_exp2f(__builtin_fmaf(sa[i2], p.c, -ms));
+                    sum += pr;
+                    pb[i2 >> 3][i2 & 7] = (__bf16)pr;
+                }
+                l += sum;
+                viol = viol | !(sum <= VIOL_SUM);
+            }
+            __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): no 16-byte read in flight when the transposing reads begin
+            __builtin_amdgcn_sched_barrier(0);
+            auto step = [&](auto f_c) __attribute__((always_inline)) {
+                constexpr int f = decltype(f_c)::value;
+                const char* vp = vrow + G::V::v_off(16 * (f / NDT)) + 64 * (f % NDT);
+                const s16x4 lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)vp);
+                const s16x4 hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vp + G::V::v_off(8)));
+                const bf16x8 a = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo4, hi4, 0, 1, 2, 3, 4, 5, 6, 7));
+                acc_mfma<f % NDT>(a, pb[f / NDT]);
+                __builtin_amdgcn_sched_barrier(0);
+            };
+            pv_steps<NVF>(step);
+        }
+        if (!exact && __builtin_amdgcn_ballot_w64(viol) != 0) {   // scores ranged too widely somewhere in these 32 rows: the item is done again, exactly
+            if (fresh_lane_id() == 0) __hip_atomic_store(sy_vote, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        } else {
+            ring_store_rows<D>(p, wr, wh, stage, tz, l);
+        }
+        if (exact) {
+            ri++;
+            continue;
+        }
+        __syncthreads();
+        if (threadIdx.x == 0 && lds_load(sy_vote) != 0) {   // (a wave may have handed the item over before the abort already)
+            const int k = lds_load(sy_nredo);
+            bool listed = false;
+            for (int r = 0; r < k; r++) listed = listed || __hip_atomic_load(&p.redo[lo + r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == idx;
+            if (!listed) {
+                __hip_atomic_store(&p.redo[lo + k], idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                lds_store(sy_nredo, k + 1);
+            }
+            lds_store(sy_vote, 0);
+        }
+        __syncthreads();
+        li++;
+    }
+    if (ri > 0 && threadIdx.x == 0) atomicAdd(&p.counters[NLIST + 3], ri);   // running total, for spinf_attn_exact_items
+    __builtin_amdgcn_s_waitcnt(0x0f70);
+}
+
+template <int D, bool WIN>
+__device__ __forceinline__ void ring_kernel_body(const AttnParams& p, char* const ring, char* const stage_all, int4* const desc) {
+    using S = RingShape<D>;
+    constexpr int TK = S::TK, NW = S::NW, HPI = S::HPI, NSLOT = S::NSLOT, NS = S::NS, NDT = S::NDT, NVF = S::NVF;
+    using G = TileGeo<D, TK, D>;
     constexpr int PFD = D >= 256 ? 2 : 8;   // fragment read-ahead: at head dim 256 one more spills a query fragment inside the tile loop
     constexpr int PF = D >= 256 ? 4 : (NS < PFD ? NS : PFD);   // K fragments are live in the score phase only, where registers are free
     constexpr int VPF = NVF < PFD ? NVF : PFD;
-    static_assert(NSLOT * G::BUFB + NW * 32 * SROW + NDESC * 16 + 256 <= 160 * 1024, "LDS budget");
-    __shared__ __attribute__((aligned(16))) char ring[NSLOT * G::BUFB];
-    __shared__ __attribute__((aligned(16))) char stage_all[NW * 32 * SROW];   // output staging, one slice per wave
-    __shared__ int4 desc[NDESC];       // {key tile, bits | DESC_FIRST | DESC_LAST, query tile | head group << 20, item index}
+    // ring: NSLOT tile slots; stage_all: output staging, one slice per wave; desc [NDESC]: {key tile, bits | DESC_FIRST | DESC_LAST,
+    // query tile | head group << 20, item index}
     __shared__ __attribute__((aligned(16))) int sy_done[MAX_SLOT];   // waves through with the tile in the slot; NW = the slot waits for somebody to recycle it (words past NSLOT stay 0)
     __shared__ int sy_issued[MAX_SLOT];   // tile the slot was last recycled for (its DMA requested)
     __shared__ int sy_gen;             // descriptors written so far
@@ -249,6 +542,8 @@ __global__ __launch_bounds__(D == 512 ? 256 : 512) void tree_attn_ring_kernel(co
     __shared__ int sy_ntiles;
     __shared__ int sy_redo[16];        // item sequence number + 1 of the last hand-over to the exact recomputation, per sequence number mod 16
     __shared__ int sy_nredo;           // items of this workgroup handed over so far (their indices: p.redo[lo ..])
+    __shared__ int sy_restart;         // after an abort: the fewest items any wave has completed (the barrier-paced pass starts there)
+    __shared__ int sy_vote;            // barrier-paced pass: some wave of the item met scores too far above its reference
 
     const Lane<D, TK, D> L(p);
     const int lo = p.list_ptr[blockIdx.x], hi = p.list_ptr[blockIdx.x + 1];
@@ -298,7 +593,7 @@ __global__ __launch_bounds__(D == 512 ? 256 : 512) void tree_attn_ring_kernel(co
         if (threadIdx.x < NSLOT) *(int*)(ring + threadIdx.x * G::BUFB + G::KTILEB + G::VTILEB + 768) = -1;   // the slot's flag: no generation yet
     }
     if (threadIdx.x < 16) sy_redo[threadIdx.x] = 0;
-    if (threadIdx.x == 0) { sy_gen = 0; sy_abort = 0; sy_ntiles = 0; sy_nredo = 0; }
+    if (threadIdx.x == 0) { sy_gen = 0; sy_abort = 0; sy_ntiles = 0; sy_nredo = 0; sy_restart = 0x7fffffff; sy_vote = 0; }
     __syncthreads();
 
     // descriptor generator (wave 0): items lo .. hi - 1, each item's plan entries in chunks of at most 64
@@ -332,6 +627,7 @@ __global__ __launch_bounds__(D == 512 ? 256 : 512) void tree_attn_ring_kernel(co
                 unsigned b = (unsigned)pbits & 0xffffu;
                 if (p_first && gl == 0) b |= DESC_FIRST;
                 if (p_last && gl == pn - 1) b |= DESC_LAST;
+                if (p.debug_expire > 0 && gen + gl == p.debug_expire - 1) b |= DESC_EXPIRE;
                 desc[(gen + gl) & (NDESC - 1)] = make_int4(pidx, (int)b, p_tz, p_item);
             }
             gen += pn;
@@ -417,75 +713,27 @@ __global__ __launch_bounds__(D == 512 ? 256 : 512) void tree_attn_ring_kernel(co
     if (L.w < NSLOT && L.w < ntiles) issue(L.w, read_desc(L.w));
 
     // ---- per-item state of this wave
-    bf16x8 qf[NS];
+    bf16x8 qf[Q_IN_ACC<D> ? 1 : NS];
     int art_q = -1, pos_q = 0;
     float M = -INFINITY, l = 0.f;
     bool viol = false;
     int iseq = 0;   // items begun
 
-    auto load_q = [&](const int tz) __attribute__((always_inline)) {
-        const int lane = fresh_lane_id();
-        const int tok = (tz & 0xfffff) * SPINF_QTILE + 32 * L.wr + (lane & 31);
-        const int tok_c = tok < p.n ? tok : p.n - 1;
-        const int h = (int)((unsigned)tz >> 20) * HPI + L.wh;
-        const __bf16* qp = p.q + (long)tok_c * p.q_tok + (long)h * p.q_head + 8 * (lane >> 5);
-#pragma unroll
-        for (int s = 0; s < NS; s++) qf[s] = *(const bf16x8*)(qp + 16 * s);
-        art_q = tok < p.n ? p.art[tok_c] : -1;
-        pos_q = WIN ? p.pos[tok_c] : 0;
-    };
+    auto load_q = [&](const int tz) __attribute__((always_inline)) { ring_load_q<D, WIN>(p, L.wr, L.wh, tz, qf, art_q, pos_q); };
     auto reset_acc = [&]() __attribute__((always_inline)) {
         M = -INFINITY;
         l = 0.f;
         acc_zero<NDT>();
         viol = false;
     };
-    // normalise O^T and store it as rows: 32 rows x 32 head dims at a time through the wave's own LDS slice, 16-byte pieces out
-    // (pieces of 8 bytes straight from the registers were measured slower: twice the requests for the same bytes)
-    auto store_rows = [&](const int tz) __attribute__((always_inline)) {
-        const int lane = fresh_lane_id(), m = lane & 31, g = lane >> 5;
-        const int tok0 = (tz & 0xfffff) * SPINF_QTILE + 32 * L.wr;
-        const int h = (int)((unsigned)tz >> 20) * HPI + L.wh;
-        const float inv = 1.0f / lane32_sum(l);
-        __bf16* ob = p.o + (long)h * p.o_head;
-        char* const stage = stage_all + L.w * 32 * SROW;
-        asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");   // the last MFMAs' results -> v_accvgpr_read
-        // tile dt is read back from the slice while tile dt + 1 is converted and written to it (the LDS takes a wave's requests
-        // in order, so the write behind the read is safe), and stored after that: no wait between a write and its read-back
-        auto put = [&](auto dt_c) __attribute__((always_inline)) {
-            constexpr int dt = decltype(dt_c)::value;
-            float r16[16];
-            acc_read<dt>(r16);
-#pragma unroll
-            for (int i4 = 0; i4 < 4; i4++) {
-                bf16x4 r;
-#pragma unroll
-                for (int jj = 0; jj < 4; jj++) r[jj] = (__bf16)(r16[4 * i4 + jj] * inv);
-                *(bf16x4*)(stage + m * SROW + (8 * i4 + 4 * g) * 2) = r;
-            }
-        };
-        auto round = [&](auto dt_c) __attribute__((always_inline)) {
-            constexpr int dt = decltype(dt_c)::value;
-            bf16x8 val[2];
-#pragma unroll
-            for (int jj = 0; jj < 2; jj++) {
-                const int c = jj * 64 + lane;
-                val[jj] = *(const bf16x8*)(stage + (c >> 2) * SROW + (c & 3) * 16);
-            }
-            if constexpr (dt + 1 < NDT) put(std::integral_constant<int, dt + 1>{});
-#pragma unroll
-            for (int jj = 0; jj < 2; jj++) {
-                const int c = jj * 64 + lane, row = c >> 2, col = c & 3;
-                if (tok0 + row < p.n) *(bf16x8*)(ob + (long)(tok0 + row) * p.o_tok + 32 * dt + col * 8) = val[jj];
-            }
-        };
-        put(std::integral_constant<int, 0>{});
-        pv_steps<NDT>(round);
-    };
+    auto store_rows = [&](const int tz) __attribute__((always_inline)) { ring_store_rows<D>(p, L.wr, L.wh, stage_all + L.w * 32 * SROW, tz, l); };
 
     {   // the first item's queries
         need_desc(0);
-        if (!dead) load_q(read_desc(0).z);
+        if (!dead) {
+            load_q(read_desc(0).z);
+            ring_wait_q<D>();
+        }
     }
 
     // ---- the tile sequence: item after item.
@@ -525,6 +773,11 @@ __global__ __launch_bounds__(D == 512 ? 256 : 512) void tree_attn_ring_kernel(co
             if (L.w < 4) claim(n0, n1, n2, n3);
             if (dead) break;
             const unsigned bits = (unsigned)d.y;
+            if ((bits & DESC_EXPIRE) && L.w == 0) {   // (test hook)
+                lds_store(&sy_abort, 1);
+                dead = true;
+                break;
+            }
             last = (bits & DESC_LAST) != 0;
             const bool act = (bits >> (2 * L.wr)) & 1u;
             if (act) {
@@ -544,19 +797,19 @@ __global__ __launch_bounds__(D == 512 ? 256 : 512) void tree_attn_ring_kernel(co
 #pragma unroll
                     for (int x = 0; x < PF; x++) kf[x] = *(const bf16x8*)(krow + 32 * x);
                     __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                    for (int x = 0; x < NS; x++) {
-                        if (x == 0) qk_first(sa, kf[x % PF], qf[x]);
-                        else if (x == NS - 1) qk_last(sa, kf[x % PF], qf[x]);
-                        else qk_next(sa, kf[x % PF], qf[x]);
+                    auto score = [&](auto x_c) __attribute__((always_inline)) {
+                        constexpr int x = decltype(x_c)::value;
+                        qk_step<D, x>(sa, kf[x % PF], qf);
                         if (x + PF < NS) kf[x % PF] = *(const bf16x8*)(krow + 32 * (x + PF));
                         __builtin_amdgcn_sched_barrier(0);
-                    }
+                    };
+                    pv_steps<NS>(score);
                 }
                 if ((bits >> (8 + 2 * L.wr)) & 1u) {
                     f32x16 sm[1] = {sa};
                     const int tok = (d.z & 0xfffff) * SPINF_QTILE + 32 * L.wr + (ln & 31);
-                    apply_mask<1, WIN, 0, TK>(sm, (const int*)(buf + G::KTILEB + G::VTILEB), d.x, 0, ln >> 5, tok, art_q, pos_q, p.window);
+                    ring_row_meta<D, WIN>(p, L.wr, d.z, art_q, pos_q);
+                    apply_mask<1, WIN, 0, TK, true>(sm, (const int*)(buf + G::KTILEB + G::VTILEB), d.x, 0, ln >> 5, tok, art_q, pos_q, p.window);
                     sa = sm[0];
                 }
                 // softmax against the row's fixed reference (the maximum of the first block it sees a key in)
@@ -654,119 +907,61 @@ __global__ __launch_bounds__(D == 512 ? 256 : 512) void tree_attn_ring_kernel(co
                     __hip_atomic_store(&p.redo[lo + k], item_done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
             }
+            ring_wait_q<D>();
         } else {
+            ring_wait_q<D>();   // (before the rows' stores: loads and stores do not return in one order, so no count tells them apart afterwards)
             store_rows(tz_done);
         }
     }
-    if (dead && fresh_lane_id() == 0) atomicAdd(&p.counters[NLIST + 4], 1);
+    if (dead && fresh_lane_id() == 0) {
+        atomicAdd(&p.counters[NLIST + 4], 1);
+        // a wave gives up inside an item or right behind its tiles, before the item's rows leave: the items it began, less that one, are complete
+        __hip_atomic_fetch_min(&sy_restart, iseq > 0 ? iseq - 1 : 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
     __builtin_amdgcn_s_waitcnt(0x0f70);
 
-    // ---- the exact recomputation.  Items in which some row met scores too far above its reference (normally none) are done
-    // again here, by the workgroup that owns them, after its list: classic online softmax over the same 32-key blocks in the same
-    // order (the reference is raised, and the accumulators rescaled, whenever a block maximum exceeds it by more than TAU_LAZY),
-    // the arithmetic of tree_attn_exact_kernel (tree_attn.hip) step for step, so the two give the same bits.  Nothing is
-    // overlapped: one tile at a time into slot 0, a workgroup barrier on either side of its request.  Whether an item comes here
-    // depends on its own rows only, so a job's output does not depend on what it is packed with.
-    __syncthreads();   // every wave is through with its list: the ring is free, the hand-overs are all in
-    const int n_redo = __builtin_amdgcn_readfirstlane(lds_load(&sy_nredo));
-    if (n_redo == 0 || __builtin_amdgcn_readfirstlane(lds_load(&sy_abort)) != 0) return;
-#pragma unroll 1
-    for (int r = 0; r < n_redo; r++) {
-        const int idx = __builtin_amdgcn_readfirstlane(__hip_atomic_load(&p.redo[lo + r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-        const int4 itv = p.items[idx];
-        const int it_t = __builtin_amdgcn_readfirstlane(itv.x), it_e0 = __builtin_amdgcn_readfirstlane(itv.y), it_z = __builtin_amdgcn_readfirstlane(itv.z);
-        const int ne = it_z & 0xfffff;
-        const int tz = it_t | (int)((unsigned)it_z >> 20 << 20);
-        const int kvh = (int)((unsigned)it_z >> 20) * HPI / p.group;
-        load_q(tz);
-        reset_acc();
-#pragma unroll 1
-        for (int e = 0; e < ne; e++) {
-            const int kt = __builtin_amdgcn_readfirstlane(p.kv_idx[it_e0 + e]);
-            const unsigned bits = (unsigned)__builtin_amdgcn_readfirstlane((int)p.kv_bits[it_e0 + e]);
-            __syncthreads();   // everyone is through with the slot
-            if (L.w == 0) {
-                using GK = Geo<D, TK>;
-                const int lane = fresh_lane_id();
-                const unsigned lane_k = (unsigned)((lane / GK::CPR) * GK::NREG * p.k_tok * 2 + (lane % GK::CPR) * 16);
-                const unsigned lane_v = (unsigned)((lane / GK::CPR) * GK::NREG * p.v_tok * 2 + (lane % GK::CPR) * 16);
-                issue_tile_wave<D, WIN>(p, lds_addr(ring), kt, kvh, 0, lane, lane_k, lane_v);
-            }
-            __builtin_amdgcn_s_waitcnt(0x0f70);   // the tile has landed (and this wave's queries)
-            __syncthreads();
-            if (!((bits >> (2 * L.wr)) & 1u)) continue;   // (wave-uniform; the barriers above are passed by every wave)
-            const int ln = fresh_lane_id();
-            const char* krow = ring + G::K::k_off(ln & 31) + 16 * (ln >> 5);
-            const char* vrow = ring + G::KTILEB + G::V::v_off(4 * (ln >> 5) + ((ln >> 2) & 3)) + 32 * ((ln >> 4) & 1) + 8 * (ln & 3);
-            // (the scheduling barriers keep the three kinds of LDS reads apart: the transposing reads of V and the 16-byte reads
-            // of K and of the keys' metadata do not complete in the order they were issued, which the compiler's counting assumes)
-            f32x16 sa;
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int x = 0; x < NS; x++) {
-                const bf16x8 kf = *(const bf16x8*)(krow + 32 * x);
-                if (x == 0) qk_first(sa, kf, qf[x]);
-                else if (x == NS - 1) qk_last(sa, kf, qf[x]);
-                else qk_next(sa, kf, qf[x]);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            if ((bits >> (8 + 2 * L.wr)) & 1u) {
-                f32x16 sm[1] = {sa};
-                const int tok = (tz & 0xfffff) * SPINF_QTILE + 32 * L.wr + (ln & 31);
-                apply_mask<1, WIN, 0, TK>(sm, (const int*)(ring + G::KTILEB + G::VTILEB), kt, 0, ln >> 5, tok, art_q, pos_q, p.window);
-                sa = sm[0];
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            bf16x8 pb[2];
-            {
-                float mx = sa[0];
-#pragma unroll
-                for (int i2 = 1; i2 < 16; i2++) mx = fmaxf(mx, sa[i2]);
-                mx = lane32_max(mx);
-                const float tm = mx * p.c;
-                const bool up = tm > M + TAU_LAZY;
-                const float mn = up ? tm : M;
-                const float alpha = up ? __builtin_amdgcn_exp2f(M - mn) : 1.0f;
-                if (__builtin_amdgcn_ballot_w64(up && M != -INFINITY) != 0) {   // rows without a key so far hold zeros
-                    asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");   // the last MFMAs' results -> v_accvgpr_read
-                    acc_scale<NDT>(alpha);
-                    asm volatile("s_nop 3" ::: "memory");                // v_accvgpr_write -> MFMA srcC
-                }
-                l *= alpha;
-                M = mn;
-                const float ms = mn == -INFINITY ? 0.f : mn;
-                float sum = 0.f;
-#pragma unroll
-                for (int i2 = 0; i2 < 16; i2++) {
-                    const float pr = __builtin_amdgcn_exp2f(__builtin_fmaf(sa[i2], p.c, -ms));
-                    sum += pr;
-                    pb[i2 >> 3][i2 & 7] = (__bf16)pr;
-                }
-                l += sum;
-            }
-            __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): no 16-byte read in flight when the transposing reads begin
-            __builtin_amdgcn_sched_barrier(0);
-            auto step = [&](auto f_c) __attribute__((always_inline)) {
-                constexpr int f = decltype(f_c)::value;
-                const char* vp = vrow + G::V::v_off(16 * (f / NDT)) + 64 * (f % NDT);
-                const s16x4 lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)vp);
-                const s16x4 hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vp + G::V::v_off(8)));
-                const bf16x8 a = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo4, hi4, 0, 1, 2, 3, 4, 5, 6, 7));
-                acc_mfma<f % NDT>(a, pb[f / NDT]);
-                __builtin_amdgcn_sched_barrier(0);
-            };
-            pv_steps<NVF>(step);
-        }
-        store_rows(tz);
+    __syncthreads();   // every wave is through with its list or has left it: the ring is free, the hand-overs are all in
+    // what is left for the barrier-paced pass: after an abort the list from the first item that some wave had not completed (a wave that
+    // was never held up has completed them all), and the items handed to the exact recomputation.  Normally nothing.
+    const bool aborted = __builtin_amdgcn_readfirstlane(lds_load(&sy_abort)) != 0;
+    if (!aborted && __builtin_amdgcn_readfirstlane(lds_load(&sy_nredo)) == 0) return;
+    int li = hi;
+    if (aborted) {
+        const int restart = __builtin_amdgcn_readfirstlane(lds_load(&sy_restart));
+        li = lo + (restart < hi - lo ? restart : hi - lo);
     }
-    if (threadIdx.x == 0) atomicAdd(&p.counters[NLIST + 3], n_redo);   // running total, for spinf_attn_exact_items
-    __builtin_amdgcn_s_waitcnt(0x0f70);
+    ring_paced_pass<D, WIN>(p, ring, stage_all, &sy_nredo, &sy_vote, lo, hi, li);
 }
 
-template <int D, bool WIN>
-int launch_ring_t(const AttnParams& p, int n_wg, hipStream_t stream) {
-    hipLaunchKernelGGL((tree_attn_ring_kernel<D, WIN>), dim3(n_wg), dim3(D == 512 ? 256 : 512), 0, stream, p);
-    const hipError_t e = hipGetLastError();
+// The tile ring, the staging slices and the descriptors are ONE block of dynamic LDS, sized at launch.  Not for flexibility: with
+// 155 KB of LDS declared in the kernel the compiler concludes that two waves per SIMD is all the kernel can ever reach and takes the
+// whole register file split evenly (128 ordinary + 128 accumulation registers), whatever limit the kernel asks for; the kernel needs
+// 60 + 196.  With the size out of its sight the limit below holds.
+extern __shared__ __attribute__((aligned(16))) char ring_lds[];
+template <int D>
+struct RingLds {
+    using S = RingShape<D>;
+    using G = TileGeo<D, S::TK, D>;
+    static constexpr int RINGB = S::NSLOT * G::BUFB, STAGEB = S::NW * 32 * SROW, BYTES = RINGB + STAGEB + NDESC * 16;
+    static_assert(BYTES + 512 <= 160 * 1024, "LDS budget");
+};
+#define RING_KERNEL(NAME, D, WIN, ATTR)                                                                                                      \
+    __global__ __launch_bounds__(D == 512 ? 256 : 512) ATTR void NAME(const AttnParams p) {                                                  \
+        ring_kernel_body<D, WIN>(p, ring_lds, ring_lds + RingLds<D>::RINGB, (int4*)(ring_lds + RingLds<D>::RINGB + RingLds<D>::STAGEB));     \
+    }
+RING_KERNEL(tree_attn_ring_kernel_256, 256, false, __attribute__((amdgpu_num_vgpr(60))))
+RING_KERNEL(tree_attn_ring_kernel_256w, 256, true, __attribute__((amdgpu_num_vgpr(60))))
+RING_KERNEL(tree_attn_ring_kernel_512, 512, false, )
+RING_KERNEL(tree_attn_ring_kernel_512w, 512, true, )
+#undef RING_KERNEL
+
+template <class K>
+int launch_ring_k(K kernel, const AttnParams& p, int n_wg, int threads, int lds_bytes, hipStream_t stream) {
+    // (more dynamic LDS than the default limit must be asked for once per kernel and device; asking again is cheap)
+    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: %d bytes of LDS for the ring kernel: %s", lds_bytes, hipGetErrorString(e));
+    hipLaunchKernelGGL(kernel, dim3(n_wg), dim3(threads), lds_bytes, stream, p);
+    e = hipGetLastError();
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: launch (ring kernel): %s", hipGetErrorString(e));
     return SPINF_OK;
 }
@@ -774,7 +969,9 @@ int launch_ring_t(const AttnParams& p, int n_wg, hipStream_t stream) {
 }  // namespace
 
 int spinf_launch_ring(const AttnParams& p, int d, bool win, int n_wg, hipStream_t stream) {
-    if (d == 256) return win ? launch_ring_t<256, true>(p, n_wg, stream) : launch_ring_t<256, false>(p, n_wg, stream);
-    if (d == 512) return win ? launch_ring_t<512, true>(p, n_wg, stream) : launch_ring_t<512, false>(p, n_wg, stream);
+    if (d == 256) return win ? launch_ring_k(tree_attn_ring_kernel_256w, p, n_wg, 512, RingLds<256>::BYTES, stream)
+                             : launch_ring_k(tree_attn_ring_kernel_256, p, n_wg, 512, RingLds<256>::BYTES, stream);
+    if (d == 512) return win ? launch_ring_k(tree_attn_ring_kernel_512w, p, n_wg, 256, RingLds<512>::BYTES, stream)
+                             : launch_ring_k(tree_attn_ring_kernel_512, p, n_wg, 256, RingLds<512>::BYTES, stream);
     return spinf_fail(SPINF_E_ARG, "tree_attn: the ring kernel takes head dim 256 or 512, not %d", d);
 }

@@ -24,7 +24,7 @@ class AttnArgs(C.Structure):
         ("kv_idx", C.c_void_p), ("kv_bits", C.c_void_p), ("items", C.c_void_p), ("list_ptr", C.c_void_p),
         ("n_items", C.c_int64), ("variant", C.c_int32),
         ("row_of", C.c_void_p), ("kv_row0", C.c_void_p),
-        ("grp", C.c_void_p), ("grp_mode", C.c_int32), ("ktile", C.c_int32), ("n_lists", C.c_int32),
+        ("grp", C.c_void_p), ("grp_mode", C.c_int32), ("ktile", C.c_int32), ("n_lists", C.c_int32), ("debug_expire", C.c_int32),
     ]
 
 

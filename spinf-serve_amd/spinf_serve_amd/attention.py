@@ -19,8 +19,9 @@ import torch
 from . import _lib
 from .masks import TreeMask
 
-# kernel tuning variant handed to the library (0 = its default choice, 1 = one head per work item, 2 = eight waves per
-# workgroup where two heads share an item); results do not depend on it
+# kernel tuning variant handed to the library (0 = its default choice: eight waves, the two heads of a GQA pair per work item, where
+# a group is even; 1 = one head per work item, four waves; 2 = four waves with two heads each, head dim <= 128); results do not
+# depend on it
 VARIANT = int(os.environ.get("SPINF_ATTN_VARIANT", "0"))
 # the kernel with decoupled waves over a static schedule, where the library has one for the geometry (0: the lockstep kernels only)
 RING = int(os.environ.get("SPINF_ATTN_RING", "-1"))      # -1 = auto
@@ -31,6 +32,32 @@ STATIC = int(os.environ.get("SPINF_ATTN_STATIC", "-1"))  # -1 = auto
 
 
 RING_MAX_ITEMS_PER_WG = 8
+
+# test hook (spinf_attn_args.debug_expire): k > 0 makes wave 0 of every workgroup of the decoupled kernel give up at its k-th tile
+DEBUG_EXPIRE = 0
+
+
+def _check_tensors(q, k, v, n_mask, compact, others=()):
+    """what every kernel launch assumes about q, k, v (and the device of whatever else it reads): raises before any launch"""
+    if q.dtype != torch.bfloat16 or k.dtype != torch.bfloat16 or v.dtype != torch.bfloat16:
+        raise ValueError("spinf::tree_attn takes bf16 q, k, v")
+    if q.dim() != 3 or k.dim() != 3 or v.dim() != 3:
+        raise ValueError("q, k, v must be [rows, heads, head dim]")
+    rows, hq, d = q.shape
+    hkv = k.shape[1]
+    if k.shape != (rows, hkv, d) or v.shape != (rows, hkv, d):
+        raise ValueError(f"k / v shapes {tuple(k.shape)} {tuple(v.shape)} do not match q {tuple(q.shape)}")
+    if hkv <= 0 or hq % hkv:
+        raise ValueError(f"{hq} query heads do not group over {hkv} key / value heads")
+    if q.stride(2) != 1 or k.stride(2) != 1 or v.stride(2) != 1:
+        raise ValueError("the head dimension must be contiguous")
+    if not compact and rows != n_mask:
+        raise ValueError(f"mask describes {n_mask} tokens, q / k / v have {rows}")
+    if not q.is_cuda:
+        raise RuntimeError("spinf::tree_attn runs on ROCm device tensors only (no CPU path)")
+    for t in (k, v, *others):
+        if t is not None and t.device != q.device:
+            raise ValueError(f"all tensors of the call must be on {q.device}, one is on {t.device}")
 
 
 def _ring_lists(q, hq, hkv, d, variant, sidx, mask):
@@ -72,6 +99,7 @@ def _attn_args(q, k, v, out, n, art, end, pos, kv_idx, kv_bits, items, list_ptr,
     a.variant = variant
     a.ktile = ktile
     a.n_lists = n_lists
+    a.debug_expire = DEBUG_EXPIRE
     if row_of is not None:
         a.row_of, a.kv_row0 = row_of.data_ptr(), kv_row0.data_ptr()
     if grp is not None:
@@ -89,16 +117,8 @@ def _tree_attn_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, art: torch.
     """q [rows, hq, d], k / v [rows, hkv, d] (any token / head strides, d contiguous) -> out [rows, hq, d] contiguous, bf16.
     rows = the stream length, or with row_of / kv_row0 (compact rows) any number of rows: the kernel maps stream positions to
     rows through row_of; rows 0 .. n_mapped-1 are the rows row_of names (each written by the kernel), later rows come back zero."""
-    if not q.is_cuda:
-        raise RuntimeError("spinf::tree_attn runs on ROCm device tensors only (no CPU path)")
-    if q.dtype != torch.bfloat16 or k.dtype != torch.bfloat16 or v.dtype != torch.bfloat16:
-        raise ValueError("spinf::tree_attn takes bf16 q, k, v")
+    _check_tensors(q, k, v, art.numel(), row_of is not None, (art, end, pos, kv_idx, kv_bits, items, list_ptr, row_of, kv_row0, grp))
     rows, hq, d = q.shape
-    hkv = k.shape[1]
-    if k.shape != (rows, hkv, d) or v.shape != (rows, hkv, d):
-        raise ValueError(f"k / v shapes {tuple(k.shape)} {tuple(v.shape)} do not match q {tuple(q.shape)}")
-    if q.stride(2) != 1 or k.stride(2) != 1 or v.stride(2) != 1:
-        raise ValueError("the head dimension must be contiguous")
     n = art.numel() if row_of is not None else rows
     if art.numel() < n:
         raise ValueError(f"mask built for {art.numel()} tokens, stream has {n}")
@@ -132,8 +152,7 @@ def tree_attn(q, k, v, mask: TreeMask, scale=None, variant=None, sidx=None):
     in place of the scatter into stream layout and the gather back (rows >= R come back zero)."""
     if not isinstance(mask, TreeMask):
         raise TypeError("attention_mask must be a TreeMask (masks.block_masks)")
-    if sidx is None and q.shape[0] != mask.n:
-        raise ValueError(f"mask describes {mask.n} tokens, q has {q.shape[0]}")
+    _check_tensors(q, k, v, mask.n, sidx is not None, (mask.art, mask.end, mask.pos, mask.kv_idx, mask.kv_bits, mask.grp, sidx))
     if sidx is not None and sidx.shape[0] > q.shape[0]:
         raise ValueError(f"sidx names {sidx.shape[0]} rows, q has {q.shape[0]}")
     scale = float(q.shape[-1] ** -0.5 if scale is None else scale)
@@ -143,10 +162,6 @@ def tree_attn(q, k, v, mask: TreeMask, scale=None, variant=None, sidx=None):
     if sidx is not None and mask.grp is not None:
         raise ValueError("image groups go with the stream layout (no sidx)")
     hq, hkv, d = q.shape[1], k.shape[1], q.shape[2]
-    if hkv <= 0 or hq % hkv:
-        raise ValueError(f"{hq} query heads do not group over {hkv} key / value heads")
-    if not q.is_cuda:
-        raise RuntimeError("spinf::tree_attn runs on ROCm device tensors only (no CPU path)")
     n_lists, ring = _ring_lists(q, hq, hkv, d, variant, sidx, mask)
     mask = mask.for_head_dim(d, ring=ring)
     per_item = _lib.load_library().spinf_attn_heads_per_item(hq, hkv, d, variant)
@@ -164,14 +179,13 @@ def tree_attn_noalloc(q, k, v, mask: TreeMask, out, scale=None):
     the device (for callers under graph capture or in loops that must not allocate; no counterpart in the reference).  The
     mask's schedule must already be on the device (any earlier call with this head geometry uploads it); stream layout only;
     at most 65,536 work items.  Same bits as tree_attn."""
-    if not q.is_cuda or q.dtype != torch.bfloat16 or k.dtype != torch.bfloat16 or v.dtype != torch.bfloat16:
-        raise ValueError("tree_attn_noalloc takes bf16 device tensors")
+    if not isinstance(mask, TreeMask):
+        raise TypeError("attention_mask must be a TreeMask (masks.block_masks)")
+    if out.shape != q.shape or out.dtype != torch.bfloat16 or not out.is_contiguous():
+        raise ValueError("out must be a contiguous bf16 tensor of q's shape")
+    _check_tensors(q, k, v, mask.n, False, (out, mask.art, mask.end, mask.pos, mask.kv_idx, mask.kv_bits, mask.grp))
     n, hq, d = q.shape
     hkv = k.shape[1]
-    if n != mask.n or out.shape != q.shape or out.dtype != torch.bfloat16 or not out.is_contiguous():
-        raise ValueError("out must be a contiguous bf16 tensor of q's shape, and the mask must describe q's rows")
-    if hkv <= 0 or hq % hkv:
-        raise ValueError(f"{hq} query heads do not group over {hkv} key / value heads")
     n_lists, ring = _ring_lists(q, hq, hkv, d, 0, None, mask)
     mask = mask.for_head_dim(d, ring=ring)
     per_item = _lib.load_library().spinf_attn_heads_per_item(hq, hkv, d, 0)

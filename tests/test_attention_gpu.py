@@ -55,6 +55,14 @@ def test_c2_shape_three_contents(dev, variant):
     _check(cfg, cfg.batches[0], dev, variant=variant)
 
 
+def _ring_aborts():
+    import ctypes
+
+    total = ctypes.c_int64(-1)
+    assert sa.load_library().spinf_attn_ring_aborts(ctypes.byref(total)) == 0
+    return total.value
+
+
 def _exact_items():
     import ctypes
 
@@ -526,6 +534,7 @@ def test_kernel_and_schedule_choices_give_the_same_bits(dev, window, monkeypatch
     q, k, v = synth.qkv(cfg, b, seed=4, device=dev)
     mask = sa.TreeMask.build(b.art, b.end, b.pos, window=window, device=dev)
     outs = []
+    aborts0 = _ring_aborts()
     for ring, static in ((0, 0), (0, 1), (1, 0)):
         monkeypatch.setattr(attention, "RING", ring)
         monkeypatch.setattr(attention, "STATIC", static)
@@ -533,8 +542,7 @@ def test_kernel_and_schedule_choices_give_the_same_bits(dev, window, monkeypatch
         outs.append(sa.tree_attn(q, k, v, mask, cfg.scale))
         torch.cuda.synchronize()
     assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
-    aborts = ctypes.c_int64(-1)
-    assert sa.load_library().spinf_attn_ring_aborts(ctypes.byref(aborts)) == 0 and aborts.value == 0
+    assert _ring_aborts() == aborts0
 
 
 @pytest.mark.parametrize("window", [None, 300])
@@ -553,14 +561,14 @@ def test_head_dim_512_kernel_choices_give_the_same_bits(dev, window, monkeypatch
     q, k, v = q[:n].contiguous(), k[:n].contiguous(), v[:n].contiguous()
     mask = sa.TreeMask.build(b.art[:n], b.end[:n], b.pos[:n], window=window, device=dev)
     outs = []
+    aborts0 = _ring_aborts()
     for ring in (0, 1):
         monkeypatch.setattr(attention, "RING", ring)
         print(f"case d512 ring={ring} window={window} n={n}", flush=True)
         outs.append(sa.tree_attn(q, k, v, mask, cfg.scale))
         torch.cuda.synchronize()
     assert torch.equal(outs[0], outs[1])
-    aborts = ctypes.c_int64(-1)
-    assert sa.load_library().spinf_attn_ring_aborts(ctypes.byref(aborts)) == 0 and aborts.value == 0
+    assert _ring_aborts() == aborts0
     # and both against the oracle on one content
     start, length, *_ = b.jobs[0]
     sl = slice(start, start + length)
@@ -640,3 +648,41 @@ def test_allocating_entry_point_under_graph_capture(dev):
         with torch.cuda.graph(g2, stream=fresh):
             sa.tree_attn(q, k, v, mask, cfg.scale)
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("d,expire,wide", [(256, 1, False), (256, 7, False), (256, 30, False), (256, 30, True), (512, 5, False), (512, 23, True)])
+def test_a_wave_that_gives_up_a_wait_costs_time_not_rows(dev, d, expire, wide, monkeypatch):
+    """the decoupled kernel's landing: wave 0 of every workgroup is told (from the host, spinf_attn_args.debug_expire) to treat its
+    wait at its expire-th tile as run out; the workgroup then leaves the ring and computes the rest of its list one tile at a time
+    between barriers.  Every kernel exits normally, the abort is counted, and the output equals the lockstep kernel's bit for bit,
+    also where items go on to the exact recomputation (wide) and with a window."""
+    from spinf_serve_amd import attention
+
+    cfg = synth.attention_config("C2" if d == 256 else "C2_512", contents=12 if d == 256 else 6)
+    b = cfg.batches[0]
+    q, k, v = synth.qkv(cfg, b, seed=9, device=dev)
+    if wide:
+        k = (k.float() * 60).to(torch.bfloat16)   # scores far above the first block's maximum: items go to the exact recomputation
+    for window in (None, 200):
+        mask = sa.TreeMask.build(b.art, b.end, b.pos, window=window, device=dev)
+        monkeypatch.setattr(attention, "RING", 0)
+        monkeypatch.setattr(attention, "DEBUG_EXPIRE", 0)
+        want = sa.tree_attn(q, k, v, mask, cfg.scale)
+        torch.cuda.synchronize()
+        monkeypatch.setattr(attention, "RING", 1)
+        before, exact0 = _ring_aborts(), _exact_items()
+        print(f"case d={d} expire={expire} wide={wide} window={window}: plain ring pass", flush=True)
+        plain = sa.tree_attn(q, k, v, mask, cfg.scale)
+        torch.cuda.synchronize()
+        assert _ring_aborts() == before
+        exact_plain = _exact_items() - exact0
+        monkeypatch.setattr(attention, "DEBUG_EXPIRE", expire)
+        print(f"case d={d} expire={expire} wide={wide} window={window}: forced abort", flush=True)
+        got = sa.tree_attn(q, k, v, mask, cfg.scale)
+        torch.cuda.synchronize()
+        monkeypatch.setattr(attention, "DEBUG_EXPIRE", 0)
+        assert _ring_aborts() > before, "no wave took the abort path"
+        assert torch.equal(plain, want)
+        assert torch.equal(got, want), float((got.float() - want.float()).abs().max())
+        if wide:
+            assert exact_plain > 0 and _exact_items() - exact0 == 2 * exact_plain   # the same items were recomputed exactly, once each
