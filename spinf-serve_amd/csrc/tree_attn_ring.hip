@@ -46,6 +46,9 @@ __device__ __forceinline__ int lds_load(const int* p) { return __hip_atomic_load
 // plain (non-atomic) reads of words other waves write, as LDS instructions: a volatile access through a generic pointer becomes a
 // flat load, which counts against the tile requests in flight
 typedef __attribute__((ext_vector_type(4))) int i32x4;
+typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 __device__ __forceinline__ int lds_peek(const int* p) { return *(const volatile __attribute__((address_space(3))) int*)(const __attribute__((address_space(3))) void*)p; }
 __device__ __forceinline__ i32x4 lds_peek4(const int* p) {
     return *(const volatile __attribute__((address_space(3))) i32x4*)(const __attribute__((address_space(3))) void*)p;
@@ -235,6 +238,22 @@ __device__ __forceinline__ void issue_tile_wave(const AttnParams& p, unsigned bu
         if (WIN) dma4_lane(p.pos + key, buf + KTILEB + VTILEB + 512);
     }
     dma4_lane(ring_seq + (gen & 63), buf + KTILEB + VTILEB + 768);   // every lane the same word: 64 copies of the flag
+}
+
+// One score of a lane's sixteen -> probability against the row's reference, row sum and (every second one) a packed pair of bf16
+// probabilities.  Assembly, so that each such slice stays between the MFMAs it is written between: left to the compiler, the sixteen
+// exponentials are all moved behind the last branch of the block.  Same instructions as the compiler's (v_fma_f32, v_exp_f32,
+// v_add_f32 in element order, v_cvt_pk_bf16_f32), same bits; the s_nop is the wait state a transcendental's result needs.
+template <int E>
+__device__ __forceinline__ void ring_sm_elem(const f32x16& sa, const float c, const float ms, float& pr_even, float& sum, unsigned (&pbn)[8]) {
+    if constexpr (E % 2 == 0) {
+        asm volatile("v_fma_f32 %0, %2, %3, -%4\n\tv_exp_f32 %0, %0\n\ts_nop 0\n\tv_add_f32 %1, %1, %0" : "=&v"(pr_even), "+v"(sum) : "v"(sa[E]), "s"(c), "v"(ms));
+    } else {
+        float pr;
+        asm volatile("v_fma_f32 %0, %3, %4, -%5\n\tv_exp_f32 %0, %0\n\ts_nop 0\n\tv_add_f32 %1, %1, %0\n\tv_cvt_pk_bf16_f32 %2, %6, %0"
+                     : "=&v"(pr), "+v"(sum), "=v"(pbn[E / 2])
+                     : "v"(sa[E]), "s"(c), "v"(ms), "v"(pr_even));
+    }
 }
 
 // A wave's place in the workgroup: four row groups x HPI heads of the item.
@@ -531,7 +550,7 @@ __device__ __forceinline__ void ring_kernel_body(const AttnParams& p, char* cons
     constexpr int TK = S::TK, NW = S::NW, HPI = S::HPI, NSLOT = S::NSLOT, NS = S::NS, NDT = S::NDT, NVF = S::NVF;
     using G = TileGeo<D, TK, D>;
     constexpr int PFD = D >= 256 ? 2 : 8;   // fragment read-ahead: at head dim 256 one more spills a query fragment inside the tile loop
-    constexpr int PF = D >= 256 ? 4 : (NS < PFD ? NS : PFD);   // K fragments are live in the score phase only, where registers are free
+    constexpr int PF = D == 256 ? 2 : D == 512 ? 4 : (NS < PFD ? NS : PFD);   // K fragment read-ahead (head dim 256: 60 ordinary registers in all)
     constexpr int VPF = NVF < PFD ? NVF : PFD;
     // ring: NSLOT tile slots; stage_all: output staging, one slice per wave; desc [NDESC]: {key tile, bits | DESC_FIRST | DESC_LAST,
     // query tile | head group << 20, item index}
@@ -544,6 +563,7 @@ __device__ __forceinline__ void ring_kernel_body(const AttnParams& p, char* cons
     __shared__ int sy_nredo;           // items of this workgroup handed over so far (their indices: p.redo[lo ..])
     __shared__ int sy_restart;         // after an abort: the fewest items any wave has completed (the barrier-paced pass starts there)
     __shared__ int sy_vote;            // barrier-paced pass: some wave of the item met scores too far above its reference
+    __shared__ int sy_gidx[64], sy_gbits[64];   // the descriptor generator's chunk of plan entries (key tiles, block bits), as it lands
 
     const Lane<D, TK, D> L(p);
     const int lo = p.list_ptr[blockIdx.x], hi = p.list_ptr[blockIdx.x + 1];
@@ -599,18 +619,19 @@ __device__ __forceinline__ void ring_kernel_body(const AttnParams& p, char* cons
     // descriptor generator (wave 0): items lo .. hi - 1, each item's plan entries in chunks of at most 64
     int gi = lo, ge = 0, gen = 0;   // next chunk: item, first entry inside it; descriptors written
     int pn = 0, p_first = 0, p_last = 0, p_tz = 0, p_item = 0;   // the requested chunk
-    int pidx = 0, pbits = 0;
-    auto gen_request = [&]() __attribute__((always_inline)) {   // loads of the next chunk's entries
+    // The chunk's plan entries come through LDS (DMA, like the tiles): as ordinary loads they would be requests in flight across the
+    // tile loop that the compiler knows of, and it then waits for "them" (in fact for every tile request of the wave) in front of
+    // whatever instruction of the loop next writes a register such a load might still be aimed at.
+    auto gen_request = [&]() __attribute__((always_inline)) {   // requests the next chunk's entries
         if (pn == 0 && gi < hi) {
             const int4 it = p.items[gi];
             const int t = __builtin_amdgcn_readfirstlane(it.x), e0 = __builtin_amdgcn_readfirstlane(it.y), z = __builtin_amdgcn_readfirstlane(it.z);
             const int ne = z & 0xfffff;
             const int n = ne - ge < 64 ? ne - ge : 64;
             const int gl = fresh_lane_id();
-            if (gl < n) {
-                pidx = p.kv_idx[e0 + ge + gl];
-                pbits = (int)p.kv_bits[e0 + ge + gl];
-            }
+            const int e = e0 + ge + (gl < n ? gl : n - 1);
+            dma4_lane(p.kv_idx + e, lds_addr(sy_gidx));
+            dma4_lane((const int*)p.kv_bits + e, lds_addr(sy_gbits));
             pn = n;
             p_first = ge == 0;
             p_last = ge + n == ne;
@@ -622,13 +643,14 @@ __device__ __forceinline__ void ring_kernel_body(const AttnParams& p, char* cons
     };
     auto gen_write = [&]() __attribute__((always_inline)) {   // descriptors of the requested chunk
         if (pn > 0) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the chunk has landed (wave 0 only, once per chunk)
             const int gl = fresh_lane_id();
             if (gl < pn) {
-                unsigned b = (unsigned)pbits & 0xffffu;
+                unsigned b = (unsigned)lds_peek(sy_gbits + gl) & 0xffffu;
                 if (p_first && gl == 0) b |= DESC_FIRST;
                 if (p_last && gl == pn - 1) b |= DESC_LAST;
                 if (p.debug_expire > 0 && gen + gl == p.debug_expire - 1) b |= DESC_EXPIRE;
-                desc[(gen + gl) & (NDESC - 1)] = make_int4(pidx, (int)b, p_tz, p_item);
+                desc[(gen + gl) & (NDESC - 1)] = make_int4(lds_peek(sy_gidx + gl), (int)b, p_tz, p_item);
             }
             gen += pn;
             pn = 0;
@@ -738,18 +760,73 @@ __device__ __forceinline__ void ring_kernel_body(const AttnParams& p, char* cons
 
     // ---- the tile sequence: item after item.
     // What a wave needs to know at the top of a tile (the tile's descriptor, the slots waiting for requests, the tile's flag) is
-    // read from LDS while the previous tile's last MFMAs run (`pf_*`), and the wave counts itself through with a tile as soon as
+    // read from LDS while the previous tile's MFMAs run (`pf_*`), and the wave counts itself through with a tile as soon as
     // its last fragment read of the tile is on its way: in the steady state no LDS round trip is waited for.
+    //
+    // Inside the wave the blocks are software-pipelined: P V of a block is put off until the scores of the wave's next block are
+    // there.  The order of a steady-state step is  S^T(j) = K Q^T  |  O^T += V^T P^T (previous block), with the softmax of block j
+    // issued between its MFMAs, a slice per MFMA .  The matrix pipe then sees one unbroken stream of MFMAs from this wave, and the
+    // softmax (vector ALU) runs in their shadow instead of between two MFMA phases.  The accumulation order of O^T and of the row
+    // sums is that of the unpipelined loop, so the bits are.  A wave keeps its hold on the previous block's slot until that block's
+    // V fragments are read; it lets go of it (P V at once, without overlap) before it skips a tile and at the end of an item, so
+    // it never holds a slot while it waits for a tile more than one place ahead (which would need that very slot recycled).
     int j = 0;
     bool have_pf = false;
     int4 pf_d = make_int4(0, 0, 0, 0);
     int pf_n0 = 0, pf_n1 = 0, pf_n2 = 0, pf_n3 = 0, pf_flag = -1;
     auto flag_word = [&](const int jj) __attribute__((always_inline)) { return (const int*)(ring + (jj & (NSLOT - 1)) * G::BUFB + G::KTILEB + G::VTILEB + 768); };
+    // V^T fragment address of this lane in slot sl (ds_read_b64_tr_b16: see Lane in attn_kernels.h), from a fresh lane index
+    auto v_lane_addr = [&](const int sl) __attribute__((always_inline)) {
+        const int ln = fresh_lane_id();
+        return ring + sl * G::BUFB + G::KTILEB + G::V::v_off(4 * (ln >> 5) + ((ln >> 2) & 3)) + 32 * ((ln >> 4) & 1) + 8 * (ln & 3);
+    };
+    // slice schedule of the softmax under the P V MFMAs: element e of the 16 scores of a lane goes behind MFMA number SM_STEP(e); the
+    // first slices wait until two MFMAs have been issued behind the last score MFMA (its result is then in the registers)
+    constexpr int SM_FIRST = 2;
+    auto sm_step_of = [](const int e) constexpr { return SM_FIRST + e * (NVF - SM_FIRST) / 16; };
     while (j < ntiles && !dead) {
         reset_acc();
         iseq++;
         int4 d = make_int4(0, 0, 0, 0);
         bool last = false;
+        bool pend = false;    // probabilities of a block wait for their P V: pbp, of the tile in slot s_pend (wave-uniform)
+        int s_pend = 0;
+        u32x4 pbp[2] = {};
+        // O^T += V^T P^T for the pending block, nothing overlapped (before a skipped tile, at the end of an item)
+        auto pv_plain = [&]() __attribute__((always_inline)) {
+            const char* const vrow = v_lane_addr(s_pend);
+            s16x4 vlo[VPF], vhi[VPF];
+            auto vload = [&](const int f, const int slot) __attribute__((always_inline)) {
+                const char* vp = vrow + G::V::v_off(16 * (f / NDT)) + 64 * (f % NDT);
+                vlo[slot] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)vp);
+                vhi[slot] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vp + G::V::v_off(8)));
+            };
+#pragma unroll
+            for (int f = 0; f < VPF; f++) vload(f, f);
+            __builtin_amdgcn_sched_barrier(0);
+            auto step = [&](auto f_c) __attribute__((always_inline)) {
+                constexpr int f = decltype(f_c)::value;
+                const bf16x8 a = __builtin_bit_cast(bf16x8, __builtin_shufflevector(vlo[f % VPF], vhi[f % VPF], 0, 1, 2, 3, 4, 5, 6, 7));
+                acc_mfma<f % NDT>(a, __builtin_bit_cast(bf16x8, pbp[f / NDT]));
+                if (f + VPF < NVF) vload(f + VPF, f % VPF);
+                if (f + VPF == NVF - 1) {   // that was the tile's last fragment read
+                    if (fresh_lane_id() == 0) __hip_atomic_fetch_add(&sy_done[s_pend], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            };
+            pv_steps<NVF>(step);
+            pend = false;
+        };
+        // the next item's queries, requested as soon as this item's last scores are there (head dim 256: the query registers are
+        // free from then on, and the request has the rest of the item to come back)
+        auto request_next_q = [&]() __attribute__((always_inline)) {
+            if constexpr (Q_IN_ACC<D>) {
+                if (last && j + 1 < ntiles) {
+                    need_desc(j + 1);
+                    if (!dead) load_q(read_desc(j + 1).z);
+                }
+            }
+        };
         do {
             const int s = j & (NSLOT - 1);
             int n0, n1, n2, n3, flag;
@@ -784,15 +861,18 @@ __device__ __forceinline__ void ring_kernel_body(const AttnParams& p, char* cons
                 if (flag != ((j / NSLOT + 1) & 63)) wait_watch(flag_word(j), (j / NSLOT + 1) & 63);
                 if (dead) break;
                 // fragment addresses from a fresh lane index (kept in registers across the tile loop they are spilled, and a reload
-                // waits for every tile request in flight): K row lane % 32 of the block, 16-byte chunk lane / 32 of each 32-byte step;
-                // V^T as ds_read_b64_tr_b16 wants it (see Lane in attn_kernels.h)
+                // waits for every tile request in flight): K row lane % 32 of the block, 16-byte chunk lane / 32 of each 32-byte step
                 const int ln = fresh_lane_id();
                 const char* buf = ring + s * G::BUFB;
                 const char* krow = buf + G::K::k_off(ln & 31) + 16 * (ln >> 5);
-                const char* vrow = buf + G::KTILEB + G::V::v_off(4 * (ln >> 5) + ((ln >> 2) & 3)) + 32 * ((ln >> 4) & 1) + 8 * (ln & 3);
-                // S^T = K Q^T
+                // S^T = K Q^T; behind the last fragment read, what the next tile's top needs is fetched (descriptor, the slots'
+                // counts, the tile's flag: 16-byte and 4-byte reads like the fragments', all back before the first transposing read of V)
                 f32x16 sa;
+                const bool pf_ok = j + 1 < ntiles && j + 1 < gen_seen;
                 {
+                    int4 dv = make_int4(0, 0, 0, 0);
+                    i32x4 nx = {0, 0, 0, 0};
+                    int fv = -1;
                     bf16x8 kf[PF];
 #pragma unroll
                     for (int x = 0; x < PF; x++) kf[x] = *(const bf16x8*)(krow + 32 * x);
@@ -801,19 +881,35 @@ __device__ __forceinline__ void ring_kernel_body(const AttnParams& p, char* cons
                         constexpr int x = decltype(x_c)::value;
                         qk_step<D, x>(sa, kf[x % PF], qf);
                         if (x + PF < NS) kf[x % PF] = *(const bf16x8*)(krow + 32 * (x + PF));
+                        if constexpr (x == NS - PF) {
+                            if (pf_ok) {
+                                dv = desc[(j + 1) & (NDESC - 1)];
+                                nx = lds_peek4(sy_done);
+                                fv = lds_peek(flag_word(j + 1));
+                            }
+                        }
                         __builtin_amdgcn_sched_barrier(0);
                     };
                     pv_steps<NS>(score);
+                    if (pf_ok) {
+                        pf_d = make_int4(__builtin_amdgcn_readfirstlane(dv.x), __builtin_amdgcn_readfirstlane(dv.y), __builtin_amdgcn_readfirstlane(dv.z), __builtin_amdgcn_readfirstlane(dv.w));
+                        pf_n0 = __builtin_amdgcn_readfirstlane(nx[0]); pf_n1 = __builtin_amdgcn_readfirstlane(nx[1]);
+                        pf_n2 = __builtin_amdgcn_readfirstlane(nx[2]); pf_n3 = __builtin_amdgcn_readfirstlane(nx[3]);
+                        pf_flag = __builtin_amdgcn_readfirstlane(fv);
+                        have_pf = true;
+                    }
                 }
-                if ((bits >> (8 + 2 * L.wr)) & 1u) {
+                const bool masked = (bits >> (8 + 2 * L.wr)) & 1u;
+                if (masked) ring_row_meta<D, WIN>(p, L.wr, d.z, art_q, pos_q);   // (before the next item's request overwrites it)
+                request_next_q();
+                if (dead) break;
+                if (masked) {
                     f32x16 sm[1] = {sa};
                     const int tok = (d.z & 0xfffff) * SPINF_QTILE + 32 * L.wr + (ln & 31);
-                    ring_row_meta<D, WIN>(p, L.wr, d.z, art_q, pos_q);
                     apply_mask<1, WIN, 0, TK, true>(sm, (const int*)(buf + G::KTILEB + G::VTILEB), d.x, 0, ln >> 5, tok, art_q, pos_q, p.window);
                     sa = sm[0];
                 }
                 // softmax against the row's fixed reference (the maximum of the first block it sees a key in)
-                bf16x8 pb[2];
                 {
                     const bool first = M == -INFINITY;
                     if (__builtin_amdgcn_ballot_w64(first) != 0) {   // only where a row meets its first keys (see the lockstep kernel)
@@ -823,31 +919,15 @@ __device__ __forceinline__ void ring_kernel_body(const AttnParams& p, char* cons
                         mx = lane32_max(mx);
                         M = first ? mx * p.c : M;
                     }
-                    const float ms = M == -INFINITY ? 0.f : M;
-                    float sum = 0.f;
-#pragma unroll
-                    for (int i2 = 0; i2 < 16; i2++) {
-                        const float pr = __builtin_amdgcn_exp2f(__builtin_fmaf(sa[i2], p.c, -ms));
-                        sum += pr;
-                        pb[i2 >> 3][i2 & 7] = (__bf16)pr;
-                    }
-                    l += sum;
-                    viol = viol | !(sum <= VIOL_SUM);
                 }
-                // O^T += V^T P^T, with what the next tile's top needs fetched meanwhile; once the last fragment read is on its way,
-                // count this wave through with the tile
-                int4 dv = make_int4(0, 0, 0, 0);
-                i32x4 nx = {0, 0, 0, 0};
-                int fv = -1;
-                const bool pf_ok = j + 1 < ntiles && j + 1 < gen_seen;
-                // (requested before the first transposing read of V: mixed in among them, a 16-byte read gave the MFMAs stale
-                // fragments, as if the two kinds of reads did not return in the order they were issued)
-                if (pf_ok) {
-                    dv = desc[(j + 1) & (NDESC - 1)];
-                    nx = lds_peek4(sy_done);
-                    fv = lds_peek(flag_word(j + 1));
-                }
-                {
+                const float ms = M == -INFINITY ? 0.f : M;
+                float sum = 0.f;
+                float pr_even = 0.f;
+                unsigned pbn[8];
+                auto sm_elem = [&](auto e_c) __attribute__((always_inline)) { ring_sm_elem<decltype(e_c)::value>(sa, p.c, ms, pr_even, sum, pbn); };
+                if (pend) {
+                    // O^T += V^T P^T of the previous block, the softmax of this one in the MFMAs' shadow
+                    const char* const vrow = v_lane_addr(s_pend);
                     s16x4 vlo[VPF], vhi[VPF];
                     auto vload = [&](const int f, const int slot) __attribute__((always_inline)) {
                         const char* vp = vrow + G::V::v_off(16 * (f / NDT)) + 64 * (f % NDT);
@@ -860,24 +940,33 @@ __device__ __forceinline__ void ring_kernel_body(const AttnParams& p, char* cons
                     auto step = [&](auto f_c) __attribute__((always_inline)) {
                         constexpr int f = decltype(f_c)::value;
                         const bf16x8 a = __builtin_bit_cast(bf16x8, __builtin_shufflevector(vlo[f % VPF], vhi[f % VPF], 0, 1, 2, 3, 4, 5, 6, 7));
-                        acc_mfma<f % NDT>(a, pb[f / NDT]);
+                        acc_mfma<f % NDT>(a, __builtin_bit_cast(bf16x8, pbp[f / NDT]));
                         if (f + VPF < NVF) vload(f + VPF, f % VPF);
-                        if (f + VPF == NVF - 1) {   // that was the tile's last fragment read
-                            if (fresh_lane_id() == 0) __hip_atomic_fetch_add(&sy_done[s], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                        if (f + VPF == NVF - 1) {   // that was the previous tile's last fragment read
+                            if (fresh_lane_id() == 0) __hip_atomic_fetch_add(&sy_done[s_pend], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                         }
+                        auto slice = [&](auto e_c) __attribute__((always_inline)) {
+                            constexpr int e = decltype(e_c)::value;
+                            if constexpr (sm_step_of(e) == f) sm_elem(e_c);
+                        };
+                        pv_steps<16>(slice);
                         __builtin_amdgcn_sched_barrier(0);
                     };
                     pv_steps<NVF>(step);
+                } else {
+                    pv_steps<16>(sm_elem);
                 }
-                if (pf_ok) {
-                    pf_d = make_int4(__builtin_amdgcn_readfirstlane(dv.x), __builtin_amdgcn_readfirstlane(dv.y), __builtin_amdgcn_readfirstlane(dv.z), __builtin_amdgcn_readfirstlane(dv.w));
-                    pf_n0 = __builtin_amdgcn_readfirstlane(nx[0]); pf_n1 = __builtin_amdgcn_readfirstlane(nx[1]);
-                    pf_n2 = __builtin_amdgcn_readfirstlane(nx[2]); pf_n3 = __builtin_amdgcn_readfirstlane(nx[3]);
-                    pf_flag = __builtin_amdgcn_readfirstlane(fv);
-                    have_pf = true;
-                }
+                l += sum;
+                viol = viol | !(sum <= VIOL_SUM);
+                pbp[0] = u32x4{pbn[0], pbn[1], pbn[2], pbn[3]};
+                pbp[1] = u32x4{pbn[4], pbn[5], pbn[6], pbn[7]};
+                s_pend = s;
+                pend = true;
             } else {
                 // nothing of this tile for these rows: the slot must have been recycled for it before this wave counts itself through
+                if (pend) pv_plain();
+                request_next_q();
+                if (dead) break;
                 wait_watch(&sy_issued[s], j);
                 if (dead) break;
                 if (fresh_lane_id() == 0) __hip_atomic_fetch_add(&sy_done[s], 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -890,11 +979,12 @@ __device__ __forceinline__ void ring_kernel_body(const AttnParams& p, char* cons
             j++;
         } while (!last);
         if (dead) break;
-        // this wave's rows of the item are complete: the next item's queries are requested (their registers are free), then the rows
-        // go out (or the item goes to the exact pass)
+        if (pend) pv_plain();
+        // this wave's rows of the item are complete: the next item's queries are requested (their registers are free; at head dim
+        // 256 that has happened behind the item's last scores), then the rows go out (or the item goes to the exact pass)
         const bool hand_over = __builtin_amdgcn_ballot_w64(viol) != 0;   // scores ranged too widely somewhere in these 32 rows
         const int tz_done = d.z, item_done = d.w;
-        if (j < ntiles) {
+        if (!Q_IN_ACC<D> && j < ntiles) {
             need_desc(j);
             if (dead) break;
             load_q(read_desc(j).z);
