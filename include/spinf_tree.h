@@ -119,8 +119,9 @@ typedef struct spinf_attn_args {
                                                variant 0; stream layout, no groups) that is the kernel with decoupled waves, which at
                                                d = 512 computes the pass in one launch instead of two */
     int32_t debug_expire;                   /* 0 in production.  Test hook of the kernel with decoupled waves (no counterpart in the reference):
-                                               k > 0 makes wave 0 of every workgroup treat its wait at its k-th tile as run out, which takes the
-                                               workgroup through the landing that a real time-out would take (the rest of its list computed one
+                                               k > 0 = polls of one wait before a wave gives up (2^18 otherwise; a healthy wait takes a handful).
+                                               With k = 1 every wave that has to wait at all gives up, which takes its workgroup through the
+                                               landing a real time-out would take (the landing kernel computes the workgroup's list again, one
                                                tile at a time between barriers).  Same results bit for bit; spinf_attn_ring_aborts counts it */
 } spinf_attn_args;
 
@@ -143,8 +144,9 @@ int spinf_tree_attn_fwd_noalloc(const spinf_attn_args* args, void* stream);
 int spinf_attn_exact_items(int64_t* total);
 /* Diagnostics (no counterpart in the reference): *total = waves of the static-schedule kernel that gave up a bounded wait on
  * the current device since the library was loaded.  Always 0 unless the kernel has a bug (or debug_expire asked for it).  The
- * results of such a pass are still complete and the same bit for bit: the workgroup finishes its list one tile at a time between
- * barriers; the count says that time was lost.  Synchronises the device. */
+ * results of such a pass are still complete and the same bit for bit: the landing kernel that follows every launch of that kernel
+ * computes the list of such a workgroup again, one tile at a time between barriers; the count says that time was lost.
+ * Synchronises the device. */
 int spinf_attn_ring_aborts(int64_t* total);
 
 /* ------------------------------------------------------------------------------------------------ Gated DeltaNet

@@ -8,6 +8,7 @@
 #include "attn_tiles.h"
 
 constexpr int NLIST = 8;       // work lists (XCDs of an MI355X)
+constexpr int LAND_CAP = 65536; // most item lists of a static schedule (the landing words of the ring kernel)
 constexpr int ENT_CAP = 256;   // plan entries of a query tile kept in LDS at a time
 
 struct AttnParams {
@@ -30,7 +31,8 @@ struct AttnParams {
     const int* grp;       // image groups (GRP kernels): -1 none; the tokens of a group see each other both ways
     bool static_lists;    // list_ptr delimits one item list per workgroup (a static schedule) instead of the eight shared lists
     bool clear_first;     // host side only: zero the cursors and counts in front of the pass (the entry point that allocates nothing)
-    int debug_expire;     // ring kernel, test hook: > 0 makes wave 0 of every workgroup give up at its tile debug_expire - 1, as if a wait had run out
+    int* land;            // ring kernel: [b] = waves of workgroup b that gave up a wait in this launch (the landing kernel then does b's list again and clears the word)
+    int spin_limit;       // ring kernel: polls of one wait before the wave gives up (a healthy wait takes a handful; tests set it to 1 to force the landing)
 };
 
 // Softmax reference point.  The fast pass fixes each row's reference at the maximum of the first 32-key block in which

@@ -556,7 +556,8 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
 // Scratch memory of the entry point that allocates nothing (spinf_tree_attn_fwd_noalloc): list cursors, counts and the redo
 // list.  In host code this name is a stand-in, not a device address: hipGetSymbolAddress gives the address, per device.
 constexpr long NOALLOC_MAX_ITEMS = 1 << 16;                            // work items (query tiles x head groups) of one call
-static __device__ __align__(256) int scratch[64 + NOALLOC_MAX_ITEMS];  // 256.25 KiB per GPU, held until the process ends
+// 64 cursors and counts | the redo list | the ring kernel's landing words (one per item list): 512.25 KiB per GPU, held until the process ends
+static __device__ __align__(256) int scratch[64 + NOALLOC_MAX_ITEMS + LAND_CAP];
 
 namespace {
 
@@ -598,7 +599,7 @@ int device_cus(int* cus) {
 }
 
 // -> the stream's block with room for n_items redo entries; *slot names it for release_block
-int acquire_block(long n_items, bool capturing, hipStream_t stream, int** ptr, int* slot, bool* dirty) {
+int acquire_block(long n_items, bool capturing, hipStream_t stream, int** ptr, int* slot, bool* dirty, long* cap) {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess || dev < 0 || dev >= 64) return spinf_fail(SPINF_E_HIP, "tree_attn: hipGetDevice: %s", hipGetErrorString(e));
@@ -612,6 +613,7 @@ int acquire_block(long n_items, bool capturing, hipStream_t stream, int** ptr, i
         *ptr = b.ptr;
         *slot = (int)i;
         *dirty = b.dirty;
+        *cap = b.cap;
         return SPINF_OK;
     }
     if (capturing)
@@ -621,15 +623,17 @@ int acquire_block(long n_items, bool capturing, hipStream_t stream, int** ptr, i
     CursorBlock b;
     b.cap = n_items < (1 << 16) ? (1 << 16) : 2 * n_items;
     b.owner = stream;
-    e = hipMalloc((void**)&b.ptr, (64 + b.cap) * sizeof(int));
+    e = hipMalloc((void**)&b.ptr, (64 + b.cap + LAND_CAP) * sizeof(int));
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: hipMalloc: %s", hipGetErrorString(e));
     e = hipMemset(b.ptr, 0, 64 * sizeof(int));   // cursors, counts and the running totals at [NLIST + 3], [NLIST + 4] start at zero
+    if (e == hipSuccess) e = hipMemset(b.ptr + 64 + b.cap, 0, LAND_CAP * sizeof(int));   // and so do the landing words (the landing kernel clears what it finds)
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: cursor block: %s", hipGetErrorString(e));
     b.taken = true;
     s.blocks.push_back(b);
     *ptr = b.ptr;
     *slot = (int)s.blocks.size() - 1;
     *dirty = false;
+    *cap = b.cap;
     return SPINF_OK;
 }
 
@@ -856,6 +860,7 @@ static int attn_fwd(const spinf_attn_args* a, void* stream, bool no_alloc) {
     hipStream_t s = (hipStream_t)stream;
     int* counters = nullptr;
     int cus = 0, slot = -1;
+    long redo_cap = NOALLOC_MAX_ITEMS;
     bool capturing = false, dirty = false;
     if (no_alloc) {
         ScratchState* st = nullptr;
@@ -867,7 +872,7 @@ static int attn_fwd(const spinf_attn_args* a, void* stream, bool no_alloc) {
         if (hipStreamIsCapturing(s, &cs) != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: hipStreamIsCapturing failed");
         capturing = cs != hipStreamCaptureStatusNone;
         if (int rc = device_cus(&cus)) return rc;
-        if (int rc = acquire_block((long)a->n_items, capturing, s, &counters, &slot, &dirty)) return rc;
+        if (int rc = acquire_block((long)a->n_items, capturing, s, &counters, &slot, &dirty, &redo_cap)) return rc;
     }
     AttnParams p;
     // A block's cursors are zero: it was cleared when allocated, and every call's exact-pass kernel, which runs after the fast pass,
@@ -888,7 +893,8 @@ static int attn_fwd(const spinf_attn_args* a, void* stream, bool no_alloc) {
     p.row_of = a->row_of; p.kv_row0 = a->kv_row0;
     p.grp = a->grp;
     p.counters = counters;
-    p.debug_expire = ring ? a->debug_expire : 0;
+    p.land = counters + 64 + redo_cap;
+    p.spin_limit = a->debug_expire > 0 ? a->debug_expire : (1 << 18);
     p.redo = counters + 64;
     const int blocks = a->n_lists > 0 ? a->n_lists : (int)(a->n_items < cus ? a->n_items : cus);
     const bool win = p.window > 0;

@@ -40,15 +40,11 @@ constexpr int GEN_AHEAD = 48;       // wave 0 keeps the descriptors this far ahe
 constexpr int SPIN_LIMIT = 1 << 18; // polls of one wait before the workgroup gives up (a healthy wait takes a handful)
 constexpr int SROW = 64 + 16;       // output staging: 32 rows x 32 head dims, 80-byte rows
 constexpr unsigned DESC_FIRST = 1u << 16, DESC_LAST = 1u << 17;
-constexpr unsigned DESC_EXPIRE = 1u << 18;   // test hook: wave 0 treats its wait for this tile as run out
 
 __device__ __forceinline__ int lds_load(const int* p) { return __hip_atomic_load(p, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP); }
 // plain (non-atomic) reads of words other waves write, as LDS instructions: a volatile access through a generic pointer becomes a
 // flat load, which counts against the tile requests in flight
 typedef __attribute__((ext_vector_type(4))) int i32x4;
-typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
-typedef __attribute__((ext_vector_type(2))) float f32x2;
-typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 __device__ __forceinline__ int lds_peek(const int* p) { return *(const volatile __attribute__((address_space(3))) int*)(const __attribute__((address_space(3))) void*)p; }
 __device__ __forceinline__ i32x4 lds_peek4(const int* p) {
     return *(const volatile __attribute__((address_space(3))) i32x4*)(const __attribute__((address_space(3))) void*)p;
@@ -149,34 +145,15 @@ __device__ __forceinline__ void acc_scale(const float alpha) {
     }
 }
 // S^T chain on ordinary registers, as assembly as well (a kernel that mixes MFMA builtins with the fixed accumulation registers
-// above would let the compiler pick accumulation registers of its own for them).
-// Where the queries live.  At head dim 256 the 16 query fragments of a wave (64 registers, constant over a work item) sit in
-// a[128:191], behind the compiler's back like the accumulators: as compiler-visible values they are what the register allocator
-// spills whenever anything else in the tile loop changes (the loop then reloads them from scratch memory in front of the first
-// MFMAs, and such a reload waits for every tile request in flight).  The kernel is limited to 60 ordinary registers
-// (amdgpu_num_vgpr), 196 accumulation registers: a[0:127] O^T, a[128:191] queries, a192 / a193 art / pos of the wave's rows.
-// At head dim 512 the accumulators take all 256 accumulation registers and the queries stay compiler-visible (205 ordinary
-// registers, one wave per SIMD: nothing is spilled there).
-template <int D>
-constexpr bool Q_IN_ACC = D == 256;
-constexpr int QBASE = 128, ROW_ART = 192, ROW_POS = 193;
-
-// step S of NS of S^T = K Q^T: sa (+)= k * q fragment S; the last step carries the wait states before the vector ALU reads the result
-template <int D, int S>
-__device__ __forceinline__ void qk_step(f32x16& sa, const bf16x8 k, const bf16x8 (&qf)[Q_IN_ACC<D> ? 1 : D / 16]) {
-    constexpr int NS = D / 16;
-    if constexpr (Q_IN_ACC<D>) {
-        if constexpr (S == 0)
-            asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, a[%c2:%c3], 0" : "=&v"(sa) : "v"(k), "n"(QBASE + 4 * S), "n"(QBASE + 4 * S + 3));
-        else if constexpr (S == NS - 1)
-            asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, a[%c2:%c3], %0\n\ts_nop 15" : "+v"(sa) : "v"(k), "n"(QBASE + 4 * S), "n"(QBASE + 4 * S + 3));
-        else
-            asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, a[%c2:%c3], %0" : "+v"(sa) : "v"(k), "n"(QBASE + 4 * S), "n"(QBASE + 4 * S + 3));
-    } else {
-        if constexpr (S == 0) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(sa) : "v"(k), "v"(qf[S]));
-        else if constexpr (S == NS - 1) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0\n\ts_nop 15" : "+v"(sa) : "v"(k), "v"(qf[S]));
-        else asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(sa) : "v"(k), "v"(qf[S]));
-    }
+// above would let the compiler pick accumulation registers of its own for them)
+__device__ __forceinline__ void qk_first(f32x16& sa, const bf16x8 k, const bf16x8 q) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(sa) : "v"(k), "v"(q));
+}
+__device__ __forceinline__ void qk_next(f32x16& sa, const bf16x8 k, const bf16x8 q) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(sa) : "v"(k), "v"(q));
+}
+__device__ __forceinline__ void qk_last(f32x16& sa, const bf16x8 k, const bf16x8 q) {   // + the wait states before the vector ALU reads the result
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0\n\ts_nop 15" : "+v"(sa) : "v"(k), "v"(q));
 }
 
 // A tile's "landed" flag is written by the DMA engine itself: the last request of a tile copies ring_seq[generation % 64] from
@@ -240,19 +217,11 @@ __device__ __forceinline__ void issue_tile_wave(const AttnParams& p, unsigned bu
     dma4_lane(ring_seq + (gen & 63), buf + KTILEB + VTILEB + 768);   // every lane the same word: 64 copies of the flag
 }
 
-// One score of a lane's sixteen -> probability against the row's reference, row sum and (every second one) a packed pair of bf16
-// probabilities.  Assembly, so that each such slice stays between the MFMAs it is written between: left to the compiler, the sixteen
-// exponentials are all moved behind the last branch of the block.  Same instructions as the compiler's (v_fma_f32, v_exp_f32,
-// v_add_f32 in element order, v_cvt_pk_bf16_f32), same bits; the s_nop is the wait state a transcendental's result needs.
-template <int E>
-__device__ __forceinline__ void ring_sm_elem(const f32x16& sa, const float c, const float ms, float& pr_even, float& sum, unsigned (&pbn)[8]) {
-    if constexpr (E % 2 == 0) {
-        asm volatile("v_fma_f32 %0, %2, %3, -%4\n\tv_exp_f32 %0, %0\n\ts_nop 0\n\tv_add_f32 %1, %1, %0" : "=&v"(pr_even), "+v"(sum) : "v"(sa[E]), "s"(c), "v"(ms));
-    } else {
-        float pr;
-        asm volatile("v_fma_f32 %0, %3, %4, -%5\n\tv_exp_f32 %0, %0\n\ts_nop 0\n\tv_add_f32 %1, %1, %0\n\tv_cvt_pk_bf16_f32 %2, %6, %0"
-                     : "=&v"(pr), "+v"(sum), "=v"(pbn[E / 2])
-                     : "v"(sa[E]), "s"(c), "v"(ms), "v"(pr_even));
+template <int N, int F = 0, class Fn>
+__device__ __forceinline__ void pv_steps(Fn& fn) {
+    if constexpr (F < N) {
+        fn(std::integral_constant<int, F>{});
+        pv_steps<N, F + 1>(fn);
     }
 }
 
@@ -268,69 +237,18 @@ struct RingShape {
     static constexpr int NVF = 2 * NDT;   // V^T fragments of one 32-key block
 };
 
-// Requests the queries of rows 32 wr .. of query tile tz & 0xfffff, head (tz >> 20) * HPI + wh (the B operands of K Q^T), and art / pos
-// of the wave's rows.  Head dim 256: into the accumulation registers, by assembly; nothing the compiler sees depends on them, so
-// the caller waits (ring_wait_q) before the item's first MFMA and before ring_row_meta.  Head dim 512: ordinary loads into qf, art_q, pos_q.
-#define RING_Q_LOAD(S) "global_load_dwordx4 a[" #S "*4+128:" #S "*4+131], %0, off offset:" #S "*32\n\t"
-#define RING_Q_CLOB(B) "a" #B
+// the queries of rows 32 wr .. of query tile tz & 0xfffff, head (tz >> 20) * HPI + wh, as B operands of K Q^T; art / pos of the wave's rows
 template <int D, bool WIN>
-__device__ __forceinline__ void ring_load_q(const AttnParams& p, const int wr, const int wh, const int tz, bf16x8 (&qf)[Q_IN_ACC<D> ? 1 : D / 16], int& art_q,
-                                            int& pos_q) {
+__device__ __forceinline__ void ring_load_q(const AttnParams& p, const int wr, const int wh, const int tz, bf16x8 (&qf)[D / 16], int& art_q, int& pos_q) {
     const int lane = fresh_lane_id();
     const int tok = (tz & 0xfffff) * SPINF_QTILE + 32 * wr + (lane & 31);
     const int tok_c = tok < p.n ? tok : p.n - 1;
     const int h = (int)((unsigned)tz >> 20) * RingShape<D>::HPI + wh;
     const __bf16* qp = p.q + (long)tok_c * p.q_tok + (long)h * p.q_head + 8 * (lane >> 5);
-    if constexpr (Q_IN_ACC<D>) {
-        asm volatile(RING_Q_LOAD(0) RING_Q_LOAD(1) RING_Q_LOAD(2) RING_Q_LOAD(3) RING_Q_LOAD(4) RING_Q_LOAD(5) RING_Q_LOAD(6) RING_Q_LOAD(7)
-                     RING_Q_LOAD(8) RING_Q_LOAD(9) RING_Q_LOAD(10) RING_Q_LOAD(11) RING_Q_LOAD(12) RING_Q_LOAD(13) RING_Q_LOAD(14) RING_Q_LOAD(15)
-                     "global_load_dword a192, %1, off"
-                     :: "v"(qp), "v"(p.art + tok_c)
-                     : "memory", RING_Q_CLOB(128), RING_Q_CLOB(129), RING_Q_CLOB(130), RING_Q_CLOB(131), RING_Q_CLOB(132), RING_Q_CLOB(133), RING_Q_CLOB(134),
-                       RING_Q_CLOB(135), RING_Q_CLOB(136), RING_Q_CLOB(137), RING_Q_CLOB(138), RING_Q_CLOB(139), RING_Q_CLOB(140), RING_Q_CLOB(141), RING_Q_CLOB(142),
-                       RING_Q_CLOB(143), RING_Q_CLOB(144), RING_Q_CLOB(145), RING_Q_CLOB(146), RING_Q_CLOB(147), RING_Q_CLOB(148), RING_Q_CLOB(149), RING_Q_CLOB(150),
-                       RING_Q_CLOB(151), RING_Q_CLOB(152), RING_Q_CLOB(153), RING_Q_CLOB(154), RING_Q_CLOB(155), RING_Q_CLOB(156), RING_Q_CLOB(157), RING_Q_CLOB(158),
-                       RING_Q_CLOB(159), RING_Q_CLOB(160), RING_Q_CLOB(161), RING_Q_CLOB(162), RING_Q_CLOB(163), RING_Q_CLOB(164), RING_Q_CLOB(165), RING_Q_CLOB(166),
-                       RING_Q_CLOB(167), RING_Q_CLOB(168), RING_Q_CLOB(169), RING_Q_CLOB(170), RING_Q_CLOB(171), RING_Q_CLOB(172), RING_Q_CLOB(173), RING_Q_CLOB(174),
-                       RING_Q_CLOB(175), RING_Q_CLOB(176), RING_Q_CLOB(177), RING_Q_CLOB(178), RING_Q_CLOB(179), RING_Q_CLOB(180), RING_Q_CLOB(181), RING_Q_CLOB(182),
-                       RING_Q_CLOB(183), RING_Q_CLOB(184), RING_Q_CLOB(185), RING_Q_CLOB(186), RING_Q_CLOB(187), RING_Q_CLOB(188), RING_Q_CLOB(189), RING_Q_CLOB(190),
-                       RING_Q_CLOB(191), RING_Q_CLOB(192));
-        if (WIN) asm volatile("global_load_dword a193, %0, off" :: "v"(p.pos + tok_c) : "memory", RING_Q_CLOB(193));
-    } else {
 #pragma unroll
-        for (int s = 0; s < D / 16; s++) qf[s] = *(const bf16x8*)(qp + 16 * s);
-        art_q = tok < p.n ? p.art[tok_c] : -1;
-        pos_q = WIN ? p.pos[tok_c] : 0;
-    }
-}
-#undef RING_Q_LOAD
-#undef RING_Q_CLOB
-// Head dim 256: waits until every request of the wave has returned, the queries with them.  (Loads and stores do not return in one
-// order, so "all but the n youngest" says nothing once stores are in flight: the wait stands in front of the item's stores, which
-// then drain while the next item is computed.)
-template <int D>
-__device__ __forceinline__ void ring_wait_q() {
-    if constexpr (Q_IN_ACC<D>) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-}
-// art / pos of this lane's query row (head dim 256: out of the accumulation registers the requests went to; the caller has waited)
-template <int D, bool WIN>
-__device__ __forceinline__ void ring_row_meta(const AttnParams& p, const int wr, const int tz, int& art_q, int& pos_q) {
-    if constexpr (Q_IN_ACC<D>) {
-        const int tok = (tz & 0xfffff) * SPINF_QTILE + 32 * wr + (fresh_lane_id() & 31);
-        int a, ps = 0;
-        asm volatile("v_accvgpr_read_b32 %0, a192" : "=v"(a));
-        if (WIN) asm volatile("v_accvgpr_read_b32 %0, a193" : "=v"(ps));
-        art_q = tok < p.n ? a : -1;
-        pos_q = ps;
-    }
-}
-
-template <int N, int F = 0, class Fn>
-__device__ __forceinline__ void pv_steps(Fn& fn) {
-    if constexpr (F < N) {
-        fn(std::integral_constant<int, F>{});
-        pv_steps<N, F + 1>(fn);
-    }
+    for (int s = 0; s < D / 16; s++) qf[s] = *(const bf16x8*)(qp + 16 * s);
+    art_q = tok < p.n ? p.art[tok_c] : -1;
+    pos_q = WIN ? p.pos[tok_c] : 0;
 }
 
 // normalise O^T and store it as rows: 32 rows x 32 head dims at a time through the wave's own LDS slice `stage`, 16-byte pieces out
@@ -378,7 +296,8 @@ __device__ __forceinline__ void ring_store_rows(const AttnParams& p, const int w
 }
 
 // ---- after the list: the barrier-paced pass over single items.  One tile at a time into slot 0 of the ring, a workgroup barrier on
-// either side of its request, nothing overlapped, no spin anywhere.  Two users:
+// either side of its request, nothing overlapped, no spin anywhere.  It is the body of the landing kernel below (a kernel of its
+// own: what it needs in registers must not weigh on the ring loop's allocation, which has none to spare).  Two uses:
 //   * the exact recomputation.  Items in which some row met scores too far above its reference (normally none) are done again by the
 //     workgroup that owns them: classic online softmax over the same 32-key blocks in the same order (the reference is raised, and
 //     the accumulators rescaled, whenever a block maximum exceeds it by more than TAU_LAZY), the arithmetic of tree_attn_exact_kernel
@@ -391,14 +310,14 @@ __device__ __forceinline__ void ring_store_rows(const AttnParams& p, const int w
 // p.redo[lo ..]; *sy_vote = 0.
 template <int D, bool WIN>
 __device__ __forceinline__ void ring_paced_pass(const AttnParams& p, char* const ring, char* const stage_all, int* const sy_nredo, int* const sy_vote,
-                                                          const int lo, const int hi, int li) {
+                                                const int lo, const int hi, int li) {
     using S = RingShape<D>;
     constexpr int TK = S::TK, HPI = S::HPI, NS = S::NS, NDT = S::NDT, NVF = S::NVF;
     using G = TileGeo<D, TK, D>;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wh = w >> 2, wr = wh ? 3 - (w & 3) : (w & 3);   // as Lane (attn_kernels.h)
     char* const stage = stage_all + w * 32 * SROW;
-    bf16x8 qf[Q_IN_ACC<D> ? 1 : NS];
+    bf16x8 qf[NS];
     int art_q = -1, pos_q = 0;
     int ri = 0;   // next entry of the redo list
 #pragma unroll 1
@@ -418,8 +337,6 @@ __device__ __forceinline__ void ring_paced_pass(const AttnParams& p, char* const
         float M = -INFINITY, l = 0.f;
         bool viol = false;
         acc_zero<NDT>();
-        ring_wait_q<D>();
-        ring_row_meta<D, WIN>(p, wr, tz, art_q, pos_q);
 #pragma unroll 1
         for (int e = 0; e < ne; e++) {
             const int kt = __builtin_amdgcn_readfirstlane(p.kv_idx[it_e0 + e]);
@@ -445,7 +362,9 @@ __device__ __forceinline__ void ring_paced_pass(const AttnParams& p, char* const
             auto score = [&](auto x_c) __attribute__((always_inline)) {
                 constexpr int x = decltype(x_c)::value;
                 const bf16x8 kf = *(const bf16x8*)(krow + 32 * x);
-                qk_step<D, x>(sa, kf, qf);
+                if (x == 0) qk_first(sa, kf, qf[x]);
+                else if (x == NS - 1) qk_last(sa, kf, qf[x]);
+                else qk_next(sa, kf, qf[x]);
             };
             pv_steps<NS>(score);
             __builtin_amdgcn_sched_barrier(0);
@@ -545,15 +464,22 @@ __device__ __forceinline__ void ring_paced_pass(const AttnParams& p, char* const
 }
 
 template <int D, bool WIN>
-__device__ __forceinline__ void ring_kernel_body(const AttnParams& p, char* const ring, char* const stage_all, int4* const desc) {
-    using S = RingShape<D>;
-    constexpr int TK = S::TK, NW = S::NW, HPI = S::HPI, NSLOT = S::NSLOT, NS = S::NS, NDT = S::NDT, NVF = S::NVF;
+__global__ __launch_bounds__(D == 512 ? 256 : 512) void tree_attn_ring_kernel(const AttnParams p) {
+    constexpr int TK = 32;
+    constexpr int NW = D == 512 ? 4 : 8;      // waves: four row groups x HPI heads of the item
+    constexpr int HPI = NW / 4;
+    constexpr int NSLOT = D == 512 ? 2 : MAX_SLOT;
     using G = TileGeo<D, TK, D>;
+    constexpr int NS = D / 16;     // contraction steps of K Q^T
+    constexpr int NDT = D / 32;    // 32-wide slices of the head dimension in O^T
+    constexpr int NVF = 2 * NDT;   // V^T fragments of one 32-key block
     constexpr int PFD = D >= 256 ? 2 : 8;   // fragment read-ahead: at head dim 256 one more spills a query fragment inside the tile loop
-    constexpr int PF = D == 256 ? 2 : D == 512 ? 4 : (NS < PFD ? NS : PFD);   // K fragment read-ahead (head dim 256: 60 ordinary registers in all)
+    constexpr int PF = D >= 256 ? 4 : (NS < PFD ? NS : PFD);   // K fragments are live in the score phase only, where registers are free
     constexpr int VPF = NVF < PFD ? NVF : PFD;
-    // ring: NSLOT tile slots; stage_all: output staging, one slice per wave; desc [NDESC]: {key tile, bits | DESC_FIRST | DESC_LAST,
-    // query tile | head group << 20, item index}
+    static_assert(NSLOT * G::BUFB + NW * 32 * SROW + NDESC * 16 + 256 <= 160 * 1024, "LDS budget");
+    __shared__ __attribute__((aligned(16))) char ring[NSLOT * G::BUFB];
+    __shared__ __attribute__((aligned(16))) char stage_all[NW * 32 * SROW];   // output staging, one slice per wave
+    __shared__ int4 desc[NDESC];       // {key tile, bits | DESC_FIRST | DESC_LAST, query tile | head group << 20, item index}
     __shared__ __attribute__((aligned(16))) int sy_done[MAX_SLOT];   // waves through with the tile in the slot; NW = the slot waits for somebody to recycle it (words past NSLOT stay 0)
     __shared__ int sy_issued[MAX_SLOT];   // tile the slot was last recycled for (its DMA requested)
     __shared__ int sy_gen;             // descriptors written so far
@@ -561,9 +487,6 @@ __device__ __forceinline__ void ring_kernel_body(const AttnParams& p, char* cons
     __shared__ int sy_ntiles;
     __shared__ int sy_redo[16];        // item sequence number + 1 of the last hand-over to the exact recomputation, per sequence number mod 16
     __shared__ int sy_nredo;           // items of this workgroup handed over so far (their indices: p.redo[lo ..])
-    __shared__ int sy_restart;         // after an abort: the fewest items any wave has completed (the barrier-paced pass starts there)
-    __shared__ int sy_vote;            // barrier-paced pass: some wave of the item met scores too far above its reference
-    __shared__ int sy_gidx[64], sy_gbits[64];   // the descriptor generator's chunk of plan entries (key tiles, block bits), as it lands
 
     const Lane<D, TK, D> L(p);
     const int lo = p.list_ptr[blockIdx.x], hi = p.list_ptr[blockIdx.x + 1];
@@ -575,7 +498,7 @@ __device__ __forceinline__ void ring_kernel_body(const AttnParams& p, char* cons
     // when all eight waves are through with some slot's tile and somebody has to recycle it, with 2 when the workgroup's abort flag is up or after SPIN_LIMIT polls.
     auto spin = [&](const int* word, const int want, const bool at_least, const bool watch) __attribute__((always_inline)) {
         const unsigned a_word = lds_addr(word), a_abort = lds_addr(&sy_abort), a_next = lds_addr(sy_done);
-        int t0, t1, n0, n1, n2, n3, v, ab, code, cnt = SPIN_LIMIT;
+        int t0, t1, n0, n1, n2, n3, v, ab, code, cnt = p.spin_limit;
 #define SPIN_ASM(CMP, WATCH)                                                                                                                         \
     asm volatile("1:\n\tds_read_b32 %0, %10\n\tds_read_b32 %1, %11\n\tds_read_b32 %2, %12\n\tds_read_b32 %3, %12 offset:4\n\t"                     \
                  "ds_read_b32 %4, %12 offset:8\n\tds_read_b32 %5, %12 offset:12\n\ts_waitcnt lgkmcnt(0)\n\t"                                        \
@@ -613,25 +536,24 @@ __device__ __forceinline__ void ring_kernel_body(const AttnParams& p, char* cons
         if (threadIdx.x < NSLOT) *(int*)(ring + threadIdx.x * G::BUFB + G::KTILEB + G::VTILEB + 768) = -1;   // the slot's flag: no generation yet
     }
     if (threadIdx.x < 16) sy_redo[threadIdx.x] = 0;
-    if (threadIdx.x == 0) { sy_gen = 0; sy_abort = 0; sy_ntiles = 0; sy_nredo = 0; sy_restart = 0x7fffffff; sy_vote = 0; }
+    if (threadIdx.x == 0) { sy_gen = 0; sy_abort = 0; sy_ntiles = 0; sy_nredo = 0; }
     __syncthreads();
 
     // descriptor generator (wave 0): items lo .. hi - 1, each item's plan entries in chunks of at most 64
     int gi = lo, ge = 0, gen = 0;   // next chunk: item, first entry inside it; descriptors written
     int pn = 0, p_first = 0, p_last = 0, p_tz = 0, p_item = 0;   // the requested chunk
-    // The chunk's plan entries come through LDS (DMA, like the tiles): as ordinary loads they would be requests in flight across the
-    // tile loop that the compiler knows of, and it then waits for "them" (in fact for every tile request of the wave) in front of
-    // whatever instruction of the loop next writes a register such a load might still be aimed at.
-    auto gen_request = [&]() __attribute__((always_inline)) {   // requests the next chunk's entries
+    int pidx = 0, pbits = 0;
+    auto gen_request = [&]() __attribute__((always_inline)) {   // loads of the next chunk's entries
         if (pn == 0 && gi < hi) {
             const int4 it = p.items[gi];
             const int t = __builtin_amdgcn_readfirstlane(it.x), e0 = __builtin_amdgcn_readfirstlane(it.y), z = __builtin_amdgcn_readfirstlane(it.z);
             const int ne = z & 0xfffff;
             const int n = ne - ge < 64 ? ne - ge : 64;
             const int gl = fresh_lane_id();
-            const int e = e0 + ge + (gl < n ? gl : n - 1);
-            dma4_lane(p.kv_idx + e, lds_addr(sy_gidx));
-            dma4_lane((const int*)p.kv_bits + e, lds_addr(sy_gbits));
+            if (gl < n) {
+                pidx = p.kv_idx[e0 + ge + gl];
+                pbits = (int)p.kv_bits[e0 + ge + gl];
+            }
             pn = n;
             p_first = ge == 0;
             p_last = ge + n == ne;
@@ -643,14 +565,12 @@ __device__ __forceinline__ void ring_kernel_body(const AttnParams& p, char* cons
     };
     auto gen_write = [&]() __attribute__((always_inline)) {   // descriptors of the requested chunk
         if (pn > 0) {
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the chunk has landed (wave 0 only, once per chunk)
             const int gl = fresh_lane_id();
             if (gl < pn) {
-                unsigned b = (unsigned)lds_peek(sy_gbits + gl) & 0xffffu;
+                unsigned b = (unsigned)pbits & 0xffffu;
                 if (p_first && gl == 0) b |= DESC_FIRST;
                 if (p_last && gl == pn - 1) b |= DESC_LAST;
-                if (p.debug_expire > 0 && gen + gl == p.debug_expire - 1) b |= DESC_EXPIRE;
-                desc[(gen + gl) & (NDESC - 1)] = make_int4(lds_peek(sy_gidx + gl), (int)b, p_tz, p_item);
+                desc[(gen + gl) & (NDESC - 1)] = make_int4(pidx, (int)b, p_tz, p_item);
             }
             gen += pn;
             pn = 0;
@@ -735,98 +655,91 @@ __device__ __forceinline__ void ring_kernel_body(const AttnParams& p, char* cons
     if (L.w < NSLOT && L.w < ntiles) issue(L.w, read_desc(L.w));
 
     // ---- per-item state of this wave
-    bf16x8 qf[Q_IN_ACC<D> ? 1 : NS];
+    bf16x8 qf[NS];
     int art_q = -1, pos_q = 0;
     float M = -INFINITY, l = 0.f;
     bool viol = false;
     int iseq = 0;   // items begun
 
-    auto load_q = [&](const int tz) __attribute__((always_inline)) { ring_load_q<D, WIN>(p, L.wr, L.wh, tz, qf, art_q, pos_q); };
+    auto load_q = [&](const int tz) __attribute__((always_inline)) {
+        const int lane = fresh_lane_id();
+        const int tok = (tz & 0xfffff) * SPINF_QTILE + 32 * L.wr + (lane & 31);
+        const int tok_c = tok < p.n ? tok : p.n - 1;
+        const int h = (int)((unsigned)tz >> 20) * HPI + L.wh;
+        const __bf16* qp = p.q + (long)tok_c * p.q_tok + (long)h * p.q_head + 8 * (lane >> 5);
+#pragma unroll
+        for (int s = 0; s < NS; s++) qf[s] = *(const bf16x8*)(qp + 16 * s);
+        art_q = tok < p.n ? p.art[tok_c] : -1;
+        pos_q = WIN ? p.pos[tok_c] : 0;
+    };
     auto reset_acc = [&]() __attribute__((always_inline)) {
         M = -INFINITY;
         l = 0.f;
         acc_zero<NDT>();
         viol = false;
     };
-    auto store_rows = [&](const int tz) __attribute__((always_inline)) { ring_store_rows<D>(p, L.wr, L.wh, stage_all + L.w * 32 * SROW, tz, l); };
+    // normalise O^T and store it as rows: 32 rows x 32 head dims at a time through the wave's own LDS slice, 16-byte pieces out
+    // (pieces of 8 bytes straight from the registers were measured slower: twice the requests for the same bytes)
+    auto store_rows = [&](const int tz) __attribute__((always_inline)) {
+        const int lane = fresh_lane_id(), m = lane & 31, g = lane >> 5;
+        const int tok0 = (tz & 0xfffff) * SPINF_QTILE + 32 * L.wr;
+        const int h = (int)((unsigned)tz >> 20) * HPI + L.wh;
+        const float inv = 1.0f / lane32_sum(l);
+        __bf16* ob = p.o + (long)h * p.o_head;
+        char* const stage = stage_all + L.w * 32 * SROW;
+        asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");   // the last MFMAs' results -> v_accvgpr_read
+        // tile dt is read back from the slice while tile dt + 1 is converted and written to it (the LDS takes a wave's requests
+        // in order, so the write behind the read is safe), and stored after that: no wait between a write and its read-back
+        auto put = [&](auto dt_c) __attribute__((always_inline)) {
+            constexpr int dt = decltype(dt_c)::value;
+            float r16[16];
+            acc_read<dt>(r16);
+#pragma unroll
+            for (int i4 = 0; i4 < 4; i4++) {
+                bf16x4 r;
+#pragma unroll
+                for (int jj = 0; jj < 4; jj++) r[jj] = (__bf16)(r16[4 * i4 + jj] * inv);
+                *(bf16x4*)(stage + m * SROW + (8 * i4 + 4 * g) * 2) = r;
+            }
+        };
+        auto round = [&](auto dt_c) __attribute__((always_inline)) {
+            constexpr int dt = decltype(dt_c)::value;
+            bf16x8 val[2];
+#pragma unroll
+            for (int jj = 0; jj < 2; jj++) {
+                const int c = jj * 64 + lane;
+                val[jj] = *(const bf16x8*)(stage + (c >> 2) * SROW + (c & 3) * 16);
+            }
+            if constexpr (dt + 1 < NDT) put(std::integral_constant<int, dt + 1>{});
+#pragma unroll
+            for (int jj = 0; jj < 2; jj++) {
+                const int c = jj * 64 + lane, row = c >> 2, col = c & 3;
+                if (tok0 + row < p.n) *(bf16x8*)(ob + (long)(tok0 + row) * p.o_tok + 32 * dt + col * 8) = val[jj];
+            }
+        };
+        put(std::integral_constant<int, 0>{});
+        pv_steps<NDT>(round);
+    };
 
     {   // the first item's queries
         need_desc(0);
-        if (!dead) {
-            load_q(read_desc(0).z);
-            ring_wait_q<D>();
-        }
+        if (!dead) load_q(read_desc(0).z);
     }
 
     // ---- the tile sequence: item after item.
     // What a wave needs to know at the top of a tile (the tile's descriptor, the slots waiting for requests, the tile's flag) is
-    // read from LDS while the previous tile's MFMAs run (`pf_*`), and the wave counts itself through with a tile as soon as
+    // read from LDS while the previous tile's last MFMAs run (`pf_*`), and the wave counts itself through with a tile as soon as
     // its last fragment read of the tile is on its way: in the steady state no LDS round trip is waited for.
-    //
-    // Inside the wave the blocks are software-pipelined: P V of a block is put off until the scores of the wave's next block are
-    // there.  The order of a steady-state step is  S^T(j) = K Q^T  |  O^T += V^T P^T (previous block), with the softmax of block j
-    // issued between its MFMAs, a slice per MFMA .  The matrix pipe then sees one unbroken stream of MFMAs from this wave, and the
-    // softmax (vector ALU) runs in their shadow instead of between two MFMA phases.  The accumulation order of O^T and of the row
-    // sums is that of the unpipelined loop, so the bits are.  A wave keeps its hold on the previous block's slot until that block's
-    // V fragments are read; it lets go of it (P V at once, without overlap) before it skips a tile and at the end of an item, so
-    // it never holds a slot while it waits for a tile more than one place ahead (which would need that very slot recycled).
     int j = 0;
     bool have_pf = false;
     int4 pf_d = make_int4(0, 0, 0, 0);
     int pf_n0 = 0, pf_n1 = 0, pf_n2 = 0, pf_n3 = 0, pf_flag = -1;
     auto flag_word = [&](const int jj) __attribute__((always_inline)) { return (const int*)(ring + (jj & (NSLOT - 1)) * G::BUFB + G::KTILEB + G::VTILEB + 768); };
-    // V^T fragment address of this lane in slot sl (ds_read_b64_tr_b16: see Lane in attn_kernels.h), from a fresh lane index
-    auto v_lane_addr = [&](const int sl) __attribute__((always_inline)) {
-        const int ln = fresh_lane_id();
-        return ring + sl * G::BUFB + G::KTILEB + G::V::v_off(4 * (ln >> 5) + ((ln >> 2) & 3)) + 32 * ((ln >> 4) & 1) + 8 * (ln & 3);
-    };
-    // slice schedule of the softmax under the P V MFMAs: element e of the 16 scores of a lane goes behind MFMA number SM_STEP(e); the
-    // first slices wait until two MFMAs have been issued behind the last score MFMA (its result is then in the registers)
-    constexpr int SM_FIRST = 2;
-    auto sm_step_of = [](const int e) constexpr { return SM_FIRST + e * (NVF - SM_FIRST) / 16; };
     while (j < ntiles && !dead) {
         reset_acc();
         iseq++;
         int4 d = make_int4(0, 0, 0, 0);
         bool last = false;
-        bool pend = false;    // probabilities of a block wait for their P V: pbp, of the tile in slot s_pend (wave-uniform)
-        int s_pend = 0;
-        u32x4 pbp[2] = {};
-        // O^T += V^T P^T for the pending block, nothing overlapped (before a skipped tile, at the end of an item)
-        auto pv_plain = [&]() __attribute__((always_inline)) {
-            const char* const vrow = v_lane_addr(s_pend);
-            s16x4 vlo[VPF], vhi[VPF];
-            auto vload = [&](const int f, const int slot) __attribute__((always_inline)) {
-                const char* vp = vrow + G::V::v_off(16 * (f / NDT)) + 64 * (f % NDT);
-                vlo[slot] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)vp);
-                vhi[slot] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vp + G::V::v_off(8)));
-            };
-#pragma unroll
-            for (int f = 0; f < VPF; f++) vload(f, f);
-            __builtin_amdgcn_sched_barrier(0);
-            auto step = [&](auto f_c) __attribute__((always_inline)) {
-                constexpr int f = decltype(f_c)::value;
-                const bf16x8 a = __builtin_bit_cast(bf16x8, __builtin_shufflevector(vlo[f % VPF], vhi[f % VPF], 0, 1, 2, 3, 4, 5, 6, 7));
-                acc_mfma<f % NDT>(a, __builtin_bit_cast(bf16x8, pbp[f / NDT]));
-                if (f + VPF < NVF) vload(f + VPF, f % VPF);
-                if (f + VPF == NVF - 1) {   // that was the tile's last fragment read
-                    if (fresh_lane_id() == 0) __hip_atomic_fetch_add(&sy_done[s_pend], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            };
-            pv_steps<NVF>(step);
-            pend = false;
-        };
-        // the next item's queries, requested as soon as this item's last scores are there (head dim 256: the query registers are
-        // free from then on, and the request has the rest of the item to come back)
-        auto request_next_q = [&]() __attribute__((always_inline)) {
-            if constexpr (Q_IN_ACC<D>) {
-                if (last && j + 1 < ntiles) {
-                    need_desc(j + 1);
-                    if (!dead) load_q(read_desc(j + 1).z);
-                }
-            }
-        };
         do {
             const int s = j & (NSLOT - 1);
             int n0, n1, n2, n3, flag;
@@ -850,66 +763,42 @@ __device__ __forceinline__ void ring_kernel_body(const AttnParams& p, char* cons
             if (L.w < 4) claim(n0, n1, n2, n3);
             if (dead) break;
             const unsigned bits = (unsigned)d.y;
-            if ((bits & DESC_EXPIRE) && L.w == 0) {   // (test hook)
-                lds_store(&sy_abort, 1);
-                dead = true;
-                break;
-            }
             last = (bits & DESC_LAST) != 0;
             const bool act = (bits >> (2 * L.wr)) & 1u;
             if (act) {
                 if (flag != ((j / NSLOT + 1) & 63)) wait_watch(flag_word(j), (j / NSLOT + 1) & 63);
                 if (dead) break;
                 // fragment addresses from a fresh lane index (kept in registers across the tile loop they are spilled, and a reload
-                // waits for every tile request in flight): K row lane % 32 of the block, 16-byte chunk lane / 32 of each 32-byte step
+                // waits for every tile request in flight): K row lane % 32 of the block, 16-byte chunk lane / 32 of each 32-byte step;
+                // V^T as ds_read_b64_tr_b16 wants it (see Lane in attn_kernels.h)
                 const int ln = fresh_lane_id();
                 const char* buf = ring + s * G::BUFB;
                 const char* krow = buf + G::K::k_off(ln & 31) + 16 * (ln >> 5);
-                // S^T = K Q^T; behind the last fragment read, what the next tile's top needs is fetched (descriptor, the slots'
-                // counts, the tile's flag: 16-byte and 4-byte reads like the fragments', all back before the first transposing read of V)
+                const char* vrow = buf + G::KTILEB + G::V::v_off(4 * (ln >> 5) + ((ln >> 2) & 3)) + 32 * ((ln >> 4) & 1) + 8 * (ln & 3);
+                // S^T = K Q^T
                 f32x16 sa;
-                const bool pf_ok = j + 1 < ntiles && j + 1 < gen_seen;
                 {
-                    int4 dv = make_int4(0, 0, 0, 0);
-                    i32x4 nx = {0, 0, 0, 0};
-                    int fv = -1;
                     bf16x8 kf[PF];
 #pragma unroll
                     for (int x = 0; x < PF; x++) kf[x] = *(const bf16x8*)(krow + 32 * x);
                     __builtin_amdgcn_sched_barrier(0);
-                    auto score = [&](auto x_c) __attribute__((always_inline)) {
-                        constexpr int x = decltype(x_c)::value;
-                        qk_step<D, x>(sa, kf[x % PF], qf);
+#pragma unroll
+                    for (int x = 0; x < NS; x++) {
+                        if (x == 0) qk_first(sa, kf[x % PF], qf[x]);
+                        else if (x == NS - 1) qk_last(sa, kf[x % PF], qf[x]);
+                        else qk_next(sa, kf[x % PF], qf[x]);
                         if (x + PF < NS) kf[x % PF] = *(const bf16x8*)(krow + 32 * (x + PF));
-                        if constexpr (x == NS - PF) {
-                            if (pf_ok) {
-                                dv = desc[(j + 1) & (NDESC - 1)];
-                                nx = lds_peek4(sy_done);
-                                fv = lds_peek(flag_word(j + 1));
-                            }
-                        }
                         __builtin_amdgcn_sched_barrier(0);
-                    };
-                    pv_steps<NS>(score);
-                    if (pf_ok) {
-                        pf_d = make_int4(__builtin_amdgcn_readfirstlane(dv.x), __builtin_amdgcn_readfirstlane(dv.y), __builtin_amdgcn_readfirstlane(dv.z), __builtin_amdgcn_readfirstlane(dv.w));
-                        pf_n0 = __builtin_amdgcn_readfirstlane(nx[0]); pf_n1 = __builtin_amdgcn_readfirstlane(nx[1]);
-                        pf_n2 = __builtin_amdgcn_readfirstlane(nx[2]); pf_n3 = __builtin_amdgcn_readfirstlane(nx[3]);
-                        pf_flag = __builtin_amdgcn_readfirstlane(fv);
-                        have_pf = true;
                     }
                 }
-                const bool masked = (bits >> (8 + 2 * L.wr)) & 1u;
-                if (masked) ring_row_meta<D, WIN>(p, L.wr, d.z, art_q, pos_q);   // (before the next item's request overwrites it)
-                request_next_q();
-                if (dead) break;
-                if (masked) {
+                if ((bits >> (8 + 2 * L.wr)) & 1u) {
                     f32x16 sm[1] = {sa};
                     const int tok = (d.z & 0xfffff) * SPINF_QTILE + 32 * L.wr + (ln & 31);
-                    apply_mask<1, WIN, 0, TK, true>(sm, (const int*)(buf + G::KTILEB + G::VTILEB), d.x, 0, ln >> 5, tok, art_q, pos_q, p.window);
+                    apply_mask<1, WIN, 0, TK>(sm, (const int*)(buf + G::KTILEB + G::VTILEB), d.x, 0, ln >> 5, tok, art_q, pos_q, p.window);
                     sa = sm[0];
                 }
                 // softmax against the row's fixed reference (the maximum of the first block it sees a key in)
+                bf16x8 pb[2];
                 {
                     const bool first = M == -INFINITY;
                     if (__builtin_amdgcn_ballot_w64(first) != 0) {   // only where a row meets its first keys (see the lockstep kernel)
@@ -919,15 +808,31 @@ __device__ __forceinline__ void ring_kernel_body(const AttnParams& p, char* cons
                         mx = lane32_max(mx);
                         M = first ? mx * p.c : M;
                     }
+                    const float ms = M == -INFINITY ? 0.f : M;
+                    float sum = 0.f;
+#pragma unroll
+                    for (int i2 = 0; i2 < 16; i2++) {
+                        const float pr = __builtin_amdgcn_exp2f(__builtin_fmaf(sa[i2], p.c, -ms));
+                        sum += pr;
+                        pb[i2 >> 3][i2 & 7] = (__bf16)pr;
+                    }
+                    l += sum;
+                    viol = viol | !(sum <= VIOL_SUM);
                 }
-                const float ms = M == -INFINITY ? 0.f : M;
-                float sum = 0.f;
-                float pr_even = 0.f;
-                unsigned pbn[8];
-                auto sm_elem = [&](auto e_c) __attribute__((always_inline)) { ring_sm_elem<decltype(e_c)::value>(sa, p.c, ms, pr_even, sum, pbn); };
-                if (pend) {
-                    // O^T += V^T P^T of the previous block, the softmax of this one in the MFMAs' shadow
-                    const char* const vrow = v_lane_addr(s_pend);
+                // O^T += V^T P^T, with what the next tile's top needs fetched meanwhile; once the last fragment read is on its way,
+                // count this wave through with the tile
+                int4 dv = make_int4(0, 0, 0, 0);
+                i32x4 nx = {0, 0, 0, 0};
+                int fv = -1;
+                const bool pf_ok = j + 1 < ntiles && j + 1 < gen_seen;
+                // (requested before the first transposing read of V: mixed in among them, a 16-byte read gave the MFMAs stale
+                // fragments, as if the two kinds of reads did not return in the order they were issued)
+                if (pf_ok) {
+                    dv = desc[(j + 1) & (NDESC - 1)];
+                    nx = lds_peek4(sy_done);
+                    fv = lds_peek(flag_word(j + 1));
+                }
+                {
                     s16x4 vlo[VPF], vhi[VPF];
                     auto vload = [&](const int f, const int slot) __attribute__((always_inline)) {
                         const char* vp = vrow + G::V::v_off(16 * (f / NDT)) + 64 * (f % NDT);
@@ -940,33 +845,24 @@ __device__ __forceinline__ void ring_kernel_body(const AttnParams& p, char* cons
                     auto step = [&](auto f_c) __attribute__((always_inline)) {
                         constexpr int f = decltype(f_c)::value;
                         const bf16x8 a = __builtin_bit_cast(bf16x8, __builtin_shufflevector(vlo[f % VPF], vhi[f % VPF], 0, 1, 2, 3, 4, 5, 6, 7));
-                        acc_mfma<f % NDT>(a, __builtin_bit_cast(bf16x8, pbp[f / NDT]));
+                        acc_mfma<f % NDT>(a, pb[f / NDT]);
                         if (f + VPF < NVF) vload(f + VPF, f % VPF);
-                        if (f + VPF == NVF - 1) {   // that was the previous tile's last fragment read
-                            if (fresh_lane_id() == 0) __hip_atomic_fetch_add(&sy_done[s_pend], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                        if (f + VPF == NVF - 1) {   // that was the tile's last fragment read
+                            if (fresh_lane_id() == 0) __hip_atomic_fetch_add(&sy_done[s], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                         }
-                        auto slice = [&](auto e_c) __attribute__((always_inline)) {
-                            constexpr int e = decltype(e_c)::value;
-                            if constexpr (sm_step_of(e) == f) sm_elem(e_c);
-                        };
-                        pv_steps<16>(slice);
                         __builtin_amdgcn_sched_barrier(0);
                     };
                     pv_steps<NVF>(step);
-                } else {
-                    pv_steps<16>(sm_elem);
                 }
-                l += sum;
-                viol = viol | !(sum <= VIOL_SUM);
-                pbp[0] = u32x4{pbn[0], pbn[1], pbn[2], pbn[3]};
-                pbp[1] = u32x4{pbn[4], pbn[5], pbn[6], pbn[7]};
-                s_pend = s;
-                pend = true;
+                if (pf_ok) {
+                    pf_d = make_int4(__builtin_amdgcn_readfirstlane(dv.x), __builtin_amdgcn_readfirstlane(dv.y), __builtin_amdgcn_readfirstlane(dv.z), __builtin_amdgcn_readfirstlane(dv.w));
+                    pf_n0 = __builtin_amdgcn_readfirstlane(nx[0]); pf_n1 = __builtin_amdgcn_readfirstlane(nx[1]);
+                    pf_n2 = __builtin_amdgcn_readfirstlane(nx[2]); pf_n3 = __builtin_amdgcn_readfirstlane(nx[3]);
+                    pf_flag = __builtin_amdgcn_readfirstlane(fv);
+                    have_pf = true;
+                }
             } else {
                 // nothing of this tile for these rows: the slot must have been recycled for it before this wave counts itself through
-                if (pend) pv_plain();
-                request_next_q();
-                if (dead) break;
                 wait_watch(&sy_issued[s], j);
                 if (dead) break;
                 if (fresh_lane_id() == 0) __hip_atomic_fetch_add(&sy_done[s], 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -979,12 +875,11 @@ __device__ __forceinline__ void ring_kernel_body(const AttnParams& p, char* cons
             j++;
         } while (!last);
         if (dead) break;
-        if (pend) pv_plain();
-        // this wave's rows of the item are complete: the next item's queries are requested (their registers are free; at head dim
-        // 256 that has happened behind the item's last scores), then the rows go out (or the item goes to the exact pass)
+        // this wave's rows of the item are complete: the next item's queries are requested (their registers are free), then the rows
+        // go out (or the item goes to the exact pass)
         const bool hand_over = __builtin_amdgcn_ballot_w64(viol) != 0;   // scores ranged too widely somewhere in these 32 rows
         const int tz_done = d.z, item_done = d.w;
-        if (!Q_IN_ACC<D> && j < ntiles) {
+        if (j < ntiles) {
             need_desc(j);
             if (dead) break;
             load_q(read_desc(j).z);
@@ -997,71 +892,152 @@ __device__ __forceinline__ void ring_kernel_body(const AttnParams& p, char* cons
                     __hip_atomic_store(&p.redo[lo + k], item_done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
             }
-            ring_wait_q<D>();
         } else {
-            ring_wait_q<D>();   // (before the rows' stores: loads and stores do not return in one order, so no count tells them apart afterwards)
             store_rows(tz_done);
         }
     }
-    if (dead && fresh_lane_id() == 0) {
-        atomicAdd(&p.counters[NLIST + 4], 1);
-        // a wave gives up inside an item or right behind its tiles, before the item's rows leave: the items it began, less that one, are complete
-        __hip_atomic_fetch_min(&sy_restart, iseq > 0 ? iseq - 1 : 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    }
+    if (dead && fresh_lane_id() == 0) atomicAdd(&p.land[blockIdx.x], 1);   // the landing kernel will do this workgroup's list again
     __builtin_amdgcn_s_waitcnt(0x0f70);
 
-    __syncthreads();   // every wave is through with its list or has left it: the ring is free, the hand-overs are all in
-    // what is left for the barrier-paced pass: after an abort the list from the first item that some wave had not completed (a wave that
-    // was never held up has completed them all), and the items handed to the exact recomputation.  Normally nothing.
-    const bool aborted = __builtin_amdgcn_readfirstlane(lds_load(&sy_abort)) != 0;
-    if (!aborted && __builtin_amdgcn_readfirstlane(lds_load(&sy_nredo)) == 0) return;
-    int li = hi;
-    if (aborted) {
-        const int restart = __builtin_amdgcn_readfirstlane(lds_load(&sy_restart));
-        li = lo + (restart < hi - lo ? restart : hi - lo);
+    // ---- the exact recomputation.  Items in which some row met scores too far above its reference (normally none) are done
+    // again here, by the workgroup that owns them, after its list: classic online softmax over the same 32-key blocks in the same
+    // order (the reference is raised, and the accumulators rescaled, whenever a block maximum exceeds it by more than TAU_LAZY),
+    // the arithmetic of tree_attn_exact_kernel (tree_attn.hip) step for step, so the two give the same bits.  Nothing is
+    // overlapped: one tile at a time into slot 0, a workgroup barrier on either side of its request.  Whether an item comes here
+    // depends on its own rows only, so a job's output does not depend on what it is packed with.
+    __syncthreads();   // every wave is through with its list: the ring is free, the hand-overs are all in
+    const int n_redo = __builtin_amdgcn_readfirstlane(lds_load(&sy_nredo));
+    if (n_redo == 0 || __builtin_amdgcn_readfirstlane(lds_load(&sy_abort)) != 0) return;
+#pragma unroll 1
+    for (int r = 0; r < n_redo; r++) {
+        const int idx = __builtin_amdgcn_readfirstlane(__hip_atomic_load(&p.redo[lo + r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+        const int4 itv = p.items[idx];
+        const int it_t = __builtin_amdgcn_readfirstlane(itv.x), it_e0 = __builtin_amdgcn_readfirstlane(itv.y), it_z = __builtin_amdgcn_readfirstlane(itv.z);
+        const int ne = it_z & 0xfffff;
+        const int tz = it_t | (int)((unsigned)it_z >> 20 << 20);
+        const int kvh = (int)((unsigned)it_z >> 20) * HPI / p.group;
+        load_q(tz);
+        reset_acc();
+#pragma unroll 1
+        for (int e = 0; e < ne; e++) {
+            const int kt = __builtin_amdgcn_readfirstlane(p.kv_idx[it_e0 + e]);
+            const unsigned bits = (unsigned)__builtin_amdgcn_readfirstlane((int)p.kv_bits[it_e0 + e]);
+            __syncthreads();   // everyone is through with the slot
+            if (L.w == 0) {
+                using GK = Geo<D, TK>;
+                const int lane = fresh_lane_id();
+                const unsigned lane_k = (unsigned)((lane / GK::CPR) * GK::NREG * p.k_tok * 2 + (lane % GK::CPR) * 16);
+                const unsigned lane_v = (unsigned)((lane / GK::CPR) * GK::NREG * p.v_tok * 2 + (lane % GK::CPR) * 16);
+                issue_tile_wave<D, WIN>(p, lds_addr(ring), kt, kvh, 0, lane, lane_k, lane_v);
+            }
+            __builtin_amdgcn_s_waitcnt(0x0f70);   // the tile has landed (and this wave's queries)
+            __syncthreads();
+            if (!((bits >> (2 * L.wr)) & 1u)) continue;   // (wave-uniform; the barriers above are passed by every wave)
+            const int ln = fresh_lane_id();
+            const char* krow = ring + G::K::k_off(ln & 31) + 16 * (ln >> 5);
+            const char* vrow = ring + G::KTILEB + G::V::v_off(4 * (ln >> 5) + ((ln >> 2) & 3)) + 32 * ((ln >> 4) & 1) + 8 * (ln & 3);
+            // (the scheduling barriers keep the three kinds of LDS reads apart: the transposing reads of V and the 16-byte reads
+            // of K and of the keys' metadata do not complete in the order they were issued, which the compiler's counting assumes)
+            f32x16 sa;
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int x = 0; x < NS; x++) {
+                const bf16x8 kf = *(const bf16x8*)(krow + 32 * x);
+                if (x == 0) qk_first(sa, kf, qf[x]);
+                else if (x == NS - 1) qk_last(sa, kf, qf[x]);
+                else qk_next(sa, kf, qf[x]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if ((bits >> (8 + 2 * L.wr)) & 1u) {
+                f32x16 sm[1] = {sa};
+                const int tok = (tz & 0xfffff) * SPINF_QTILE + 32 * L.wr + (ln & 31);
+                apply_mask<1, WIN, 0, TK>(sm, (const int*)(ring + G::KTILEB + G::VTILEB), kt, 0, ln >> 5, tok, art_q, pos_q, p.window);
+                sa = sm[0];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            bf16x8 pb[2];
+            {
+                float mx = sa[0];
+#pragma unroll
+                for (int i2 = 1; i2 < 16; i2++) mx = fmaxf(mx, sa[i2]);
+                mx = lane32_max(mx);
+                const float tm = mx * p.c;
+                const bool up = tm > M + TAU_LAZY;
+                const float mn = up ? tm : M;
+                const float alpha = up ? __builtin_amdgcn_exp2f(M - mn) : 1.0f;
+                if (__builtin_amdgcn_ballot_w64(up && M != -INFINITY) != 0) {   // rows without a key so far hold zeros
+                    asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");   // the last MFMAs' results -> v_accvgpr_read
+                    acc_scale<NDT>(alpha);
+                    asm volatile("s_nop 3" ::: "memory");                // v_accvgpr_write -> MFMA srcC
+                }
+                l *= alpha;
+                M = mn;
+                const float ms = mn == -INFINITY ? 0.f : mn;
+                float sum = 0.f;
+#pragma unroll
+                for (int i2 = 0; i2 < 16; i2++) {
+                    const float pr = __builtin_amdgcn_exp2f(__builtin_fmaf(sa[i2], p.c, -ms));
+                    sum += pr;
+                    pb[i2 >> 3][i2 & 7] = (__bf16)pr;
+                }
+                l += sum;
+            }
+            __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): no 16-byte read in flight when the transposing reads begin
+            __builtin_amdgcn_sched_barrier(0);
+            auto step = [&](auto f_c) __attribute__((always_inline)) {
+                constexpr int f = decltype(f_c)::value;
+                const char* vp = vrow + G::V::v_off(16 * (f / NDT)) + 64 * (f % NDT);
+                const s16x4 lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)vp);
+                const s16x4 hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vp + G::V::v_off(8)));
+                const bf16x8 a = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo4, hi4, 0, 1, 2, 3, 4, 5, 6, 7));
+                acc_mfma<f % NDT>(a, pb[f / NDT]);
+                __builtin_amdgcn_sched_barrier(0);
+            };
+            pv_steps<NVF>(step);
+        }
+        store_rows(tz);
     }
-    ring_paced_pass<D, WIN>(p, ring, stage_all, &sy_nredo, &sy_vote, lo, hi, li);
+    if (threadIdx.x == 0) atomicAdd(&p.counters[NLIST + 3], n_redo);   // running total, for spinf_attn_exact_items
+    __builtin_amdgcn_s_waitcnt(0x0f70);
 }
 
-// The tile ring, the staging slices and the descriptors are ONE block of dynamic LDS, sized at launch.  Not for flexibility: with
-// 155 KB of LDS declared in the kernel the compiler concludes that two waves per SIMD is all the kernel can ever reach and takes the
-// whole register file split evenly (128 ordinary + 128 accumulation registers), whatever limit the kernel asks for; the kernel needs
-// 60 + 196.  With the size out of its sight the limit below holds.
-extern __shared__ __attribute__((aligned(16))) char ring_lds[];
-template <int D>
-struct RingLds {
+// The landing kernel: launched behind every launch of the ring kernel, with the same grid.  A workgroup whose ring-kernel twin left no
+// word (p.land[b] == 0: every launch but a faulty one) returns at once; otherwise it computes that workgroup's whole list again.
+template <int D, bool WIN>
+__global__ __launch_bounds__(D == 512 ? 256 : 512) void tree_attn_ring_landing_kernel(const AttnParams p) {
+    const int gave_up = p.land[blockIdx.x];   // waves of the ring kernel's workgroup b that gave up a wait
+    if (gave_up == 0) return;
     using S = RingShape<D>;
     using G = TileGeo<D, S::TK, D>;
-    static constexpr int RINGB = S::NSLOT * G::BUFB, STAGEB = S::NW * 32 * SROW, BYTES = RINGB + STAGEB + NDESC * 16;
-    static_assert(BYTES + 512 <= 160 * 1024, "LDS budget");
-};
-#define RING_KERNEL(NAME, D, WIN, ATTR)                                                                                                      \
-    __global__ __launch_bounds__(D == 512 ? 256 : 512) ATTR void NAME(const AttnParams p) {                                                  \
-        ring_kernel_body<D, WIN>(p, ring_lds, ring_lds + RingLds<D>::RINGB, (int4*)(ring_lds + RingLds<D>::RINGB + RingLds<D>::STAGEB));     \
+    __shared__ __attribute__((aligned(16))) char ring[G::BUFB];
+    __shared__ __attribute__((aligned(16))) char stage_all[S::NW * 32 * SROW];
+    __shared__ int sy_nredo, sy_vote;
+    const int lo = p.list_ptr[blockIdx.x], hi = p.list_ptr[blockIdx.x + 1];
+    if (threadIdx.x == 0) {
+        sy_nredo = 0;   // (the ring kernel's workgroup left without its exact recomputations: whatever the list needs is found again here)
+        sy_vote = 0;
+        atomicAdd(&p.counters[NLIST + 4], gave_up);   // running total, for spinf_attn_ring_aborts
     }
-RING_KERNEL(tree_attn_ring_kernel_256, 256, false, __attribute__((amdgpu_num_vgpr(60))))
-RING_KERNEL(tree_attn_ring_kernel_256w, 256, true, __attribute__((amdgpu_num_vgpr(60))))
-RING_KERNEL(tree_attn_ring_kernel_512, 512, false, )
-RING_KERNEL(tree_attn_ring_kernel_512w, 512, true, )
-#undef RING_KERNEL
+    __syncthreads();
+    ring_paced_pass<D, WIN>(p, ring, stage_all, &sy_nredo, &sy_vote, lo, hi, lo);
+    if (threadIdx.x == 0) p.land[blockIdx.x] = 0;   // (the word is per launch: the next one starts clean)
+}
 
-template <class K>
-int launch_ring_k(K kernel, const AttnParams& p, int n_wg, int threads, int lds_bytes, hipStream_t stream) {
-    // (more dynamic LDS than the default limit must be asked for once per kernel and device; asking again is cheap)
-    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: %d bytes of LDS for the ring kernel: %s", lds_bytes, hipGetErrorString(e));
-    hipLaunchKernelGGL(kernel, dim3(n_wg), dim3(threads), lds_bytes, stream, p);
-    e = hipGetLastError();
+template <int D, bool WIN>
+int launch_ring_t(const AttnParams& p, int n_wg, hipStream_t stream) {
+    hipLaunchKernelGGL((tree_attn_ring_kernel<D, WIN>), dim3(n_wg), dim3(D == 512 ? 256 : 512), 0, stream, p);
+    hipError_t e = hipGetLastError();
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: launch (ring kernel): %s", hipGetErrorString(e));
+    hipLaunchKernelGGL((tree_attn_ring_landing_kernel<D, WIN>), dim3(n_wg), dim3(D == 512 ? 256 : 512), 0, stream, p);
+    e = hipGetLastError();
+    if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: launch (landing kernel): %s", hipGetErrorString(e));
     return SPINF_OK;
 }
 
 }  // namespace
 
 int spinf_launch_ring(const AttnParams& p, int d, bool win, int n_wg, hipStream_t stream) {
-    if (d == 256) return win ? launch_ring_k(tree_attn_ring_kernel_256w, p, n_wg, 512, RingLds<256>::BYTES, stream)
-                             : launch_ring_k(tree_attn_ring_kernel_256, p, n_wg, 512, RingLds<256>::BYTES, stream);
-    if (d == 512) return win ? launch_ring_k(tree_attn_ring_kernel_512w, p, n_wg, 256, RingLds<512>::BYTES, stream)
-                             : launch_ring_k(tree_attn_ring_kernel_512, p, n_wg, 256, RingLds<512>::BYTES, stream);
+    if (d == 256) return win ? launch_ring_t<256, true>(p, n_wg, stream) : launch_ring_t<256, false>(p, n_wg, stream);
+    if (d == 512) return win ? launch_ring_t<512, true>(p, n_wg, stream) : launch_ring_t<512, false>(p, n_wg, stream);
     return spinf_fail(SPINF_E_ARG, "tree_attn: the ring kernel takes head dim 256 or 512, not %d", d);
 }

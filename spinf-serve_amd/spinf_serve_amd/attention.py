@@ -33,7 +33,7 @@ STATIC = int(os.environ.get("SPINF_ATTN_STATIC", "-1"))  # -1 = auto
 
 RING_MAX_ITEMS_PER_WG = 8
 
-# test hook (spinf_attn_args.debug_expire): k > 0 makes wave 0 of every workgroup of the decoupled kernel give up at its k-th tile
+# test hook (spinf_attn_args.debug_expire): k > 0 = polls after which a wave of the decoupled kernel gives up a wait (2^18 otherwise)
 DEBUG_EXPIRE = 0
 
 

@@ -650,12 +650,13 @@ def test_allocating_entry_point_under_graph_capture(dev):
     torch.cuda.synchronize()
 
 
-@pytest.mark.parametrize("d,expire,wide", [(256, 1, False), (256, 7, False), (256, 30, False), (256, 30, True), (512, 5, False), (512, 23, True)])
-def test_a_wave_that_gives_up_a_wait_costs_time_not_rows(dev, d, expire, wide, monkeypatch):
-    """the decoupled kernel's landing: wave 0 of every workgroup is told (from the host, spinf_attn_args.debug_expire) to treat its
-    wait at its expire-th tile as run out; the workgroup then leaves the ring and computes the rest of its list one tile at a time
-    between barriers.  Every kernel exits normally, the abort is counted, and the output equals the lockstep kernel's bit for bit,
-    also where items go on to the exact recomputation (wide) and with a window."""
+@pytest.mark.parametrize("d,limit,wide", [(256, 1, False), (256, 1, True), (256, 3, False), (512, 1, False), (512, 1, True)])
+def test_a_wave_that_gives_up_a_wait_costs_time_not_rows(dev, d, limit, wide, monkeypatch):
+    """the decoupled kernel's landing: the waves are told (from the host, spinf_attn_args.debug_expire) to give up a wait after
+    `limit` polls instead of 2^18, so every wave that has to wait for a tile at all gives up, as after a real time-out; its
+    workgroup leaves the ring and the landing kernel computes that workgroup's list again, one tile at a time between barriers.
+    Every kernel exits normally, the aborts are counted, and the output equals the lockstep kernel's bit for bit, also where items
+    go on to the exact recomputation (wide) and with a window."""
     from spinf_serve_amd import attention
 
     cfg = synth.attention_config("C2" if d == 256 else "C2_512", contents=12 if d == 256 else 6)
@@ -671,13 +672,13 @@ def test_a_wave_that_gives_up_a_wait_costs_time_not_rows(dev, d, expire, wide, m
         torch.cuda.synchronize()
         monkeypatch.setattr(attention, "RING", 1)
         before, exact0 = _ring_aborts(), _exact_items()
-        print(f"case d={d} expire={expire} wide={wide} window={window}: plain ring pass", flush=True)
+        print(f"case d={d} limit={limit} wide={wide} window={window}: plain ring pass", flush=True)
         plain = sa.tree_attn(q, k, v, mask, cfg.scale)
         torch.cuda.synchronize()
         assert _ring_aborts() == before
         exact_plain = _exact_items() - exact0
-        monkeypatch.setattr(attention, "DEBUG_EXPIRE", expire)
-        print(f"case d={d} expire={expire} wide={wide} window={window}: forced abort", flush=True)
+        monkeypatch.setattr(attention, "DEBUG_EXPIRE", limit)
+        print(f"case d={d} limit={limit} wide={wide} window={window}: waits run out after {limit} polls", flush=True)
         got = sa.tree_attn(q, k, v, mask, cfg.scale)
         torch.cuda.synchronize()
         monkeypatch.setattr(attention, "DEBUG_EXPIRE", 0)
@@ -686,3 +687,6 @@ def test_a_wave_that_gives_up_a_wait_costs_time_not_rows(dev, d, expire, wide, m
         assert torch.equal(got, want), float((got.float() - want.float()).abs().max())
         if wide:
             assert exact_plain > 0 and _exact_items() - exact0 == 2 * exact_plain   # the same items were recomputed exactly, once each
+        again = sa.tree_attn(q, k, v, mask, cfg.scale)   # and the next launch starts clean
+        torch.cuda.synchronize()
+        assert torch.equal(again, want) and _ring_aborts() == before + (_ring_aborts() - before)
