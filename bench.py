@@ -122,6 +122,38 @@ def gdn_record(sa, synth, torch, np, args, steps, warmup):
     return rec, cfg, t
 
 
+def attn_record(sa, synth, torch, np, workload, seed, steps, warmup):
+    """one of the other attention configurations, whole (every pass, every layer of a step), inputs drawn on the device -> record"""
+    dev = torch.device("cuda:0")
+    cfg = synth.attention_config(workload, seed=seed)
+    layers = [None] if cfg.window is None else [cfg.window, None]
+    work = []
+    for b in cfg.batches:
+        masks = sa.block_masks(b, sliding_window=cfg.window, device=dev)
+        work.append((synth.qkv_device(cfg, b, seed=seed, device=dev), masks))
+    torch.cuda.synchronize()
+
+    def step():
+        out = None
+        for (q, k, v), masks in work:
+            for w in layers:
+                out = sa.tree_attn(q, k, v, masks["sliding_attention" if w else "full_attention"], cfg.scale)
+        return out
+
+    wall, kern = timed(step, steps, warmup, torch)
+    ms = float(np.mean(kern))
+    flops = sum(cfg.flops(w) for w in layers)
+    nbytes = cfg.bytes() * len(layers)
+    tfl = flops / (ms * 1e-3) / 1e12
+    return {"metric": "packed query tokens/s + % bf16 MFMA peak (useful FLOPs), tree-mask attn", "value": cfg.n_real * len(layers) * steps / wall, "unit": "tokens/s",
+            "ms_per_step": 1e3 * wall / steps, "steps": steps, "warmup": warmup, "dtype": "bf16", "data": "synthetic (seeded numpy trees; Q/K/V from the device generator)",
+            "config": {"workload": WORKLOADS[workload], "contents": len(cfg.trees), "packed_tokens": cfg.n_real, "stream_tokens": sum(b.length for b in cfg.batches),
+                       "passes": len(cfg.batches), "layers_per_step": len(layers), "visible_pairs": [cfg.pairs(w) for w in layers]},
+            "roofline": {"bound": "mfma", "achieved": tfl, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": tfl / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_BYTES.get(workload),
+                         "kernel_ms": ms, "useful_flops": flops, "algorithmic_bytes": nbytes,
+                         "mfma_floor_ms": flops / (PEAK_BF16_TFLOPS * 1e12) * 1e3, "hbm_floor_ms": nbytes / (PEAK_HBM_GBS * 1e9) * 1e3}}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -134,6 +166,7 @@ def main():
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--variant", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-big", action="store_true", help="C2 only: skip the C3 / C4 sub-records")
     ap.add_argument("--nsplit", type=int, default=None, help="XDEC workloads: splits of a (group, kv head) key stream (default: the library's choice)")
     ap.add_argument("--rows", default="stream", choices=["stream", "compact", "scatter"],
                     help="attention workloads: stream layout (default); compact = real rows only, read through the kernel's row map; "
@@ -405,6 +438,11 @@ def main():
         # the other half of the hot path, timed in the same run: C5 through the Gated DeltaNet tree scan
         work = None
         line["gdn"] = gdn_record(sa, synth, torch, np, args, max(10, args.steps // 4), max(5, args.warmup // 4))[0]
+        # and the two bigger attention configurations, whole, a few steps each (C3: 13 passes x 2 layers a step; C4: one launch of 659,200 tokens)
+        if not args.no_big:
+            for name, key in (("C3", "c3"), ("C4", "c4")):
+                torch.cuda.empty_cache()
+                line[key] = attn_record(sa, synth, torch, np, name, args.seed, 4, 1)
     print(json.dumps(line))
 
 

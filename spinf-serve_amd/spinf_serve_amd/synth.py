@@ -135,6 +135,25 @@ def qkv(cfg: AttnConfig, batch, seed: int = 0, device="cuda"):
     return mk(cfg.hq), mk(cfg.hkv), mk(cfg.hkv)
 
 
+def qkv_device(cfg: AttnConfig, batch, seed: int = 0, device="cuda"):
+    """Q, K, V of qkv()'s shapes and value distribution, drawn by the device's generator: for streams of several GB, where the
+    host generator takes half a minute.  (Other values than qkv()'s for the same seed.)"""
+    import torch
+
+    gen = torch.Generator(device=device).manual_seed(seed + 7919 * batch.length)
+    n = batch.length
+
+    def mk(h):
+        out = torch.empty((n, h, cfg.d), dtype=torch.bfloat16, device=device)
+        step = max(1, (1 << 26) // (h * cfg.d))
+        for a in range(0, n, step):
+            b = min(n, a + step)
+            out[a:b] = (torch.randn((b - a, h, cfg.d), generator=gen, device=device) * cfg.std).to(torch.bfloat16)
+        return out
+
+    return mk(cfg.hq), mk(cfg.hkv), mk(cfg.hkv)
+
+
 # ------------------------------------------------------------------------------------------------ Gated DeltaNet
 @dataclass
 class GdnConfig:
