@@ -315,6 +315,12 @@ int spinf_xdecode_attn_fwd(const spinf_xdec_args* args, void* stream);
  * *flops receives the floating-point operations of the launch.  Timing is the caller's (events on the stream).
  */
 int spinf_diag_mfma_rate(int64_t iters, float* out, int64_t out_floats, double* flops, void* stream);
+/* Diagnostics (no counterpart in the reference): do a wave's LDS reads of different kinds (ds_read_b64_tr_b16, ds_read_b128) return
+ * in issue order, as every s_waitcnt lgkmcnt(n) of the kernels above assumes?  `workgroups` workgroups of four waves each run
+ * `iters` rounds of six interleavings of eight reads, waiting with the partial counts an in-order LDS allows, and compare with the
+ * same reads done one at a time.  out: 7 device ints, zeroed by the caller: [0..5] += mismatches per interleaving, [6] += workgroups
+ * that ran.  Any nonzero count in [0..5] means out-of-order returns. */
+int spinf_diag_lds_order(int32_t iters, int32_t workgroups, int32_t* out, void* stream);
 
 #ifdef __cplusplus
 }

@@ -38,7 +38,124 @@ __global__ __launch_bounds__(512) void mfma_rate_kernel(const long iters, float*
     out[(long)blockIdx.x * blockDim.x + threadIdx.x] = s;   // keeps the loop alive
 }
 
+// ---- do LDS reads of different kinds return in the order they were issued?
+// The attention and scan kernels mix three kinds of LDS reads in one wave: transposing 8-byte reads (ds_read_b64_tr_b16: V^T
+// fragments), 16-byte reads (K fragments, key metadata, descriptors) and 4-byte reads, and wait for them with partial counts
+// (s_waitcnt lgkmcnt(n): "all but the n youngest have returned"), which is only right if a wave's LDS reads return in issue order
+// whatever their kind.  This kernel checks exactly that, under load: every wave issues eight reads of mixed kinds back to back,
+// waits with the partial count an in-order LDS allows before it touches each result (registers poisoned beforehand, so a read that
+// has not returned shows), and compares with the same reads done one at a time with a full wait.  Assembly throughout, so that the
+// waits are the ones written here and nothing else.
+typedef __attribute__((ext_vector_type(2))) unsigned u32x2;
+typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
+constexpr int LDS_ORDER_WORDS = 8192;    // 32 KB of pattern
+constexpr int LDS_ORDER_PATTERNS = 6;
+
+__device__ __forceinline__ void lds_rd_tr(u32x2& d, const unsigned addr) { asm volatile("ds_read_b64_tr_b16 %0, %1" : "+v"(d) : "v"(addr) : "memory"); }
+__device__ __forceinline__ void lds_rd_16(u32x4& d, const unsigned addr) { asm volatile("ds_read_b128 %0, %1" : "+v"(d) : "v"(addr) : "memory"); }
+template <int N>
+__device__ __forceinline__ void lds_wait(u32x2& d) { asm volatile("s_waitcnt lgkmcnt(%c1)" : "+v"(d) : "n"(N) : "memory"); }
+template <int N>
+__device__ __forceinline__ void lds_wait(u32x4& d) { asm volatile("s_waitcnt lgkmcnt(%c1)" : "+v"(d) : "n"(N) : "memory"); }
+__device__ __forceinline__ unsigned fold(const u32x2 d) { return d[0] * 3u + d[1]; }
+__device__ __forceinline__ unsigned fold(const u32x4 d) { return ((d[0] * 3u + d[1]) * 3u + d[2]) * 3u + d[3]; }
+
+// KINDS: bit k set = read k is a 16-byte read, clear = a transposing 8-byte read
+template <unsigned KINDS, int K = 0>
+__device__ __forceinline__ void lds_order_issue(u32x2 (&t)[8], u32x4 (&b)[8], const unsigned (&at)[8], const unsigned (&ab)[8]) {
+    if constexpr (K < 8) {
+        if constexpr ((KINDS >> K) & 1u) lds_rd_16(b[K], ab[K]);
+        else lds_rd_tr(t[K], at[K]);
+        lds_order_issue<KINDS, K + 1>(t, b, at, ab);
+    }
+}
+template <unsigned KINDS, int K = 0>
+__device__ __forceinline__ void lds_order_take(u32x2 (&t)[8], u32x4 (&b)[8], unsigned (&got)[8]) {
+    if constexpr (K < 8) {
+        if constexpr ((KINDS >> K) & 1u) {
+            lds_wait<7 - K>(b[K]);
+            got[K] = fold(b[K]);
+        } else {
+            lds_wait<7 - K>(t[K]);
+            got[K] = fold(t[K]);
+        }
+        lds_order_take<KINDS, K + 1>(t, b, got);
+    }
+}
+template <unsigned KINDS, int K = 0>
+__device__ __forceinline__ void lds_order_serial(const unsigned (&at)[8], const unsigned (&ab)[8], unsigned (&want)[8]) {
+    if constexpr (K < 8) {
+        if constexpr ((KINDS >> K) & 1u) {
+            u32x4 d = {0xdeadbeefu, 0xdeadbeefu, 0xdeadbeefu, 0xdeadbeefu};
+            lds_rd_16(d, ab[K]);
+            lds_wait<0>(d);
+            want[K] = fold(d);
+        } else {
+            u32x2 d = {0xdeadbeefu, 0xdeadbeefu};
+            lds_rd_tr(d, at[K]);
+            lds_wait<0>(d);
+            want[K] = fold(d);
+        }
+        lds_order_serial<KINDS, K + 1>(at, ab, want);
+    }
+}
+
+template <unsigned KINDS>
+__device__ __forceinline__ int lds_order_round(const unsigned base, const int it) {
+    const unsigned lane = threadIdx.x & 63u;
+    unsigned at[8], ab[8];
+#pragma unroll
+    for (int k = 0; k < 8; k++) {   // strides that change with the round: conflict-free and conflicting patterns both come by
+        at[k] = base + ((lane * 8u * (1u + (unsigned)((it + k) % 9)) + 64u * (unsigned)k * (unsigned)(it % 7 + 1)) & (LDS_ORDER_WORDS * 4u - 8u));
+        ab[k] = base + ((lane * 16u * (1u + (unsigned)((it + 3 * k) % 5)) + 256u * (unsigned)k + 16u * (unsigned)(it % 11)) & (LDS_ORDER_WORDS * 4u - 16u));
+    }
+    u32x2 t[8];
+    u32x4 b[8];
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        t[k] = u32x2{0xdeadbeefu, 0xdeadbeefu};
+        b[k] = u32x4{0xdeadbeefu, 0xdeadbeefu, 0xdeadbeefu, 0xdeadbeefu};
+    }
+    unsigned got[8], want[8];
+    lds_order_issue<KINDS>(t, b, at, ab);
+    lds_order_take<KINDS>(t, b, got);
+    lds_order_serial<KINDS>(at, ab, want);
+    int bad = 0;
+#pragma unroll
+    for (int k = 0; k < 8; k++) bad += got[k] != want[k];
+    return bad;
+}
+
+__global__ __launch_bounds__(256) void lds_order_kernel(const int iters, int* out) {
+    __shared__ __attribute__((aligned(16))) unsigned pat[LDS_ORDER_WORDS];
+    for (int i = threadIdx.x; i < LDS_ORDER_WORDS; i += blockDim.x) pat[i] = (unsigned)i * 2654435761u ^ ((unsigned)i >> 3) ^ (blockIdx.x * 40503u);
+    __syncthreads();
+    const unsigned base = (unsigned)(size_t)(const __attribute__((address_space(3))) unsigned*)pat;
+    int bad[LDS_ORDER_PATTERNS] = {0, 0, 0, 0, 0, 0};
+    for (int it = 0; it < iters; it++) {
+        bad[0] += lds_order_round<0xaau>(base, it);   // T B T B T B T B
+        bad[1] += lds_order_round<0x55u>(base, it);   // B T B T B T B T
+        bad[2] += lds_order_round<0xf0u>(base, it);   // T T T T B B B B
+        bad[3] += lds_order_round<0x0fu>(base, it);   // B B B B T T T T
+        bad[4] += lds_order_round<0xccu>(base, it);   // T T B B T T B B
+        bad[5] += lds_order_round<0x24u>(base, it);   // T T B T T B T T: a 16-byte read among transposing ones
+    }
+#pragma unroll
+    for (int v = 0; v < LDS_ORDER_PATTERNS; v++)
+        if (bad[v]) atomicAdd(&out[v], bad[v]);
+    if (threadIdx.x == 0) atomicAdd(&out[LDS_ORDER_PATTERNS], 1);   // workgroups that ran
+}
+
 }  // namespace
+
+extern "C" int spinf_diag_lds_order(int32_t iters, int32_t workgroups, int32_t* out, void* stream) {
+    if (iters <= 0 || iters > 100000 || workgroups <= 0 || workgroups > 65536 || !out)
+        return spinf_fail(SPINF_E_ARG, "diag_lds_order: iters in 1 .. 100,000, workgroups in 1 .. 65,536, out not null");
+    hipLaunchKernelGGL(lds_order_kernel, dim3(workgroups), dim3(256), 0, (hipStream_t)stream, (int)iters, (int*)out);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "diag_lds_order: launch: %s", hipGetErrorString(e));
+    return SPINF_OK;
+}
 
 extern "C" int spinf_diag_mfma_rate(int64_t iters, float* out, int64_t out_floats, double* flops, void* stream) {
     if (iters <= 0 || iters > (1 << 24) || !out || !flops) return spinf_fail(SPINF_E_ARG, "diag_mfma_rate: iters in 1 .. 2^24, out and flops not null");

@@ -108,6 +108,59 @@ def test_ops_have_no_cpu_path(lib):
         sa.tree_attn(q, k, k, mask, cfg.scale)
 
 
+@pytest.mark.parametrize("entry", ["tree_attn", "tree_attn_noalloc"])
+def test_both_attention_entry_points_check_their_tensors_before_any_launch(lib, entry):
+    """one shared check in front of spinf_tree_attn_fwd and spinf_tree_attn_fwd_noalloc: a wrong dtype, shape, head grouping,
+    stride or row count raises ValueError on the host (the kernels index by these and would read out of bounds)"""
+    import torch
+
+    from spinf_serve_amd import attention
+
+    cfg = synth.attention_config("C1")
+    b = cfg.batches[0]
+    n, hq, hkv, d = b.length, cfg.hq, cfg.hkv, cfg.d
+    mask = sa.TreeMask.build(b.art, b.end, b.pos, device="cpu")
+
+    def call(q, k, v, out=None):
+        if entry == "tree_attn":
+            return sa.tree_attn(q, k, v, mask, cfg.scale)
+        return attention.tree_attn_noalloc(q, k, v, mask, torch.empty_like(q) if out is None else out, cfg.scale)
+
+    def z(rows, heads, dim, dtype=torch.bfloat16):
+        return torch.zeros((rows, heads, dim), dtype=dtype)
+
+    q, k = z(n, hq, d), z(n, hkv, d)
+    with pytest.raises(ValueError, match="bf16"):
+        call(z(n, hq, d, torch.float16), k, k)
+    with pytest.raises(ValueError, match="bf16"):
+        call(q, k, z(n, hkv, d, torch.float32))
+    with pytest.raises(ValueError, match="heads, head dim"):
+        call(q.reshape(n, hq * d), k, k)
+    with pytest.raises(ValueError, match="do not match"):
+        call(q, z(n - 1, hkv, d), k)
+    with pytest.raises(ValueError, match="do not match"):
+        call(q, k, z(n, hkv, d // 2))
+    with pytest.raises(ValueError, match="do not match"):
+        call(q, k, z(n, hkv + 1, d))
+    with pytest.raises(ValueError, match="do not group"):
+        call(z(n, 3, d), z(n, 2, d), z(n, 2, d))
+    with pytest.raises(ValueError, match="contiguous"):
+        call(z(n, hq, 2 * d)[:, :, ::2], k, k)
+    with pytest.raises(ValueError, match="mask describes"):
+        call(z(n + 64, hq, d), z(n + 64, hkv, d), z(n + 64, hkv, d))
+    with pytest.raises(TypeError, match="TreeMask"):
+        (sa.tree_attn if entry == "tree_attn" else attention.tree_attn_noalloc)(q, k, k, None, *(() if entry == "tree_attn" else (q,)))
+    if entry == "tree_attn_noalloc":
+        with pytest.raises(ValueError, match="out must be"):
+            call(q, k, k, out=z(n, hq, d, torch.float32))
+        with pytest.raises(ValueError, match="out must be"):
+            call(q, k, k, out=z(n + 1, hq, d))
+        with pytest.raises(ValueError, match="out must be"):
+            call(q, k, k, out=z(n, 2 * hq, d)[:, ::2])
+    with pytest.raises(RuntimeError, match="ROCm"):   # everything in order except the device: still no CPU path
+        call(q, k, k)
+
+
 # ------------------------------------------------------------------------------------------------ stream layout
 def _golden_trees(case):
     return [TokenTree(t["prefix"], t["branches"], list(t["parents"]), tuple(t["aligned"])) for t in case["trees"]]
