@@ -321,6 +321,13 @@ int spinf_diag_mfma_rate(int64_t iters, float* out, int64_t out_floats, double* 
  * same reads done one at a time.  out: 7 device ints, zeroed by the caller: [0..5] += mismatches per interleaving, [6] += workgroups
  * that ran.  Any nonzero count in [0..5] means out-of-order returns. */
 int spinf_diag_lds_order(int32_t iters, int32_t workgroups, int32_t* out, void* stream);
+/* Diagnostics (no counterpart in the reference): the wait states around an MFMA issued from inline assembly, which the compiler's
+ * hazard recogniser does not see.  out: 21 device ints, zeroed by the caller: [5 kind + g] += lanes with a wrong result for gap g
+ * of (0, 1, 2, 4, 8) instructions; kind 0: v_mov writes the B registers, gap, MFMA; kind 1: MFMA, gap, v_mov overwrites B; kind 2:
+ * v_exp_f32 -> v_cvt_pk_bf16_f32 writes B, gap, MFMA; kind 3: as 2 with, in place of the five gaps: one satisfied s_waitcnt
+ * lgkmcnt(0), two of them, a satisfied s_waitcnt vmcnt(0), v_nop, s_waitcnt + s_nop 0; [20] += workgroups (of eight waves) that
+ * ran.  out: 21 device ints. */
+int spinf_diag_mfma_hazard(int32_t iters, int32_t workgroups, int32_t* out, void* stream);
 
 #ifdef __cplusplus
 }

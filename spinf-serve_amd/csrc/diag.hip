@@ -146,7 +146,87 @@ __global__ __launch_bounds__(256) void lds_order_kernel(const int iters, int* ou
     if (threadIdx.x == 0) atomicAdd(&out[LDS_ORDER_PATTERNS], 1);   // workgroups that ran
 }
 
+// ---- what must lie between a VALU write of an MFMA's A / B registers and the MFMA, and between the MFMA and the next VALU write of
+// them?  The attention kernels issue their MFMAs from inline assembly (the accumulators live in registers the compiler must not see),
+// so the compiler's hazard recogniser does not know that those blocks read their operands as an MFMA does: whatever wait states
+// the hardware wants around them must come from the source.  Each case runs four MFMAs to have the matrix pipe busy, then the
+// sequence under test with GAP independent instructions (s_nop) in between, and counts lanes whose 16 results are not the expected
+// value.  KIND 0: v_mov writes B, then the MFMA reads it.  KIND 1: the MFMA reads B, then v_mov overwrites it.  KIND 2: as 0, but B
+// comes out of v_exp_f32 -> v_cvt_pk_bf16_f32, the chain the softmax feeds the P V product with.  KIND 3: as 2, with other things
+// in the gap: one satisfied s_waitcnt lgkmcnt(0), two of them, a satisfied s_waitcnt vmcnt(0), v_nop, s_waitcnt + s_nop 0.
+typedef __attribute__((ext_vector_type(16))) float diag_f32x16;
+constexpr int MFMA_HAZARD_GAPS = 5;     // 0, 1, 2, 4, 8 instructions
+constexpr int MFMA_HAZARD_KINDS = 4;
+
+#define SPINF_DIAG_FILL                                                                                                              \
+    "v_mov_b32 v20, %1\n\tv_mov_b32 v21, %1\n\tv_mov_b32 v22, %1\n\tv_mov_b32 v23, %1\n\t"                                           \
+    "v_mov_b32 v24, %1\n\tv_mov_b32 v25, %1\n\tv_mov_b32 v26, %1\n\tv_mov_b32 v27, %1\n\tv_mov_b32 v29, 1.0\n\ts_nop 7\n\t"          \
+    "v_mfma_f32_32x32x16_bf16 v[32:47], v[20:23], v[24:27], 0\n\tv_mfma_f32_32x32x16_bf16 v[48:63], v[20:23], v[24:27], 0\n\t"      \
+    "v_mfma_f32_32x32x16_bf16 v[64:79], v[20:23], v[24:27], 0\n\tv_mfma_f32_32x32x16_bf16 v[80:95], v[20:23], v[24:27], 0\n\t"
+#define SPINF_DIAG_CLOB                                                                                                              \
+    "v20", "v21", "v22", "v23", "v24", "v25", "v26", "v27", "v28", "v29", "v32", "v33", "v34", "v35", "v36", "v37", "v38", "v39", "v40", "v41", "v42",   \
+        "v43", "v44", "v45", "v46", "v47", "v48", "v49", "v50", "v51", "v52", "v53", "v54", "v55", "v56", "v57", "v58", "v59", "v60", "v61", "v62",     \
+        "v63", "v64", "v65", "v66", "v67", "v68", "v69", "v70", "v71", "v72", "v73", "v74", "v75", "v76", "v77", "v78", "v79", "v80", "v81", "v82",     \
+        "v83", "v84", "v85", "v86", "v87", "v88", "v89", "v90", "v91", "v92", "v93", "v94", "v95", "memory"
+#define SPINF_DIAG_WRITE_B "v_mov_b32 v24, %2\n\tv_mov_b32 v25, %2\n\tv_mov_b32 v26, %2\n\tv_mov_b32 v27, %2\n\t"
+#define SPINF_DIAG_CVT_B                                                                                                             \
+    "v_exp_f32 v28, v29\n\ts_nop 0\n\tv_cvt_pk_bf16_f32 v24, v28, v28\n\tv_cvt_pk_bf16_f32 v25, v28, v28\n\t"                        \
+    "v_cvt_pk_bf16_f32 v26, v28, v28\n\tv_cvt_pk_bf16_f32 v27, v28, v28\n\t"
+#define SPINF_DIAG_MFMA "v_mfma_f32_32x32x16_bf16 %0, v[20:23], v[24:27], 0\n\t"
+#define SPINF_DIAG_DRAIN "s_nop 15\n\ts_nop 15\n\t"
+
+template <int KIND>
+__device__ __forceinline__ int mfma_hazard_bad(const diag_f32x16 acc) {
+    const float want = KIND == 1 ? 16.f : 32.f;   // 16 products of 1 x 1, or of 1 x 2
+    bool bad = false;
+#pragma unroll
+    for (int i = 0; i < 16; i++) bad = bad || acc[i] != want;
+    return bad ? 1 : 0;
+}
+#define SPINF_DIAG_CASE(KIND, G, GAPTEXT)                                                                                            \
+    {                                                                                                                                \
+        diag_f32x16 acc;                                                                                                             \
+        if (KIND == 0) asm volatile(SPINF_DIAG_FILL SPINF_DIAG_WRITE_B GAPTEXT SPINF_DIAG_MFMA SPINF_DIAG_DRAIN : "=&v"(acc) : "v"(one2), "v"(two2) : SPINF_DIAG_CLOB);   \
+        if (KIND == 1) asm volatile(SPINF_DIAG_FILL SPINF_DIAG_MFMA GAPTEXT SPINF_DIAG_WRITE_B SPINF_DIAG_DRAIN : "=&v"(acc) : "v"(one2), "v"(two2) : SPINF_DIAG_CLOB);   \
+        if (KIND >= 2) asm volatile(SPINF_DIAG_FILL SPINF_DIAG_CVT_B GAPTEXT SPINF_DIAG_MFMA SPINF_DIAG_DRAIN : "=&v"(acc) : "v"(one2), "v"(two2) : SPINF_DIAG_CLOB);     \
+        bad[KIND * MFMA_HAZARD_GAPS + G] += mfma_hazard_bad<KIND>(acc);                                                              \
+    }
+#define SPINF_DIAG_KIND(KIND)                                                                                                        \
+    SPINF_DIAG_CASE(KIND, 0, "")                                                                                                     \
+    SPINF_DIAG_CASE(KIND, 1, "s_nop 0\n\t")                                                                                          \
+    SPINF_DIAG_CASE(KIND, 2, "s_nop 1\n\t")                                                                                          \
+    SPINF_DIAG_CASE(KIND, 3, "s_nop 3\n\t")                                                                                          \
+    SPINF_DIAG_CASE(KIND, 4, "s_nop 7\n\t")
+
+__global__ __launch_bounds__(512) void mfma_hazard_kernel(const int iters, int* out) {
+    const unsigned one2 = 0x3f803f80u, two2 = 0x40004000u;   // bf16 pairs of 1.0 and 2.0
+    int bad[MFMA_HAZARD_KINDS * MFMA_HAZARD_GAPS] = {};
+    for (int it = 0; it < iters; it++) {
+        SPINF_DIAG_KIND(0)
+        SPINF_DIAG_KIND(1)
+        SPINF_DIAG_KIND(2)
+        SPINF_DIAG_CASE(3, 0, "s_waitcnt lgkmcnt(0)\n\t")
+        SPINF_DIAG_CASE(3, 1, "s_waitcnt lgkmcnt(0)\n\ts_waitcnt lgkmcnt(0)\n\t")
+        SPINF_DIAG_CASE(3, 2, "s_waitcnt vmcnt(0)\n\t")
+        SPINF_DIAG_CASE(3, 3, "v_nop\n\t")
+        SPINF_DIAG_CASE(3, 4, "s_waitcnt lgkmcnt(0)\n\ts_nop 0\n\t")
+    }
+#pragma unroll
+    for (int v = 0; v < MFMA_HAZARD_KINDS * MFMA_HAZARD_GAPS; v++)
+        if (bad[v]) atomicAdd(&out[v], bad[v]);
+    if (threadIdx.x == 0) atomicAdd(&out[MFMA_HAZARD_KINDS * MFMA_HAZARD_GAPS], 1);
+}
+
 }  // namespace
+
+extern "C" int spinf_diag_mfma_hazard(int32_t iters, int32_t workgroups, int32_t* out, void* stream) {
+    if (iters <= 0 || iters > 100000 || workgroups <= 0 || workgroups > 65536 || !out)
+        return spinf_fail(SPINF_E_ARG, "diag_mfma_hazard: iters in 1 .. 100,000, workgroups in 1 .. 65,536, out not null");
+    hipLaunchKernelGGL(mfma_hazard_kernel, dim3(workgroups), dim3(512), 0, (hipStream_t)stream, (int)iters, (int*)out);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "diag_mfma_hazard: launch: %s", hipGetErrorString(e));
+    return SPINF_OK;
+}
 
 extern "C" int spinf_diag_lds_order(int32_t iters, int32_t workgroups, int32_t* out, void* stream) {
     if (iters <= 0 || iters > 100000 || workgroups <= 0 || workgroups > 65536 || !out)

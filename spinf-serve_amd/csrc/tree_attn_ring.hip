@@ -355,8 +355,12 @@ __device__ __forceinline__ void ring_paced_pass(const AttnParams& p, char* const
             const int ln = fresh_lane_id();
             const char* krow = ring + G::K::k_off(ln & 31) + 16 * (ln >> 5);
             const char* vrow = ring + G::KTILEB + G::V::v_off(4 * (ln >> 5) + ((ln >> 2) & 3)) + 32 * ((ln >> 4) & 1) + 8 * (ln & 3);
-            // (the scheduling barriers keep the three kinds of LDS reads apart, and every read of one kind has returned before the
-            // first of the next kind is issued: the MFMAs are assembly, so nothing else orders the loads that feed them)
+            // (the scheduling barriers keep the phases apart.  The MFMAs are assembly, which the compiler's hazard recogniser does
+            // not look into: left to interleave the softmax of the block's second half with the P V products of the first, it
+            // put the conversion that writes a P fragment directly in front of the MFMA that reads it, and an MFMA that issues in
+            // the cycle after a vector write of its A / B registers reads the old values (spinf_diag_mfma_hazard measures it).
+            // With the phases apart, V fragment reads lie between the conversions and the first MFMA; the build scans the
+            // generated assembly for the pattern.)
             f32x16 sa;
             __builtin_amdgcn_sched_barrier(0);
             auto score = [&](auto x_c) __attribute__((always_inline)) {
@@ -423,7 +427,7 @@ __device__ __forceinline__ void ring_paced_pass(const AttnParams& p, char* const
                 l += sum;
                 viol = viol | !(sum <= VIOL_SUM);
             }
-            __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): no 16-byte read in flight when the transposing reads begin
+            __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): the softmax phase ends here, the waits below are for V fragments only
             __builtin_amdgcn_sched_barrier(0);
             auto step = [&](auto f_c) __attribute__((always_inline)) {
                 constexpr int f = decltype(f_c)::value;
@@ -825,8 +829,10 @@ __global__ __launch_bounds__(D == 512 ? 256 : 512) void tree_attn_ring_kernel(co
                 i32x4 nx = {0, 0, 0, 0};
                 int fv = -1;
                 const bool pf_ok = j + 1 < ntiles && j + 1 < gen_seen;
-                // (requested before the first transposing read of V: mixed in among them, a 16-byte read gave the MFMAs stale
-                // fragments, as if the two kinds of reads did not return in the order they were issued)
+                // (requested before the first transposing read of V, so that every wait inside the MFMA sequence is for V
+                // fragments alone and stalls: a wait that is already satisfied takes no time, and then a vector write of an
+                // operand could end up in the issue cycle before the assembly MFMA that reads it; LDS reads of different kinds
+                // do return in issue order, spinf_diag_lds_order checks it)
                 if (pf_ok) {
                     dv = desc[(j + 1) & (NDESC - 1)];
                     nx = lds_peek4(sy_done);
@@ -936,8 +942,8 @@ __global__ __launch_bounds__(D == 512 ? 256 : 512) void tree_attn_ring_kernel(co
             const int ln = fresh_lane_id();
             const char* krow = ring + G::K::k_off(ln & 31) + 16 * (ln >> 5);
             const char* vrow = ring + G::KTILEB + G::V::v_off(4 * (ln >> 5) + ((ln >> 2) & 3)) + 32 * ((ln >> 4) & 1) + 8 * (ln & 3);
-            // (the scheduling barriers keep the three kinds of LDS reads apart: the transposing reads of V and the 16-byte reads
-            // of K and of the keys' metadata do not complete in the order they were issued, which the compiler's counting assumes)
+            // (the scheduling barriers keep the phases apart, as in ring_paced_pass: no vector write of a P fragment directly in
+            // front of the assembly MFMA that reads it)
             f32x16 sa;
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -982,7 +988,7 @@ __global__ __launch_bounds__(D == 512 ? 256 : 512) void tree_attn_ring_kernel(co
                 }
                 l += sum;
             }
-            __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): no 16-byte read in flight when the transposing reads begin
+            __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): the softmax phase ends here, the waits below are for V fragments only
             __builtin_amdgcn_sched_barrier(0);
             auto step = [&](auto f_c) __attribute__((always_inline)) {
                 constexpr int f = decltype(f_c)::value;

@@ -22,3 +22,25 @@ def test_lds_reads_of_mixed_kinds_return_in_issue_order(dev, lib):
     got = out.cpu().tolist()
     assert got[6] == wgs, got
     assert got[:6] == [0] * 6, f"LDS reads returned out of order: mismatches per interleaving {got[:6]} of {wgs * 256 * iters * 8} reads each"
+
+
+def test_an_mfma_needs_one_instruction_after_a_vector_write_of_its_operands(dev, lib):
+    """The ring kernel issues its MFMAs from inline assembly, where the compiler's hazard recogniser does not look, so the gap
+    the hardware wants between a vector write of an MFMA's A / B registers and the MFMA must come from the source (the build
+    scans the generated assembly for it).  Measured here: with the MFMA in the very next issue cycle it multiplies the
+    registers' OLD contents (v_mov as well as v_exp -> v_cvt_pk writers); with one instruction or more in between, or with
+    the write behind the MFMA, every product is right."""
+    out = torch.zeros(21, dtype=torch.int32, device=dev)
+    wgs, iters = 1024, 20
+    _lib.check(lib.spinf_diag_mfma_hazard(iters, wgs, out.data_ptr(), C.c_void_p(torch.cuda.current_stream().cuda_stream)), "spinf_diag_mfma_hazard")
+    torch.cuda.synchronize()
+    got = out.cpu().tolist()
+    lanes = wgs * 512 * iters
+    assert got[20] == wgs, got
+    write_then_mfma, mfma_then_write, cvt_then_mfma, other_gaps = got[0:5], got[5:10], got[10:15], got[15:20]
+    print(f"lanes with wrong products of {lanes} per case, gaps of 0 1 2 4 8 instructions: v_mov -> MFMA {write_then_mfma}, MFMA -> v_mov "
+          f"{mfma_then_write}, v_exp -> v_cvt_pk -> MFMA {cvt_then_mfma}; s_waitcnt x1, x2, vmcnt, v_nop, s_waitcnt + s_nop in the gap {other_gaps}")
+    assert write_then_mfma[1:] == [0] * 4 and cvt_then_mfma[1:] == [0] * 4, got
+    assert mfma_then_write == [0] * 5, got
+    assert other_gaps[3:] == [0] * 2, got
+    assert write_then_mfma[0] > 0 and cvt_then_mfma[0] > 0, f"no wrong product without a gap any more: {got} (the assembly scan of the build could go)"
