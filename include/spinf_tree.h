@@ -131,7 +131,7 @@ int spinf_tree_attn_fwd(const spinf_attn_args* args, void* stream);
 /* The same pass with nothing allocated.  No counterpart in the reference: it is for callers that cannot call hipMalloc (code
  * under HIP graph capture, tight serving loops, harnesses that forbid allocation).  spinf_tree_attn_fwd keeps its list cursors,
  * counts and redo list in a buffer that the library allocates (and regrows) on the device; this entry point keeps them in a
- * file-scope device array of 64 + 65,536 ints (256.25 KiB per GPU, held until the process ends) and calls no hipMalloc /
+ * file-scope device array of 64 + 65,536 + 4,096 ints (272.25 KiB per GPU, held until the process ends) and calls no hipMalloc /
  * hipFree nor any allocating routine.  Same arguments, same kernels, same results bit for bit.  Limit: n_items (query tiles x
  * head groups) <= 65,536, more is SPINF_E_ARG.  The cursors and counts are cleared by a small kernel in front of every pass that
  * uses them (the kernel with decoupled waves uses none: such a call is one launch), so a call does not depend on what the
@@ -246,8 +246,9 @@ int spinf_lm_logprobs(const spinf_lm_args* args, void* stream);
 /* The whole read-out in one pass: replaces the row gather Hf[sel], the chunked logits GEMM, the soft-capping, the log-softmax and
  * the column selection of Scorer._forward / Scorer._logprobs (spinf_serve/scorer.py:247-261 and :340-355).  The logits matrix is
  * never stored: out[r, c] = log_softmax(cap(h[sel[r]] . W^T))[cols[c]], or the whole row with cols == NULL (scorer.py:260).
- *   h [*, h_ld >= hidden] bf16: the final hidden states (after the final norm); sel [rows] int64 device: their rows to read,
- *   NULL = rows 0 .. rows-1; w [vocab, w_ld >= hidden] bf16: the lm head's weight (nn.Linear layout); hidden a multiple of 64;
+ *   h [h_rows, h_ld >= hidden] bf16: the final hidden states (after the final norm); sel [rows] int64 device: their rows to read,
+ *   each in -h_rows .. h_rows-1 (a negative entry counts from the end, as the reference's tensor indexing Hf[sel] does; any other
+ *   entry reads nothing outside h and gives a row of NaN), NULL = rows 0 .. rows-1 (rows <= h_rows); w [vocab, w_ld >= hidden] bf16: the lm head's weight (nn.Linear layout); hidden a multiple of 64;
  *   rows of h and w 16-byte aligned.
  *   logits_dtype 0: the logits stay fp32 (the reference's "f32out" and "fp32" modes, scorer.py:345-348); 1: they are rounded to
  *   bf16 and soft-capped in bf16 steps, as `h @ W.t()` on bf16 tensors gives them (scorer.py:349-352).
@@ -265,6 +266,7 @@ typedef struct spinf_lm_head_args {
     const int64_t* cols; int64_t n_cols;
     float* out; int64_t out_ld;
     void* workspace; int64_t workspace_bytes;
+    int64_t h_rows;                          /* rows of h (> 0): what sel is checked against */
 } spinf_lm_head_args;
 int spinf_lm_head_workspace(const spinf_lm_head_args* args, int64_t* bytes);
 int spinf_lm_head_fwd(const spinf_lm_head_args* args, void* stream);

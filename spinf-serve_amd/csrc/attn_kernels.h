@@ -8,7 +8,7 @@
 #include "attn_tiles.h"
 
 constexpr int NLIST = 8;       // work lists (XCDs of an MI355X)
-constexpr int LAND_CAP = 65536; // most item lists of a static schedule (the landing words of the ring kernel)
+constexpr int LAND_CAP = 4096;  // most item lists of a static schedule (one landing word of the ring kernel each; a schedule has one list per compute unit)
 constexpr int ENT_CAP = 256;   // plan entries of a query tile kept in LDS at a time
 
 struct AttnParams {

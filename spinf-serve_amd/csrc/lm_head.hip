@@ -35,7 +35,7 @@ constexpr float LOG2E = 1.4426950408889634f;
 
 struct HeadParams {
     const __bf16* h; long h_ld;
-    const long* sel; int rows;
+    const long* sel; int rows; long h_rows;
     const __bf16* w; long w_ld;
     int vocab, hidden;
     float cap, inv_cap;
@@ -81,7 +81,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     for (int i = 0; i < 8; i++) {
         const int row = (tid >> 3) + 32 * i;
         const int rr = r0 + row < p.rows ? r0 + row : p.rows - 1;
-        row_h[i] = p.sel ? (int)p.sel[rr] : rr;
+        long hr = p.sel ? p.sel[rr] : rr;           // an entry of the row list counts from the end when negative, as tensor indexing does
+        hr = hr < 0 ? hr + p.h_rows : hr;
+        row_h[i] = hr >= 0 && hr < p.h_rows ? (int)hr : 0;   // (an entry outside h reads row 0; the finishing kernel turns its row into NaN)
     }
     // The row list's loads end here: a value that still counts as "in flight" when the loop is entered makes the compiler wait
     // for it at every use, and such a wait also waits for every tile load issued before it.
@@ -300,8 +302,10 @@ __global__ __launch_bounds__(256) void lm_head_finish_kernel(const HeadParams p)
     const float lse = m + logf(s);
     float* out = p.out + (long)row * p.out_ld;
     const int n = p.cols ? p.n_cols : p.vocab;
+    const long hr = p.sel ? p.sel[row] : row;
+    const bool row_known = hr >= -p.h_rows && hr < p.h_rows;   // a row list entry that names no row of h
     for (int i = threadIdx.x; i < n; i += 256) {
-        const bool known = !p.cols || (p.cols[i] >= 0 && p.cols[i] < p.vocab);   // no tile wrote a column outside the vocabulary
+        const bool known = row_known && (!p.cols || (p.cols[i] >= 0 && p.cols[i] < p.vocab));   // no tile wrote a column outside the vocabulary
         out[i] = known ? out[i] - lse : __builtin_nanf("");
     }
 }
@@ -314,6 +318,9 @@ int check(const spinf_lm_head_args* a) {
     if (a->softcap < 0.f || a->softcap > 40.f) return spinf_fail(SPINF_E_ARG, "lm_head: softcap %g outside 0 .. 40", (double)a->softcap);
     if (a->logits_dtype != 0 && a->logits_dtype != 1) return spinf_fail(SPINF_E_ARG, "lm_head: logits_dtype %d (0 = fp32, 1 = bf16)", a->logits_dtype);
     if ((a->cols == nullptr) != (a->n_cols == 0) || a->n_cols < 0) return spinf_fail(SPINF_E_ARG, "lm_head: cols and n_cols come together");
+    if (a->h_rows < 0 || a->h_rows > (1ll << 31) - 1 || (a->rows > 0 && a->h_rows == 0))
+        return spinf_fail(SPINF_E_ARG, "lm_head: h_rows %lld (the rows of h) out of range", (long long)a->h_rows);
+    if (!a->sel && a->rows > a->h_rows) return spinf_fail(SPINF_E_ARG, "lm_head: %lld rows to read without a row list, h has %lld", (long long)a->rows, (long long)a->h_rows);
     return SPINF_OK;
 }
 
@@ -339,7 +346,7 @@ extern "C" int spinf_lm_head_fwd(const spinf_lm_head_args* a, void* stream) {
         return spinf_fail(SPINF_E_ARG, "lm_head: workspace of %lld bytes, %lld needed (spinf_lm_head_workspace)", (long long)a->workspace_bytes,
                           (long long)(a->rows * parts_of(a) * (int64_t)sizeof(float2)));
     HeadParams p;
-    p.h = (const __bf16*)a->h; p.h_ld = a->h_ld; p.sel = a->sel; p.rows = (int)a->rows;
+    p.h = (const __bf16*)a->h; p.h_ld = a->h_ld; p.sel = a->sel; p.rows = (int)a->rows; p.h_rows = a->h_rows;
     p.w = (const __bf16*)a->w; p.w_ld = a->w_ld; p.vocab = (int)a->vocab; p.hidden = (int)a->hidden;
     p.cap = a->softcap; p.inv_cap = a->softcap > 0.f ? 1.0f / a->softcap : 0.f;
     p.cols = a->cols; p.n_cols = (int)a->n_cols; p.out = a->out; p.out_ld = a->out_ld;

@@ -556,7 +556,7 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
 // Scratch memory of the entry point that allocates nothing (spinf_tree_attn_fwd_noalloc): list cursors, counts and the redo
 // list.  In host code this name is a stand-in, not a device address: hipGetSymbolAddress gives the address, per device.
 constexpr long NOALLOC_MAX_ITEMS = 1 << 16;                            // work items (query tiles x head groups) of one call
-// 64 cursors and counts | the redo list | the ring kernel's landing words (one per item list): 512.25 KiB per GPU, held until the process ends
+// 64 cursors and counts | the redo list | the ring kernel's landing words (one per item list): 272.25 KiB per GPU, held until the process ends
 static __device__ __align__(256) int scratch[64 + NOALLOC_MAX_ITEMS + LAND_CAP];
 
 namespace {
@@ -565,13 +565,15 @@ namespace {
 // stream it was first used on: calls on one stream follow each other in stream order and share it, calls on different streams
 // (or from host threads that use different streams) never share cursors, and no event or query is needed to tell when a block is
 // free.  Blocks are never freed before the process ends: a bigger schedule gets a new block for its stream, and a launch
-// recorded into a graph keeps the block it was recorded with for good (replays may run at any time).
+// recorded into a graph keeps the block it was recorded with for good (replays may run at any time): the calls that ONE capture
+// records on a stream share that block (the graph runs them in the order they were recorded), no other call gets it again.
 struct CursorBlock {
     int* ptr = nullptr;
     long cap = 0;               // redo entries
     hipStream_t owner = nullptr;
     bool taken = false;         // between acquire and release on some host thread
-    bool pinned = false;        // recorded into a graph
+    bool pinned = false;        // recorded into a graph ...
+    unsigned long long capture = 0;   // ... by the capture with this id
     bool dirty = false;         // a call on it failed to get all its kernels onto the stream: clear it before the next use
 };
 struct DeviceState {
@@ -599,17 +601,20 @@ int device_cus(int* cus) {
 }
 
 // -> the stream's block with room for n_items redo entries; *slot names it for release_block
-int acquire_block(long n_items, bool capturing, hipStream_t stream, int** ptr, int* slot, bool* dirty, long* cap) {
+int acquire_block(long n_items, bool capturing, unsigned long long capture, hipStream_t stream, int** ptr, int* slot, bool* dirty, long* cap) {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess || dev < 0 || dev >= 64) return spinf_fail(SPINF_E_HIP, "tree_attn: hipGetDevice: %s", hipGetErrorString(e));
     std::lock_guard<std::mutex> lock(g_mu);
     DeviceState& s = g_dev[dev];
+    for (int pass = 0; pass < 2; pass++)   // a capture's later calls take the block its first call pinned, before a fresh one
     for (size_t i = 0; i < s.blocks.size(); i++) {
         CursorBlock& b = s.blocks[i];
-        if (b.taken || b.pinned || b.owner != stream || b.cap < n_items) continue;
+        if (b.taken || b.owner != stream || b.cap < n_items) continue;
+        if (pass == 0 ? !(capturing && b.pinned && b.capture == capture) : b.pinned) continue;
         b.taken = true;
         b.pinned = capturing;
+        b.capture = capturing ? capture : 0;
         *ptr = b.ptr;
         *slot = (int)i;
         *dirty = b.dirty;
@@ -617,8 +622,9 @@ int acquire_block(long n_items, bool capturing, hipStream_t stream, int** ptr, i
         return SPINF_OK;
     }
     if (capturing)
-        return spinf_fail(SPINF_E_ARG, "tree_attn: this stream has no cursor block of this size yet and none can be allocated during capture: "
-                                       "run one call of this size on the stream before the capture, or record spinf_tree_attn_fwd_noalloc");
+        return spinf_fail(SPINF_E_ARG, "tree_attn: this stream has no free cursor block of this size (a block recorded into an earlier graph stays with that "
+                                       "graph) and none can be allocated during capture: run one call of this size on the stream before the capture, or "
+                                       "record spinf_tree_attn_fwd_noalloc");
     if (s.blocks.size() >= MAX_CURSOR_BLOCKS) return spinf_fail(SPINF_E_NOMEM, "tree_attn: %zu cursor blocks on one device (one per stream in use)", s.blocks.size());
     CursorBlock b;
     b.cap = n_items < (1 << 16) ? (1 << 16) : 2 * n_items;
@@ -834,7 +840,7 @@ static int attn_fwd(const spinf_attn_args* a, void* stream, bool no_alloc) {
     pick_kernel(a->hq, a->hkv, a->d, a->variant, &rt, &nhw);
     if ((a->row_of != nullptr) != (a->kv_row0 != nullptr)) return spinf_fail(SPINF_E_ARG, "tree_attn: row_of and kv_row0 come together");
     if (a->row_of && rt != 1) return spinf_fail(SPINF_E_ARG, "tree_attn: variant %d does not take compact rows", a->variant);
-    if (a->n_lists < 0 || a->n_lists > 65536) return spinf_fail(SPINF_E_ARG, "tree_attn: %d item lists, at most 65,536", a->n_lists);
+    if (a->n_lists < 0 || a->n_lists > LAND_CAP) return spinf_fail(SPINF_E_ARG, "tree_attn: %d item lists, at most %d", a->n_lists, LAND_CAP);
     const bool ring = a->n_lists > 0 && a->ktile == 32;   // static schedule over 32-key entries: the ring kernel
     if (ring) {
         if (!((a->d == 256 && nhw == 2 && rt == 1) || a->d == 512) || a->row_of || a->grp)
@@ -869,10 +875,11 @@ static int attn_fwd(const spinf_attn_args* a, void* stream, bool no_alloc) {
         cus = st->cus;
     } else {
         hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
-        if (hipStreamIsCapturing(s, &cs) != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: hipStreamIsCapturing failed");
+        unsigned long long capture = 0;
+        if (hipStreamGetCaptureInfo(s, &cs, &capture) != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: hipStreamGetCaptureInfo failed");
         capturing = cs != hipStreamCaptureStatusNone;
         if (int rc = device_cus(&cus)) return rc;
-        if (int rc = acquire_block((long)a->n_items, capturing, s, &counters, &slot, &dirty, &redo_cap)) return rc;
+        if (int rc = acquire_block((long)a->n_items, capturing, capture, s, &counters, &slot, &dirty, &redo_cap)) return rc;
     }
     AttnParams p;
     // A block's cursors are zero: it was cleared when allocated, and every call's exact-pass kernel, which runs after the fast pass,

@@ -63,6 +63,7 @@ class LmHeadArgs(C.Structure):
         ("cols", C.c_void_p), ("n_cols", C.c_int64),
         ("out", C.c_void_p), ("out_ld", C.c_int64),
         ("workspace", C.c_void_p), ("workspace_bytes", C.c_int64),
+        ("h_rows", C.c_int64),
     ]
 
 

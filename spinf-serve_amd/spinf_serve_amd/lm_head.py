@@ -76,7 +76,7 @@ def _head_op(h: torch.Tensor, sel: Optional[torch.Tensor], w: torch.Tensor, cols
     rows, vocab = (h.shape[0] if sel is None else sel.numel()), w.shape[0]
     out = torch.empty((rows, vocab if cols is None else cols.numel()), dtype=torch.float32, device=h.device)
     a = _lib.LmHeadArgs()
-    a.h, a.h_ld, a.rows = h.data_ptr(), h.stride(0), rows
+    a.h, a.h_ld, a.rows, a.h_rows = h.data_ptr(), h.stride(0), rows, h.shape[0]
     a.sel = sel.data_ptr() if sel is not None else None
     a.w, a.w_ld, a.vocab, a.hidden = w.data_ptr(), w.stride(0), vocab, h.shape[1]
     a.softcap, a.logits_dtype = softcap, int(bf16_logits)
@@ -103,8 +103,9 @@ def lm_head_logprobs(h, sel, w, cols=None, softcap=None, logits="fp32"):
     """h [*, hidden] bf16 (the final hidden states), sel int64 device vector of the rows to read (None: all), w [vocab, hidden] bf16
     -> log_softmax(softcap * tanh(h[sel] @ w.T / softcap)) fp32, the columns ``cols`` of it or with cols None all of it.
     logits "fp32": the logits keep their fp32 accumulators (the reference's "f32out" / "fp32" modes); "bf16": rounded to bf16 and
-    capped in bf16 steps, as the reference's `h @ W.t()` on bf16 tensors.  A negative column counts from the end, as in torch
-    indexing; a column outside the vocabulary gives NaN."""
+    capped in bf16 steps, as the reference's `h @ W.t()` on bf16 tensors.  A negative column or row of ``sel`` counts from the end,
+    as in torch indexing; a column outside the vocabulary gives NaN, an entry of ``sel`` outside h a whole row of NaN (where
+    torch's indexing would raise: the list is a device tensor, and checking it on the host would cost a synchronisation)."""
     if logits not in ("fp32", "bf16"):
         raise ValueError(f"logits mode {logits!r}")
     if cols is not None:

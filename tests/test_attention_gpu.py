@@ -650,6 +650,54 @@ def test_allocating_entry_point_under_graph_capture(dev):
     torch.cuda.synchronize()
 
 
+@pytest.mark.parametrize("ring", [0, 1])
+def test_several_calls_recorded_by_one_capture_share_the_streams_block(dev, ring, monkeypatch):
+    """a layer stack records one attention call per layer into one graph: the calls of ONE capture on a stream share the stream's
+    cursor block (the graph runs them in recorded order); a second graph on the same stream needs a block of its own, which an
+    eager call between the captures provides.  Both kernels (lockstep with its cursors, decoupled with its redo list)."""
+    from spinf_serve_amd import attention
+
+    monkeypatch.setattr(attention, "RING", ring)
+    cfg = synth.attention_config("C2", contents=3)
+    b = cfg.batches[0]
+    q, k, v = synth.qkv(cfg, b, seed=13, device=dev)
+    q2 = (q.float() * 0.5 + 0.25).to(torch.bfloat16)
+    mask = sa.TreeMask.build(b.art, b.end, b.pos, device=dev)
+    want1, want2 = sa.tree_attn(q, k, v, mask, cfg.scale), sa.tree_attn(q2, k, v, mask, cfg.scale)
+    torch.cuda.synchronize()
+    s = torch.cuda.Stream(device=dev)
+    with torch.cuda.stream(s):
+        sa.tree_attn(q, k, v, mask, cfg.scale)
+    s.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=s):
+        out1 = sa.tree_attn(q, k, v, mask, cfg.scale)
+        out2 = sa.tree_attn(q2, k, v, mask, cfg.scale)
+        out3 = sa.tree_attn(out2, k, v, mask, cfg.scale)   # a call that depends on the one before it
+    want3 = sa.tree_attn(want2, k, v, mask, cfg.scale)
+    for rep in range(3):
+        for o in (out1, out2, out3):
+            o.zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out1, want1) and torch.equal(out2, want2) and torch.equal(out3, want3), rep
+    g2 = torch.cuda.CUDAGraph()
+    with pytest.raises(ValueError, match="stays with that graph"):   # the stream's only block went with the first graph
+        with torch.cuda.graph(g2, stream=s):
+            sa.tree_attn(q, k, v, mask, cfg.scale)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(s):
+        sa.tree_attn(q, k, v, mask, cfg.scale)   # takes a new block for the stream
+    s.synchronize()
+    g3 = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g3, stream=s):
+        out4 = sa.tree_attn(q2, k, v, mask, cfg.scale)
+    g3.replay()
+    g.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(out4, want2) and torch.equal(out1, want1) and torch.equal(out3, want3)
+
+
 @pytest.mark.parametrize("d,limit,wide", [(256, 1, False), (256, 1, True), (256, 3, False), (512, 1, False), (512, 1, True)])
 def test_a_wave_that_gives_up_a_wait_costs_time_not_rows(dev, d, limit, wide, monkeypatch):
     """the decoupled kernel's landing: the waves are told (from the host, spinf_attn_args.debug_expire) to give up a wait after

@@ -13,7 +13,8 @@ from oracle import gdn as ogdn
 from spinf_serve_amd import synth
 
 pytestmark = pytest.mark.gpu
-TOL = 2e-2
+TOL = 2e-2       # attention: bf16 outputs of up to ~4 in size against float64
+GDN_TOL = 2e-3   # the delta-rule scan: outputs of unit scale (measured 3e-4)
 
 
 def _np(t):
@@ -48,7 +49,7 @@ def test_c2_full_pack_is_invariant_and_matches_the_oracle(dev):
     real = one.art[:n] >= 0
     err = float(np.abs(_np(out[s0 : s0 + n])[real] - want[real]).max())
     print(f"C2 full pack, content 5: max abs err {err:.3e}", flush=True)
-    assert err <= TOL
+    assert err <= TOL, f"C2 full pack, content 5: max abs error {err:.3e} against the float64 oracle, tolerance {TOL:.0e}"
 
 
 def test_c5_full_stream_properties(dev):
@@ -80,7 +81,7 @@ def test_c5_full_stream_properties(dev):
             want = ogdn.tree_scan(*(_np(z(t[x])) for x in ("q", "k", "v", "g", "beta")), one.batch.prev, one.batch.art >= 0)
             err = float(np.abs(_np(alone) - want).max())
             print(f"C5 full stream, content 77: max abs err {err:.3e}", flush=True)
-            assert err <= TOL
+            assert err <= GDN_TOL, f"C5 full stream, content 77: max abs error {err:.3e} against the float64 recurrence, tolerance {GDN_TOL:.0e}"
 
 
 def _device_qkv(cfg, n, dev, seed):
@@ -124,8 +125,9 @@ def _check_pack(cfg, b, trees, slots, oracle_slot, oracle_heads, window, dev, se
                                 pos=one.pos[:n], window=window, scale=cfg.scale)
     real = one.art[:n] >= 0
     err = float(np.abs(_np(out[s0 : s0 + n, :oracle_heads])[real] - want[real]).max())
-    print(f"{cfg.name} pack of {b.length} tokens, window {window}, content {oracle_slot} ({n} tokens, {oracle_heads} heads): max abs err {err:.3e}", flush=True)
-    assert err <= TOL
+    what = f"{cfg.name} pack of {b.length} tokens, window {window}, content {oracle_slot} ({n} tokens, {oracle_heads} heads)"
+    print(f"{what}: max abs err {err:.3e}", flush=True)
+    assert err <= TOL, f"{what}: max abs error {err:.3e} against the float64 oracle, tolerance {TOL:.0e}"
 
 
 @pytest.mark.parametrize("window", [None, 1024])

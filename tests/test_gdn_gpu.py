@@ -1,7 +1,8 @@
 """GPU parity of the Gated DeltaNet kernels (through the C ABI) against the float64 recurrence of the oracle
-(spinf_serve/models/qwen35/gdn.py:176-186).  Tolerance: 2e-2 max abs on outputs of unit scale (bf16 inputs and bf16 MFMA
-operands with fp32 accumulation; the reference quotes 4.9e-4 for its own fork identity in bf16, docs/QWEN.md:51-52, measured
-values are printed)."""
+(spinf_serve/models/qwen35/gdn.py:176-186).  Tolerances, max abs: 2e-3 on the outputs (unit scale; bf16 inputs and bf16 MFMA
+operands with fp32 accumulation, bf16 outputs: measured 2.1e-4 .. 3.8e-4; the reference quotes 4.9e-4 for its own fork identity
+in bf16, docs/QWEN.md:51-52) and 5e-3 on the final states (fp32, sums over up to 200 tokens: measured 1.6e-3 .. 2.2e-3).  Every
+assertion carries the measured value, and the file's last test prints the largest ones."""
 
 import numpy as np
 import pytest
@@ -12,12 +13,24 @@ from oracle import gdn as ogdn
 from spinf_serve_amd import synth
 
 pytestmark = pytest.mark.gpu
-TOL = 2e-2
-STATE_TOL = 2e-2
+TOL = 2e-3
+STATE_TOL = 5e-3
 
 
 def _np(t):
     return t.float().cpu().numpy()
+
+
+WORST = {"out": 0.0, "state": 0.0}
+
+
+def _within(got, want, tol, what):
+    """max abs error of a device tensor against the oracle's array, with the measured value in the failure message"""
+    err = float(np.abs(_np(got) - want).max()) if want.size else 0.0
+    key = "state" if tol is STATE_TOL else "out"
+    WORST[key] = max(WORST[key], err)
+    assert err <= tol, f"{what}: max abs error {err:.3e} against the float64 recurrence, tolerance {tol:.0e}"
+    return err
 
 
 def _inputs(T, H, HV, dev, seed=0, K=128, V=128):
@@ -50,10 +63,9 @@ def test_flat_segments_match_recurrence(dev, mode, lens):
     for s in range(n):
         a, b = int(cu_cpu[s]), int(cu_cpu[s + 1])
         want, S = ogdn.recurrent(*(_np(t[x][a:b]) for x in ("q", "k", "v", "g", "beta")), h0=_np(h0[s]) if s % 2 == 0 else None)
-        worst = max(worst, float(np.abs(_np(o[0, a:b]) - want).max()) if b > a else 0.0)   # (an empty segment only hands its state on)
-        worst_s = max(worst_s, float(np.abs(_np(ht[s]) - S).max()))
+        worst = max(worst, _within(o[0, a:b], want, TOL, f"{mode} lens={lens} segment {s}"))   # (an empty segment only hands its state on)
+        worst_s = max(worst_s, _within(ht[s], S, STATE_TOL, f"{mode} lens={lens} state {s}"))
     print(f"  max abs err o={worst:.3e} state={worst_s:.3e}", flush=True)
-    assert worst <= TOL and worst_s <= STATE_TOL
 
 
 def test_rows_by_index_and_skipped_states(dev):
@@ -80,7 +92,7 @@ def test_rows_by_index_and_skipped_states(dev):
         for a, b in ((0, 90), (90, 110)):
             r = rows[a:b]
             want, _ = ogdn.recurrent(*(_np(t[x][r]) for x in ("q", "k", "v", "g", "beta")))
-            assert np.abs(_np(o[0, r]) - want).max() <= TOL, mode
+            _within(o[0, r], want, TOL, f"{mode} rows {a}..{b}")
 
 
 @pytest.mark.parametrize("mode", ["recurrent", "chunked"])
@@ -108,9 +120,9 @@ def test_segments_forked_from_one_state(dev, mode):
     for s in range(n):
         a, b = int(cu_cpu[s]), int(cu_cpu[s + 1])
         want, S = ogdn.recurrent(*(_np(t[x][a:b]) for x in ("q", "k", "v", "g", "beta")), h0=_np(h0[src[s]]) if src[s] >= 0 else None)
-        assert float(np.abs(_np(o[0, a:b]) - want).max()) <= TOL, s
+        _within(o[0, a:b], want, TOL, f"{mode} segment {s}")
         if s in kept:
-            assert float(np.abs(_np(ht[s]) - S).max()) <= STATE_TOL, s
+            _within(ht[s], S, STATE_TOL, f"{mode} state {s}")
         else:
             assert torch.isnan(ht[s]).all(), s
 
@@ -134,9 +146,9 @@ def test_recurrent_other_value_dims(dev, V):
     for s in range(n):
         a, b = int(cu_cpu[s]), int(cu_cpu[s + 1])
         want, S = ogdn.recurrent(*(_np(t[x][a:b]) for x in ("q", "k", "v", "g", "beta")), h0=_np(h0[s]) if int(h0_idx[s]) >= 0 else None)
-        assert float(np.abs(_np(o[0, a:b]) - want).max()) <= TOL, s
+        _within(o[0, a:b], want, TOL, f"value dim {V} segment {s}")
         if int(ht_idx[s]) >= 0:
-            assert float(np.abs(_np(ht[s]) - S).max()) <= STATE_TOL, s
+            _within(ht[s], S, STATE_TOL, f"value dim {V} state {s}")
         else:
             assert torch.isnan(ht[s]).all(), s
 
@@ -151,13 +163,12 @@ def test_tree_scan_forks_from_trunk_state(dev):
     torch.cuda.synchronize()
     b = cfg.batch
     want = ogdn.tree_scan(*(_np(t[x]) for x in ("q", "k", "v", "g", "beta")), b.prev, b.art >= 0)
-    err = float(np.abs(_np(o) - want).max())
+    err = _within(o, want, TOL, "C5 x2 contents")
     print(f"C5 x2 contents: max abs err {err:.3e}", flush=True)
-    assert err <= TOL
     assert (o[torch.from_numpy(b.art < 0).to(dev)] == 0).all()
     # the short-segment threshold only picks the kernel: a plan that runs everything chunked agrees
     o2 = sa.gdn_tree(t["q"], t["k"], t["v"], t["g"], t["beta"], cfg.plan(dev, short=4))
-    assert float(np.abs(_np(o2) - want).max()) <= TOL
+    _within(o2, want, TOL, "C5 x2 contents, all chunked")
 
 
 def test_deep_trie(dev):
@@ -177,7 +188,7 @@ def test_deep_trie(dev):
     t = synth.gdn_inputs(cfg, seed=2, device=dev)
     o = sa.gdn_tree(t["q"], t["k"], t["v"], t["g"], t["beta"], cfg.plan(dev))
     want = ogdn.tree_scan(*(_np(t[x]) for x in ("q", "k", "v", "g", "beta")), cfg.batch.prev, cfg.batch.art >= 0)
-    assert float(np.abs(_np(o) - want).max()) <= TOL
+    _within(o, want, TOL, "deep tree")
 
 
 def test_decoder_steps_rerun_the_recurrence_from_the_prefix_state(dev):
@@ -205,8 +216,14 @@ def test_decoder_steps_rerun_the_recurrence_from_the_prefix_state(dev):
         torch.cuda.synchronize()
         for s, r in enumerate(rows):
             want, _ = ogdn.recurrent(*(_np(t[x][r]) for x in ("q", "k", "v", "g", "beta")), h0=_np(states[slot_group[s]]))
-            assert float(np.abs(_np(o_buf[0, r[-1]]) - want[-1]).max()) <= TOL, (step, s)   # the decoder reads the new token's row
-            assert float(np.abs(_np(o_buf[0, r]) - want).max()) <= TOL
+            _within(o_buf[0, r[-1]], want[-1], TOL, f"decoder step {step} slot {s}, the new token's row")   # (the row the decoder reads)
+            _within(o_buf[0, r], want, TOL, f"decoder step {step} slot {s}")
     used = sorted(x for r in rows for x in r)
     untouched = np.setdiff1d(np.arange(R), used)
     assert torch.isnan(o_buf[0, untouched].float()).all()                         # rows of no slot are never written
+
+
+def test_zz_report_worst_errors():
+    """(runs last in this file) the largest errors the tests above measured, for the record"""
+    print(f"gdn kernels against the float64 recurrence: worst max abs error outputs {WORST['out']:.3e} (tolerance {TOL:.0e}), "
+          f"states {WORST['state']:.3e} (tolerance {STATE_TOL:.0e})", flush=True)

@@ -161,6 +161,32 @@ def test_both_attention_entry_points_check_their_tensors_before_any_launch(lib, 
         call(q, k, k)
 
 
+def test_build_scan_of_the_ring_assembly_catches_what_it_is_there_for():
+    """the scan build() runs over tree_attn_ring.s, on hand-made listings: a vector write of an MFMA operand in the issue cycle
+    before an assembly MFMA (a wait on a memory counter in between does not count), a compiler-owned accumulation register,
+    too many spills; and what it must let pass"""
+    import __graft_entry__ as ge
+
+    def listing(*body):
+        return ["_Zkernel:", *("\t" + b for b in body)]
+
+    mfma = ["\t;;#ASMSTART", "\tv_mfma_f32_32x32x16_bf16 a[0:15], v[0:3], v[4:7], a[0:15]", "\t;;#ASMEND"]
+    ge._scan_ring_assembly(listing("v_cvt_pk_bf16_f32 v7, v14, v15", "ds_read_b64_tr_b16 v[0:1], v89") + mfma)
+    ge._scan_ring_assembly(listing("v_cvt_pk_bf16_f32 v7, v14, v15", "s_nop 0") + mfma)
+    ge._scan_ring_assembly(listing("v_cvt_pk_bf16_f32 v8, v14, v15", "s_waitcnt lgkmcnt(0)") + mfma)
+    ge._scan_ring_assembly(listing("v_cvt_pk_bf16_f32 v7, v14, v15") + [".LBB0_1:"] + mfma)   # (a branch target: the writer is not the predecessor)
+    with pytest.raises(RuntimeError, match="issue cycle before"):
+        ge._scan_ring_assembly(listing("v_cvt_pk_bf16_f32 v7, v14, v15", "s_waitcnt lgkmcnt(0)") + mfma)
+    with pytest.raises(RuntimeError, match="issue cycle before"):
+        ge._scan_ring_assembly(listing("v_mov_b32_e32 v2, v9") + mfma)
+    with pytest.raises(RuntimeError, match="accumulation register of its own"):
+        ge._scan_ring_assembly(listing("v_accvgpr_write_b32 a130, v3"))
+    meta = ["    .name:           _ZN12_GLOBAL__N_121tree_attn_ring_kernelILi256ELb0EEEv10AttnParams", "    .vgpr_spill_count: 16"]
+    with pytest.raises(RuntimeError, match="spills 16"):
+        ge._scan_ring_assembly(meta)
+    ge._scan_ring_assembly([meta[0], "    .vgpr_spill_count: 2"])
+
+
 # ------------------------------------------------------------------------------------------------ stream layout
 def _golden_trees(case):
     return [TokenTree(t["prefix"], t["branches"], list(t["parents"]), tuple(t["aligned"])) for t in case["trees"]]

@@ -59,12 +59,16 @@ def test_argument_checks_come_before_any_launch():
     with pytest.raises(RuntimeError):
         sa.lm_logprobs(torch.zeros(2, 64), None, 30.0)   # no CPU path
     b = _lib.LmHeadArgs()
-    b.rows, b.vocab, b.hidden = 4, 100, 100
+    b.rows, b.vocab, b.hidden, b.h_rows = 4, 100, 100, 4
     need = C.c_int64()
     assert lib.spinf_lm_head_workspace(C.byref(b), C.byref(need)) != 0 and b"multiple of 64" in lib.spinf_last_error()
     b.hidden = 128
     assert lib.spinf_lm_head_workspace(C.byref(b), C.byref(need)) == 0 and need.value == 4 * 2 * 8
     assert lib.spinf_lm_head_fwd(C.byref(b), None) != 0 and b"null pointer" in lib.spinf_last_error()
+    b.h_rows = 0
+    assert lib.spinf_lm_head_workspace(C.byref(b), C.byref(need)) != 0 and b"h_rows" in lib.spinf_last_error()
+    b.h_rows = 3   # no row list: rows 0 .. 3 of an h of three rows
+    assert lib.spinf_lm_head_workspace(C.byref(b), C.byref(need)) != 0 and b"without a row list" in lib.spinf_last_error()
     with pytest.raises(RuntimeError):
         sa.lm_head_logprobs(torch.zeros(2, 64, dtype=torch.bfloat16), None, torch.zeros(8, 64, dtype=torch.bfloat16))   # no CPU path
 
@@ -140,6 +144,24 @@ def test_fused_head_matches_the_oracle(dev, rows, vocab, hidden, cap):
     # without a row list: rows 0 .. of h itself
     head = sa.lm_head_logprobs(hd[:rows], None, wd, torch.from_numpy(cols).to(dev), cap).cpu().numpy()
     assert np.abs(head - olm.head_logprobs(h.float().numpy()[:rows], w.float().numpy(), None, cols, cap)).max() <= TOL
+
+
+@pytest.mark.gpu
+def test_fused_head_row_list_entries_are_checked_on_the_device(dev):
+    """sel is a device tensor: a negative entry counts from the end (Hf[sel] in the reference, spinf_serve/scorer.py:247-261), an
+    entry outside h reads nothing outside h and gives a row of NaN; the rows beside it are not affected"""
+    rng = np.random.default_rng(5)
+    n = 40
+    h, w = _bf16_values(rng, (n, 128), 1.0).to(dev), _bf16_values(rng, (1000, 128), 1.0).to(dev)
+    good = torch.tensor([0, 39, 17, 17, 5], device=dev)
+    want = sa.lm_head_logprobs(h, good, w, None, 30.0)
+    sel = torch.tensor([0, -1, n, 17, -n - 1, -23, 1 << 40, 5, -(1 << 40)], device=dev)
+    got = sa.lm_head_logprobs(h, sel, w, None, 30.0)
+    assert torch.equal(got[[0, 1, 3, 5, 7]], want)
+    assert torch.isnan(got[[2, 4, 6, 8]]).all()
+    cols = torch.tensor([3, 999, 500], device=dev)
+    part = sa.lm_head_logprobs(h, sel, w, cols, 30.0)
+    assert torch.equal(part[[0, 1, 3, 5, 7]], want[:, cols]) and torch.isnan(part[[2, 4, 6, 8]]).all()
 
 
 @pytest.mark.gpu

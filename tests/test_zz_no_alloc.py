@@ -94,6 +94,56 @@ def test_noalloc_head_dim_512_one_launch_and_graph_replay(dev):
         assert torch.equal(again, want)
 
 
+@pytest.mark.parametrize("ring", [0, 1])
+def test_noalloc_takes_no_device_memory_and_replays_with_cursors_and_wide_scores(dev, ring, monkeypatch):
+    """head dim 256 through both kernels (ring 0: the lockstep kernel, whose cursors, counts and redo list are the scratch array's,
+    cleared by a kernel in front of the pass; ring 1: the kernel with decoupled waves), on scores wide enough that items go to the
+    exact recomputation: the device's free memory and the number of allocations torch has made are the same after the calls as before, and a
+    graph that recorded the call replays to the allocating entry point's bits every time, with eager calls of both entry
+    points in between"""
+    from spinf_serve_amd import attention
+
+    monkeypatch.setattr(attention, "RING", ring)
+    cfg = synth.attention_config("C2", contents=3)
+    b = cfg.batches[0]
+    want, got = _pair(cfg, b, dev, seed=6, scale_keys=(200, 50.0))
+    assert torch.equal(want, got)
+    q, k, v = synth.qkv(cfg, b, seed=6, device=dev)
+    k = k.clone()
+    k[200:] *= 50.0
+    mask = sa.TreeMask.build(b.art, b.end, b.pos, device=dev)
+    assert torch.equal(sa.tree_attn(q, k, v, mask, cfg.scale), want)     # uploads this mask's schedule
+    out = torch.zeros_like(want)
+    lib = sa.load_library()
+    total = ctypes.c_int64(0)
+    assert lib.spinf_attn_exact_items(ctypes.byref(total)) == 0          # (synchronises)
+    before = total.value
+    free0, made0 = torch.cuda.mem_get_info(dev)[0], torch.cuda.memory_stats(dev)["allocation.all.allocated"]
+    for _ in range(3):
+        sa.tree_attn_noalloc(q, k, v, mask, out, cfg.scale)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info(dev)[0] == free0, "device memory was taken"
+    assert torch.cuda.memory_stats(dev)["allocation.all.allocated"] == made0, "torch's allocator was asked for memory"
+    assert torch.equal(out, want)
+    assert lib.spinf_attn_exact_items(ctypes.byref(total)) == 0
+    assert total.value > before, "the wide items went through the exact recomputation"
+    side = torch.cuda.Stream(device=dev)
+    g = torch.cuda.CUDAGraph()
+    print(f"no-alloc case d256 ring={ring} wide scores under capture", flush=True)
+    with torch.cuda.graph(g, stream=side):
+        sa.tree_attn_noalloc(q, k, v, mask, out, cfg.scale)
+    for rep in range(3):
+        out.zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), rep
+        again = sa.tree_attn(q, k, v, mask, cfg.scale)                     # eager work between the replays, both entry points
+        eager = torch.zeros_like(want)
+        sa.tree_attn_noalloc(q, k, v, mask, eager, cfg.scale)
+        torch.cuda.synchronize()
+        assert torch.equal(again, want) and torch.equal(eager, want)
+
+
 def test_noalloc_rejects_more_items_than_its_array_holds(dev):
     a = sa._lib.AttnArgs()
     one = torch.zeros(8, dtype=torch.int32, device=dev)
