@@ -1,6 +1,6 @@
 """Benchmark of the tree-mask packed-prefill attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K=200] [--warmup W=100] [--workload C2|C3|C4|C5|XDEC|LM|LM_head|copy|mfma_peak ...] [--seed S] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K=200] [--warmup W=100] [--workload C2|C2_stream|C3|C4|C5|XDEC|LM|LM_head|copy|mfma_peak ...] [--seed S] [--no-cpu]
 
 A step is one pass of the attention op (one layer's call through the C ABI) over one packed synthetic stream already
 resident in HBM; the tile plan is compiled once per stream, outside the timed region, as the reference builds its block
@@ -30,6 +30,7 @@ WORKLOADS = {
     "C2_512": "C2's stream at the head geometry of the Gemma-4 full-attention layers: 16 query heads / 1 KV head, head_dim 512, global layer",
     "C3": "C3: 512 contents, trunk lognormal(median 800, sigma 0.6) clipped 64..4096, U{8..64} branches of U{4..24}, passes <= 65,536 tokens, 16/8 heads, head_dim 256, one sliding (W=1024) + one global layer per pass",
     "C4": "C4: contents x (8192-token trunk + 16 nodes x 32 + 192 leaves of U{6..10}), 32/16 heads, head_dim 128, one varlen pass",
+    "C2_stream": "C2's byte pattern with nothing computed: the same work items on the same static schedule, query loads, every K / V tile through the LDS ring by the same DMA requests (four in flight), output stores in the kernel's pattern; no MFMA, no softmax, no mask (spinf_diag_attn_stream)",
     "copy": "plain device copy of 1 GiB (reads 1 GiB, writes 1 GiB per launch): the yardstick the FETCH_SIZE / WRITE_SIZE counters are scaled by",
     "C5": "C5: Gated DeltaNet, contents x (2048-token trunk + 32 branches x 12), 16 qk / 32 v heads, 128 x 128 fp32 state",
     "C5_prologue": "C5's stream through the Gated DeltaNet layer's prologue: path convolution (4 taps) + silu + q/k l2 norm + beta + g from the input projection's rows",
@@ -201,6 +202,43 @@ def main():
                     config={"workload": WORKLOADS["copy"], "bytes_read": n, "bytes_written": n},
                     roofline={"bound": "hbm", "achieved": 2 * n / (ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                               "frac": 2 * n / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": 2 * n, "kernel_ms": ms})
+        print(json.dumps(line))
+        return
+
+    if args.workload == "C2_stream":
+        # the floor that data movement alone sets for C2 on its schedule, and the product kernel beside it in the same run
+        from spinf_serve_amd import attention
+
+        cfg = synth.attention_config("C2", seed=args.seed, contents=args.contents)
+        b = cfg.batches[0]
+        mask = sa.block_masks(b, sliding_window=None, device=dev)["full_attention"]
+        q, k, v = synth.qkv(cfg, b, seed=args.seed, device=dev)
+        out = torch.empty_like(q)
+        status = torch.zeros(2, dtype=torch.int32, device=dev)
+        want = sa.tree_attn(q, k, v, mask, cfg.scale)   # (uploads the schedule)
+        wall, kern = timed(lambda: attention.tree_attn_byte_pattern(q, k, v, mask, out, status), args.steps, args.warmup, torch)
+        ms, ms_min = float(np.mean(kern)), float(timed.min_ms)
+        gave_up = int(status[0])
+        assert gave_up == 0 and bool((out == 1).all()), "the yardstick did not run to its end"
+        _, kern2 = timed(lambda: sa.tree_attn(q, k, v, mask, cfg.scale), args.steps, args.warmup, torch)
+        ms2 = float(np.mean(kern2))
+        ms_tiles = float(np.mean(timed(lambda: attention.tree_attn_byte_pattern(q, k, v, mask, out, status, parts=1), args.steps, args.warmup, torch)[1]))
+        ms_rows = float(np.mean(timed(lambda: attention.tree_attn_byte_pattern(q, k, v, mask, out, status, parts=2), args.steps, args.warmup, torch)[1]))
+        by_slots = {n: float(np.mean(timed(lambda: attention.tree_attn_byte_pattern(q, k, v, mask, out, status, parts=1, nslot=n), args.steps, args.warmup, torch)[1]))
+                    for n in (1, 2, 3)}
+        by_slots[4] = ms_tiles
+        dealt = {n: float(np.mean(timed(lambda: attention.tree_attn_byte_pattern(q, k, v, mask, out, status, parts=5, nslot=n), args.steps, args.warmup, torch)[1]))
+                 for n in (1, 2, 4)}
+        plan = mask.for_head_dim(cfg.d, ring=True).plan
+        tile_bytes = len(plan.kv_idx) * (cfg.hq // 2) * 32 * cfg.d * 2 * 2   # K and V of every 32-key tile of every work item: what goes into LDS
+        gbs = cfg.bytes() / (ms * 1e-3) / 1e9
+        line.update(metric="tree-mask attn byte pattern, nothing computed", unit="ms", value=ms, higher_is_better=False, ms_per_step=1e3 * wall / args.steps,
+                    dtype="bf16", config={"workload": WORKLOADS["C2_stream"], "contents": len(cfg.trees), "packed_tokens": cfg.n_real, "stream_tokens": b.length},
+                    roofline={"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS, "traffic": None,
+                              "kernel_ms": ms, "kernel_ms_min": ms_min, "algorithmic_bytes": cfg.bytes(), "bytes_into_lds": tile_bytes,
+                              "lds_fill_gbs": tile_bytes / (ms * 1e-3) / 1e9, "tiles_only_ms": ms_tiles, "tiles_only_ms_by_requests_in_flight": by_slots, "tiles_only_ms_requests_dealt_over_the_waves": dealt, "queries_and_outputs_only_ms": ms_rows, "product_kernel_ms": ms2, "product_over_floor": ms2 / ms,
+                              "frac_of_bf16_peak_if_the_product_ran_at_this_floor": cfg.flops(None) / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS})
+        assert torch.equal(sa.tree_attn(q, k, v, mask, cfg.scale), want)
         print(json.dumps(line))
         return
 

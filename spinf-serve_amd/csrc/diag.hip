@@ -4,6 +4,8 @@
 
 #include "spinf_tree.h"
 #include "common.h"
+#include "attn_kernels.h"
+#include "attn_ring_io.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
@@ -217,7 +219,199 @@ __global__ __launch_bounds__(512) void mfma_hazard_kernel(const int iters, int* 
     if (threadIdx.x == 0) atomicAdd(&out[MFMA_HAZARD_KINDS * MFMA_HAZARD_GAPS], 1);
 }
 
+// ---- the byte pattern of a tree-attention pass with nothing computed: what does moving the data alone cost?
+// The same work items in the same static lists as the kernel with decoupled waves (tree_attn_ring.hip, head dim 256, two heads
+// per item, eight waves): per item every wave loads the queries of its 32 rows (16 bytes per lane and contraction step), every
+// 32-key K / V tile of the item's plan entries comes into a four-slot LDS ring by the same whole-wave DMA requests
+// (issue_tile_wave, four tiles in flight, issued by waves 0 .. 3, the landing flag written by the DMA itself), and at the item's
+// end every wave writes its 32 output rows in the kernel's store pattern (16-byte pieces, four lanes to a row's 64 bytes).
+// No MFMA, no softmax, no mask, no LDS fragment reads: the outputs are a constant.  One workgroup barrier per tile keeps the
+// ring's slots in order, which costs nothing here (the waves have nothing else to do).  status[0] += waves that gave up a bounded
+// wait (never), status[1] += tiles seen landed.  parts: 1 = the K / V tiles only, 2 = the queries and outputs only, 3 = both;
+// nslot (1 .. 4): slots of the ring in use = tile requests in flight.  parts 5: the tiles only, with every tile's requests dealt out
+// over the eight waves and awaited by request count and barrier, as the lockstep kernel does (one wave per tile otherwise).
+template <int D>
+__global__ __launch_bounds__(512) void attn_stream_kernel(const AttnParams p, int* status, const int parts, const int nslot) {
+    using G = TileGeo<D, 32, D>;
+    using GK = Geo<D, 32>;
+    constexpr int NSLOT = 4, NS = D / 16, NDT = D / 32, HPI = 2;
+    __shared__ __attribute__((aligned(16))) char ring[NSLOT * G::BUFB];
+    __shared__ int sy_abort;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wh = w >> 2, wr = w & 3;
+    const int lo = p.list_ptr[blockIdx.x], hi = p.list_ptr[blockIdx.x + 1];
+    auto flag_word = [&](const int slot) { return (int*)(ring + slot * G::BUFB + G::KTILEB + G::VTILEB + 768); };
+    if (threadIdx.x < NSLOT * 64) flag_word(threadIdx.x >> 6)[threadIdx.x & 63] = 0;
+    if (threadIdx.x == 0) sy_abort = 0;
+    int total = 0;
+    for (int i = lo; i < hi; i++) total += __builtin_amdgcn_readfirstlane(p.items[i].z) & 0xfffff;
+    __syncthreads();
+
+    struct Cursor { int item, e, ne, e0, kvh, tz; };
+    auto open = [&](Cursor& c) {
+        while (c.item < hi) {
+            const int4 it = p.items[c.item];
+            c.e0 = __builtin_amdgcn_readfirstlane(it.y);
+            const int z = __builtin_amdgcn_readfirstlane(it.z);
+            c.ne = z & 0xfffff;
+            c.kvh = (int)((unsigned)z >> 20) * HPI / p.group;
+            c.tz = __builtin_amdgcn_readfirstlane(it.x) | (int)((unsigned)z >> 20 << 20);
+            c.e = 0;
+            if (c.ne > 0) break;
+            c.item++;
+        }
+    };
+    auto step = [&](Cursor& c) {
+        if (++c.e >= c.ne) {
+            c.item++;
+            open(c);
+        }
+    };
+    const int lane = fresh_lane_id();
+    const unsigned lane_k = (unsigned)((lane / GK::CPR) * GK::NREG * p.k_tok * 2 + (lane % GK::CPR) * 16);
+    const unsigned lane_v = (unsigned)((lane / GK::CPR) * GK::NREG * p.v_tok * 2 + (lane % GK::CPR) * 16);
+    auto request = [&](const Cursor& c, const int j) {   // tile j of the list into slot j % NSLOT
+        const int kt = __builtin_amdgcn_readfirstlane(p.kv_idx[c.e0 + c.e]);
+        issue_tile_wave<D, false>(p, lds_addr(ring + (j % nslot) * G::BUFB), kt, c.kvh, j / nslot + 1, lane, lane_k, lane_v);
+    };
+    auto load_q = [&](const int tz, bf16x8 (&qf)[NS]) {
+        const int tok = (tz & 0xfffff) * SPINF_QTILE + 32 * wr + (lane & 31);
+        const int tok_c = tok < p.n ? tok : p.n - 1;
+        const int h = (int)((unsigned)tz >> 20) * HPI + wh;
+        const __bf16* qp = p.q + (long)tok_c * p.q_tok + (long)h * p.q_head + 8 * (lane >> 5);
+#pragma unroll
+        for (int s2 = 0; s2 < NS; s2++) qf[s2] = *(const bf16x8*)(qp + 16 * s2);
+    };
+
+    Cursor ahead{lo, 0, 0, 0, 0, 0}, here{lo, 0, 0, 0, 0, 0};
+    open(ahead);
+    open(here);
+    if (parts == 5) {   // the tiles alone, every tile's requests dealt out over the eight waves (as the lockstep kernel does over its four)
+        auto share = [&](const Cursor& c, const int j) {
+            const int kt = __builtin_amdgcn_readfirstlane(p.kv_idx[c.e0 + c.e]);
+            issue_tile<D, 8, false, 0, 32, D>(p, lds_addr(ring + (j % nslot) * G::BUFB), kt, -1, c.kvh, w, lane, lane_k, lane_v);
+        };
+        for (int j = 0; j < nslot && ahead.item < hi; j++) {
+            share(ahead, j);
+            step(ahead);
+        }
+        const int mine = 4 + (w < 3);   // requests of this wave per tile
+        int seen = 0;
+#pragma unroll 1
+        for (int j = 0; j < total; j++) {
+            const int left = total - 1 - j < nslot - 1 ? total - 1 - j : nslot - 1;   // younger tiles on their way
+            switch (left * mine) {
+                case 0: __builtin_amdgcn_s_waitcnt(0x0f70); break;
+                case 4: __builtin_amdgcn_s_waitcnt(0x0f74); break;
+                case 5: __builtin_amdgcn_s_waitcnt(0x0f75); break;
+                case 8: __builtin_amdgcn_s_waitcnt(0x0f78); break;
+                case 10: __builtin_amdgcn_s_waitcnt(0x0f7a); break;
+                case 12: __builtin_amdgcn_s_waitcnt(0x0f7c); break;
+                default: __builtin_amdgcn_s_waitcnt(0x0f7f); break;   // 15
+            }
+            __syncthreads();   // tile j has landed, whoever requested which part of it; its slot can take tile j + nslot
+            seen++;
+            if (ahead.item < hi) {
+                share(ahead, j + nslot);
+                step(ahead);
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        if (threadIdx.x == 0) atomicAdd(&status[1], seen);
+        return;
+    }
+    const bool tiles = parts & 1, rows = parts & 2;
+    if (tiles && w < nslot) {   // wave w requests the tiles j = w, w + nslot, ...: the first one now
+        for (int i = 0; i < w && ahead.item < hi; i++) step(ahead);
+        if (ahead.item < hi) request(ahead, w);
+    }
+    bf16x8 qf[NS];
+    if (rows && here.item < hi) load_q(here.tz, qf);
+    int seen = 0;
+#pragma unroll 1
+    for (int j = 0; j < total; j++) {
+        const int want = (j / nslot + 1) & 63;
+        int polls = 0;
+        while (tiles && *(volatile int*)flag_word(j % nslot) != want && *(volatile int*)&sy_abort == 0) {
+            if (++polls > (1 << 20)) {
+                sy_abort = 1;
+                if (lane == 0) atomicAdd(&status[0], 1);
+            }
+            __builtin_amdgcn_s_sleep(1);
+        }
+        if (tiles) __syncthreads();   // every wave has seen tile j: its slot can take tile j + nslot
+        if (*(volatile int*)&sy_abort != 0) break;
+        seen++;
+        if (tiles && w == j % nslot) {
+            for (int i = 0; i < nslot && ahead.item < hi; i++) step(ahead);
+            if (ahead.item < hi) request(ahead, j + nslot);
+        }
+        if (here.e == here.ne - 1 && !rows) {
+            step(here);
+        } else if (here.e == here.ne - 1) {   // the item's last tile: the next queries are requested, then this item's rows leave
+            const int tz = here.tz;
+            step(here);
+            bf16x8 qn[NS];
+            if (here.item < hi) load_q(here.tz, qn);
+#pragma unroll
+            for (int s2 = 0; s2 < NS; s2++) asm volatile("" ::"v"(qf[s2]));   // the queries did arrive in registers
+            const int tok0 = (tz & 0xfffff) * SPINF_QTILE + 32 * wr;
+            const int h = (int)((unsigned)tz >> 20) * HPI + wh;
+            __bf16* ob = p.o + (long)h * p.o_head;
+            bf16x8 one;
+#pragma unroll
+            for (int i = 0; i < 8; i++) one[i] = (__bf16)1.0f;
+#pragma unroll
+            for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+                for (int jj = 0; jj < 2; jj++) {
+                    const int c = jj * 64 + lane, row = c >> 2, col = c & 3;
+                    if (tok0 + row < p.n) *(bf16x8*)(ob + (long)(tok0 + row) * p.o_tok + 32 * dt + col * 8) = one;
+                }
+            if (here.item < hi) {
+#pragma unroll
+                for (int s2 = 0; s2 < NS; s2++) qf[s2] = qn[s2];
+            }
+        } else {
+            step(here);
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(0x0f70);   // no DMA of this workgroup is still on its way into LDS when it ends
+    if (threadIdx.x == 0) atomicAdd(&status[1], seen);
+}
+
 }  // namespace
+
+extern "C" int spinf_diag_attn_stream(const spinf_attn_args* a, int32_t parts, int32_t nslot, int32_t* status, void* stream) {
+    if (!a || !status) return spinf_fail(SPINF_E_ARG, "diag_attn_stream: null pointer");
+    if ((parts < 1 || parts > 3) && parts != 5)
+        return spinf_fail(SPINF_E_ARG, "diag_attn_stream: parts %d not in 1 (tiles), 2 (queries and outputs), 3 (both), 5 (tiles, requests dealt over the waves)", parts);
+    if (parts == 5 && !a->pos) return spinf_fail(SPINF_E_ARG, "diag_attn_stream: null pointer");
+    if (nslot < 1 || nslot > 4) return spinf_fail(SPINF_E_ARG, "diag_attn_stream: %d slots, 1 .. 4", nslot);
+    if (!a->q || !a->k || !a->v || !a->out || !a->art || !a->end || !a->kv_idx || !a->items || !a->list_ptr)
+        return spinf_fail(SPINF_E_ARG, "diag_attn_stream: null pointer");
+    if (a->d != 256 || a->ktile != 32 || a->n_lists <= 0 || a->n_lists > LAND_CAP || a->hkv <= 0 || a->hq % (2 * a->hkv) || a->row_of || a->grp || a->n <= 0)
+        return spinf_fail(SPINF_E_ARG, "diag_attn_stream: takes what the kernel with decoupled waves takes at head dim 256: a static schedule over 32-key "
+                                       "entries, an even number of query heads per key / value head, stream layout");
+    const int64_t strides[8] = {a->q_tok, a->q_head, a->k_tok, a->k_head, a->v_tok, a->v_head, a->o_tok, a->o_head};
+    for (int i = 0; i < 8; i++)
+        if (strides[i] % 8) return spinf_fail(SPINF_E_ARG, "diag_attn_stream: strides must be multiples of 8 elements");
+    const uintptr_t ptrs[4] = {(uintptr_t)a->q, (uintptr_t)a->k, (uintptr_t)a->v, (uintptr_t)a->out};
+    for (int i = 0; i < 4; i++)
+        if (ptrs[i] % 16) return spinf_fail(SPINF_E_ARG, "diag_attn_stream: tensors must be 16-byte aligned");
+    AttnParams p = {};
+    p.q = (const __bf16*)a->q; p.k = (const __bf16*)a->k; p.v = (const __bf16*)a->v; p.o = (__bf16*)a->out;
+    p.q_tok = a->q_tok; p.q_head = a->q_head; p.k_tok = a->k_tok; p.k_head = a->k_head;
+    p.v_tok = a->v_tok; p.v_head = a->v_head; p.o_tok = a->o_tok; p.o_head = a->o_head;
+    p.n = (int)a->n; p.group = a->hq / a->hkv;
+    p.art = a->art; p.end = a->end; p.pos = a->pos;
+    p.kv_idx = a->kv_idx; p.kv_bits = a->kv_bits;
+    p.items = (const int4*)a->items; p.list_ptr = a->list_ptr;
+    hipLaunchKernelGGL(attn_stream_kernel<256>, dim3(a->n_lists), dim3(512), 0, (hipStream_t)stream, p, (int*)status, (int)parts, (int)nslot);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "diag_attn_stream: launch: %s", hipGetErrorString(e));
+    return SPINF_OK;
+}
 
 extern "C" int spinf_diag_mfma_hazard(int32_t iters, int32_t workgroups, int32_t* out, void* stream) {
     if (iters <= 0 || iters > 100000 || workgroups <= 0 || workgroups > 65536 || !out)

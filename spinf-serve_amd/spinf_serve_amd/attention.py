@@ -202,6 +202,42 @@ def tree_attn_noalloc(q, k, v, mask: TreeMask, out, scale=None):
     return out
 
 
+def tree_attn_byte_pattern(q, k, v, mask: TreeMask, out, status, parts=3, nslot=4):
+    """A yardstick, not an operator (spinf_diag_attn_stream): the data movement of tree_attn's kernel with decoupled waves for these
+    tensors (head dim 256, the same static schedule: query loads, every K / V tile of every work item through the LDS ring by the
+    same DMA requests, output stores in the kernel's pattern) with nothing computed; ``out`` [n, hq, d] comes back as ones on the
+    real rows.  status: 2 int32 on the device, zeroed by the caller: [0] += waves that gave up a wait, [1] += tiles seen landed.
+    parts: 3 = all of it, 1 = the K / V tiles only, 2 = the queries and outputs only; nslot: ring slots in use (tile requests in
+    flight), 1 .. 4."""
+    if not isinstance(mask, TreeMask):
+        raise TypeError("attention_mask must be a TreeMask (masks.block_masks)")
+    if out.shape != q.shape or out.dtype != torch.bfloat16 or not out.is_contiguous():
+        raise ValueError("out must be a contiguous bf16 tensor of q's shape")
+    if status.dtype != torch.int32 or status.numel() < 2 or not status.is_contiguous():
+        raise ValueError("status must be 2 contiguous int32")
+    _check_tensors(q, k, v, mask.n, False, (out, status, mask.art, mask.end, mask.pos, mask.kv_idx, mask.kv_bits))
+    n, hq, d = q.shape
+    hkv = k.shape[1]
+    if d != 256 or (hq // hkv) % 2 or mask.grp is not None:
+        raise ValueError("the byte-pattern yardstick covers head dim 256 with an even number of query heads per key / value head, no image groups")
+    n_lists = _static_lists_of(q.device)
+    mask = mask.for_head_dim(d, ring=True)
+    items, list_ptr, n_items = mask.schedule(hq // 2, n_lists)
+    a = _attn_args(q, k, v, out, n, mask.art, mask.end, mask.pos, mask.kv_idx, mask.kv_bits, items, list_ptr, n_items, float(d ** -0.5), int(mask.window), 0,
+                   None, None, None, 0, int(mask.plan.ktile), n_lists)
+    lib = _lib.load_library()
+    with torch.cuda.device(q.device):
+        stream = torch.cuda.current_stream(q.device).cuda_stream
+        _lib.check(lib.spinf_diag_attn_stream(C.byref(a), int(parts), int(nslot), C.c_void_p(status.data_ptr()), C.c_void_p(stream)), "spinf_diag_attn_stream")
+    return out
+
+
+def _static_lists_of(device):
+    from .masks import _static_lists
+
+    return _static_lists(device)
+
+
 # K/V capture for extraction, as spinf_serve/models/gemma4.py:66-70: while CAPTURE[device] = {"window", "ranges": [(start, n, key)],
 # "kv": {}} is set, every call keeps the layer's keys / values of the ranges (sliding layers only their last window - 1)
 CAPTURE: dict = {}

@@ -44,3 +44,24 @@ def test_an_mfma_needs_one_instruction_after_a_vector_write_of_its_operands(dev,
     assert mfma_then_write == [0] * 5, got
     assert other_gaps[3:] == [0] * 2, got
     assert write_then_mfma[0] > 0 and cvt_then_mfma[0] > 0, f"no wrong product without a gap any more: {got} (the assembly scan of the build could go)"
+
+
+def test_byte_pattern_yardstick_moves_every_tile_and_writes_every_row(dev, lib):
+    """spinf_diag_attn_stream on a scaled-down C2: every tile of every work item is seen landed (the count equals the plan
+    entries of the 32-key plan x head groups), no wait is given up, and every row of the stream is written"""
+    import spinf_serve_amd as sa
+    from spinf_serve_amd import attention, synth
+
+    cfg = synth.attention_config("C2", contents=3)
+    b = cfg.batches[0]
+    q, k, v = synth.qkv(cfg, b, seed=1, device=dev)
+    mask = sa.TreeMask.build(b.art, b.end, b.pos, device=dev)
+    out = torch.zeros_like(q)
+    status = torch.zeros(2, dtype=torch.int32, device=dev)
+    attention.tree_attn_byte_pattern(q, k, v, mask, out, status)
+    torch.cuda.synchronize()
+    plan = mask.for_head_dim(cfg.d, ring=True).plan
+    gave_up, tiles = status.cpu().tolist()
+    assert gave_up == 0
+    assert tiles == len(plan.kv_idx) * (cfg.hq // 2)
+    assert (out == 1).all()
