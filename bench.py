@@ -168,6 +168,7 @@ def main():
     ap.add_argument("--variant", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-big", action="store_true", help="C2 only: skip the C3 / C4 sub-records")
+    ap.add_argument("--parts-only", action="store_true", help="C2_stream only: time the whole pattern alone, none of its parts and variants (for a profile of one kernel shape)")
     ap.add_argument("--nsplit", type=int, default=None, help="XDEC workloads: splits of a (group, kv head) key stream (default: the library's choice)")
     ap.add_argument("--rows", default="stream", choices=["stream", "compact", "scatter"],
                     help="attention workloads: stream layout (default); compact = real rows only, read through the kernel's row map; "
@@ -220,6 +221,13 @@ def main():
         ms, ms_min = float(np.mean(kern)), float(timed.min_ms)
         gave_up = int(status[0])
         assert gave_up == 0 and bool((out == 1).all()), "the yardstick did not run to its end"
+        if args.parts_only:
+            line.update(metric="tree-mask attn byte pattern, nothing computed", unit="ms", value=ms, higher_is_better=False, ms_per_step=1e3 * wall / args.steps,
+                        dtype="bf16", config={"workload": WORKLOADS["C2_stream"], "contents": len(cfg.trees), "packed_tokens": cfg.n_real, "stream_tokens": b.length},
+                        roofline={"bound": "hbm", "achieved": cfg.bytes() / (ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                  "frac": cfg.bytes() / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": None, "kernel_ms": ms, "kernel_ms_min": ms_min})
+            print(json.dumps(line))
+            return
         _, kern2 = timed(lambda: sa.tree_attn(q, k, v, mask, cfg.scale), args.steps, args.warmup, torch)
         ms2 = float(np.mean(kern2))
         ms_tiles = float(np.mean(timed(lambda: attention.tree_attn_byte_pattern(q, k, v, mask, out, status, parts=1), args.steps, args.warmup, torch)[1]))
@@ -229,6 +237,9 @@ def main():
         by_slots[4] = ms_tiles
         dealt = {n: float(np.mean(timed(lambda: attention.tree_attn_byte_pattern(q, k, v, mask, out, status, parts=5, nslot=n), args.steps, args.warmup, torch)[1]))
                  for n in (1, 2, 4)}
+        out.zero_()
+        ms_dealt = float(np.mean(timed(lambda: attention.tree_attn_byte_pattern(q, k, v, mask, out, status, parts=7), args.steps, args.warmup, torch)[1]))
+        assert int(status[0]) == 0 and bool((out == 1).all())
         plan = mask.for_head_dim(cfg.d, ring=True).plan
         tile_bytes = len(plan.kv_idx) * (cfg.hq // 2) * 32 * cfg.d * 2 * 2   # K and V of every 32-key tile of every work item: what goes into LDS
         gbs = cfg.bytes() / (ms * 1e-3) / 1e9
@@ -236,7 +247,7 @@ def main():
                     dtype="bf16", config={"workload": WORKLOADS["C2_stream"], "contents": len(cfg.trees), "packed_tokens": cfg.n_real, "stream_tokens": b.length},
                     roofline={"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS, "traffic": None,
                               "kernel_ms": ms, "kernel_ms_min": ms_min, "algorithmic_bytes": cfg.bytes(), "bytes_into_lds": tile_bytes,
-                              "lds_fill_gbs": tile_bytes / (ms * 1e-3) / 1e9, "tiles_only_ms": ms_tiles, "tiles_only_ms_by_requests_in_flight": by_slots, "tiles_only_ms_requests_dealt_over_the_waves": dealt, "queries_and_outputs_only_ms": ms_rows, "product_kernel_ms": ms2, "product_over_floor": ms2 / ms,
+                              "lds_fill_gbs": tile_bytes / (ms * 1e-3) / 1e9, "tiles_only_ms": ms_tiles, "tiles_only_ms_by_requests_in_flight": by_slots, "tiles_only_ms_requests_dealt_over_the_waves": dealt, "kernel_ms_requests_dealt_over_the_waves": ms_dealt, "queries_and_outputs_only_ms": ms_rows, "product_kernel_ms": ms2, "product_over_floor": ms2 / ms,
                               "frac_of_bf16_peak_if_the_product_ran_at_this_floor": cfg.flops(None) / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS})
         assert torch.equal(sa.tree_attn(q, k, v, mask, cfg.scale), want)
         print(json.dumps(line))

@@ -229,7 +229,8 @@ __global__ __launch_bounds__(512) void mfma_hazard_kernel(const int iters, int* 
 // ring's slots in order, which costs nothing here (the waves have nothing else to do).  status[0] += waves that gave up a bounded
 // wait (never), status[1] += tiles seen landed.  parts: 1 = the K / V tiles only, 2 = the queries and outputs only, 3 = both;
 // nslot (1 .. 4): slots of the ring in use = tile requests in flight.  parts 5: the tiles only, with every tile's requests dealt out
-// over the eight waves and awaited by request count and barrier, as the lockstep kernel does (one wave per tile otherwise).
+// over the eight waves and awaited by request count and barrier, as the lockstep kernel does (one wave per tile otherwise); parts 7:
+// the whole pattern that way, with a landing flag per wave.
 template <int D>
 __global__ __launch_bounds__(512) void attn_stream_kernel(const AttnParams p, int* status, const int parts, const int nslot) {
     using G = TileGeo<D, 32, D>;
@@ -320,8 +321,21 @@ __global__ __launch_bounds__(512) void attn_stream_kernel(const AttnParams p, in
         if (threadIdx.x == 0) atomicAdd(&status[1], seen);
         return;
     }
-    const bool tiles = parts & 1, rows = parts & 2;
-    if (tiles && w < nslot) {   // wave w requests the tiles j = w, w + nslot, ...: the first one now
+    const bool tiles = parts & 1, rows = parts & 2, dealt = parts == 7;
+    // parts 7: the whole pattern with every tile's requests dealt out over the eight waves; wave w's last request of a tile writes
+    // word w of the slot's flag area (one lane of a 4-byte request), and a tile has landed when all eight words show its generation
+    auto share = [&](const Cursor& c, const int j) {
+        const int kt = __builtin_amdgcn_readfirstlane(p.kv_idx[c.e0 + c.e]);
+        const unsigned buf = lds_addr(ring + (j % nslot) * G::BUFB);
+        issue_tile<D, 8, false, 0, 32, D>(p, buf, kt, -1, c.kvh, w, lane, lane_k, lane_v);
+        if (lane == w) dma4_lane(ring_seq + ((j / nslot + 1) & 63), buf + G::KTILEB + G::VTILEB + 768);
+    };
+    if (dealt) {
+        for (int j = 0; j < nslot && ahead.item < hi; j++) {
+            share(ahead, j);
+            step(ahead);
+        }
+    } else if (tiles && w < nslot) {   // wave w requests the tiles j = w, w + nslot, ...: the first one now
         for (int i = 0; i < w && ahead.item < hi; i++) step(ahead);
         if (ahead.item < hi) request(ahead, w);
     }
@@ -332,17 +346,36 @@ __global__ __launch_bounds__(512) void attn_stream_kernel(const AttnParams p, in
     for (int j = 0; j < total; j++) {
         const int want = (j / nslot + 1) & 63;
         int polls = 0;
-        while (tiles && *(volatile int*)flag_word(j % nslot) != want && *(volatile int*)&sy_abort == 0) {
-            if (++polls > (1 << 20)) {
-                sy_abort = 1;
-                if (lane == 0) atomicAdd(&status[0], 1);
+        if (dealt) {
+            const volatile int* f = flag_word(j % nslot);
+            while (true) {
+                bool all = true;
+                for (int i = 0; i < 8; i++) all = all && f[i] == want;
+                if (all || *(volatile int*)&sy_abort != 0) break;
+                if (++polls > (1 << 20)) {
+                    sy_abort = 1;
+                    if (lane == 0) atomicAdd(&status[0], 1);
+                }
+                __builtin_amdgcn_s_sleep(1);
             }
-            __builtin_amdgcn_s_sleep(1);
+        } else {
+            while (tiles && *(volatile int*)flag_word(j % nslot) != want && *(volatile int*)&sy_abort == 0) {
+                if (++polls > (1 << 20)) {
+                    sy_abort = 1;
+                    if (lane == 0) atomicAdd(&status[0], 1);
+                }
+                __builtin_amdgcn_s_sleep(1);
+            }
         }
         if (tiles) __syncthreads();   // every wave has seen tile j: its slot can take tile j + nslot
         if (*(volatile int*)&sy_abort != 0) break;
         seen++;
-        if (tiles && w == j % nslot) {
+        if (dealt) {
+            if (ahead.item < hi) {
+                share(ahead, j + nslot);
+                step(ahead);
+            }
+        } else if (tiles && w == j % nslot) {
             for (int i = 0; i < nslot && ahead.item < hi; i++) step(ahead);
             if (ahead.item < hi) request(ahead, j + nslot);
         }
@@ -384,9 +417,9 @@ __global__ __launch_bounds__(512) void attn_stream_kernel(const AttnParams p, in
 
 extern "C" int spinf_diag_attn_stream(const spinf_attn_args* a, int32_t parts, int32_t nslot, int32_t* status, void* stream) {
     if (!a || !status) return spinf_fail(SPINF_E_ARG, "diag_attn_stream: null pointer");
-    if ((parts < 1 || parts > 3) && parts != 5)
-        return spinf_fail(SPINF_E_ARG, "diag_attn_stream: parts %d not in 1 (tiles), 2 (queries and outputs), 3 (both), 5 (tiles, requests dealt over the waves)", parts);
-    if (parts == 5 && !a->pos) return spinf_fail(SPINF_E_ARG, "diag_attn_stream: null pointer");
+    if ((parts < 1 || parts > 3) && parts != 5 && parts != 7)
+        return spinf_fail(SPINF_E_ARG, "diag_attn_stream: parts %d not in 1 (tiles), 2 (queries and outputs), 3 (both), 5 / 7 (as 1 / 3 with a tile's requests dealt over the waves)", parts);
+    if (parts >= 5 && !a->pos) return spinf_fail(SPINF_E_ARG, "diag_attn_stream: null pointer");
     if (nslot < 1 || nslot > 4) return spinf_fail(SPINF_E_ARG, "diag_attn_stream: %d slots, 1 .. 4", nslot);
     if (!a->q || !a->k || !a->v || !a->out || !a->art || !a->end || !a->kv_idx || !a->items || !a->list_ptr)
         return spinf_fail(SPINF_E_ARG, "diag_attn_stream: null pointer");

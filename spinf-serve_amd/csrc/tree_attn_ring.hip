@@ -947,26 +947,36 @@ __global__ __launch_bounds__(D == 512 ? 256 : 512) void tree_attn_ring_kernel(co
     __builtin_amdgcn_s_waitcnt(0x0f70);
 }
 
-// The landing kernel: launched behind every launch of the ring kernel, with the same grid.  A workgroup whose ring-kernel twin left no
-// word (p.land[b] == 0: every launch but a faulty one) returns at once; otherwise it computes that workgroup's whole list again.
+// The landing kernel: launched behind every launch of the ring kernel, a few workgroups that go through the ring kernel's workgroups
+// b = 0 .. n_wg - 1 between them.  Where b left no word (p.land[b] == 0: every launch but a faulty one) there is nothing to do;
+// otherwise b's whole list is computed again.  (A grid as wide as the ring kernel's cost 4.1 us per call just to start and end.)
+constexpr int LANDING_WGS = 16;
 template <int D, bool WIN>
-__global__ __launch_bounds__(D == 512 ? 256 : 512) void tree_attn_ring_landing_kernel(const AttnParams p) {
-    const int gave_up = p.land[blockIdx.x];   // waves of the ring kernel's workgroup b that gave up a wait
-    if (gave_up == 0) return;
+__global__ __launch_bounds__(D == 512 ? 256 : 512) void tree_attn_ring_landing_kernel(const AttnParams p, const int n_wg) {
     using S = RingShape<D>;
     using G = TileGeo<D, S::TK, D>;
     __shared__ __attribute__((aligned(16))) char ring[G::BUFB];
     __shared__ __attribute__((aligned(16))) char stage_all[S::NW * 32 * SROW];
     __shared__ int sy_nredo, sy_vote;
-    const int lo = p.list_ptr[blockIdx.x], hi = p.list_ptr[blockIdx.x + 1];
-    if (threadIdx.x == 0) {
-        sy_nredo = 0;   // (the ring kernel's workgroup left without its exact recomputations: whatever the list needs is found again here)
-        sy_vote = 0;
-        atomicAdd(&p.counters[NLIST + 4], gave_up);   // running total, for spinf_attn_ring_aborts
+    // every launch but a faulty one ends here: one word per thread, all of them zero
+    int mine = 0;
+    for (int b = blockIdx.x + gridDim.x * threadIdx.x; b < n_wg; b += gridDim.x * blockDim.x) mine |= p.land[b];
+    if (__syncthreads_or(mine) == 0) return;
+#pragma unroll 1
+    for (int b = blockIdx.x; b < n_wg; b += gridDim.x) {
+        const int gave_up = __builtin_amdgcn_readfirstlane(p.land[b]);   // waves of the ring kernel's workgroup b that gave up a wait
+        if (gave_up == 0) continue;
+        const int lo = p.list_ptr[b], hi = p.list_ptr[b + 1];
+        __syncthreads();   // (the previous list's last reads of the words below)
+        if (threadIdx.x == 0) {
+            sy_nredo = 0;   // (the ring kernel's workgroup left without its exact recomputations: whatever the list needs is found again here)
+            sy_vote = 0;
+            atomicAdd(&p.counters[NLIST + 4], gave_up);   // running total, for spinf_attn_ring_aborts
+        }
+        __syncthreads();
+        ring_paced_pass<D, WIN>(p, ring, stage_all, &sy_nredo, &sy_vote, lo, hi, lo);
+        if (threadIdx.x == 0) p.land[b] = 0;   // (the word is per launch: the next one starts clean)
     }
-    __syncthreads();
-    ring_paced_pass<D, WIN>(p, ring, stage_all, &sy_nredo, &sy_vote, lo, hi, lo);
-    if (threadIdx.x == 0) p.land[blockIdx.x] = 0;   // (the word is per launch: the next one starts clean)
 }
 
 template <int D, bool WIN>
@@ -974,7 +984,7 @@ int launch_ring_t(const AttnParams& p, int n_wg, hipStream_t stream) {
     hipLaunchKernelGGL((tree_attn_ring_kernel<D, WIN>), dim3(n_wg), dim3(D == 512 ? 256 : 512), 0, stream, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: launch (ring kernel): %s", hipGetErrorString(e));
-    hipLaunchKernelGGL((tree_attn_ring_landing_kernel<D, WIN>), dim3(n_wg), dim3(D == 512 ? 256 : 512), 0, stream, p);
+    hipLaunchKernelGGL((tree_attn_ring_landing_kernel<D, WIN>), dim3(n_wg < LANDING_WGS ? n_wg : LANDING_WGS), dim3(D == 512 ? 256 : 512), 0, stream, p, n_wg);
     e = hipGetLastError();
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: launch (landing kernel): %s", hipGetErrorString(e));
     return SPINF_OK;

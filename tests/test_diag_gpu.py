@@ -56,12 +56,13 @@ def test_byte_pattern_yardstick_moves_every_tile_and_writes_every_row(dev, lib):
     b = cfg.batches[0]
     q, k, v = synth.qkv(cfg, b, seed=1, device=dev)
     mask = sa.TreeMask.build(b.art, b.end, b.pos, device=dev)
-    out = torch.zeros_like(q)
-    status = torch.zeros(2, dtype=torch.int32, device=dev)
-    attention.tree_attn_byte_pattern(q, k, v, mask, out, status)
-    torch.cuda.synchronize()
     plan = mask.for_head_dim(cfg.d, ring=True).plan
-    gave_up, tiles = status.cpu().tolist()
-    assert gave_up == 0
-    assert tiles == len(plan.kv_idx) * (cfg.hq // 2)
-    assert (out == 1).all()
+    for parts in (3, 7):   # a tile's requests made by one wave, as in the kernel; dealt out over the eight waves
+        out = torch.zeros_like(q)
+        status = torch.zeros(2, dtype=torch.int32, device=dev)
+        attention.tree_attn_byte_pattern(q, k, v, mask, out, status, parts=parts)
+        torch.cuda.synchronize()
+        gave_up, tiles = status.cpu().tolist()
+        assert gave_up == 0, parts
+        assert tiles == len(plan.kv_idx) * (cfg.hq // 2), parts
+        assert (out == 1).all(), parts
