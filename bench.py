@@ -462,6 +462,18 @@ def main():
                           # the two roofs at the published peaks: whichever floor is higher binds the workload
                           "mfma_floor_ms": flops / (PEAK_BF16_TFLOPS * 1e12) * 1e3, "hbm_floor_ms": cfg.bytes() * len(layers) / (PEAK_HBM_GBS * 1e9) * 1e3},
                 plan_build_ms_host=plan_ms, setup_s=setup_s)
+    if args.workload == "C2" and args.rows == "stream" and args.variant == 0:
+        # the same work items with nothing computed (spinf_diag_attn_stream, --workload C2_stream): what moving this pass's bytes in the
+        # kernel's pattern takes on this box right now
+        from spinf_serve_amd import attention
+
+        (q, k, v), masks = work[0]
+        ybuf, ystat = torch.empty_like(q), torch.zeros(2, dtype=torch.int32, device=dev)
+        _, ykern = timed(lambda: attention.tree_attn_byte_pattern(q, k, v, masks["full_attention"], ybuf, ystat), args.steps, args.warmup, torch)
+        if int(ystat[0]) == 0 and bool((ybuf == 1).all()):
+            line["roofline"]["byte_pattern_ms"] = float(np.mean(ykern))
+            line["roofline"]["kernel_ms_over_byte_pattern_ms"] = ms / line["roofline"]["byte_pattern_ms"]
+        del ybuf
     # what a pure MFMA loop sustains on this part right now, next to the published constant the fraction is priced against
     line["roofline"]["reachable_peak"] = mfma_rate(torch)[0]
     line["roofline"]["frac_of_reachable_peak"] = tfl / line["roofline"]["reachable_peak"]
