@@ -121,8 +121,8 @@ typedef struct spinf_attn_args {
     int32_t debug_expire;                   /* 0 in production.  Test hook of the kernel with decoupled waves (no counterpart in the reference):
                                                k > 0 = polls of one wait before a wave gives up (2^18 otherwise; a healthy wait takes a handful).
                                                With k = 1 every wave that has to wait at all gives up, which takes its workgroup through the
-                                               landing a real time-out would take (the landing kernel computes the workgroup's list again, one
-                                               tile at a time between barriers).  Same results bit for bit; spinf_attn_ring_aborts counts it */
+                                               landing a real time-out would take (every wave leaves the ring and the workgroup computes its list
+                                               again, one tile at a time between barriers).  Same results bit for bit; spinf_attn_ring_aborts counts it */
 } spinf_attn_args;
 
 /* query heads one work item covers for this geometry (1 or 2); 0 for an invalid geometry */
@@ -131,7 +131,7 @@ int spinf_tree_attn_fwd(const spinf_attn_args* args, void* stream);
 /* The same pass with nothing allocated.  No counterpart in the reference: it is for callers that cannot call hipMalloc (code
  * under HIP graph capture, tight serving loops, harnesses that forbid allocation).  spinf_tree_attn_fwd keeps its list cursors,
  * counts and redo list in a buffer that the library allocates (and regrows) on the device; this entry point keeps them in a
- * file-scope device array of 64 + 65,536 + 4,096 ints (272.25 KiB per GPU, held until the process ends) and calls no hipMalloc /
+ * file-scope device array of 64 + 65,536 ints (256.25 KiB per GPU, held until the process ends) and calls no hipMalloc /
  * hipFree nor any allocating routine.  Same arguments, same kernels, same results bit for bit.  Limit: n_items (query tiles x
  * head groups) <= 65,536, more is SPINF_E_ARG.  The cursors and counts are cleared by a small kernel in front of every pass that
  * uses them (the kernel with decoupled waves uses none: such a call is one launch), so a call does not depend on what the
@@ -144,8 +144,8 @@ int spinf_tree_attn_fwd_noalloc(const spinf_attn_args* args, void* stream);
 int spinf_attn_exact_items(int64_t* total);
 /* Diagnostics (no counterpart in the reference): *total = waves of the static-schedule kernel that gave up a bounded wait on
  * the current device since the library was loaded.  Always 0 unless the kernel has a bug (or debug_expire asked for it).  The
- * results of such a pass are still complete and the same bit for bit: the landing kernel that follows every launch of that kernel
- * computes the list of such a workgroup again, one tile at a time between barriers; the count says that time was lost.
+ * results of such a pass are still complete and the same bit for bit: such a workgroup computes its list again before it ends,
+ * one tile at a time between barriers; the count says that time was lost.
  * Synchronises the device. */
 int spinf_attn_ring_aborts(int64_t* total);
 

@@ -8,7 +8,7 @@
 #include "attn_tiles.h"
 
 constexpr int NLIST = 8;       // work lists (XCDs of an MI355X)
-constexpr int LAND_CAP = 4096;  // most item lists of a static schedule (one landing word of the ring kernel each; a schedule has one list per compute unit)
+constexpr int LAND_CAP = 4096;  // most item lists of a static schedule (a schedule has one list per compute unit)
 constexpr int ENT_CAP = 256;   // plan entries of a query tile kept in LDS at a time
 
 struct AttnParams {
@@ -22,7 +22,8 @@ struct AttnParams {
     const int4* items;    // work items {query tile, first entry, entries | head group << 20, first key tile}, list by list
     const int* list_ptr;  // [NLIST + 1] offsets of the lists in items
     int* counters;        // [0..NLIST) next item of each list, [NLIST] workgroups done, [NLIST+1] items awaiting the exact pass,
-                          // [NLIST+2] exact-pass workgroups done; each kernel's last workgroup resets what it used
+                          // [NLIST+2] exact-pass workgroups done; each kernel's last workgroup resets what it used; running totals:
+                          // [NLIST+3] items recomputed exactly, [NLIST+4] waves of the ring kernel that gave up a wait
     int* redo;            // indices (into items) of the work items the fast pass handed to the exact pass (the ring kernel: entries
                           // list_ptr[b] .. of workgroup b's own hand-overs, which it recomputes itself)
     // compact rows (ROWS kernels): q, k, v, o hold the real tokens only; row_of[stream position] = row, -1 for a pad position;
@@ -31,8 +32,8 @@ struct AttnParams {
     const int* grp;       // image groups (GRP kernels): -1 none; the tokens of a group see each other both ways
     bool static_lists;    // list_ptr delimits one item list per workgroup (a static schedule) instead of the eight shared lists
     bool clear_first;     // host side only: zero the cursors and counts in front of the pass (the entry point that allocates nothing)
-    int* land;            // ring kernel: [b] = waves of workgroup b that gave up a wait in this launch (the landing kernel then does b's list again and clears the word)
-    int spin_limit;       // ring kernel: polls of one wait before the wave gives up (a healthy wait takes a handful; tests set it to 1 to force the landing)
+    int spin_limit;       // ring kernel: polls of one wait before the wave gives up and its workgroup lands in the barrier-paced pass (a healthy
+                          // wait takes a handful; tests set it to 1 to force the landing)
 };
 
 // Softmax reference point.  The fast pass fixes each row's reference at the maximum of the first 32-key block in which

@@ -556,8 +556,8 @@ __global__ __launch_bounds__(256 * NHW) void tree_attn_kernel(const AttnParams p
 // Scratch memory of the entry point that allocates nothing (spinf_tree_attn_fwd_noalloc): list cursors, counts and the redo
 // list.  In host code this name is a stand-in, not a device address: hipGetSymbolAddress gives the address, per device.
 constexpr long NOALLOC_MAX_ITEMS = 1 << 16;                            // work items (query tiles x head groups) of one call
-// 64 cursors and counts | the redo list | the ring kernel's landing words (one per item list): 272.25 KiB per GPU, held until the process ends
-static __device__ __align__(256) int scratch[64 + NOALLOC_MAX_ITEMS + LAND_CAP];
+// 64 cursors and counts | the redo list: 256.25 KiB per GPU, held until the process ends
+static __device__ __align__(256) int scratch[64 + NOALLOC_MAX_ITEMS];
 
 namespace {
 
@@ -629,10 +629,9 @@ int acquire_block(long n_items, bool capturing, unsigned long long capture, hipS
     CursorBlock b;
     b.cap = n_items < (1 << 16) ? (1 << 16) : 2 * n_items;
     b.owner = stream;
-    e = hipMalloc((void**)&b.ptr, (64 + b.cap + LAND_CAP) * sizeof(int));
+    e = hipMalloc((void**)&b.ptr, (64 + b.cap) * sizeof(int));
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: hipMalloc: %s", hipGetErrorString(e));
     e = hipMemset(b.ptr, 0, 64 * sizeof(int));   // cursors, counts and the running totals at [NLIST + 3], [NLIST + 4] start at zero
-    if (e == hipSuccess) e = hipMemset(b.ptr + 64 + b.cap, 0, LAND_CAP * sizeof(int));   // and so do the landing words (the landing kernel clears what it finds)
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: cursor block: %s", hipGetErrorString(e));
     b.taken = true;
     s.blocks.push_back(b);
@@ -900,7 +899,6 @@ static int attn_fwd(const spinf_attn_args* a, void* stream, bool no_alloc) {
     p.row_of = a->row_of; p.kv_row0 = a->kv_row0;
     p.grp = a->grp;
     p.counters = counters;
-    p.land = counters + 64 + redo_cap;
     p.spin_limit = a->debug_expire > 0 ? a->debug_expire : (1 << 18);
     p.redo = counters + 64;
     const int blocks = a->n_lists > 0 ? a->n_lists : (int)(a->n_items < cus ? a->n_items : cus);

@@ -236,8 +236,8 @@ __device__ __forceinline__ void ring_store_rows(const AttnParams& p, const int w
 }
 
 // ---- after the list: the barrier-paced pass over single items.  One tile at a time into slot 0 of the ring, a workgroup barrier on
-// either side of its request, nothing overlapped, no spin anywhere.  It is the body of the landing kernel below (a kernel of its
-// own: what it needs in registers must not weigh on the ring loop's allocation, which has none to spare).  Two uses:
+// either side of its request, nothing overlapped, no spin anywhere.  Every workgroup of the ring kernel ends in it (normally with
+// nothing to do).  Two uses:
 //   * the exact recomputation.  Items in which some row met scores too far above its reference (normally none) are done again by the
 //     workgroup that owns them: classic online softmax over the same 32-key blocks in the same order (the reference is raised, and
 //     the accumulators rescaled, whenever a block maximum exceeds it by more than TAU_LAZY), the arithmetic of tree_attn_exact_kernel
@@ -428,6 +428,7 @@ __global__ __launch_bounds__(D == 512 ? 256 : 512) void tree_attn_ring_kernel(co
     __shared__ int sy_issued[MAX_SLOT];   // tile the slot was last recycled for (its DMA requested)
     __shared__ int sy_gen;             // descriptors written so far
     __shared__ int sy_abort;
+    __shared__ int sy_gave_up;         // waves that gave up a wait
     __shared__ int sy_ntiles;
     __shared__ int sy_redo[16];        // item sequence number + 1 of the last hand-over to the exact recomputation, per sequence number mod 16
     __shared__ int sy_nredo;           // items of this workgroup handed over so far (their indices: p.redo[lo ..])
@@ -480,7 +481,7 @@ __global__ __launch_bounds__(D == 512 ? 256 : 512) void tree_attn_ring_kernel(co
         if (threadIdx.x < NSLOT) *(int*)(ring + threadIdx.x * G::BUFB + G::KTILEB + G::VTILEB + 768) = -1;   // the slot's flag: no generation yet
     }
     if (threadIdx.x < 16) sy_redo[threadIdx.x] = 0;
-    if (threadIdx.x == 0) { sy_gen = 0; sy_abort = 0; sy_ntiles = 0; sy_nredo = 0; }
+    if (threadIdx.x == 0) { sy_gen = 0; sy_abort = 0; sy_gave_up = 0; sy_ntiles = 0; sy_nredo = 0; }
     __syncthreads();
 
     // descriptor generator (wave 0): items lo .. hi - 1, each item's plan entries in chunks of at most 64
@@ -842,7 +843,7 @@ __global__ __launch_bounds__(D == 512 ? 256 : 512) void tree_attn_ring_kernel(co
             store_rows(tz_done);
         }
     }
-    if (dead && fresh_lane_id() == 0) atomicAdd(&p.land[blockIdx.x], 1);   // the landing kernel will do this workgroup's list again
+    if (dead && fresh_lane_id() == 0) __hip_atomic_fetch_add(&sy_gave_up, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);   // (the list is done again below)
     __builtin_amdgcn_s_waitcnt(0x0f70);
 
     // ---- the exact recomputation.  Items in which some row met scores too far above its reference (normally none) are done
@@ -852,131 +853,18 @@ __global__ __launch_bounds__(D == 512 ? 256 : 512) void tree_attn_ring_kernel(co
     // overlapped: one tile at a time into slot 0, a workgroup barrier on either side of its request.  Whether an item comes here
     // depends on its own rows only, so a job's output does not depend on what it is packed with.
     __syncthreads();   // every wave is through with its list: the ring is free, the hand-overs are all in
-    const int n_redo = __builtin_amdgcn_readfirstlane(lds_load(&sy_nredo));
-    if (n_redo == 0 || __builtin_amdgcn_readfirstlane(lds_load(&sy_abort)) != 0) return;
-#pragma unroll 1
-    for (int r = 0; r < n_redo; r++) {
-        const int idx = __builtin_amdgcn_readfirstlane(__hip_atomic_load(&p.redo[lo + r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-        const int4 itv = p.items[idx];
-        const int it_t = __builtin_amdgcn_readfirstlane(itv.x), it_e0 = __builtin_amdgcn_readfirstlane(itv.y), it_z = __builtin_amdgcn_readfirstlane(itv.z);
-        const int ne = it_z & 0xfffff;
-        const int tz = it_t | (int)((unsigned)it_z >> 20 << 20);
-        const int kvh = (int)((unsigned)it_z >> 20) * HPI / p.group;
-        load_q(tz);
-        reset_acc();
-#pragma unroll 1
-        for (int e = 0; e < ne; e++) {
-            const int kt = __builtin_amdgcn_readfirstlane(p.kv_idx[it_e0 + e]);
-            const unsigned bits = (unsigned)__builtin_amdgcn_readfirstlane((int)p.kv_bits[it_e0 + e]);
-            __syncthreads();   // everyone is through with the slot
-            if (L.w == 0) {
-                using GK = Geo<D, TK>;
-                const int lane = fresh_lane_id();
-                const unsigned lane_k = (unsigned)((lane / GK::CPR) * GK::NREG * p.k_tok * 2 + (lane % GK::CPR) * 16);
-                const unsigned lane_v = (unsigned)((lane / GK::CPR) * GK::NREG * p.v_tok * 2 + (lane % GK::CPR) * 16);
-                issue_tile_wave<D, WIN>(p, lds_addr(ring), kt, kvh, 0, lane, lane_k, lane_v);
-            }
-            __builtin_amdgcn_s_waitcnt(0x0f70);   // the tile has landed (and this wave's queries)
-            __syncthreads();
-            if (!((bits >> (2 * L.wr)) & 1u)) continue;   // (wave-uniform; the barriers above are passed by every wave)
-            const int ln = fresh_lane_id();
-            const char* krow = ring + G::K::k_off(ln & 31) + 16 * (ln >> 5);
-            const char* vrow = ring + G::KTILEB + G::V::v_off(4 * (ln >> 5) + ((ln >> 2) & 3)) + 32 * ((ln >> 4) & 1) + 8 * (ln & 3);
-            // (the scheduling barriers keep the phases apart, as in ring_paced_pass: no vector write of a P fragment directly in
-            // front of the assembly MFMA that reads it)
-            f32x16 sa;
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int x = 0; x < NS; x++) {
-                const bf16x8 kf = *(const bf16x8*)(krow + 32 * x);
-                if (x == 0) qk_first(sa, kf, qf[x]);
-                else if (x == NS - 1) qk_last(sa, kf, qf[x]);
-                else qk_next(sa, kf, qf[x]);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            if ((bits >> (8 + 2 * L.wr)) & 1u) {
-                f32x16 sm[1] = {sa};
-                const int tok = (tz & 0xfffff) * SPINF_QTILE + 32 * L.wr + (ln & 31);
-                apply_mask<1, WIN, 0, TK>(sm, (const int*)(ring + G::KTILEB + G::VTILEB), kt, 0, ln >> 5, tok, art_q, pos_q, p.window);
-                sa = sm[0];
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            bf16x8 pb[2];
-            {
-                float mx = sa[0];
-#pragma unroll
-                for (int i2 = 1; i2 < 16; i2++) mx = fmaxf(mx, sa[i2]);
-                mx = lane32_max(mx);
-                const float tm = mx * p.c;
-                const bool up = tm > M + TAU_LAZY;
-                const float mn = up ? tm : M;
-                const float alpha = up ? __builtin_amdgcn_exp2f(M - mn) : 1.0f;
-                if (__builtin_amdgcn_ballot_w64(up && M != -INFINITY) != 0) {   // rows without a key so far hold zeros
-                    asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");   // the last MFMAs' results -> v_accvgpr_read
-                    acc_scale<NDT>(alpha);
-                    asm volatile("s_nop 3" ::: "memory");                // v_accvgpr_write -> MFMA srcC
-                }
-                l *= alpha;
-                M = mn;
-                const float ms = mn == -INFINITY ? 0.f : mn;
-                float sum = 0.f;
-#pragma unroll
-                for (int i2 = 0; i2 < 16; i2++) {
-                    const float pr = __builtin_amdgcn_exp2f(__builtin_fmaf(sa[i2], p.c, -ms));
-                    sum += pr;
-                    pb[i2 >> 3][i2 & 7] = (__bf16)pr;
-                }
-                l += sum;
-            }
-            __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): the softmax phase ends here, the waits below are for V fragments only
-            __builtin_amdgcn_sched_barrier(0);
-            auto step = [&](auto f_c) __attribute__((always_inline)) {
-                constexpr int f = decltype(f_c)::value;
-                const char* vp = vrow + G::V::v_off(16 * (f / NDT)) + 64 * (f % NDT);
-                const s16x4 lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)vp);
-                const s16x4 hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vp + G::V::v_off(8)));
-                const bf16x8 a = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo4, hi4, 0, 1, 2, 3, 4, 5, 6, 7));
-                acc_mfma<f % NDT>(a, pb[f / NDT]);
-                __builtin_amdgcn_sched_barrier(0);
-            };
-            pv_steps<NVF>(step);
-        }
-        store_rows(tz);
-    }
-    if (threadIdx.x == 0) atomicAdd(&p.counters[NLIST + 3], n_redo);   // running total, for spinf_attn_exact_items
-    __builtin_amdgcn_s_waitcnt(0x0f70);
-}
-
-// The landing kernel: launched behind every launch of the ring kernel, a few workgroups that go through the ring kernel's workgroups
-// b = 0 .. n_wg - 1 between them.  Where b left no word (p.land[b] == 0: every launch but a faulty one) there is nothing to do;
-// otherwise b's whole list is computed again.  (A grid as wide as the ring kernel's cost 4.1 us per call just to start and end.)
-constexpr int LANDING_WGS = 16;
-template <int D, bool WIN>
-__global__ __launch_bounds__(D == 512 ? 256 : 512) void tree_attn_ring_landing_kernel(const AttnParams p, const int n_wg) {
-    using S = RingShape<D>;
-    using G = TileGeo<D, S::TK, D>;
-    __shared__ __attribute__((aligned(16))) char ring[G::BUFB];
-    __shared__ __attribute__((aligned(16))) char stage_all[S::NW * 32 * SROW];
-    __shared__ int sy_nredo, sy_vote;
-    // every launch but a faulty one ends here: one word per thread, all of them zero
-    int mine = 0;
-    for (int b = blockIdx.x + gridDim.x * threadIdx.x; b < n_wg; b += gridDim.x * blockDim.x) mine |= p.land[b];
-    if (__syncthreads_or(mine) == 0) return;
-#pragma unroll 1
-    for (int b = blockIdx.x; b < n_wg; b += gridDim.x) {
-        const int gave_up = __builtin_amdgcn_readfirstlane(p.land[b]);   // waves of the ring kernel's workgroup b that gave up a wait
-        if (gave_up == 0) continue;
-        const int lo = p.list_ptr[b], hi = p.list_ptr[b + 1];
-        __syncthreads();   // (the previous list's last reads of the words below)
+    const bool gave_up = __builtin_amdgcn_readfirstlane(lds_load(&sy_abort)) != 0;
+    if (!gave_up && __builtin_amdgcn_readfirstlane(lds_load(&sy_nredo)) == 0) return;
+    __shared__ int sy_vote;
+    if (gave_up) {   // some wave gave up a wait: the whole list again, one tile at a time between barriers (same bits)
         if (threadIdx.x == 0) {
-            sy_nredo = 0;   // (the ring kernel's workgroup left without its exact recomputations: whatever the list needs is found again here)
-            sy_vote = 0;
-            atomicAdd(&p.counters[NLIST + 4], gave_up);   // running total, for spinf_attn_ring_aborts
+            sy_nredo = 0;   // (whatever the list needs recomputed exactly is found again on the way)
+            atomicAdd(&p.counters[NLIST + 4], lds_load(&sy_gave_up));   // running total, for spinf_attn_ring_aborts
         }
-        __syncthreads();
-        ring_paced_pass<D, WIN>(p, ring, stage_all, &sy_nredo, &sy_vote, lo, hi, lo);
-        if (threadIdx.x == 0) p.land[b] = 0;   // (the word is per launch: the next one starts clean)
     }
+    if (threadIdx.x == 0) sy_vote = 0;
+    __syncthreads();
+    ring_paced_pass<D, WIN>(p, ring, stage_all, &sy_nredo, &sy_vote, lo, gave_up ? hi : lo, lo);
 }
 
 template <int D, bool WIN>
@@ -984,9 +872,6 @@ int launch_ring_t(const AttnParams& p, int n_wg, hipStream_t stream) {
     hipLaunchKernelGGL((tree_attn_ring_kernel<D, WIN>), dim3(n_wg), dim3(D == 512 ? 256 : 512), 0, stream, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: launch (ring kernel): %s", hipGetErrorString(e));
-    hipLaunchKernelGGL((tree_attn_ring_landing_kernel<D, WIN>), dim3(n_wg < LANDING_WGS ? n_wg : LANDING_WGS), dim3(D == 512 ? 256 : 512), 0, stream, p, n_wg);
-    e = hipGetLastError();
-    if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "tree_attn: launch (landing kernel): %s", hipGetErrorString(e));
     return SPINF_OK;
 }
 

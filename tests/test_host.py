@@ -181,6 +181,12 @@ def test_build_scan_of_the_ring_assembly_catches_what_it_is_there_for():
         ge._scan_ring_assembly(listing("v_mov_b32_e32 v2, v9") + mfma)
     with pytest.raises(RuntimeError, match="accumulation register of its own"):
         ge._scan_ring_assembly(listing("v_accvgpr_write_b32 a130, v3"))
+    reload = ["_ZN12_GLOBAL__N_121tree_attn_ring_kernelILi256ELb0EEEv10AttnParams: ; @kernel", ".LBB0_7:    ;   in Loop: Header=BB0_3 Depth=2",
+              "\tscratch_load_dwordx4 v[4:7], off, off offset:16"]
+    with pytest.raises(RuntimeError, match="16-byte reload"):
+        ge._scan_ring_assembly(reload)
+    ge._scan_ring_assembly([reload[0], ".LBB0_7:", reload[2]])                                  # outside any loop: tolerated
+    ge._scan_ring_assembly([reload[0], reload[1], "\tscratch_load_dword v4, off, off offset:16"])   # a single register: tolerated
     meta = ["    .name:           _ZN12_GLOBAL__N_121tree_attn_ring_kernelILi256ELb0EEEv10AttnParams", "    .vgpr_spill_count: 16"]
     with pytest.raises(RuntimeError, match="spills 16"):
         ge._scan_ring_assembly(meta)
