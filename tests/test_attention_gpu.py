@@ -702,7 +702,7 @@ def test_several_calls_recorded_by_one_capture_share_the_streams_block(dev, ring
 def test_a_wave_that_gives_up_a_wait_costs_time_not_rows(dev, d, limit, wide, monkeypatch):
     """the decoupled kernel's landing: the waves are told (from the host, spinf_attn_args.debug_expire) to give up a wait after
     `limit` polls instead of 2^18, so every wave that has to wait for a tile at all gives up, as after a real time-out; its
-    workgroup leaves the ring and the landing kernel computes that workgroup's list again, one tile at a time between barriers.
+    workgroup leaves the ring and computes its list again before it ends, one tile at a time between barriers.
     Every kernel exits normally, the aborts are counted, and the output equals the lockstep kernel's bit for bit, also where items
     go on to the exact recomputation (wide) and with a window."""
     from spinf_serve_amd import attention
