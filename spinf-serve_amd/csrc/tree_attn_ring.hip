@@ -25,7 +25,8 @@
 //     and it requests its next queries right away.
 //
 // Every wait is a bounded spin on an LDS word; a wave that runs out of spins sets the workgroup's abort flag (and a counter the
-// host can read), which makes every wave of the workgroup leave at its next wait.
+// host can read), which makes every wave of the workgroup leave the ring at its next wait; the workgroup then computes its list
+// again, one tile at a time between barriers (ring_paced_pass): the same bits, later.
 #include <hip/hip_runtime.h>
 
 #include <type_traits>
@@ -846,12 +847,9 @@ __global__ __launch_bounds__(D == 512 ? 256 : 512) void tree_attn_ring_kernel(co
     if (dead && fresh_lane_id() == 0) __hip_atomic_fetch_add(&sy_gave_up, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);   // (the list is done again below)
     __builtin_amdgcn_s_waitcnt(0x0f70);
 
-    // ---- the exact recomputation.  Items in which some row met scores too far above its reference (normally none) are done
-    // again here, by the workgroup that owns them, after its list: classic online softmax over the same 32-key blocks in the same
-    // order (the reference is raised, and the accumulators rescaled, whenever a block maximum exceeds it by more than TAU_LAZY),
-    // the arithmetic of tree_attn_exact_kernel (tree_attn.hip) step for step, so the two give the same bits.  Nothing is
-    // overlapped: one tile at a time into slot 0, a workgroup barrier on either side of its request.  Whether an item comes here
-    // depends on its own rows only, so a job's output does not depend on what it is packed with.
+    // ---- after the list: normally nothing.  Items in which some row met scores too far above its reference are done again, exactly,
+    // by ring_paced_pass; and if some wave gave up a wait (every wave has then left the ring), so is the whole list, with the ring
+    // pass's own arithmetic: an abort costs time, never rows.
     __syncthreads();   // every wave is through with its list: the ring is free, the hand-overs are all in
     const bool gave_up = __builtin_amdgcn_readfirstlane(lds_load(&sy_abort)) != 0;
     if (!gave_up && __builtin_amdgcn_readfirstlane(lds_load(&sy_nredo)) == 0) return;
