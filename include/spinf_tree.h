@@ -336,8 +336,15 @@ int spinf_diag_mfma_hazard(int32_t iters, int32_t workgroups, int32_t* out, void
  * (four in flight), and the output stores in the kernel's pattern; out comes back as 1.0 on the stream's rows.  status: 2 device
  * ints, zeroed by the caller: [0] += waves that gave up a bounded wait (never), [1] += tiles seen landed (the schedule's plan
  * entries x head groups).  parts: 3 = all of it, 1 = the K / V tiles only, 2 = the queries and outputs only (out is written
- * with 2 and 3), 5 / 7 = as 1 / 3 with each tile's requests dealt out over the eight waves instead of made by one; nslot (1 .. 4): ring slots in use, i.e. tile requests in flight (the kernel has 4).  Its time is the floor that data movement alone sets for that kernel on that schedule. */
+ * with 2 and 3), 5 / 7 = as 1 / 3 with each tile's requests dealt out over the eight waves instead of made by one; nslot (1 .. 4):
+ * ring slots in use, i.e. tile requests in flight (the kernel has 4).  Its time is the floor that data movement alone sets for that
+ * kernel on that schedule. */
 int spinf_diag_attn_stream(const spinf_attn_args* args, int32_t parts, int32_t nslot, int32_t* status, void* stream);
+
+/* For bindings in other languages (no counterpart in the reference): sizes[0..6] = sizeof of spinf_attn_args, spinf_gdn_args,
+ * spinf_gdn_pre_args, spinf_gdn_gate_args, spinf_lm_args, spinf_lm_head_args, spinf_xdec_args as this library was built (n must be
+ * 7): a binding compares them with its own mirrors of the structures before its first call. */
+int spinf_struct_sizes(int64_t* sizes, int32_t n);
 
 #ifdef __cplusplus
 }

@@ -107,6 +107,14 @@ def load_library():
     if not os.path.exists(path):
         raise RuntimeError(f"{path} is missing: build the HIP library first (python __graft_entry__.py); there is no fallback path")
     lib = C.CDLL(path)
+    try:
+        return _bind(lib, path)
+    except AttributeError as e:   # a symbol of include/spinf_tree.h that this library does not export
+        raise RuntimeError(f"{path} is of another version than this package ({e}): rebuild it (python __graft_entry__.py); there is no fallback path") from None
+
+
+def _bind(lib, path):
+    global _LIB
     lib.spinf_last_error.restype = C.c_char_p
     lib.spinf_version.restype = C.c_int
     lib.spinf_tileplan_build.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.POINTER(C.c_void_p)]
@@ -139,12 +147,19 @@ def load_library():
     lib.spinf_lm_head_fwd.argtypes = [C.POINTER(LmHeadArgs), C.c_void_p]
     lib.spinf_diag_lds_order.argtypes = [C.c_int32, C.c_int32, C.c_void_p, C.c_void_p]
     lib.spinf_diag_mfma_hazard.argtypes = [C.c_int32, C.c_int32, C.c_void_p, C.c_void_p]
+    lib.spinf_struct_sizes.argtypes = [C.POINTER(C.c_int64), C.c_int32]
     lib.spinf_diag_attn_stream.argtypes = [C.POINTER(AttnArgs), C.c_int32, C.c_int32, C.c_void_p, C.c_void_p]
     lib.spinf_xdecode_plan.argtypes = [C.POINTER(XdecArgs), C.POINTER(C.c_int32), C.POINTER(C.c_int64)]
     lib.spinf_xdecode_attn_fwd.argtypes = [C.POINTER(XdecArgs), C.c_void_p]
     lib.spinf_xdecode_tiles.argtypes = [C.POINTER(XdecArgs), C.POINTER(C.c_int32)]
-    for name in ("spinf_diag_attn_stream", "spinf_diag_lds_order", "spinf_diag_mfma_hazard", "spinf_diag_mfma_rate", "spinf_lm_head_workspace", "spinf_lm_head_fwd", "spinf_gdn_plan_build", "spinf_gdn_plan_counts", "spinf_gdn_plan_export", "spinf_tileplan_schedule_static", "spinf_attn_ring_aborts", "spinf_tileplan_build", "spinf_tileplan_build_groups", "spinf_tileplan_build_ktile", "spinf_tileplan_counts", "spinf_tileplan_export", "spinf_tileplan_schedule", "spinf_tileplan_row0", "spinf_tree_attn_fwd", "spinf_tree_attn_fwd_noalloc", "spinf_attn_exact_items", "spinf_gdn_fwd", "spinf_gdn_prologue", "spinf_gdn_gate", "spinf_lm_logprobs", "spinf_xdecode_plan", "spinf_xdecode_tiles", "spinf_xdecode_attn_fwd"):
+    for name in ("spinf_struct_sizes", "spinf_diag_attn_stream", "spinf_diag_lds_order", "spinf_diag_mfma_hazard", "spinf_diag_mfma_rate", "spinf_lm_head_workspace", "spinf_lm_head_fwd", "spinf_gdn_plan_build", "spinf_gdn_plan_counts", "spinf_gdn_plan_export", "spinf_tileplan_schedule_static", "spinf_attn_ring_aborts", "spinf_tileplan_build", "spinf_tileplan_build_groups", "spinf_tileplan_build_ktile", "spinf_tileplan_counts", "spinf_tileplan_export", "spinf_tileplan_schedule", "spinf_tileplan_row0", "spinf_tree_attn_fwd", "spinf_tree_attn_fwd_noalloc", "spinf_attn_exact_items", "spinf_gdn_fwd", "spinf_gdn_prologue", "spinf_gdn_gate", "spinf_lm_logprobs", "spinf_xdecode_plan", "spinf_xdecode_tiles", "spinf_xdecode_attn_fwd"):
         getattr(lib, name).restype = C.c_int
+    # the argument blocks above mirror include/spinf_tree.h: a library built from another version of the header would read them wrongly
+    mirrors = (AttnArgs, GdnArgs, GdnPreArgs, GdnGateArgs, LmArgs, LmHeadArgs, XdecArgs)
+    sizes = (C.c_int64 * len(mirrors))()
+    if lib.spinf_struct_sizes(sizes, len(mirrors)) != 0 or list(sizes) != [C.sizeof(m) for m in mirrors]:
+        raise RuntimeError(f"{path}: argument blocks of {list(sizes)} bytes, this package's are {[C.sizeof(m) for m in mirrors]}: "
+                           "the library and the package are of different versions (rebuild: python __graft_entry__.py); no fallback")
     _LIB = lib
     return lib
 

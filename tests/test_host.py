@@ -631,3 +631,25 @@ def test_gdn_plan_compiler_edge_cases():
         sa.tree_plan(prev, real[:2].astype(bool), "cpu")
     with pytest.raises(ValueError):
         sa.tree_plan(prev, real.astype(bool), "cpu", path="sideways")
+
+
+def test_argument_blocks_have_the_size_the_library_was_built_with(lib, monkeypatch):
+    """spinf_struct_sizes: the ctypes mirrors of the seven argument blocks against sizeof in the built library (load_library checks the
+    same at load time and refuses a library of another version instead of passing it misread arguments)"""
+    import ctypes as C
+
+    from spinf_serve_amd import _lib
+
+    sizes = (C.c_int64 * 7)()
+    assert lib.spinf_struct_sizes(sizes, 7) == 0
+    mirrors = (_lib.AttnArgs, _lib.GdnArgs, _lib.GdnPreArgs, _lib.GdnGateArgs, _lib.LmArgs, _lib.LmHeadArgs, _lib.XdecArgs)
+    assert list(sizes) == [C.sizeof(m) for m in mirrors]
+    assert lib.spinf_struct_sizes(sizes, 6) == -1 and b"7 sizes" in lib.spinf_last_error()
+
+    class Grown(C.Structure):
+        _fields_ = list(_lib.LmHeadArgs._fields_) + [("more", C.c_int64)]
+
+    monkeypatch.setattr(_lib, "_LIB", None)
+    monkeypatch.setattr(_lib, "LmHeadArgs", Grown)
+    with pytest.raises(RuntimeError, match="different versions"):
+        _lib.load_library()
