@@ -1,6 +1,6 @@
 """Benchmark of the tree-mask packed-prefill attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K=200] [--warmup W=100] [--workload C2|C2_stream|C3|C4|C5|XDEC|LM|LM_head|copy|mfma_peak ...] [--seed S] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K=200] [--warmup W=100] [--workload C2|C2_stream|C3|C4|C5|XDEC|LM|LM_head|copy|mfma_peak|mfma_valu ...] [--seed S] [--no-cpu]
 
 A step is one pass of the attention op (one layer's call through the C ABI) over one packed synthetic stream already
 resident in HBM; the tile plan is compiled once per stream, outside the timed region, as the reference builds its block
@@ -39,6 +39,7 @@ WORKLOADS = {
     "XDEC_long": "extraction-decode attention step: 64 groups x (U{1024..4096}-token prefix + 8 slots with templates of U{8..16} tokens) x 6 beams, 33 generated entries (step 32), 16 / 8 heads, head_dim 256, global layer",
     "XDEC_qwen": "XDEC's step at the Qwen-hybrid attention geometry: 24 query heads / 4 KV heads, head_dim 256 (288 rows per (group, kv head): three row chunks)",
     "XDEC_512": "XDEC's step at the head geometry of the Gemma-4 full-attention layers: 16 query heads / 1 KV head, head_dim 512 (output computed 256 head dims at a time, two launches)",
+    "mfma_valu": "rounds of one v_mfma_f32_32x32x16_bf16 and nv independent vector instructions per wave, one, two and four waves per SIMD: clocks per round of a wave and of its SIMD (spinf_diag_mfma_valu)",
     "mfma_peak": "pure v_mfma_f32_32x32x16_bf16 loop, one workgroup of eight waves on every compute unit, operands in registers: the yardstick for what the matrix cores sustain on this part",
     "LM_head": "lm head of one chunk of 1,024 read rows gathered from a 65,536-row stream: h[sel] W^T (hidden 2,560, vocabulary 262,144, bf16 MFMA, fp32 logits) + soft-capping (30) + log-softmax + 8 option columns in one pass, no logits matrix",
     "LM": "lm head read-out of one chunk of 1,024 read rows: soft-capping (30) + log-softmax over 262,144 fp32 logits + 8 option columns",
@@ -250,6 +251,30 @@ def main():
                               "lds_fill_gbs": tile_bytes / (ms * 1e-3) / 1e9, "tiles_only_ms": ms_tiles, "tiles_only_ms_by_requests_in_flight": by_slots, "tiles_only_ms_requests_dealt_over_the_waves": dealt, "kernel_ms_requests_dealt_over_the_waves": ms_dealt, "queries_and_outputs_only_ms": ms_rows, "product_kernel_ms": ms2, "product_over_floor": ms2 / ms,
                               "frac_of_bf16_peak_if_the_product_ran_at_this_floor": cfg.flops(None) / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS})
         assert torch.equal(sa.tree_attn(q, k, v, mask, cfg.scale), want)
+        print(json.dumps(line))
+        return
+
+    if args.workload == "mfma_valu":
+        import ctypes as C
+
+        from spinf_serve_amd import _lib
+
+        lib = _lib.load_library()
+        iters = 20000
+        table = {}
+        for kind, kname in ((0, "v_fma_f32"), (1, "v_exp_f32")):
+            for wps in (1, 2, 4):
+                for nv in (0, 2, 4, 6, 8, 12, 16):
+                    out = torch.zeros(2 * 4 * wps, dtype=torch.int64, device=dev)
+                    _lib.check(lib.spinf_diag_mfma_valu(nv, kind, wps, iters, out.data_ptr(), C.c_void_p(torch.cuda.current_stream().cuda_stream)), "spinf_diag_mfma_valu")
+                    torch.cuda.synchronize()
+                    t = out.cpu().view(-1, 2)
+                    simd0 = t[0::4]   # the waves of SIMD 0: wave 0 (the oldest, favoured by the arbiter), 4, 8, 12
+                    table[f"{kname} nv={nv} waves_per_simd={wps}"] = {
+                        "clocks_per_round_oldest_wave": round(float(simd0[0, 1] - simd0[0, 0]) / iters, 1),
+                        "clocks_per_mfma_simd": round(float(simd0[:, 1].max() - simd0[:, 0].min()) / (iters * wps), 1)}
+        line.update(metric="clocks per MFMA of a SIMD, MFMA + nv vector instructions per round", unit="clocks", value=table["v_fma_f32 nv=6 waves_per_simd=2"]["clocks_per_mfma_simd"],
+                    higher_is_better=False, ms_per_step=None, dtype="bf16", config={"workload": WORKLOADS["mfma_valu"], "iters": iters}, table=table)
         print(json.dumps(line))
         return
 

@@ -330,6 +330,12 @@ int spinf_diag_lds_order(int32_t iters, int32_t workgroups, int32_t* out, void* 
  * lgkmcnt(0), two of them, a satisfied s_waitcnt vmcnt(0), v_nop, s_waitcnt + s_nop 0; [20] += workgroups (of eight waves) that
  * ran.  out: 21 device ints. */
 int spinf_diag_mfma_hazard(int32_t iters, int32_t workgroups, int32_t* out, void* stream);
+/* Diagnostics (no counterpart in the reference): do a wave's vector instructions run in the shadow of its own MFMAs?  One workgroup
+ * per compute unit, waves_per_simd (1, 2 or 4) waves on every SIMD, each wave iters rounds of { one v_mfma_f32_32x32x16_bf16 on one
+ * accumulator, nv (0, 2, 4, 6, 8, 12 or 16) independent vector instructions: v_fma_f32 (kind 0) or v_exp_f32 (kind 1) }.  out:
+ * 2 x 4 x waves_per_simd device int64: the clock before and after the loop of every wave of workgroup 0 (wave w = SIMD w % 4).
+ * Clocks per round of a wave alone on its SIMD: 36 + 4 nv measured (36 + 8 nv for v_exp_f32), i.e. nothing runs in the shadow. */
+int spinf_diag_mfma_valu(int32_t nv, int32_t kind, int32_t waves_per_simd, int32_t iters, int64_t* out, void* stream);
 /* Diagnostics (no counterpart in the reference): the byte pattern of spinf_tree_attn_fwd's kernel with decoupled waves, with
  * nothing computed.  args as for a head-dim-256 call with a static schedule over 32-key entries (n_lists > 0, ktile 32, stream
  * layout, no image groups): per work item the query loads, every K / V tile through a four-slot LDS ring by the same DMA requests

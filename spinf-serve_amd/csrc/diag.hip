@@ -40,6 +40,51 @@ __global__ __launch_bounds__(512) void mfma_rate_kernel(const long iters, float*
     out[(long)blockIdx.x * blockDim.x + threadIdx.x] = s;   // keeps the loop alive
 }
 
+// ---- do a wave's vector instructions run in the shadow of its own MFMAs?
+// Every wave runs iters x { one v_mfma_f32_32x32x16_bf16 (32 clocks of the matrix pipe) on a single accumulator, then NV vector
+// instructions that depend on nothing the MFMA touches: v_fma_f32 (KIND 0) or v_exp_f32 (KIND 1) }, with one, two or four waves per
+// SIMD.  Every wave of workgroup 0 records the clock before and after its loop (s_memtime ticks, which count core clocks here: the bare
+// MFMA chain reads 32.3 per MFMA).  If the vector instructions ran under the MFMA a wave would need max(36, 4 + 4 NV) clocks per round;
+// measured on MI355X it needs 36 + 4 NV (8 NV for v_exp_f32): they do not, the two add up, and only ANOTHER wave of the SIMD can use
+// the vector ALU while an MFMA runs.  This is what bounds the attention kernels at head dim 128, where a 32 x 32 block is 16 MFMAs
+// (512 clocks) and about as many clocks of softmax per wave.
+template <int NV, int KIND>
+__global__ __launch_bounds__(1024) void mfma_valu_kernel(const int iters, long long* out) {
+    bf16x8 a, b;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        a[i] = (__bf16)(0.001f * (float)((threadIdx.x + i) & 15));
+        b[i] = (__bf16)(0.002f * (float)((threadIdx.x * 3 + i) & 7));
+    }
+    f32x16 acc;
+#pragma unroll
+    for (int i = 0; i < 16; i++) acc[i] = 0.f;
+    float v[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) v[i] = 0.5f + 0.01f * (float)i + 0.0001f * (float)(threadIdx.x & 63);
+    const float c = 0.999f, d = 0.0001f;
+    __syncthreads();
+    const long long t0 = __builtin_readcyclecounter();
+    for (int it = 0; it < iters; it++) {
+        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
+#pragma unroll
+        for (int j = 0; j < NV; j++) {
+            if (KIND == 0) asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(v[j % 16]) : "v"(c), "v"(d));
+            else asm volatile("v_exp_f32 %0, %0" : "+v"(v[j % 16]));
+        }
+    }
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");   // the last MFMA's result -> vector ALU reads (assembly: the compiler adds no wait states)
+    const long long t1 = __builtin_readcyclecounter();
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) sum += acc[i] + v[i];
+    if (sum == 12345.678f) out[0] = 0;   // keeps the loop alive (never true)
+    if (blockIdx.x == 0 && (threadIdx.x & 63) == 0) {
+        out[2 * (threadIdx.x >> 6)] = t0;
+        out[2 * (threadIdx.x >> 6) + 1] = t1;
+    }
+}
+
 // ---- do LDS reads of different kinds return in the order they were issued?
 // The attention and scan kernels mix three kinds of LDS reads in one wave: transposing 8-byte reads (ds_read_b64_tr_b16: V^T
 // fragments), 16-byte reads (K fragments, key metadata, descriptors) and 4-byte reads, and wait for them with partial counts
@@ -452,6 +497,35 @@ extern "C" int spinf_diag_mfma_hazard(int32_t iters, int32_t workgroups, int32_t
     hipLaunchKernelGGL(mfma_hazard_kernel, dim3(workgroups), dim3(512), 0, (hipStream_t)stream, (int)iters, (int*)out);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "diag_mfma_hazard: launch: %s", hipGetErrorString(e));
+    return SPINF_OK;
+}
+
+template <int KIND>
+static void launch_mfma_valu(int nv, int wgs, int threads, int iters, long long* out, hipStream_t stream) {
+    switch (nv) {
+        case 0: hipLaunchKernelGGL((mfma_valu_kernel<0, KIND>), dim3(wgs), dim3(threads), 0, stream, iters, out); break;
+        case 2: hipLaunchKernelGGL((mfma_valu_kernel<2, KIND>), dim3(wgs), dim3(threads), 0, stream, iters, out); break;
+        case 4: hipLaunchKernelGGL((mfma_valu_kernel<4, KIND>), dim3(wgs), dim3(threads), 0, stream, iters, out); break;
+        case 6: hipLaunchKernelGGL((mfma_valu_kernel<6, KIND>), dim3(wgs), dim3(threads), 0, stream, iters, out); break;
+        case 8: hipLaunchKernelGGL((mfma_valu_kernel<8, KIND>), dim3(wgs), dim3(threads), 0, stream, iters, out); break;
+        case 12: hipLaunchKernelGGL((mfma_valu_kernel<12, KIND>), dim3(wgs), dim3(threads), 0, stream, iters, out); break;
+        default: hipLaunchKernelGGL((mfma_valu_kernel<16, KIND>), dim3(wgs), dim3(threads), 0, stream, iters, out); break;
+    }
+}
+
+extern "C" int spinf_diag_mfma_valu(int32_t nv, int32_t kind, int32_t waves_per_simd, int32_t iters, int64_t* out, void* stream) {
+    if ((nv != 0 && nv != 2 && nv != 4 && nv != 6 && nv != 8 && nv != 12 && nv != 16) || kind < 0 || kind > 1)
+        return spinf_fail(SPINF_E_ARG, "diag_mfma_valu: nv %d not in {0, 2, 4, 6, 8, 12, 16} or kind %d not in {0, 1}", nv, kind);
+    if ((waves_per_simd != 1 && waves_per_simd != 2 && waves_per_simd != 4) || iters <= 0 || iters > (1 << 22) || !out)
+        return spinf_fail(SPINF_E_ARG, "diag_mfma_valu: waves per SIMD in {1, 2, 4}, iters in 1 .. 2^22, out not null");
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return spinf_fail(SPINF_E_HIP, "diag_mfma_valu: no device");
+    const int threads = 256 * waves_per_simd;
+    if (kind == 0) launch_mfma_valu<0>(nv, prop.multiProcessorCount, threads, iters, (long long*)out, (hipStream_t)stream);
+    else launch_mfma_valu<1>(nv, prop.multiProcessorCount, threads, iters, (long long*)out, (hipStream_t)stream);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "diag_mfma_valu: launch: %s", hipGetErrorString(e));
     return SPINF_OK;
 }
 

@@ -147,12 +147,13 @@ def _bind(lib, path):
     lib.spinf_lm_head_fwd.argtypes = [C.POINTER(LmHeadArgs), C.c_void_p]
     lib.spinf_diag_lds_order.argtypes = [C.c_int32, C.c_int32, C.c_void_p, C.c_void_p]
     lib.spinf_diag_mfma_hazard.argtypes = [C.c_int32, C.c_int32, C.c_void_p, C.c_void_p]
+    lib.spinf_diag_mfma_valu.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p]
     lib.spinf_struct_sizes.argtypes = [C.POINTER(C.c_int64), C.c_int32]
     lib.spinf_diag_attn_stream.argtypes = [C.POINTER(AttnArgs), C.c_int32, C.c_int32, C.c_void_p, C.c_void_p]
     lib.spinf_xdecode_plan.argtypes = [C.POINTER(XdecArgs), C.POINTER(C.c_int32), C.POINTER(C.c_int64)]
     lib.spinf_xdecode_attn_fwd.argtypes = [C.POINTER(XdecArgs), C.c_void_p]
     lib.spinf_xdecode_tiles.argtypes = [C.POINTER(XdecArgs), C.POINTER(C.c_int32)]
-    for name in ("spinf_struct_sizes", "spinf_diag_attn_stream", "spinf_diag_lds_order", "spinf_diag_mfma_hazard", "spinf_diag_mfma_rate", "spinf_lm_head_workspace", "spinf_lm_head_fwd", "spinf_gdn_plan_build", "spinf_gdn_plan_counts", "spinf_gdn_plan_export", "spinf_tileplan_schedule_static", "spinf_attn_ring_aborts", "spinf_tileplan_build", "spinf_tileplan_build_groups", "spinf_tileplan_build_ktile", "spinf_tileplan_counts", "spinf_tileplan_export", "spinf_tileplan_schedule", "spinf_tileplan_row0", "spinf_tree_attn_fwd", "spinf_tree_attn_fwd_noalloc", "spinf_attn_exact_items", "spinf_gdn_fwd", "spinf_gdn_prologue", "spinf_gdn_gate", "spinf_lm_logprobs", "spinf_xdecode_plan", "spinf_xdecode_tiles", "spinf_xdecode_attn_fwd"):
+    for name in ("spinf_struct_sizes", "spinf_diag_attn_stream", "spinf_diag_lds_order", "spinf_diag_mfma_hazard", "spinf_diag_mfma_valu", "spinf_diag_mfma_rate", "spinf_lm_head_workspace", "spinf_lm_head_fwd", "spinf_gdn_plan_build", "spinf_gdn_plan_counts", "spinf_gdn_plan_export", "spinf_tileplan_schedule_static", "spinf_attn_ring_aborts", "spinf_tileplan_build", "spinf_tileplan_build_groups", "spinf_tileplan_build_ktile", "spinf_tileplan_counts", "spinf_tileplan_export", "spinf_tileplan_schedule", "spinf_tileplan_row0", "spinf_tree_attn_fwd", "spinf_tree_attn_fwd_noalloc", "spinf_attn_exact_items", "spinf_gdn_fwd", "spinf_gdn_prologue", "spinf_gdn_gate", "spinf_lm_logprobs", "spinf_xdecode_plan", "spinf_xdecode_tiles", "spinf_xdecode_attn_fwd"):
         getattr(lib, name).restype = C.c_int
     # the argument blocks above mirror include/spinf_tree.h: a library built from another version of the header would read them wrongly
     mirrors = (AttnArgs, GdnArgs, GdnPreArgs, GdnGateArgs, LmArgs, LmHeadArgs, XdecArgs)

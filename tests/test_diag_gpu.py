@@ -46,6 +46,29 @@ def test_an_mfma_needs_one_instruction_after_a_vector_write_of_its_operands(dev,
     assert write_then_mfma[0] > 0 and cvt_then_mfma[0] > 0, f"no wrong product without a gap any more: {got} (the assembly scan of the build could go)"
 
 
+def test_a_waves_vector_instructions_do_not_run_in_the_shadow_of_its_own_mfmas(dev, lib):
+    """What bounds the attention kernels at head dim 128 (16 MFMAs and about as many clocks of softmax per 32 x 32 block and wave):
+    a wave that issues { MFMA 32x32x16, nv independent v_fma_f32 } per round needs 36 + 4 nv clocks per round, not max(36, 4 nv):
+    its vector instructions wait for its MFMA.  Only another wave of the SIMD fills the gap: with two waves per SIMD and 4 vector
+    instructions per MFMA the matrix pipe is busy all the time (32 clocks per MFMA of the SIMD)."""
+    iters = 20000
+
+    def run(nv, wps):
+        out = torch.zeros(2 * 4 * wps, dtype=torch.int64, device=dev)
+        _lib.check(lib.spinf_diag_mfma_valu(nv, 0, wps, iters, out.data_ptr(), C.c_void_p(torch.cuda.current_stream().cuda_stream)), "spinf_diag_mfma_valu")
+        torch.cuda.synchronize()
+        t = out.cpu().view(-1, 2)[0::4]   # the waves of SIMD 0
+        return float(t[0, 1] - t[0, 0]) / iters, float(t[:, 1].max() - t[:, 0].min()) / (iters * wps)
+
+    alone = {nv: run(nv, 1)[0] for nv in (0, 8, 16)}
+    pair = run(4, 2)[1]
+    print(f"clocks per round of a wave alone on its SIMD: {alone}; clocks per MFMA of a SIMD with two waves, 4 vector instructions per MFMA: {pair:.1f}")
+    assert 30 <= alone[0] <= 36, alone            # the counter counts core clocks: a 32x32x16 MFMA chain is 32 per link
+    assert alone[8] >= alone[0] + 0.8 * 32, f"vector instructions now run under a wave's own MFMA: {alone} (the two-block pipeline of the lockstep kernel would pay)"
+    assert alone[16] >= alone[0] + 0.8 * 64, alone
+    assert pair <= 36, f"a second wave no longer fills the matrix pipe: {pair}"
+
+
 def test_byte_pattern_yardstick_moves_every_tile_and_writes_every_row(dev, lib):
     """spinf_diag_attn_stream on a scaled-down C2: every tile of every work item is seen landed (the count equals the plan
     entries of the 32-key plan x head groups), no wait is given up, and every row of the stream is written"""
