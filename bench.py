@@ -273,6 +273,15 @@ def main():
                     table[f"{kname} nv={nv} waves_per_simd={wps}"] = {
                         "clocks_per_round_oldest_wave": round(float(simd0[0, 1] - simd0[0, 0]) / iters, 1),
                         "clocks_per_mfma_simd": round(float(simd0[:, 1].max() - simd0[:, 0].min()) / (iters * wps), 1)}
+        for wps in (1, 2, 4):   # rounds shaped like an attention block at head dim 128 (16 MFMAs; 48 v_fma_f32 + 16 v_exp_f32 at nv = 16)
+            for nv in (0, 8, 16):
+                out = torch.zeros(2 * 4 * wps, dtype=torch.int64, device=dev)
+                _lib.check(lib.spinf_diag_mfma_valu(nv, 2, wps, iters // 8, out.data_ptr(), C.c_void_p(torch.cuda.current_stream().cuda_stream)), "spinf_diag_mfma_valu")
+                torch.cuda.synchronize()
+                simd0 = out.cpu().view(-1, 2)[0::4]
+                table[f"block-shaped rounds nv={nv} waves_per_simd={wps}"] = {
+                    "clocks_per_block_oldest_wave": round(float(simd0[0, 1] - simd0[0, 0]) / (iters // 8), 1),
+                    "clocks_per_block_simd": round(float(simd0[:, 1].max() - simd0[:, 0].min()) / ((iters // 8) * wps), 1)}
         line.update(metric="clocks per MFMA of a SIMD, MFMA + nv vector instructions per round", unit="clocks", value=table["v_fma_f32 nv=6 waves_per_simd=2"]["clocks_per_mfma_simd"],
                     higher_is_better=False, ms_per_step=None, dtype="bf16", config={"workload": WORKLOADS["mfma_valu"], "iters": iters}, table=table)
         print(json.dumps(line))

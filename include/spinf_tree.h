@@ -332,7 +332,9 @@ int spinf_diag_lds_order(int32_t iters, int32_t workgroups, int32_t* out, void* 
 int spinf_diag_mfma_hazard(int32_t iters, int32_t workgroups, int32_t* out, void* stream);
 /* Diagnostics (no counterpart in the reference): do a wave's vector instructions run in the shadow of its own MFMAs?  One workgroup
  * per compute unit, waves_per_simd (1, 2 or 4) waves on every SIMD, each wave iters rounds of { one v_mfma_f32_32x32x16_bf16 on one
- * accumulator, nv (0, 2, 4, 6, 8, 12 or 16) independent vector instructions: v_fma_f32 (kind 0) or v_exp_f32 (kind 1) }.  out:
+ * accumulator, nv (0, 2, 4, 6, 8, 12 or 16) independent vector instructions: v_fma_f32 (kind 0) or v_exp_f32 (kind 1) } (kind 2:
+ * rounds shaped like a 32 x 32 attention block at head dim 128: 8 chained MFMAs, 3 nv v_fma_f32 + nv v_exp_f32, 8 MFMAs on four
+ * accumulators).  out:
  * 2 x 4 x waves_per_simd device int64: the clock before and after the loop of every wave of workgroup 0 (wave w = SIMD w % 4).
  * Clocks per round of a wave alone on its SIMD: 36 + 4 nv measured (36 + 8 nv for v_exp_f32), i.e. nothing runs in the shadow. */
 int spinf_diag_mfma_valu(int32_t nv, int32_t kind, int32_t waves_per_simd, int32_t iters, int64_t* out, void* stream);

@@ -43,7 +43,8 @@ __global__ __launch_bounds__(512) void mfma_rate_kernel(const long iters, float*
 // ---- do a wave's vector instructions run in the shadow of its own MFMAs?
 // Every wave runs iters x { one v_mfma_f32_32x32x16_bf16 (32 clocks of the matrix pipe) on a single accumulator, then NV vector
 // instructions that depend on nothing the MFMA touches: v_fma_f32 (KIND 0) or v_exp_f32 (KIND 1) }, with one, two or four waves per
-// SIMD.  Every wave of workgroup 0 records the clock before and after its loop (s_memtime ticks, which count core clocks here: the bare
+// SIMD (KIND 2: rounds shaped like a 32 x 32 attention block at head dim 128: 8 chained MFMAs, 3 NV v_fma_f32 + NV v_exp_f32, 8 MFMAs
+// on four accumulators).  Every wave of workgroup 0 records the clock before and after its loop (s_memtime ticks, which count core clocks here: the bare
 // MFMA chain reads 32.3 per MFMA).  If the vector instructions ran under the MFMA a wave would need max(36, 4 + 4 NV) clocks per round;
 // measured on MI355X it needs 36 + 4 NV (8 NV for v_exp_f32): they do not, the two add up, and only ANOTHER wave of the SIMD can use
 // the vector ALU while an MFMA runs.  This is what bounds the attention kernels at head dim 128, where a 32 x 32 block is 16 MFMAs
@@ -65,7 +66,23 @@ __global__ __launch_bounds__(1024) void mfma_valu_kernel(const int iters, long l
     const float c = 0.999f, d = 0.0001f;
     __syncthreads();
     const long long t0 = __builtin_readcyclecounter();
+    f32x16 o[4];   // (KIND 2)
+#pragma unroll
+    for (int n = 0; n < 4; n++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) o[n][i] = 0.f;
     for (int it = 0; it < iters; it++) {
+        if (KIND == 2) {   // an attention block's phases: 8 chained MFMAs, the softmax's vector instructions, 8 MFMAs on four accumulators
+#pragma unroll
+            for (int x = 0; x < 8; x++) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
+#pragma unroll
+            for (int j = 0; j < 3 * NV; j++) asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(v[j % 16]) : "v"(c), "v"(d));
+#pragma unroll
+            for (int j = 0; j < NV; j++) asm volatile("v_exp_f32 %0, %0" : "+v"(v[j % 16]));
+#pragma unroll
+            for (int x = 0; x < 8; x++) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(o[x & 3]) : "v"(a), "v"(b));
+            continue;
+        }
         asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
 #pragma unroll
         for (int j = 0; j < NV; j++) {
@@ -77,7 +94,7 @@ __global__ __launch_bounds__(1024) void mfma_valu_kernel(const int iters, long l
     const long long t1 = __builtin_readcyclecounter();
     float sum = 0.f;
 #pragma unroll
-    for (int i = 0; i < 16; i++) sum += acc[i] + v[i];
+    for (int i = 0; i < 16; i++) sum += acc[i] + v[i] + o[0][i] + o[1][i] + o[2][i] + o[3][i];
     if (sum == 12345.678f) out[0] = 0;   // keeps the loop alive (never true)
     if (blockIdx.x == 0 && (threadIdx.x & 63) == 0) {
         out[2 * (threadIdx.x >> 6)] = t0;
@@ -514,8 +531,8 @@ static void launch_mfma_valu(int nv, int wgs, int threads, int iters, long long*
 }
 
 extern "C" int spinf_diag_mfma_valu(int32_t nv, int32_t kind, int32_t waves_per_simd, int32_t iters, int64_t* out, void* stream) {
-    if ((nv != 0 && nv != 2 && nv != 4 && nv != 6 && nv != 8 && nv != 12 && nv != 16) || kind < 0 || kind > 1)
-        return spinf_fail(SPINF_E_ARG, "diag_mfma_valu: nv %d not in {0, 2, 4, 6, 8, 12, 16} or kind %d not in {0, 1}", nv, kind);
+    if ((nv != 0 && nv != 2 && nv != 4 && nv != 6 && nv != 8 && nv != 12 && nv != 16) || kind < 0 || kind > 2)
+        return spinf_fail(SPINF_E_ARG, "diag_mfma_valu: nv %d not in {0, 2, 4, 6, 8, 12, 16} or kind %d not in {0, 1, 2}", nv, kind);
     if ((waves_per_simd != 1 && waves_per_simd != 2 && waves_per_simd != 4) || iters <= 0 || iters > (1 << 22) || !out)
         return spinf_fail(SPINF_E_ARG, "diag_mfma_valu: waves per SIMD in {1, 2, 4}, iters in 1 .. 2^22, out not null");
     int dev = 0;
@@ -523,6 +540,7 @@ extern "C" int spinf_diag_mfma_valu(int32_t nv, int32_t kind, int32_t waves_per_
     if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return spinf_fail(SPINF_E_HIP, "diag_mfma_valu: no device");
     const int threads = 256 * waves_per_simd;
     if (kind == 0) launch_mfma_valu<0>(nv, prop.multiProcessorCount, threads, iters, (long long*)out, (hipStream_t)stream);
+    else if (kind == 2) launch_mfma_valu<2>(nv, prop.multiProcessorCount, threads, iters, (long long*)out, (hipStream_t)stream);
     else launch_mfma_valu<1>(nv, prop.multiProcessorCount, threads, iters, (long long*)out, (hipStream_t)stream);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return spinf_fail(SPINF_E_HIP, "diag_mfma_valu: launch: %s", hipGetErrorString(e));
