@@ -108,7 +108,8 @@ typedef struct spinf_attn_args {
     int64_t n_items;
     int32_t variant;   /* 0 = default kernel choice (eight waves, two heads of a GQA group per work item, where the group is even);
                           1 = one head per work item, four waves; 2 = four waves with two heads each (head dim <= 128,
-                          no compact rows) */
+                          no compact rows); 3 = the kernel with decoupled waves at head dim 128 (items as for 0; needs an even
+                          group, a static schedule (n_lists > 0) over 64-key entries, the stream layout, no image groups) */
     const int32_t* row_of; const int32_t* kv_row0;
     const int32_t* grp; int32_t grp_mode;   /* image groups, as given to spinf_tileplan_build_groups (device copy of grp), or NULL */
     int32_t ktile;                          /* keys per plan entry: 0 or 64; 32 with d = 512, and with a static schedule */

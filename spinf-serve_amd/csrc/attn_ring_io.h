@@ -32,24 +32,25 @@ __device__ __forceinline__ void dma_regions(const char* base, unsigned stride, u
                  : "memory", "m0", "scc");
 }
 
-// One wave requests a whole 32-key tile: K and V regions, art / end / pos of the keys, then the flag (generation gen).
-template <int D, bool WIN>
+// One wave requests a whole tile of TK keys (32; 64 at head dim 128): K and V regions, art / end / pos of the keys, then the flag
+// (generation gen).
+template <int D, bool WIN, int TK = 32>
 __device__ __forceinline__ void issue_tile_wave(const AttnParams& p, unsigned buf, int kt, int kvh, int gen, int lane, unsigned lane_k, unsigned lane_v) {
-    using GK = Geo<D, 32>;
+    using GK = Geo<D, TK>;
     constexpr int KTILEB = GK::KTILEB, VTILEB = GK::VTILEB;
     const char* kbase = (const char*)(p.k + (long)kvh * p.k_head);
     const char* vbase = (const char*)(p.v + (long)kvh * p.v_head);
-    if (kt * 32 + 32 <= p.n) {
-        const long first = (long)kt * 32;
+    if (kt * TK + TK <= p.n) {
+        const long first = (long)kt * TK;
         dma_regions<GK::NREG, GK::KRS>(kbase + first * p.k_tok * 2, (unsigned)(p.k_tok * 2), lane_k, buf);
         dma_regions<GK::NREG, GK::VRS>(vbase + first * p.v_tok * 2, (unsigned)(p.v_tok * 2), lane_v, buf + KTILEB);
-        const int key = kt * 32 + (lane & 31);
+        const int key = kt * TK + (lane & (TK - 1));
         dma4_lane(p.art + key, buf + KTILEB + VTILEB);
         dma4_lane(p.end + key, buf + KTILEB + VTILEB + 256);
         if (WIN) dma4_lane(p.pos + key, buf + KTILEB + VTILEB + 512);
     } else {   // the stream's last, partial tile: rows clamped per lane
         auto row_at = [&](const int reg, const int slot) {
-            const long grow = (long)kt * 32 + reg + GK::NREG * slot;
+            const long grow = (long)kt * TK + reg + GK::NREG * slot;
             return grow < p.n ? grow : (long)p.n - 1;
         };
 #pragma unroll 1   // (rolled: unrolled, the 32 per-lane addresses are all computed up front and take 64 registers)
@@ -58,7 +59,7 @@ __device__ __forceinline__ void issue_tile_wave(const AttnParams& p, unsigned bu
 #pragma unroll 1
         for (int reg = 0; reg < GK::NREG; reg++)
             dma16_lane(vbase + row_at(reg, lane / GK::CPR) * p.v_tok * 2 + (lane % GK::CPR) * 16, buf + KTILEB + reg * GK::VRS);
-        int key = kt * 32 + (lane & 31);
+        int key = kt * TK + (lane & (TK - 1));
         key = key < p.n ? key : p.n - 1;
         dma4_lane(p.art + key, buf + KTILEB + VTILEB);
         dma4_lane(p.end + key, buf + KTILEB + VTILEB + 256);

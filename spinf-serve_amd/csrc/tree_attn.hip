@@ -714,7 +714,7 @@ void pick_kernel(int hq, int hkv, int d, int variant, int* rt, int* nhw) {
     *rt = 1;
     *nhw = 1;
     if (d > 256) return;   // head dim 512: one head per item, the single-pass kernel
-    if (variant == 0 && pairs) *nhw = 2;
+    if ((variant == 0 || variant == 3) && pairs) *nhw = 2;
     if (variant == 2 && pairs && d <= 128) *rt = 2;
 }
 
@@ -840,8 +840,13 @@ static int attn_fwd(const spinf_attn_args* a, void* stream, bool no_alloc) {
     if ((a->row_of != nullptr) != (a->kv_row0 != nullptr)) return spinf_fail(SPINF_E_ARG, "tree_attn: row_of and kv_row0 come together");
     if (a->row_of && rt != 1) return spinf_fail(SPINF_E_ARG, "tree_attn: variant %d does not take compact rows", a->variant);
     if (a->n_lists < 0 || a->n_lists > LAND_CAP) return spinf_fail(SPINF_E_ARG, "tree_attn: %d item lists, at most %d", a->n_lists, LAND_CAP);
-    const bool ring = a->n_lists > 0 && a->ktile == 32;   // static schedule over 32-key entries: the ring kernel
-    if (ring) {
+    // the ring kernel: a static schedule over 32-key entries (head dim 256 and 512), or variant 3 at head dim 128 (64-key entries)
+    const bool ring128 = a->variant == 3;
+    const bool ring = a->n_lists > 0 && (a->ktile == 32 || ring128);
+    if (ring128 && !(a->d == 128 && a->n_lists > 0 && (a->ktile == 0 || a->ktile == 64) && nhw == 2 && rt == 1 && !a->row_of && !a->grp))
+        return spinf_fail(SPINF_E_ARG, "tree_attn: variant 3 (the kernel with decoupled waves at head dim 128) takes head dim 128, an even number of query heads per "
+                                       "key / value head, a static schedule over 64-key entries, the stream layout and no image groups");
+    if (ring && !ring128) {
         if (!((a->d == 256 && nhw == 2 && rt == 1) || a->d == 512) || a->row_of || a->grp)
             return spinf_fail(SPINF_E_ARG, "tree_attn: a static schedule over 32-key entries goes with head dim 512, or head dim 256 with an even number of query heads "
                                            "per key / value head and variant 0; with the stream layout and no image groups");

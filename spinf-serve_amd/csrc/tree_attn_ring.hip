@@ -169,7 +169,8 @@ __device__ __forceinline__ void pv_steps(Fn& fn) {
 // A wave's place in the workgroup: four row groups x HPI heads of the item.
 template <int D>
 struct RingShape {
-    static constexpr int TK = 32;
+    static constexpr int TK = D == 128 ? 64 : 32;    // keys per tile: at head dim 128 a 32-key tile is too little work per ring slot
+    static constexpr int NSUB = TK / 32;             // 32-key blocks per tile
     static constexpr int NW = D == 512 ? 4 : 8;      // waves: four row groups x HPI heads of the item
     static constexpr int HPI = NW / 4;
     static constexpr int NSLOT = D == 512 ? 2 : MAX_SLOT;
@@ -288,14 +289,16 @@ __device__ __forceinline__ void ring_paced_pass(const AttnParams& p, char* const
                 const int lane = fresh_lane_id();
                 const unsigned lane_k = (unsigned)((lane / GK::CPR) * GK::NREG * p.k_tok * 2 + (lane % GK::CPR) * 16);
                 const unsigned lane_v = (unsigned)((lane / GK::CPR) * GK::NREG * p.v_tok * 2 + (lane % GK::CPR) * 16);
-                issue_tile_wave<D, WIN>(p, lds_addr(ring), kt, kvh, 0, lane, lane_k, lane_v);
+                issue_tile_wave<D, WIN, TK>(p, lds_addr(ring), kt, kvh, 0, lane, lane_k, lane_v);
             }
             __builtin_amdgcn_s_waitcnt(0x0f70);   // the tile has landed (and this wave's queries)
             __syncthreads();
-            if (!((bits >> (2 * wr)) & 1u)) continue;   // (wave-uniform; the barriers above are passed by every wave)
+#pragma unroll 1
+            for (int sub = 0; sub < S::NSUB; sub++) {   // the tile's 32-key blocks
+            if (!((bits >> (2 * wr + sub)) & 1u)) continue;   // (wave-uniform; the barriers above are passed by every wave)
             const int ln = fresh_lane_id();
-            const char* krow = ring + G::K::k_off(ln & 31) + 16 * (ln >> 5);
-            const char* vrow = ring + G::KTILEB + G::V::v_off(4 * (ln >> 5) + ((ln >> 2) & 3)) + 32 * ((ln >> 4) & 1) + 8 * (ln & 3);
+            const char* krow = ring + G::K::k_off(ln & 31) + 16 * (ln >> 5) + sub * G::KSUB;
+            const char* vrow = ring + G::KTILEB + G::V::v_off(4 * (ln >> 5) + ((ln >> 2) & 3)) + 32 * ((ln >> 4) & 1) + 8 * (ln & 3) + sub * G::VSUB;
             // (the scheduling barriers keep the phases apart.  The MFMAs are assembly, which the compiler's hazard recogniser does
             // not look into: left to interleave the softmax of the block's second half with the P V products of the first, it
             // put the conversion that writes a P fragment directly in front of the MFMA that reads it, and an MFMA that issues in
@@ -313,10 +316,10 @@ __device__ __forceinline__ void ring_paced_pass(const AttnParams& p, char* const
             };
             pv_steps<NS>(score);
             __builtin_amdgcn_sched_barrier(0);
-            if ((bits >> (8 + 2 * wr)) & 1u) {
+            if ((bits >> (8 + 2 * wr + sub)) & 1u) {
                 f32x16 sm[1] = {sa};
                 const int tok = (tz & 0xfffff) * SPINF_QTILE + 32 * wr + (ln & 31);
-                apply_mask<1, WIN, 0, TK>(sm, (const int*)(ring + G::KTILEB + G::VTILEB), kt, 0, ln >> 5, tok, art_q, pos_q, p.window);
+                apply_mask<1, WIN, 0, TK>(sm, (const int*)(ring + G::KTILEB + G::VTILEB), kt, sub, ln >> 5, tok, art_q, pos_q, p.window);
                 sa = sm[0];
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -380,6 +383,7 @@ __device__ __forceinline__ void ring_paced_pass(const AttnParams& p, char* const
                 __builtin_amdgcn_sched_barrier(0);
             };
             pv_steps<NVF>(step);
+            }
         }
         if (!exact && __builtin_amdgcn_ballot_w64(viol) != 0) {   // scores ranged too widely somewhere in these 32 rows: the item is done again, exactly
             if (fresh_lane_id() == 0) __hip_atomic_store(sy_vote, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -410,7 +414,7 @@ __device__ __forceinline__ void ring_paced_pass(const AttnParams& p, char* const
 
 template <int D, bool WIN>
 __global__ __launch_bounds__(D == 512 ? 256 : 512) void tree_attn_ring_kernel(const AttnParams p) {
-    constexpr int TK = 32;
+    constexpr int TK = RingShape<D>::TK, NSUB = RingShape<D>::NSUB;
     constexpr int NW = D == 512 ? 4 : 8;      // waves: four row groups x HPI heads of the item
     constexpr int HPI = NW / 4;
     constexpr int NSLOT = D == 512 ? 2 : MAX_SLOT;
@@ -421,6 +425,7 @@ __global__ __launch_bounds__(D == 512 ? 256 : 512) void tree_attn_ring_kernel(co
     constexpr int PFD = D >= 256 ? 2 : 8;   // fragment read-ahead: at head dim 256 one more spills a query fragment inside the tile loop
     constexpr int PF = D >= 256 ? 4 : (NS < PFD ? NS : PFD);   // K fragments are live in the score phase only, where registers are free
     constexpr int VPF = NVF < PFD ? NVF : PFD;
+    constexpr int DONE_AT = NVF - 1 - VPF > 0 ? NVF - 1 - VPF : 0;   // the P V step behind which a block's last V fragment read is on its way
     static_assert(NSLOT * G::BUFB + NW * 32 * SROW + NDESC * 16 + 256 <= 160 * 1024, "LDS budget");
     __shared__ __attribute__((aligned(16))) char ring[NSLOT * G::BUFB];
     __shared__ __attribute__((aligned(16))) char stage_all[NW * 32 * SROW];   // output staging, one slice per wave
@@ -555,7 +560,7 @@ __global__ __launch_bounds__(D == 512 ? 256 : 512) void tree_attn_ring_kernel(co
         const int lane = fresh_lane_id();
         const unsigned lane_k = (unsigned)((lane / GK::CPR) * GK::NREG * p.k_tok * 2 + (lane % GK::CPR) * 16);
         const unsigned lane_v = (unsigned)((lane / GK::CPR) * GK::NREG * p.v_tok * 2 + (lane % GK::CPR) * 16);
-        issue_tile_wave<D, WIN>(p, lds_addr(ring + (j & (NSLOT - 1)) * G::BUFB), d.x, kvh, j / NSLOT + 1, lane, lane_k, lane_v);
+        issue_tile_wave<D, WIN, TK>(p, lds_addr(ring + (j & (NSLOT - 1)) * G::BUFB), d.x, kvh, j / NSLOT + 1, lane, lane_k, lane_v);
     };
 
     // When all eight waves are through with a slot's tile (its count stands at 8), whichever wave comes by first recycles the slot:
@@ -710,7 +715,9 @@ __global__ __launch_bounds__(D == 512 ? 256 : 512) void tree_attn_ring_kernel(co
             if (dead) break;
             const unsigned bits = (unsigned)d.y;
             last = (bits & DESC_LAST) != 0;
-            const bool act = (bits >> (2 * L.wr)) & 1u;
+            // the tile's 32-key blocks that this wave's rows see something of (one bit per block)
+            const unsigned ab = (bits >> (2 * L.wr)) & (NSUB == 2 ? 3u : 1u);
+            const bool act = ab != 0;
             if (act) {
                 if (flag != ((j / NSLOT + 1) & 63)) wait_watch(flag_word(j), (j / NSLOT + 1) & 63);
                 if (dead) break;
@@ -719,88 +726,107 @@ __global__ __launch_bounds__(D == 512 ? 256 : 512) void tree_attn_ring_kernel(co
                 // V^T as ds_read_b64_tr_b16 wants it (see Lane in attn_kernels.h)
                 const int ln = fresh_lane_id();
                 const char* buf = ring + s * G::BUFB;
-                const char* krow = buf + G::K::k_off(ln & 31) + 16 * (ln >> 5);
-                const char* vrow = buf + G::KTILEB + G::V::v_off(4 * (ln >> 5) + ((ln >> 2) & 3)) + 32 * ((ln >> 4) & 1) + 8 * (ln & 3);
-                // S^T = K Q^T
-                f32x16 sa;
-                {
-                    bf16x8 kf[PF];
-#pragma unroll
-                    for (int x = 0; x < PF; x++) kf[x] = *(const bf16x8*)(krow + 32 * x);
-                    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                    for (int x = 0; x < NS; x++) {
-                        if (x == 0) qk_first(sa, kf[x % PF], qf[x]);
-                        else if (x == NS - 1) qk_last(sa, kf[x % PF], qf[x]);
-                        else qk_next(sa, kf[x % PF], qf[x]);
-                        if (x + PF < NS) kf[x % PF] = *(const bf16x8*)(krow + 32 * (x + PF));
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
-                }
-                if ((bits >> (8 + 2 * L.wr)) & 1u) {
-                    f32x16 sm[1] = {sa};
-                    const int tok = (d.z & 0xfffff) * SPINF_QTILE + 32 * L.wr + (ln & 31);
-                    apply_mask<1, WIN, 0, TK>(sm, (const int*)(buf + G::KTILEB + G::VTILEB), d.x, 0, ln >> 5, tok, art_q, pos_q, p.window);
-                    sa = sm[0];
-                }
-                // softmax against the row's fixed reference (the maximum of the first block it sees a key in)
-                bf16x8 pb[2];
-                {
-                    const bool first = M == -INFINITY;
-                    if (__builtin_amdgcn_ballot_w64(first) != 0) {   // only where a row meets its first keys (see the lockstep kernel)
-                        float mx = sa[0];
-#pragma unroll
-                        for (int i2 = 1; i2 < 16; i2++) mx = fmaxf(mx, sa[i2]);
-                        mx = lane32_max(mx);
-                        M = first ? mx * p.c : M;
-                    }
-                    const float ms = M == -INFINITY ? 0.f : M;
-                    float sum = 0.f;
-#pragma unroll
-                    for (int i2 = 0; i2 < 16; i2++) {
-                        const float pr = __builtin_amdgcn_exp2f(__builtin_fmaf(sa[i2], p.c, -ms));
-                        sum += pr;
-                        pb[i2 >> 3][i2 & 7] = (__bf16)pr;
-                    }
-                    l += sum;
-                    viol = viol | !(sum <= VIOL_SUM);
-                }
-                // O^T += V^T P^T, with what the next tile's top needs fetched meanwhile; once the last fragment read is on its way,
-                // count this wave through with the tile
+                // what the next tile's top needs, fetched under the last block's P V products
                 int4 dv = make_int4(0, 0, 0, 0);
                 i32x4 nx = {0, 0, 0, 0};
                 int fv = -1;
                 const bool pf_ok = j + 1 < ntiles && j + 1 < gen_seen;
-                // (requested before the first transposing read of V, so that every wait inside the MFMA sequence is for V
-                // fragments alone and stalls: a wait that is already satisfied takes no time, and then a vector write of an
-                // operand could end up in the issue cycle before the assembly MFMA that reads it; LDS reads of different kinds
-                // do return in issue order, spinf_diag_lds_order checks it)
-                if (pf_ok) {
-                    dv = desc[(j + 1) & (NDESC - 1)];
-                    nx = lds_peek4(sy_done);
-                    fv = lds_peek(flag_word(j + 1));
-                }
-                {
-                    s16x4 vlo[VPF], vhi[VPF];
-                    auto vload = [&](const int f, const int slot) __attribute__((always_inline)) {
-                        const char* vp = vrow + G::V::v_off(16 * (f / NDT)) + 64 * (f % NDT);
-                        vlo[slot] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)vp);
-                        vhi[slot] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vp + G::V::v_off(8)));
-                    };
+                // one 32-key block: K Q^T, mask, softmax, P V.  TAIL: the last block of the tile that this wave computes
+                auto block = [&](const int sub, auto tail_c) __attribute__((always_inline)) {
+                    constexpr bool TAIL = decltype(tail_c)::value;
+                    const char* krow = buf + G::K::k_off(ln & 31) + 16 * (ln >> 5) + sub * G::KSUB;
+                    const char* vrow = buf + G::KTILEB + G::V::v_off(4 * (ln >> 5) + ((ln >> 2) & 3)) + 32 * ((ln >> 4) & 1) + 8 * (ln & 3) + sub * G::VSUB;
+                    // S^T = K Q^T
+                    f32x16 sa;
+                    {
+                        bf16x8 kf[PF];
 #pragma unroll
-                    for (int f = 0; f < VPF; f++) vload(f, f);
-                    __builtin_amdgcn_sched_barrier(0);
-                    auto step = [&](auto f_c) __attribute__((always_inline)) {
-                        constexpr int f = decltype(f_c)::value;
-                        const bf16x8 a = __builtin_bit_cast(bf16x8, __builtin_shufflevector(vlo[f % VPF], vhi[f % VPF], 0, 1, 2, 3, 4, 5, 6, 7));
-                        acc_mfma<f % NDT>(a, pb[f / NDT]);
-                        if (f + VPF < NVF) vload(f + VPF, f % VPF);
-                        if (f + VPF == NVF - 1) {   // that was the tile's last fragment read
-                            if (fresh_lane_id() == 0) __hip_atomic_fetch_add(&sy_done[s], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                        }
+                        for (int x = 0; x < PF; x++) kf[x] = *(const bf16x8*)(krow + 32 * x);
                         __builtin_amdgcn_sched_barrier(0);
-                    };
-                    pv_steps<NVF>(step);
+#pragma unroll
+                        for (int x = 0; x < NS; x++) {
+                            if (x == 0) qk_first(sa, kf[x % PF], qf[x]);
+                            else if (x == NS - 1) qk_last(sa, kf[x % PF], qf[x]);
+                            else qk_next(sa, kf[x % PF], qf[x]);
+                            if (x + PF < NS) kf[x % PF] = *(const bf16x8*)(krow + 32 * (x + PF));
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                    }
+                    if ((bits >> (8 + 2 * L.wr + sub)) & 1u) {
+                        f32x16 sm[1] = {sa};
+                        const int tok = (d.z & 0xfffff) * SPINF_QTILE + 32 * L.wr + (ln & 31);
+                        apply_mask<1, WIN, 0, TK>(sm, (const int*)(buf + G::KTILEB + G::VTILEB), d.x, sub, ln >> 5, tok, art_q, pos_q, p.window);
+                        sa = sm[0];
+                    }
+                    // softmax against the row's fixed reference (the maximum of the first block it sees a key in)
+                    bf16x8 pb[2];
+                    {
+                        const bool first = M == -INFINITY;
+                        if (__builtin_amdgcn_ballot_w64(first) != 0) {   // only where a row meets its first keys (see the lockstep kernel)
+                            float mx = sa[0];
+#pragma unroll
+                            for (int i2 = 1; i2 < 16; i2++) mx = fmaxf(mx, sa[i2]);
+                            mx = lane32_max(mx);
+                            M = first ? mx * p.c : M;
+                        }
+                        const float ms = M == -INFINITY ? 0.f : M;
+                        float sum = 0.f;
+#pragma unroll
+                        for (int i2 = 0; i2 < 16; i2++) {
+                            const float pr = __builtin_amdgcn_exp2f(__builtin_fmaf(sa[i2], p.c, -ms));
+                            sum += pr;
+                            pb[i2 >> 3][i2 & 7] = (__bf16)pr;
+                        }
+                        l += sum;
+                        viol = viol | !(sum <= VIOL_SUM);
+                    }
+                    // O^T += V^T P^T, with what the next tile's top needs fetched meanwhile; once the last fragment read is on its way,
+                    // count this wave through with the tile
+                    // (requested before the first transposing read of V, so that every wait inside the MFMA sequence is for V
+                    // fragments alone and stalls: a wait that is already satisfied takes no time, and then a vector write of an
+                    // operand could end up in the issue cycle before the assembly MFMA that reads it; LDS reads of different kinds
+                    // do return in issue order, spinf_diag_lds_order checks it)
+                    if (TAIL && pf_ok) {
+                        dv = desc[(j + 1) & (NDESC - 1)];
+                        nx = lds_peek4(sy_done);
+                        fv = lds_peek(flag_word(j + 1));
+                    }
+                    {
+                        s16x4 vlo[VPF], vhi[VPF];
+                        auto vload = [&](const int f, const int slot) __attribute__((always_inline)) {
+                            const char* vp = vrow + G::V::v_off(16 * (f / NDT)) + 64 * (f % NDT);
+                            vlo[slot] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)vp);
+                            vhi[slot] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vp + G::V::v_off(8)));
+                        };
+#pragma unroll
+                        for (int f = 0; f < VPF; f++) vload(f, f);
+                        __builtin_amdgcn_sched_barrier(0);
+                        // (head dim 128 reads all of a block's V fragments ahead, and the compiler then sinks the conversions that write
+                        // the P fragments below those reads, right in front of the first MFMA, which would multiply the registers' old
+                        // contents: one instruction in between)
+                        if constexpr (VPF >= NVF) asm volatile("s_nop 0" ::: "memory");
+                        auto step = [&](auto f_c) __attribute__((always_inline)) {
+                            constexpr int f = decltype(f_c)::value;
+                            const bf16x8 a = __builtin_bit_cast(bf16x8, __builtin_shufflevector(vlo[f % VPF], vhi[f % VPF], 0, 1, 2, 3, 4, 5, 6, 7));
+                            acc_mfma<f % NDT>(a, pb[f / NDT]);
+                            if (f + VPF < NVF) vload(f + VPF, f % VPF);
+                            if (TAIL && f == DONE_AT) {   // that was the tile's last fragment read
+                                if (fresh_lane_id() == 0) __hip_atomic_fetch_add(&sy_done[s], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                            }
+                            __builtin_amdgcn_sched_barrier(0);
+                        };
+                        pv_steps<NVF>(step);
+                    }
+                };
+                if constexpr (NSUB == 1) {
+                    block(0, std::true_type{});
+                } else {
+                    if (ab == 3u) {
+                        block(0, std::false_type{});
+                        block(1, std::true_type{});
+                    } else {
+                        block((int)(ab >> 1), std::true_type{});
+                    }
                 }
                 if (pf_ok) {
                     pf_d = make_int4(__builtin_amdgcn_readfirstlane(dv.x), __builtin_amdgcn_readfirstlane(dv.y), __builtin_amdgcn_readfirstlane(dv.z), __builtin_amdgcn_readfirstlane(dv.w));
@@ -876,7 +902,8 @@ int launch_ring_t(const AttnParams& p, int n_wg, hipStream_t stream) {
 }  // namespace
 
 int spinf_launch_ring(const AttnParams& p, int d, bool win, int n_wg, hipStream_t stream) {
+    if (d == 128) return win ? launch_ring_t<128, true>(p, n_wg, stream) : launch_ring_t<128, false>(p, n_wg, stream);
     if (d == 256) return win ? launch_ring_t<256, true>(p, n_wg, stream) : launch_ring_t<256, false>(p, n_wg, stream);
     if (d == 512) return win ? launch_ring_t<512, true>(p, n_wg, stream) : launch_ring_t<512, false>(p, n_wg, stream);
-    return spinf_fail(SPINF_E_ARG, "tree_attn: the ring kernel takes head dim 256 or 512, not %d", d);
+    return spinf_fail(SPINF_E_ARG, "tree_attn: the ring kernel takes head dim 128, 256 or 512, not %d", d);
 }

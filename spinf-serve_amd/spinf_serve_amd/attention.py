@@ -20,8 +20,8 @@ from . import _lib
 from .masks import TreeMask
 
 # kernel tuning variant handed to the library (0 = its default choice: eight waves, the two heads of a GQA pair per work item, where
-# a group is even; 1 = one head per work item, four waves; 2 = four waves with two heads each, head dim <= 128); results do not
-# depend on it
+# a group is even; 1 = one head per work item, four waves; 2 = four waves with two heads each, head dim <= 128; 3 is set by
+# tree_attn itself where head dim 128 goes to the kernel with decoupled waves); results do not depend on it
 VARIANT = int(os.environ.get("SPINF_ATTN_VARIANT", "0"))
 # the kernel with decoupled waves over a static schedule, where the library has one for the geometry (0: the lockstep kernels only)
 RING = int(os.environ.get("SPINF_ATTN_RING", "-1"))      # -1 = auto
@@ -32,6 +32,8 @@ STATIC = int(os.environ.get("SPINF_ATTN_STATIC", "-1"))  # -1 = auto
 
 
 RING_MAX_ITEMS_PER_WG = 8
+# head dim 128: the kernel with decoupled waves over 64-key tiles (the library's variant 3) where the geometry allows
+RING_128 = False
 
 # test hook (spinf_attn_args.debug_expire): k > 0 = polls after which a wave of the decoupled kernel gives up a wait (2^18 otherwise)
 DEBUG_EXPIRE = 0
@@ -67,13 +69,15 @@ def _ring_lists(q, hq, hkv, d, variant, sidx, mask):
     its waves run through the item boundaries; with many items per workgroup (C3's 65,536-token passes: 16) the lockstep kernel
     is 6 - 10 % faster.  The lockstep kernel takes the static lists on sliding layers (5 % faster there than its queue) and its
     queue on global layers (4 % faster).  SPINF_ATTN_RING / SPINF_ATTN_STATIC = 0 / 1 switch the two for every call where the
-    geometry allows, "auto" (the default) follows the measurements."""
+    geometry allows, "auto" (the default) follows the measurements.  Head dim 128 has the decoupled kernel too (the library's
+    variant 3, 64-key tiles): 55.5 against 48.5 ms on C4, so "auto" leaves it to the lockstep kernel (RING_128 or
+    SPINF_ATTN_RING=1 select it)."""
     from .masks import _static_lists
 
     n_wg = _static_lists(q.device)
-    ring = (d == 512 or (variant == 0 and d == 256 and (hq // hkv) % 2 == 0)) and sidx is None and mask.grp is None
+    ring = (d == 512 or (variant == 0 and d in (128, 256) and (hq // hkv) % 2 == 0)) and sidx is None and mask.grp is None
     if ring and RING < 0:
-        ring = d == 512 or mask.plan.n_qtiles * (hq // 2) <= RING_MAX_ITEMS_PER_WG * n_wg
+        ring = d == 512 or (d == 256 and mask.plan.n_qtiles * (hq // 2) <= RING_MAX_ITEMS_PER_WG * n_wg) or (d == 128 and RING_128)
     elif not RING:
         ring = False
     static = d != 512 and (int(mask.window) > 0 if STATIC < 0 else bool(STATIC))
@@ -163,7 +167,9 @@ def tree_attn(q, k, v, mask: TreeMask, scale=None, variant=None, sidx=None):
         raise ValueError("image groups go with the stream layout (no sidx)")
     hq, hkv, d = q.shape[1], k.shape[1], q.shape[2]
     n_lists, ring = _ring_lists(q, hq, hkv, d, variant, sidx, mask)
-    mask = mask.for_head_dim(d, ring=ring)
+    if ring and d == 128:
+        variant = 3   # (64-key plan entries, as the lockstep kernels take)
+    mask = mask.for_head_dim(d, ring=ring and d != 128)
     per_item = _lib.load_library().spinf_attn_heads_per_item(hq, hkv, d, variant)
     if per_item <= 0:
         raise ValueError(f"{hq} query heads do not group over {hkv} key / value heads")
@@ -187,13 +193,14 @@ def tree_attn_noalloc(q, k, v, mask: TreeMask, out, scale=None):
     n, hq, d = q.shape
     hkv = k.shape[1]
     n_lists, ring = _ring_lists(q, hq, hkv, d, 0, None, mask)
-    mask = mask.for_head_dim(d, ring=ring)
-    per_item = _lib.load_library().spinf_attn_heads_per_item(hq, hkv, d, 0)
+    variant = 3 if ring and d == 128 else 0
+    mask = mask.for_head_dim(d, ring=ring and d != 128)
+    per_item = _lib.load_library().spinf_attn_heads_per_item(hq, hkv, d, variant)
     if per_item <= 0:
         raise ValueError(f"{hq} query heads do not group over {hkv} key / value heads")
     items, list_ptr, n_items = mask.schedule(hq // per_item, n_lists)
     scale = float(d ** -0.5 if scale is None else scale)
-    a = _attn_args(q, k, v, out, n, mask.art, mask.end, mask.pos, mask.kv_idx, mask.kv_bits, items, list_ptr, n_items, scale, int(mask.window), 0,
+    a = _attn_args(q, k, v, out, n, mask.art, mask.end, mask.pos, mask.kv_idx, mask.kv_bits, items, list_ptr, n_items, scale, int(mask.window), variant,
                    None, None, mask.grp, int(mask.grp_mode), int(mask.plan.ktile), n_lists)
     lib = _lib.load_library()
     with torch.cuda.device(q.device):

@@ -101,7 +101,7 @@ def test_wide_score_range_takes_the_exact_pass(dev, d, hq, hkv):
     assert float(np.abs(out2.float().cpu().numpy() - _oracle(q, k2, v, b, cfg.scale)).max()) <= TOL
 
 
-@pytest.mark.parametrize("d,hq,hkv", [(256, 4, 2), (512, 4, 1)])
+@pytest.mark.parametrize("d,hq,hkv", [(128, 4, 2), (256, 4, 2), (512, 4, 1)])
 @pytest.mark.parametrize("window", [None, 150])
 def test_exact_recomputation_is_the_same_in_both_kernels(dev, d, hq, hkv, window, monkeypatch):
     """the kernel with decoupled waves recomputes the items with too wide a score range itself, after its list; the lockstep
@@ -545,6 +545,36 @@ def test_kernel_and_schedule_choices_give_the_same_bits(dev, window, monkeypatch
     assert _ring_aborts() == aborts0
 
 
+@pytest.mark.parametrize("window", [None, 200])
+def test_head_dim_128_decoupled_kernel_gives_the_lockstep_bits(dev, window, monkeypatch):
+    """the kernel with decoupled waves at head dim 128 (the library's variant 3: 64-key tiles, two 32-key blocks per tile and wave;
+    not the default there, the lockstep kernel is faster on long trunks): the same bits as the lockstep kernel on a two-level tree
+    with a long trunk, on short ragged trees, and through the entry point that allocates nothing; no wave gives up a wait"""
+    from spinf_serve_amd import attention
+
+    rng = np.random.default_rng(31)
+    cases = [synth.attention_config("C4", contents=1), synth.attention_config("smoke"),
+             synth.AttnConfig("ragged", 8, 2, 128, 128 ** -0.5, 1.0, None, [synth._tree(rng, 333, [17, 5, 64, 9]), synth._tree(rng, 70, []), synth._tree(rng, 1, [3])])]
+    cases[2].batches = synth.pack(cases[2].trees)
+    for cfg in cases:
+        b = cfg.batches[0]
+        q, k, v = synth.qkv(cfg, b, seed=12, device=dev)
+        mask = sa.TreeMask.build(b.art, b.end, b.pos, window=window, device=dev)
+        monkeypatch.setattr(attention, "RING", 0)
+        want = sa.tree_attn(q, k, v, mask, cfg.scale)
+        torch.cuda.synchronize()
+        monkeypatch.setattr(attention, "RING", 1)
+        before = _ring_aborts()
+        print(f"case d=128 decoupled kernel {cfg.name} n={b.length} window={window}", flush=True)
+        got = sa.tree_attn(q, k, v, mask, cfg.scale)
+        out = torch.full_like(want, float("nan"))
+        sa.tree_attn_noalloc(q, k, v, mask, out, cfg.scale)
+        torch.cuda.synchronize()
+        assert _ring_aborts() == before
+        assert torch.equal(got, want), float((got.float() - want.float()).abs().max())
+        assert torch.equal(out, want)
+
+
 @pytest.mark.parametrize("window", [None, 300])
 def test_head_dim_512_kernel_choices_give_the_same_bits(dev, window, monkeypatch):
     """head dim 512: the kernel with decoupled waves (one launch, the whole output row in accumulation registers) and the lockstep
@@ -698,7 +728,7 @@ def test_several_calls_recorded_by_one_capture_share_the_streams_block(dev, ring
     assert torch.equal(out4, want2) and torch.equal(out1, want1) and torch.equal(out3, want3)
 
 
-@pytest.mark.parametrize("d,limit,wide", [(256, 1, False), (256, 1, True), (256, 3, False), (512, 1, False), (512, 1, True)])
+@pytest.mark.parametrize("d,limit,wide", [(128, 1, False), (128, 1, True), (256, 1, False), (256, 1, True), (256, 3, False), (512, 1, False), (512, 1, True)])
 def test_a_wave_that_gives_up_a_wait_costs_time_not_rows(dev, d, limit, wide, monkeypatch):
     """the decoupled kernel's landing: the waves are told (from the host, spinf_attn_args.debug_expire) to give up a wait after
     `limit` polls instead of 2^18, so every wave that has to wait for a tile at all gives up, as after a real time-out; its
@@ -707,7 +737,7 @@ def test_a_wave_that_gives_up_a_wait_costs_time_not_rows(dev, d, limit, wide, mo
     go on to the exact recomputation (wide) and with a window."""
     from spinf_serve_amd import attention
 
-    cfg = synth.attention_config("C2" if d == 256 else "C2_512", contents=12 if d == 256 else 6)
+    cfg = synth.attention_config({128: "C4", 256: "C2", 512: "C2_512"}[d], contents={128: 1, 256: 12, 512: 6}[d])
     b = cfg.batches[0]
     q, k, v = synth.qkv(cfg, b, seed=9, device=dev)
     if wide:

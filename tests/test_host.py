@@ -179,8 +179,12 @@ def test_build_scan_of_the_ring_assembly_catches_what_it_is_there_for():
         ge._scan_ring_assembly(listing("v_cvt_pk_bf16_f32 v7, v14, v15", "s_waitcnt lgkmcnt(0)") + mfma)
     with pytest.raises(RuntimeError, match="issue cycle before"):
         ge._scan_ring_assembly(listing("v_mov_b32_e32 v2, v9") + mfma)
-    with pytest.raises(RuntimeError, match="accumulation register of its own"):
+    with pytest.raises(RuntimeError, match="accumulation register that the assembly owns"):
         ge._scan_ring_assembly(listing("v_accvgpr_write_b32 a130, v3"))
+    k128 = "_ZN12_GLOBAL__N_121tree_attn_ring_kernelILi128ELb0EEEv10AttnParams: ; @kernel"
+    ge._scan_ring_assembly([k128, "\tv_accvgpr_write_b32 a66, v3"])        # head dim 128: the assembly owns a[0:63] only
+    with pytest.raises(RuntimeError, match="accumulation register that the assembly owns"):
+        ge._scan_ring_assembly([k128, "\tv_accvgpr_read_b32 v3, a63"])
     reload = ["_ZN12_GLOBAL__N_121tree_attn_ring_kernelILi256ELb0EEEv10AttnParams: ; @kernel", ".LBB0_7:    ;   in Loop: Header=BB0_3 Depth=2",
               "\tscratch_load_dwordx4 v[4:7], off, off offset:16"]
     with pytest.raises(RuntimeError, match="16-byte reload"):
