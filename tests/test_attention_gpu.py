@@ -519,6 +519,8 @@ def test_argument_errors(dev):
         sa.tree_attn(q.float(), k, v, mask, cfg.scale)
     with pytest.raises(RuntimeError):
         sa.tree_attn(q.cpu(), k.cpu(), v.cpu(), mask, cfg.scale)  # no CPU path
+    with pytest.raises(Exception, match="variant 3"):
+        sa.tree_attn(q, k, v, mask, cfg.scale, variant=3)         # the decoupled kernel at head dim 128 wants a static schedule
 
 
 @pytest.mark.parametrize("window", [None, 256])

@@ -50,6 +50,12 @@ def test_c_abi_rejects_bad_arguments(lib):
     counts = (ctypes.c_int64 * 5)()
     assert lib.spinf_tileplan_counts(out, counts) == 0 and list(counts) == [0, 0, 0, 0, 0]
     lib.spinf_tileplan_free(out)
+    # the yardsticks check their arguments before they touch the GPU
+    buf = (ctypes.c_int64 * 32)()
+    assert lib.spinf_diag_mfma_valu(3, 0, 2, 100, buf, None) == -1 and b"nv 3" in lib.spinf_last_error()
+    assert lib.spinf_diag_mfma_valu(4, 3, 2, 100, buf, None) == -1 and b"kind 3" in lib.spinf_last_error()
+    assert lib.spinf_diag_mfma_valu(4, 0, 3, 100, buf, None) == -1 and b"waves per SIMD" in lib.spinf_last_error()
+    assert lib.spinf_diag_mfma_valu(4, 0, 2, 100, None, None) == -1
 
 
 def test_heads_per_item_follows_the_kernel_choice(lib):
@@ -61,6 +67,7 @@ def test_heads_per_item_follows_the_kernel_choice(lib):
         assert f(6, 2, d, 0) == 1 and f(4, 4, d, 0) == 1 and f(3, 1, d, 0) == 1
         assert f(16, 8, d, 1) == 1
         assert f(16, 8, d, 2) == (2 if d <= 128 else 1)
+        assert f(16, 8, d, 3) == 2 and f(6, 2, d, 3) == 1     # (variant 3, the decoupled kernel at head dim 128: items as for variant 0)
     assert f(0, 1, 128, 0) == 0 and f(5, 2, 128, 0) == 0      # not a head geometry
 
 
