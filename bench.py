@@ -49,7 +49,7 @@ WORKLOADS = {
 # HBM bytes per launch of the dominant kernel(s), from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE runs of this file (KiB per
 # dispatch), each scaled by what the same counter reads for `--workload copy` (whose traffic is known).  The figures and the
 # commands are in profiles/*_counters.md; a workload without a counter run has None.
-TRAFFIC_BYTES = {"C2": 786_454_852, "C2_512": 1_301_296_466, "C3": 55_747_249_459, "C4": 22_633_866_199, "C5": 8_754_360_320, "C5_prologue": 10_777_077_760, "C5_gate": 7_650_867_200,
+TRAFFIC_BYTES = {"C2": 786_454_852, "C2_512": 1_301_296_466, "C3": 49_766_912_684, "C4": 22_633_866_199, "C5": 8_754_360_320, "C5_prologue": 10_777_077_760, "C5_gate": 7_650_867_200,
                  "XDEC": 525_321_216, "XDEC_long": 2_324_807_680}
 
 

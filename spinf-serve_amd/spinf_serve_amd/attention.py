@@ -67,9 +67,10 @@ def _ring_lists(q, hq, hkv, d, variant, sidx, mask):
 
     Measured on MI355X: the decoupled kernel wins where a workgroup gets only a handful of items (C2: 6.75 per workgroup), since
     its waves run through the item boundaries; with many items per workgroup (C3's 65,536-token passes: 16) the lockstep kernel
-    is 6 - 10 % faster.  The lockstep kernel takes the static lists on sliding layers (5 % faster there than its queue) and its
-    queue on global layers (4 % faster).  SPINF_ATTN_RING / SPINF_ATTN_STATIC = 0 / 1 switch the two for every call where the
-    geometry allows, "auto" (the default) follows the measurements.  Head dim 128 has the decoupled kernel too (the library's
+    is 6 - 10 % faster.  The lockstep kernel takes its shared queues (measured over C3's 13 passes, the variants taking turns: sliding
+    layers 9.64 ms on the queues, 10.33 on static lists, 10.39 on the decoupled kernel; global layers 11.38 / 12.11 / 12.20).
+    SPINF_ATTN_RING / SPINF_ATTN_STATIC = 0 / 1 switch the two for every call where the geometry allows, "auto" (the default)
+    follows the measurements.  Head dim 128 has the decoupled kernel too (the library's
     variant 3, 64-key tiles): 55.5 against 48.5 ms on C4, so "auto" leaves it to the lockstep kernel (RING_128 or
     SPINF_ATTN_RING=1 select it)."""
     from .masks import _static_lists
@@ -80,7 +81,7 @@ def _ring_lists(q, hq, hkv, d, variant, sidx, mask):
         ring = d == 512 or (d == 256 and mask.plan.n_qtiles * (hq // 2) <= RING_MAX_ITEMS_PER_WG * n_wg) or (d == 128 and RING_128)
     elif not RING:
         ring = False
-    static = d != 512 and (int(mask.window) > 0 if STATIC < 0 else bool(STATIC))
+    static = d != 512 and STATIC > 0
     if ring or static:
         return n_wg, ring
     return 0, False
